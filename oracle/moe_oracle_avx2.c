@@ -1,0 +1,119 @@
+/*
+ * AVX2 inner loops of the CPU oracle.  TEST INFRASTRUCTURE ONLY.
+ *
+ * These restate the x86 vec_dot kernels the reference runs when it is built with
+ * `target-cpu=native` (its .cargo/config.toml:1-2):
+ *   vec_dot_q4_0_q8_0  candle-core/src/quantized/avx.rs:50-68
+ *   vec_dot_q8_0_q8_0  candle-core/src/quantized/avx.rs:71-87
+ *   vec_dot_q4k_q8k    candle-core/src/quantized/avx.rs:443-525
+ * The integer parts are exact; the f32 accumulation order differs from the scalar
+ * vec_dot_unopt, which the reference's own tests allow up to 1e-6 * k
+ * (candle-core/tests/quantized_tests.rs:869-876).  Used for the CPU-baseline timing.
+ */
+#include "moe_oracle.h"
+#include <immintrin.h>
+#include <math.h>
+#include <string.h>
+
+static inline float hsum_float_8(__m256 x) { /* avx.rs:26-32 */
+    __m128 res = _mm256_extractf128_ps(x, 1);
+    res = _mm_add_ps(res, _mm256_castps256_ps128(x));
+    res = _mm_add_ps(res, _mm_movehl_ps(res, res));
+    res = _mm_add_ss(res, _mm_movehdup_ps(res));
+    return _mm_cvtss_f32(res);
+}
+static inline __m256 mul_sum_i8_pairs_float(__m256i x, __m256i y) { /* avx.rs:12-24,43-48 */
+    __m256i ax = _mm256_sign_epi8(x, x);
+    __m256i sy = _mm256_sign_epi8(y, x);
+    __m256i dot = _mm256_maddubs_epi16(ax, sy);
+    __m256i summed = _mm256_madd_epi16(_mm256_set1_epi16(1), dot);
+    return _mm256_cvtepi32_ps(summed);
+}
+static inline __m256i bytes_from_nibbles_32(const uint8_t* p) { /* avx.rs:34-41 */
+    __m128i tmp = _mm_loadu_si128((const __m128i*)p);
+    __m256i bytes = _mm256_insertf128_si256(_mm256_castsi128_si256(tmp), _mm_srli_epi16(tmp, 4), 1);
+    return _mm256_and_si256(_mm256_set1_epi8(0xF), bytes);
+}
+
+static float dot_q4_0(int64_t n, const orc_block_q4_0* xs, const orc_block_q8_0* ys) {
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t b = 0; b < n / 32; b++) {
+        __m256 d = _mm256_set1_ps(orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d));
+        __m256i bx = _mm256_sub_epi8(bytes_from_nibbles_32(xs[b].qs), _mm256_set1_epi8(8));
+        __m256i by = _mm256_loadu_si256((const __m256i*)ys[b].qs);
+        acc = _mm256_fmadd_ps(d, mul_sum_i8_pairs_float(bx, by), acc);
+    }
+    return hsum_float_8(acc);
+}
+static float dot_q8_0(int64_t n, const orc_block_q8_0* xs, const orc_block_q8_0* ys) {
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t b = 0; b < n / 32; b++) {
+        __m256 d = _mm256_set1_ps(orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d));
+        __m256i bx = _mm256_loadu_si256((const __m256i*)xs[b].qs);
+        __m256i by = _mm256_loadu_si256((const __m256i*)ys[b].qs);
+        acc = _mm256_fmadd_ps(d, mul_sum_i8_pairs_float(bx, by), acc);
+    }
+    return hsum_float_8(acc);
+}
+static float dot_q4k(int64_t n, const orc_block_q4k* xs, const orc_block_q8k* ys) {
+    const uint32_t KMASK1 = 0x3f3f3f3f, KMASK2 = 0x0f0f0f0f, KMASK3 = 0x03030303;
+    const __m256i m4 = _mm256_set1_epi8(0xF);
+    __m256 acc = _mm256_setzero_ps();
+    __m128 acc_m = _mm_setzero_ps();
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q4k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        float d = y->d * orc_f16_to_f32(x->d);
+        float dmin = -y->d * orc_f16_to_f32(x->dmin);
+        uint32_t utmp[4];
+        memcpy(utmp, x->scales, 12);
+        utmp[3] = ((utmp[2] >> 4) & KMASK2) | (((utmp[1] >> 6) & KMASK3) << 4);
+        uint32_t uaux = utmp[1] & KMASK1;
+        utmp[1] = (utmp[2] & KMASK2) | (((utmp[0] >> 6) & KMASK3) << 4);
+        utmp[2] = uaux;
+        utmp[0] &= KMASK1;
+        const uint8_t* q4 = x->qs;
+        const int8_t* q8 = y->qs;
+        __m256i mins_and_scales = _mm256_cvtepu8_epi16(
+            _mm_set_epi32((int)utmp[3], (int)utmp[2], (int)utmp[1], (int)utmp[0]));
+        __m256i q8sums = _mm256_loadu_si256((const __m256i*)y->bsums);
+        __m128i q8s = _mm_hadd_epi16(_mm256_extracti128_si256(q8sums, 0), _mm256_extracti128_si256(q8sums, 1));
+        __m128i prod = _mm_madd_epi16(_mm256_extracti128_si256(mins_and_scales, 1), q8s);
+        acc_m = _mm_fmadd_ps(_mm_set1_ps(dmin), _mm_cvtepi32_ps(prod), acc_m);
+        __m128i sc128 = _mm256_extracti128_si256(mins_and_scales, 0);
+        __m256i scales = _mm256_set_m128i(sc128, sc128);
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < 4; j++) {
+            /* 16-bit scale 2j (resp. 2j+1) broadcast to every lane: bytes {2s, 2s+1} repeated */
+            __m256i shuf_l = _mm256_set1_epi16((short)(((4 * j + 1) << 8) | (4 * j)));
+            __m256i shuf_h = _mm256_set1_epi16((short)(((4 * j + 3) << 8) | (4 * j + 2)));
+            __m256i scale_l = _mm256_shuffle_epi8(scales, shuf_l);
+            __m256i scale_h = _mm256_shuffle_epi8(scales, shuf_h);
+            __m256i q4bits = _mm256_loadu_si256((const __m256i*)q4);
+            q4 += 32;
+            __m256i q4l = _mm256_and_si256(q4bits, m4);
+            __m256i q4h = _mm256_and_si256(_mm256_srli_epi16(q4bits, 4), m4);
+            __m256i q8l = _mm256_loadu_si256((const __m256i*)q8);
+            q8 += 32;
+            __m256i p16l = _mm256_madd_epi16(scale_l, _mm256_maddubs_epi16(q4l, q8l));
+            sumi = _mm256_add_epi32(sumi, p16l);
+            __m256i q8h = _mm256_loadu_si256((const __m256i*)q8);
+            q8 += 32;
+            __m256i p16h = _mm256_madd_epi16(scale_h, _mm256_maddubs_epi16(q4h, q8h));
+            sumi = _mm256_add_epi32(sumi, p16h);
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    acc_m = _mm_add_ps(acc_m, _mm_movehl_ps(acc_m, acc_m));
+    acc_m = _mm_add_ss(acc_m, _mm_movehdup_ps(acc_m));
+    return hsum_float_8(acc) + _mm_cvtss_f32(acc_m);
+}
+
+float orc_vec_dot_avx2(int dtype, int64_t n, const void* w, const void* a) {
+    switch (dtype) {
+        case ORC_Q4_0: return dot_q4_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
+        case ORC_Q8_0: return dot_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
+        case ORC_Q4K: return dot_q4k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        default: return orc_vec_dot(dtype, n, w, a);
+    }
+}

@@ -1,0 +1,216 @@
+"""Pins the CPU oracle's block formats against the reference's own known answers."""
+import numpy as np
+import pytest
+
+from rand09 import std_rng_f32
+
+
+def ramp(bound, size=1024):
+    # get_test_vector2, candle-core/tests/quantized_tests.rs:393-405
+    i = np.arange(size, dtype=np.float32)
+    return (i - np.float32(size / 2)) * np.float32(bound) / np.float32(size / 2)
+
+
+def ggml_like(offset, n=4096):
+    # create_ggml_like_vector, quantized_tests.rs:428-432 (f32 cos of an f32 argument)
+    i = np.arange(n, dtype=np.float32) + np.float32(offset)
+    return (np.float32(0.1) + np.float32(2.0) * np.cos(i, dtype=np.float32)).astype(np.float32)
+
+
+def test_f16_exhaustive(O):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([O.f16_to_f32(int(v)) for v in h], dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(got[np.isnan(want)]).all()
+    # every representable half converts back to itself
+    fin = ~np.isnan(want)
+    back = np.array([O.f32_to_f16(float(v)) for v in want[fin]], dtype=np.uint16)
+    assert np.array_equal(back, h[fin])
+
+
+def test_f32_to_f16_rounding(O):
+    rng = np.random.default_rng(7)
+    bits = rng.integers(0, 2**32, size=200000, dtype=np.uint64).astype(np.uint32)
+    # concentrate half of the samples around the f16 range incl. subnormals and ties
+    e = rng.integers(127 - 27, 127 + 17, size=100000).astype(np.uint32)
+    bits[:100000] = (bits[:100000] & np.uint32(0x807FFFFF)) | (e << np.uint32(23))
+    bits[:20000] &= np.uint32(0xFFFFF000)  # many exact ties
+    f = bits.view(np.float32)
+    f = f[~np.isnan(f)]
+    with np.errstate(over="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    got = np.array([O.f32_to_f16(float(v)) for v in f], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_q4_0_roundtrip_known_answer(O, golden):
+    src = np.arange(128, dtype=np.float32)
+    dst = O.dequantize(O.Q4_0, O.quantize(O.Q4_0, src), 128)
+    want = np.array(golden["q4_0_roundtrip_0_127"]["expected"], dtype=np.float32)
+    assert np.array_equal(dst.view(np.uint32), want.view(np.uint32))  # includes the two -0.0
+
+
+@pytest.mark.parametrize("simd", [False, True])
+def test_q4_0_matmul_known_answers(O, golden, simd):
+    m, k, n = 3, 64, 4
+    lhs = np.arange(m * k, dtype=np.float32).reshape(m, k)
+    rhs = np.arange(k * n, dtype=np.float32)
+    got = O.matmul(O.Q4_0, lhs, O.quantize(O.Q4_0, rhs), n, simd=simd)
+    assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_3_64_4"]["expected_rounded"]
+    lhs = (np.arange(m * k, dtype=np.float32) - np.float32(m * k / 2.0)).reshape(m, k)
+    rhs = np.arange(k * n, dtype=np.float32) - np.float32(k * n / 3.0)
+    got = O.matmul(O.Q4_0, lhs, O.quantize(O.Q4_0, rhs), n, simd=simd)
+    assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_neg_3_64_4"]["expected_rounded"]
+
+
+@pytest.mark.parametrize("name,dt", [("q4k_ramp", 12), ("q8k_ramp", 15)])
+def test_kquant_ramp_spot_values(O, golden, name, dt):
+    g = golden[name]
+    idx = golden["ramp_spot_indices"]
+    src = ramp(0.5)
+    assert src[idx].tolist() == np.array(golden["ramp_src_spot"]["expected"], dtype=np.float32).tolist()
+    dst = O.dequantize(dt, O.quantize(dt, src), 1024)
+    assert np.abs(dst - src).max() < g["max_abs_err_bound_0p5"]
+    got = (np.round(np.float32(1000.0) * dst[idx]) / np.float32(1000.0)).astype(np.float32)
+    assert got.tolist() == np.array(g["spot_rounded_3"], dtype=np.float32).tolist()
+    big = ramp(128.0)
+    dbig = O.dequantize(dt, O.quantize(dt, big), 1024)
+    assert np.abs(dbig - big).max() < g["max_abs_err_bound_128"]
+
+
+@pytest.mark.parametrize("dt", [2, 8, 12, 15])
+def test_ggml_quantization_rmse(O, golden, dt):
+    src = ggml_like(0.0)
+    dst = O.dequantize(dt, O.quantize(dt, src), src.size)
+    rmse = np.sqrt(np.sum((src - dst).astype(np.float32) ** 2, dtype=np.float32)) / src.size
+    assert rmse <= golden["ggml_quantization_rmse_bound"]["bound"]
+
+
+@pytest.mark.parametrize("dt", [2, 8, 12, 15])
+def test_ggml_dot_error(O, golden, dt):
+    # ggml_matmul_error_test, quantized_tests.rs:846-911
+    g = golden["ggml_dot_error"]
+    n = 4096
+    cases = [(ggml_like(0.0), ggml_like(1.0), 1.0),
+             (np.arange(n, dtype=np.float32) / np.float32(n), np.arange(n, dtype=np.float32) / np.float32(n), 2.0)]
+    for a, b, err_m in cases:
+        aq = O.quantize(dt, a)
+        bq = O.quantize(O.VECDOT[dt], b)
+        r_unopt = O.vec_dot(dt, n, aq, bq)
+        r_opt = O.vec_dot(dt, n, aq, bq, simd=True)
+        assert abs(r_opt - r_unopt) / n <= 1e-6
+        r_mm = float(O.matmul(dt, b.reshape(1, n), aq, 1)[0, 0])
+        assert abs(r_mm - r_unopt) / n <= 1e-6
+        ref = float(np.sum(a * b, dtype=np.float32))
+        for r in (r_unopt, r_opt, r_mm):
+            err = abs(r - ref) / n
+            assert err <= g["max_dot_product_error"]
+            assert err - g["leniency"] <= g["reference_error"][str(dt)] * err_m
+
+
+def test_vec_dot_matches_dequantised_float64(O):
+    # brute force: the integer block dot must equal the float dot of the dequantised operands
+    rng = np.random.default_rng(3)
+    n = 2048
+    for dt in (O.Q4_0, O.Q8_0, O.Q4K):
+        w = rng.normal(0, 0.02, n).astype(np.float32)
+        x = rng.normal(0, 1.0, n).astype(np.float32)
+        wq, xq = O.quantize(dt, w), O.quantize(O.VECDOT[dt], x)
+        wd = O.dequantize(dt, wq, n).astype(np.float64)
+        xd = O.dequantize(O.VECDOT[dt], xq, n).astype(np.float64)
+        want = float(wd @ xd)
+        for simd in (False, True):
+            got = O.vec_dot(dt, n, wq, xq, simd=simd)
+            assert abs(got - want) <= 2e-5 * np.sqrt(n) * np.abs(wd).max() * np.abs(xd).max() * 8
+
+
+@pytest.mark.parametrize("simd", [False, True])
+def test_seeded_matmul_spot_values(O, golden, simd):
+    g = golden["seeded_matmul_11_512_21"]
+    m, k, n = 11, 512, 21
+    v = std_rng_f32(g["seed"], (m + n) * k)
+    lhs = (v[: m * k] - np.float32(0.5)).reshape(m, k)
+    rhs = (v[m * k:] - np.float32(0.5)).reshape(n, k)
+    pick = [0, m * n // 3, m * n * 2 // 3, m * n - 1]
+    r3 = lambda a: [float(np.round(np.float32(1000.0) * np.float32(x)) / np.float32(1000.0)) for x in a]
+    dense = (lhs.astype(np.float64) @ rhs.astype(np.float64).T).reshape(-1)
+    assert r3(dense[pick]) == r3(g["dense"])  # validates the StdRng restatement itself
+    for key, dt in (("q4k", O.Q4K), ("q8k", O.Q8K)):
+        mm = O.matmul(dt, lhs, O.quantize(dt, rhs), n, simd=simd).reshape(-1)
+        assert r3(mm[pick]) == r3(g[key])
+
+
+def test_matmul_batch_invariance_and_threads(O):
+    # qmm_batch, quantized_tests.rs:221-256: identical rows give identical outputs at any batch
+    rng = np.random.default_rng(11)
+    k, n = 512, 300
+    w = O.quantize(O.Q4K, rng.normal(0, 0.02, (n, k)).astype(np.float32))
+    lhs = rng.normal(0, 1, (2, k)).astype(np.float32)
+    mm = O.matmul(O.Q4K, lhs, w, n)
+    mm6 = O.matmul(O.Q4K, np.concatenate([lhs] * 3), w, n, threads=4)
+    assert np.array_equal(mm6[2:4], mm) and np.array_equal(mm6[4:], mm)
+
+
+def test_q8_quantizer_closed_forms(O):
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 1, 256).astype(np.float32)
+    x[17] = -4.5  # largest magnitude is negative: Q8K must map it to +... -128*-1 -> clipped 127? no: iscale=-128/max
+    b = O.quantize(O.Q8K, x)
+    d = b[:4].view(np.float32)[0]
+    qs = b[4:260].view(np.int8)
+    bs = b[260:].view(np.int16)
+    iscale = np.float32(-128.0) / np.float32(-4.5)
+    assert d == np.float32(1.0) / iscale
+    assert qs[17] == -128
+    want = np.minimum(np.sign(iscale * x) * np.floor(np.abs(iscale * x) + np.float32(0.5)), 127).astype(np.int8)
+    assert np.array_equal(qs, want)
+    assert np.array_equal(bs, qs.astype(np.int32).reshape(16, 16).sum(1).astype(np.int16))
+    # positive maximum: the maximum itself would be -128*... = -128 -> stays in range, others clip at 127
+    x2 = -x
+    q2 = O.quantize(O.Q8K, x2)[4:260].view(np.int8)
+    assert q2[17] == -128 and q2.max() <= 127
+    # Q8_0: d = amax/127 stored as f16, quants use the unrounded f32 reciprocal
+    y = rng.normal(0, 1, 32).astype(np.float32)
+    b0 = O.quantize(O.Q8_0, y)
+    d32 = np.abs(y).max() / np.float32(127.0)
+    assert b0[:2].view(np.float16)[0] == np.float16(d32)
+    idv = np.float32(1.0) / d32
+    t = y * idv
+    want0 = (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).astype(np.int8)
+    assert np.array_equal(b0[2:].view(np.int8), want0)
+    # all-zero blocks
+    assert not O.quantize(O.Q8K, np.zeros(256, np.float32)).any()
+    assert not O.quantize(O.Q8_0, np.zeros(32, np.float32)).any()
+    z4 = O.quantize(O.Q4_0, np.zeros(32, np.float32))  # d = 0/-8 = -0.0, every nibble 8
+    assert z4[:2].view(np.uint16)[0] == 0x8000 and (z4[2:] == 0x88).all()
+
+
+def test_q4k_layout_against_independent_decoder(O):
+    # independent numpy decoder of the published Q4_K layout (d, dmin, 12 packed 6-bit scale/min bytes,
+    # 128 nibble bytes: byte l of each 32-byte group holds element l (low) and l+32 (high))
+    rng = np.random.default_rng(9)
+    x = rng.normal(0, 0.02, 1024).astype(np.float32)
+    blocks = O.quantize(O.Q4K, x).reshape(4, 144)
+    out = np.empty((4, 256), dtype=np.float32)
+    for b in range(4):
+        raw = blocks[b]
+        d = np.float32(raw[0:2].view(np.float16)[0])
+        dmin = np.float32(raw[2:4].view(np.float16)[0])
+        s = raw[4:16].astype(np.int32)
+        sc = np.zeros(8, np.int32)
+        mn = np.zeros(8, np.int32)
+        for j in range(8):
+            if j < 4:
+                sc[j], mn[j] = s[j] & 63, s[j + 4] & 63
+            else:
+                sc[j] = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4)
+                mn[j] = (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+        qs = raw[16:].reshape(4, 32)
+        for g in range(4):
+            lo = (qs[g] & 0xF).astype(np.float32)
+            hi = (qs[g] >> 4).astype(np.float32)
+            out[b, 64 * g: 64 * g + 32] = (d * np.float32(sc[2 * g])) * lo - dmin * np.float32(mn[2 * g])
+            out[b, 64 * g + 32: 64 * g + 64] = (d * np.float32(sc[2 * g + 1])) * hi - dmin * np.float32(mn[2 * g + 1])
+    got = O.dequantize(O.Q4K, blocks.reshape(-1), 1024)
+    assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
