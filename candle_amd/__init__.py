@@ -1,0 +1,11 @@
+"""MI355X (gfx950) implementation of candle's quantized sparse-MoE block.
+
+The product is the C-ABI shared library ``candle_amd/lib/libcandle_amd_moe.so`` (HIP kernels,
+declared in ``include/candle_amd_moe.h``).  This package is a thin ctypes front end over it whose
+classes mirror the names of the reference (``MlpOrMoe``/``SparseMoeBlock`` with ``forward``).
+There is no CPU fallback: every call fails if the library or a gfx950 device is missing.
+"""
+from .moe import (  # noqa: F401
+    GGML_Q4_0, GGML_Q8_0, GGML_Q4K, GGML_Q8K, MoeError, SparseMoeBlock, MlpOrMoe,
+    dequantize, quantize_act, route, qmatmul, device_arch, debug_expf, lib_path, load_library,
+)

@@ -1,0 +1,79 @@
+// Wave-level activation quantisers.  They restate, per block, exactly what candle's
+// k_quants::matmul applies to every lhs row before the integer dot products:
+//   BlockQ8K::from_float   candle-core/src/quantized/k_quants.rs:1819-1856
+//   BlockQ8_0::from_float  candle-core/src/quantized/k_quants.rs:605-634
+// so the int8 operands are bit-identical to the CPU path's.
+#pragma once
+#include "moe_common.hpp"
+
+namespace moe {
+
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Byte offset of element k (0..K) inside a Q8K-quantised activation row (see moe_common.hpp).
+__host__ __device__ inline int q8k_act_offset(int k) {
+    return (k / 64) * 64 + ((k % 32) / 8) * 16 + ((k / 32) % 2) * 8 + (k % 8);
+}
+
+// One wave quantises one 256-element block; lane l holds elements 4l..4l+3 in v.
+//   qs_block : the block's 256 quant bytes (device layout), d_out / bs_out: scale and 16 bsums.
+__device__ inline void quantize_q8k_block(float4 v, int lane, int8_t* qs_block, float* d_out, __half* bs_out) {
+    // first element of largest magnitude, scanning in index order with a strict '<'
+    float amax = 0.f, mx = 0.f;
+    float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float a = fabsf(e[i]);
+        if (amax < a) { amax = a; mx = e[i]; }
+    }
+    float wmax = wave_max(amax);
+    if (wmax == 0.f) {
+        *reinterpret_cast<uint32_t*>(qs_block + q8k_act_offset(4 * lane)) = 0u;
+        if (lane == 0) *d_out = 0.f;
+        if (lane < 16) bs_out[lane] = __float2half(0.f);
+        return;
+    }
+    unsigned long long winners = __ballot(amax == wmax);
+    int first = __ffsll((long long)winners) - 1;
+    float max = __shfl(mx, first, 64);
+    float iscale = -128.0f / max;
+    int sum = 0;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float r = roundf(iscale * e[i]);
+        int q = sat_i8(fminf(r, 127.f));
+        sum += q;
+        packed |= (uint32_t)(uint8_t)q << (8 * i);
+    }
+    *reinterpret_cast<uint32_t*>(qs_block + q8k_act_offset(4 * lane)) = packed;
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    if ((lane & 3) == 0) bs_out[lane >> 2] = __int2half_rn(sum);
+    if (lane == 0) *d_out = 1.0f / iscale;
+}
+
+// Half a wave (32 lanes) quantises one 32-element block; lane holds element (lane & 31).
+//   q_out: the element's quant byte; d_out: f16-rounded scale widened to f32; bsum_out: sum of quants.
+__device__ inline void quantize_q8_0_block(float x, int lane, int8_t* q_out, float* d_out, int32_t* bsum_out) {
+    float amax = fabsf(x);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    float d = amax / 127.0f;
+    float id = (d != 0.f) ? 1.0f / d : 0.f;
+    int q = sat_i8(roundf(x * id));
+    *q_out = (int8_t)q;
+    int sum = q;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    if ((lane & 31) == 0) {
+        *d_out = __half2float(__float2half_rn(d));
+        *bsum_out = sum;
+    }
+}
+
+}  // namespace moe

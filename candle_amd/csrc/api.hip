@@ -1,0 +1,510 @@
+// C ABI of the library (see include/candle_amd_moe.h): layer objects, device memory and the
+// sequence of kernel launches of one forward pass.
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "kernels.hpp"
+
+namespace moe {
+
+static thread_local std::string g_err;
+void set_error(int, const std::string& msg) { g_err = msg; }
+int fail(int code, const std::string& msg) {
+    g_err = msg;
+    return code;
+}
+
+static std::once_flag g_dev_once;
+static int g_dev_rc = MOE_E_NODEVICE;
+static std::string g_dev_msg, g_arch;
+
+int ensure_device() {
+    std::call_once(g_dev_once, [] {
+        int n = 0;
+        hipError_t e = hipGetDeviceCount(&n);
+        if (e != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            g_dev_msg = std::string("no HIP device visible (") + (e != hipSuccess ? hipGetErrorString(e) : "device count 0") +
+                        "); this library has no CPU fallback";
+            g_dev_rc = MOE_E_NODEVICE;
+            return;
+        }
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) {
+            g_dev_msg = std::string("hipGetDeviceProperties: ") + hipGetErrorString(e);
+            g_dev_rc = MOE_E_HIP;
+            return;
+        }
+        g_arch = prop.gcnArchName;
+        if (g_arch.rfind("gfx950", 0) != 0) {
+            g_dev_msg = "device architecture is " + g_arch + "; the kernels are built for gfx950 only";
+            g_dev_rc = MOE_E_NODEVICE;
+            return;
+        }
+        g_dev_rc = MOE_OK;
+    });
+    if (g_dev_rc != MOE_OK) g_err = g_dev_msg;
+    return g_dev_rc;
+}
+
+// ------------------------------------------------------------------ device buffers
+struct DevBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    DevBuf() = default;
+    DevBuf(const DevBuf&) = delete;
+    DevBuf& operator=(const DevBuf&) = delete;
+    int reserve(size_t bytes) {
+        if (bytes <= cap) return MOE_OK;
+        if (p) MOE_HIP_CHECK(hipFree(p));
+        p = nullptr;
+        cap = 0;
+        size_t want = std::max<size_t>(bytes, 256);
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) {
+            p = nullptr;
+            return fail(MOE_E_NOMEM, std::string("hipMalloc(") + std::to_string(want) + "): " + hipGetErrorString(e));
+        }
+        cap = want;
+        return MOE_OK;
+    }
+    template <typename T>
+    T* as() const { return reinterpret_cast<T*>(p); }
+};
+
+struct ActStore {
+    DevBuf qs, d, bsum;
+    int reserve(int vdt, int64_t rows, int64_t k) {
+        int rc;
+        if ((rc = qs.reserve(act_qs_bytes(rows, k)))) return rc;
+        if ((rc = d.reserve(act_d_bytes(vdt, rows, k)))) return rc;
+        return bsum.reserve(act_bsum_bytes(vdt, rows, k));
+    }
+    ActBuf view() const {
+        ActBuf a;
+        a.qs = qs.as<int8_t>();
+        a.d = d.as<float>();
+        a.bsum = bsum.p;
+        return a;
+    }
+};
+
+struct RouteStore {
+    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots, counter;
+    int reserve(int64_t T, int E, int k, bool shared) {
+        int rc;
+        const int64_t S = T * k + (shared ? T : 0);
+        if ((rc = logits.reserve((size_t)T * E * 4))) return rc;
+        if ((rc = topk_idx.reserve((size_t)T * k * 4))) return rc;
+        if ((rc = topk_w.reserve((size_t)T * k * 4))) return rc;
+        if ((rc = shared_w.reserve((size_t)T * 4))) return rc;
+        if ((rc = offsets.reserve((size_t)(E + 2) * 4))) return rc;
+        if ((rc = perm_token.reserve((size_t)S * 4))) return rc;
+        if ((rc = perm_w.reserve((size_t)S * 4))) return rc;
+        if ((rc = tok_slots.reserve((size_t)T * (k + 1) * 4))) return rc;
+        if (!counter.p) {
+            if ((rc = counter.reserve(256))) return rc;
+            MOE_HIP_CHECK(hipMemset(counter.p, 0, 256));
+        }
+        return MOE_OK;
+    }
+    RouteBufs view() const {
+        RouteBufs r;
+        r.logits = logits.as<float>();
+        r.topk_idx = topk_idx.as<int32_t>();
+        r.topk_w = topk_w.as<float>();
+        r.shared_w = shared_w.as<float>();
+        r.offsets = offsets.as<int32_t>();
+        r.perm_token = perm_token.as<int32_t>();
+        r.perm_w = perm_w.as<float>();
+        r.tok_slots = tok_slots.as<int32_t>();
+        r.counter = counter.as<uint32_t>();
+        return r;
+    }
+};
+
+}  // namespace moe
+
+using namespace moe;
+
+struct moe_layer {
+    int64_t H = 0, F = 0, E = 0, k = 0, Fs = 0;
+    int dt = 0, vdt = 0, norm_topk = 1;
+    bool has_bias = false, has_rms = false;
+    float rms_eps = 0.f;
+    DevBuf weights;                 // all re-laid expert matrices
+    DevBuf gate, gate_bias, shared_gate, rms_alpha, groups;
+    std::vector<GroupWeights> host_groups;  // E routed (+1 shared)
+    // per-call workspace, grown on demand
+    std::mutex mu;
+    int64_t cap_T = -1;
+    RouteStore route;
+    ActStore xq, hq, hq_shared;
+    DevBuf yw, x_dev, y_dev;
+    hipStream_t stream = nullptr;   // used by the host-pointer entry
+    hipEvent_t done = nullptr;      // end of the last enqueued forward
+    int64_t last_T = 0;
+};
+
+static int reserve_workspace(moe_layer* L, int64_t T) {
+    if (T <= L->cap_T) return MOE_OK;
+    int rc;
+    const bool shared = L->Fs > 0;
+    const int64_t S = T * L->k + (shared ? T : 0);
+    if ((rc = L->route.reserve(T, (int)L->E, (int)L->k, shared))) return rc;
+    if ((rc = L->xq.reserve(L->vdt, T, L->H))) return rc;
+    if ((rc = L->hq.reserve(L->vdt, T * L->k, L->F))) return rc;
+    if (shared && (rc = L->hq_shared.reserve(L->vdt, T, L->Fs))) return rc;
+    if ((rc = L->yw.reserve((size_t)S * L->H * 4))) return rc;
+    L->cap_T = T;
+    return MOE_OK;
+}
+
+static int check_desc(const moe_desc* d) {
+    if (!d) return fail(MOE_E_INVALID, "desc is NULL");
+    const int dt = d->ggml_dtype;
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
+        return fail(MOE_E_INVALID, "unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q4K=12)");
+    const int64_t be = block_elems(dt);
+    if (d->hidden <= 0 || d->ffn <= 0) return fail(MOE_E_INVALID, "hidden and ffn must be positive");
+    // the reference rejects a last dimension that is not a multiple of the block size
+    // (candle-core/src/quantized/mod.rs:310-322)
+    if (d->hidden % be || d->ffn % be)
+        return fail(MOE_E_INVALID, "hidden and ffn must be multiples of the block size " + std::to_string(be));
+    if (d->hidden % 16 || d->ffn % 32) return fail(MOE_E_INVALID, "hidden must be a multiple of 16 and ffn of 32");
+    if (d->hidden > 16384) return fail(MOE_E_INVALID, "hidden > 16384 is not supported");
+    if (d->n_experts < 1 || d->n_experts > 256) return fail(MOE_E_INVALID, "n_experts must be in 1..256");
+    // top_k = 0 makes the reference return zeros (quantized_llama.rs:507-512 defaults the key to 0);
+    // that degenerate case is rejected here rather than silently reproduced
+    if (d->top_k < 1 || d->top_k > d->n_experts || d->top_k > 16)
+        return fail(MOE_E_INVALID, "top_k must be in 1..min(n_experts,16)");
+    if (!d->gate || !d->w1 || !d->w2 || !d->w3) return fail(MOE_E_INVALID, "gate, w1, w2, w3 must be set");
+    for (int64_t e = 0; e < d->n_experts; e++)
+        if (!d->w1[e] || !d->w2[e] || !d->w3[e]) return fail(MOE_E_INVALID, "expert " + std::to_string(e) + " has a NULL matrix");
+    if (d->shared_ffn < 0) return fail(MOE_E_INVALID, "shared_ffn < 0");
+    if (d->shared_ffn > 0) {
+        if (d->shared_ffn % be || d->shared_ffn % 32) return fail(MOE_E_INVALID, "shared_ffn must be a multiple of the block size and of 32");
+        if (!d->shared_w1 || !d->shared_w2 || !d->shared_w3 || !d->shared_gate)
+            return fail(MOE_E_INVALID, "shared expert needs shared_w1, shared_w2, shared_w3 and shared_gate");
+    }
+    return MOE_OK;
+}
+
+static int upload_f32(DevBuf& b, const float* src, size_t n) {
+    int rc = b.reserve(n * 4);
+    if (rc) return rc;
+    MOE_HIP_CHECK(hipMemcpy(b.p, src, n * 4, hipMemcpyHostToDevice));
+    return MOE_OK;
+}
+
+extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
+    if (!out) return fail(MOE_E_INVALID, "out is NULL");
+    *out = nullptr;
+    int rc = ensure_device();
+    if (rc) return rc;
+    if ((rc = check_desc(d))) return rc;
+    moe_layer* L = new moe_layer();
+    auto bail = [&](int code) {
+        moe_layer_destroy(L);
+        return code;
+    };
+    L->H = d->hidden; L->F = d->ffn; L->E = d->n_experts; L->k = d->top_k; L->Fs = d->shared_ffn;
+    L->dt = d->ggml_dtype; L->vdt = vecdot_dtype(L->dt); L->norm_topk = d->norm_topk ? 1 : 0;
+    L->rms_eps = d->rms_eps;
+    if ((rc = upload_f32(L->gate, d->gate, (size_t)L->E * L->H))) return bail(rc);
+    if (d->gate_bias) {
+        L->has_bias = true;
+        if ((rc = upload_f32(L->gate_bias, d->gate_bias, (size_t)L->E))) return bail(rc);
+    }
+    if (L->Fs > 0 && (rc = upload_f32(L->shared_gate, d->shared_gate, (size_t)L->H))) return bail(rc);
+    if (d->rms_alpha) {
+        L->has_rms = true;
+        if ((rc = upload_f32(L->rms_alpha, d->rms_alpha, (size_t)L->H))) return bail(rc);
+    }
+    // one allocation for all matrices
+    const size_t mat = (size_t)relaid_bytes(L->dt, L->F, L->H);      // w1/w3: [F,H]; w2: [H,F] has the same size
+    const size_t smat = L->Fs ? (size_t)relaid_bytes(L->dt, L->Fs, L->H) : 0;
+    const size_t total = mat * 3 * L->E + smat * 3;
+    if ((rc = L->weights.reserve(total))) return bail(rc);
+    const size_t raw_mat = (size_t)(L->F * L->H / block_elems(L->dt) * block_bytes(L->dt));
+    const size_t raw_smat = (size_t)(L->Fs * L->H / block_elems(L->dt) * block_bytes(L->dt));
+    DevBuf staging;
+    if ((rc = staging.reserve(std::max(raw_mat, raw_smat)))) return bail(rc);
+    uint8_t* wbase = L->weights.as<uint8_t>();
+    size_t off = 0;
+    auto put = [&](const void* src, size_t raw_bytes, int64_t rows, int64_t cols, const uint8_t** dst) -> int {
+        hipError_t e = hipMemcpy(staging.p, src, raw_bytes, hipMemcpyHostToDevice);
+        if (e != hipSuccess) return fail(MOE_E_HIP, std::string("hipMemcpy(weights): ") + hipGetErrorString(e));
+        e = launch_relayout(L->dt, staging.as<uint8_t>(), wbase + off, rows, cols, nullptr);
+        if (e == hipSuccess) e = hipDeviceSynchronize();
+        if (e != hipSuccess) return fail(MOE_E_HIP, std::string("relayout: ") + hipGetErrorString(e));
+        *dst = wbase + off;
+        off += (size_t)relaid_bytes(L->dt, rows, cols);
+        return MOE_OK;
+    };
+    L->host_groups.resize(L->E + (L->Fs ? 1 : 0));
+    for (int64_t e = 0; e < L->E; e++) {
+        GroupWeights& g = L->host_groups[e];
+        if ((rc = put(d->w1[e], raw_mat, L->F, L->H, &g.w1))) return bail(rc);
+        if ((rc = put(d->w3[e], raw_mat, L->F, L->H, &g.w3))) return bail(rc);
+        if ((rc = put(d->w2[e], raw_mat, L->H, L->F, &g.w2))) return bail(rc);
+    }
+    if (L->Fs) {
+        GroupWeights& g = L->host_groups[L->E];
+        if ((rc = put(d->shared_w1, raw_smat, L->Fs, L->H, &g.w1))) return bail(rc);
+        if ((rc = put(d->shared_w3, raw_smat, L->Fs, L->H, &g.w3))) return bail(rc);
+        if ((rc = put(d->shared_w2, raw_smat, L->H, L->Fs, &g.w2))) return bail(rc);
+    }
+    if ((rc = L->groups.reserve(L->host_groups.size() * sizeof(GroupWeights)))) return bail(rc);
+    hipError_t e = hipMemcpy(L->groups.p, L->host_groups.data(), L->host_groups.size() * sizeof(GroupWeights), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&L->done, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        fail(MOE_E_HIP, std::string("layer setup: ") + hipGetErrorString(e));
+        return bail(MOE_E_HIP);
+    }
+    *out = L;
+    return MOE_OK;
+}
+
+extern "C" void moe_layer_destroy(moe_layer* L) {
+    if (!L) return;
+    (void)hipDeviceSynchronize();
+    if (L->stream) (void)hipStreamDestroy(L->stream);
+    if (L->done) (void)hipEventDestroy(L->done);
+    delete L;
+}
+
+// Enqueue one forward on `s`.  Caller holds L->mu.
+static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s) {
+    int rc = reserve_workspace(L, T);
+    if (rc) return rc;
+    // a previous call may still be running on another stream and shares the workspace
+    MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
+    const bool shared = L->Fs > 0;
+    FrontParams fp;
+    fp.x = d_x; fp.T = T; fp.H = (int)L->H; fp.E = (int)L->E; fp.k = (int)L->k; fp.norm_topk = L->norm_topk;
+    fp.gate = L->gate.as<float>();
+    fp.gate_bias = L->has_bias ? L->gate_bias.as<float>() : nullptr;
+    fp.shared_gate = shared ? L->shared_gate.as<float>() : nullptr;
+    fp.rms_alpha = L->has_rms ? L->rms_alpha.as<float>() : nullptr;
+    fp.rms_eps = L->rms_eps;
+    fp.vdt = L->vdt;
+    fp.xq = L->xq.view();
+    fp.rb = L->route.view();
+    MOE_HIP_CHECK(launch_front(fp, s));
+
+    ExpertParams ep;
+    ep.dt = L->dt; ep.H = (int)L->H; ep.F = (int)L->F;
+    ep.n_groups = (int)L->E; ep.group0 = 0;
+    ep.groups = L->groups.as<GroupWeights>();
+    ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = L->hq.view(); ep.slot_origin = 0;
+    ep.yw = L->yw.as<float>();
+    ep.max_rows = T;
+    ep.slot_tiles = (T * L->k > 9 * L->E) ? 2 : 1;   // expected rows per expert above ~9: carry 32 slots per pass
+    MOE_HIP_CHECK(launch_expert_up(ep, s));
+    MOE_HIP_CHECK(launch_expert_down(ep, s));
+    if (shared) {
+        ExpertParams sp = ep;
+        sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E;
+        sp.groups = L->groups.as<GroupWeights>() + L->E;
+        sp.hq = L->hq_shared.view(); sp.slot_origin = (int)(T * L->k);
+        sp.max_rows = T; sp.slot_tiles = T > 16 ? 2 : 1;
+        MOE_HIP_CHECK(launch_expert_up(sp, s));
+        MOE_HIP_CHECK(launch_expert_down(sp, s));
+    }
+    MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb.tok_slots, (int)L->k + (shared ? 1 : 0),
+                                 L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    MOE_HIP_CHECK(hipEventRecord(L->done, s));
+    L->last_T = T;
+    return MOE_OK;
+}
+
+extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream) {
+    if (!L || T < 0 || (T > 0 && (!d_x || !d_y))) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_device");
+    if (d_x == d_y && T > 0) return fail(MOE_E_INVALID, "d_x and d_y must not alias");
+    if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (T == 0) { L->last_T = 0; return MOE_OK; }
+    return enqueue_forward(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int moe_layer_forward(moe_layer* L, const float* x, int64_t T, float* y) {
+    if (!L || T < 0 || (T > 0 && (!x || !y))) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward");
+    if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (T == 0) { L->last_T = 0; return MOE_OK; }
+    int rc;
+    const size_t bytes = (size_t)T * L->H * 4;
+    if ((rc = L->x_dev.reserve(bytes))) return rc;
+    if ((rc = L->y_dev.reserve(bytes))) return rc;
+    MOE_HIP_CHECK(hipMemcpyAsync(L->x_dev.p, x, bytes, hipMemcpyHostToDevice, L->stream));
+    if ((rc = enqueue_forward(L, L->x_dev.as<float>(), T, L->y_dev.as<float>(), L->stream))) return rc;
+    MOE_HIP_CHECK(hipMemcpyAsync(y, L->y_dev.p, bytes, hipMemcpyDeviceToHost, L->stream));
+    MOE_HIP_CHECK(hipStreamSynchronize(L->stream));
+    return MOE_OK;
+}
+
+static int d2h(void* dst, const void* src, size_t bytes) {
+    if (!dst || bytes == 0) return MOE_OK;
+    MOE_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return MOE_OK;
+}
+
+extern "C" int moe_layer_last_logits(moe_layer* L, float* logits, int64_t T) {
+    if (!L || !logits) return fail(MOE_E_INVALID, "bad argument to moe_layer_last_logits");
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
+    MOE_HIP_CHECK(hipEventSynchronize(L->done));
+    return d2h(logits, L->route.logits.p, (size_t)T * L->E * 4);
+}
+
+extern "C" int moe_layer_last_routing(moe_layer* L, int64_t T, int32_t* topk_idx, float* topk_w, int32_t* offsets,
+                                      int32_t* perm_token, float* perm_w) {
+    if (!L) return fail(MOE_E_INVALID, "layer is NULL");
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
+    MOE_HIP_CHECK(hipEventSynchronize(L->done));
+    int rc;
+    const size_t A = (size_t)T * L->k;
+    if ((rc = d2h(topk_idx, L->route.topk_idx.p, A * 4))) return rc;
+    if ((rc = d2h(topk_w, L->route.topk_w.p, A * 4))) return rc;
+    if ((rc = d2h(offsets, L->route.offsets.p, (size_t)(L->E + 1) * 4))) return rc;
+    if ((rc = d2h(perm_token, L->route.perm_token.p, A * 4))) return rc;
+    return d2h(perm_w, L->route.perm_w.p, A * 4);
+}
+
+extern "C" int moe_layer_dequantize_weight(moe_layer* L, int64_t expert, int which, float* out, int64_t n_elems) {
+    if (!L || !out) return fail(MOE_E_INVALID, "bad argument to moe_layer_dequantize_weight");
+    if (expert < 0 || expert >= (int64_t)L->host_groups.size() || which < 1 || which > 3)
+        return fail(MOE_E_INVALID, "expert / which out of range");
+    const int64_t F = expert == L->E ? L->Fs : L->F;
+    const int64_t rows = which == 2 ? L->H : F, cols = which == 2 ? F : L->H;
+    if (n_elems != rows * cols) return fail(MOE_E_INVALID, "n_elems must be rows*cols = " + std::to_string(rows * cols));
+    const GroupWeights& g = L->host_groups[expert];
+    const uint8_t* src = which == 1 ? g.w1 : which == 2 ? g.w2 : g.w3;
+    DevBuf tmp;
+    int rc = tmp.reserve((size_t)n_elems * 4);
+    if (rc) return rc;
+    MOE_HIP_CHECK(launch_dequant_tiled(L->dt, src, tmp.as<float>(), rows, cols, nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(out, tmp.p, (size_t)n_elems * 4);
+}
+
+extern "C" int moe_route(const float* logits, int64_t T, int64_t E, int64_t k, int32_t norm_topk, int32_t* topk_idx,
+                         float* topk_w, int32_t* offsets, int32_t* perm_token, float* perm_w) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if (T < 0 || E < 1 || E > 256 || k < 1 || k > E || k > 16) return fail(MOE_E_INVALID, "moe_route: need 1<=E<=256, 1<=k<=min(E,16)");
+    if (T > 0 && !logits) return fail(MOE_E_INVALID, "logits is NULL");
+    if (T == 0) {
+        if (offsets) std::memset(offsets, 0, (size_t)(E + 1) * 4);
+        return MOE_OK;
+    }
+    RouteStore rs;
+    DevBuf dl;
+    if ((rc = rs.reserve(T, (int)E, (int)k, false))) return rc;
+    if ((rc = dl.reserve((size_t)T * E * 4))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(dl.p, logits, (size_t)T * E * 4, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_route_from_logits(dl.as<float>(), T, (int)E, (int)k, norm_topk ? 1 : 0, rs.view(), nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    const size_t A = (size_t)T * k;
+    if ((rc = d2h(topk_idx, rs.topk_idx.p, A * 4))) return rc;
+    if ((rc = d2h(topk_w, rs.topk_w.p, A * 4))) return rc;
+    if ((rc = d2h(offsets, rs.offsets.p, (size_t)(E + 1) * 4))) return rc;
+    if ((rc = d2h(perm_token, rs.perm_token.p, A * 4))) return rc;
+    return d2h(perm_w, rs.perm_w.p, A * 4);
+}
+
+extern "C" int moe_dequantize(int32_t dt, const void* blocks, int64_t n, float* out) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    const int64_t be = block_elems(dt);
+    if (be < 0) return fail(MOE_E_INVALID, "moe_dequantize: unsupported dtype " + std::to_string(dt));
+    if (n < 0 || n % be) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
+    if (n == 0) return MOE_OK;
+    if (!blocks || !out) return fail(MOE_E_INVALID, "NULL pointer");
+    DevBuf src, dst;
+    const size_t bytes = (size_t)(n / be * block_bytes(dt));
+    if ((rc = src.reserve(bytes))) return rc;
+    if ((rc = dst.reserve((size_t)n * 4))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(src.p, blocks, bytes, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_dequant_std(dt, src.as<uint8_t>(), dst.as<float>(), n, nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(out, dst.p, (size_t)n * 4);
+}
+
+extern "C" int moe_quantize_act(int32_t vdt, const float* x, int64_t rows, int64_t k, void* out) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if (vdt != MOE_GGML_Q8_0 && vdt != MOE_GGML_Q8K) return fail(MOE_E_INVALID, "vecdot_dtype must be Q8_0 (8) or Q8K (15)");
+    const int64_t be = block_elems(vdt);
+    if (rows < 0 || k <= 0 || k % be || k > (1 << 24)) return fail(MOE_E_INVALID, "k must be a positive multiple of the block size");
+    if (rows == 0) return MOE_OK;
+    if (!x || !out) return fail(MOE_E_INVALID, "NULL pointer");
+    DevBuf dx, dout;
+    ActStore as;
+    const size_t out_bytes = (size_t)(rows * k / be * block_bytes(vdt));
+    if ((rc = dx.reserve((size_t)rows * k * 4))) return rc;
+    if ((rc = dout.reserve(out_bytes))) return rc;
+    if ((rc = as.reserve(vdt, rows, k))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(dx.p, x, (size_t)rows * k * 4, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_quantize_rows(vdt, dx.as<float>(), rows, (int)k, as.view(), nullptr));
+    MOE_HIP_CHECK(launch_actbuf_to_std(vdt, as.view(), rows, (int)k, dout.as<uint8_t>(), nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(out, dout.p, out_bytes);
+}
+
+extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_qmatmul: unsupported dtype");
+    const int64_t be = block_elems(dt);
+    if (n <= 0 || n % 16 || k <= 0 || k % be || m < 0) return fail(MOE_E_INVALID, "moe_qmatmul: need n % 16 == 0 and k a multiple of the block size");
+    if (m == 0) return MOE_OK;
+    if (!w_blocks || !x || !y) return fail(MOE_E_INVALID, "NULL pointer");
+    const int vdt = vecdot_dtype(dt);
+    DevBuf raw, tiled, dx, dy, grp;
+    ActStore as;
+    RouteStore rs;
+    const size_t raw_bytes = (size_t)(n * k / be * block_bytes(dt));
+    if ((rc = raw.reserve(raw_bytes))) return rc;
+    if ((rc = tiled.reserve((size_t)relaid_bytes(dt, n, k)))) return rc;
+    if ((rc = dx.reserve((size_t)m * k * 4))) return rc;
+    if ((rc = dy.reserve((size_t)m * n * 4))) return rc;
+    if ((rc = grp.reserve(sizeof(GroupWeights)))) return rc;
+    if ((rc = as.reserve(vdt, m, k))) return rc;
+    if ((rc = rs.reserve(m, 1, 1, false))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(raw.p, w_blocks, raw_bytes, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(hipMemcpy(dx.p, x, (size_t)m * k * 4, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_relayout(dt, raw.as<uint8_t>(), tiled.as<uint8_t>(), n, k, nullptr));
+    GroupWeights g{nullptr, nullptr, tiled.as<uint8_t>()};
+    MOE_HIP_CHECK(hipMemcpy(grp.p, &g, sizeof g, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_quantize_rows(vdt, dx.as<float>(), m, (int)k, as.view(), nullptr));
+    MOE_HIP_CHECK(launch_identity_routing(rs.view(), m, nullptr));
+    ExpertParams ep;
+    ep.dt = dt; ep.H = (int)n; ep.F = (int)k; ep.n_groups = 1; ep.group0 = 0;
+    ep.groups = grp.as<GroupWeights>();
+    ep.rb = rs.view(); ep.hq = as.view(); ep.slot_origin = 0; ep.yw = dy.as<float>();
+    ep.max_rows = m; ep.slot_tiles = m > 16 ? 2 : 1;
+    MOE_HIP_CHECK(launch_expert_down(ep, nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(y, dy.p, (size_t)m * n * 4);
+}
+
+extern "C" const char* moe_last_error(void) { return g_err.c_str(); }
+
+extern "C" const char* moe_device_arch(void) {
+    if (ensure_device()) return nullptr;
+    return g_arch.c_str();
+}
+
+extern "C" float moe_debug_expf(float x) { return expf_glibc(x); }

@@ -1,0 +1,90 @@
+// Launchers of the gfx950 kernels (definitions in the kernels_*.hip files).
+#pragma once
+#include "moe_common.hpp"
+
+namespace moe {
+
+// Routing state of one forward call (all device pointers).  "Groups" are the E routed experts
+// plus, when the layer has one, the always-on shared expert as group E.
+struct RouteBufs {
+    float* logits = nullptr;        // [T, E]
+    int32_t* topk_idx = nullptr;    // [T, k] rank order
+    float* topk_w = nullptr;        // [T, k]
+    float* shared_w = nullptr;      // [T] sigmoid gate of the shared expert (or null)
+    int32_t* offsets = nullptr;     // [G+1] slot ranges per group
+    int32_t* perm_token = nullptr;  // [S] token row of every slot
+    float* perm_w = nullptr;        // [S] routing weight of every slot
+    int32_t* tok_slots = nullptr;   // [T, k(+1)] slots of a token, ascending expert index
+    uint32_t* counter = nullptr;    // one word, zero between launches
+};
+
+struct FrontParams {
+    const float* x = nullptr;       // [T, H]
+    int64_t T = 0;
+    int H = 0, E = 0, k = 0, norm_topk = 1;
+    const float* gate = nullptr;        // [E, H]
+    const float* gate_bias = nullptr;   // [E] or null
+    const float* shared_gate = nullptr; // [H] or null
+    const float* rms_alpha = nullptr;   // [H] or null
+    float rms_eps = 0.f;
+    int vdt = MOE_GGML_Q8K;             // activation format
+    ActBuf xq;                          // token-indexed quantised activations (output)
+    RouteBufs rb;
+};
+// rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token; the
+// last workgroup to finish builds the per-expert lists.
+hipError_t launch_front(const FrontParams& p, hipStream_t s);
+// softmax + top-k + lists from given logits (parity hook).
+hipError_t launch_route_from_logits(const float* logits, int64_t T, int E, int k, int norm_topk,
+                                    const RouteBufs& rb, hipStream_t s);
+
+struct GroupWeights {
+    const uint8_t* w1;
+    const uint8_t* w3;
+    const uint8_t* w2;
+};
+
+struct ExpertParams {
+    int dt = 0;
+    int H = 0, F = 0;
+    int n_groups = 0;               // groups handled by this launch
+    int group0 = 0;                 // index of the first of them in rb.offsets
+    const GroupWeights* groups = nullptr;  // device array [n_groups]
+    RouteBufs rb;
+    ActBuf xq;                      // token-indexed, K = H
+    ActBuf hq;                      // slot-indexed (row = slot - slot_origin), K = F
+    int slot_origin = 0;
+    float* yw = nullptr;            // [S, H] weighted expert outputs, slot-indexed (absolute)
+    int64_t max_rows = 0;           // upper bound of rows in any group of this launch
+    int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1 or 2)
+};
+// h = silu(W1 x) * (W3 x), quantised to the activation format, for every slot of every group.
+hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s);
+// yw[slot] = (W2 h[slot]) * perm_w[slot]
+hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
+
+// y[t] = sum over the token's slots (ascending expert index) of yw[slot] (+ residual[t]).
+hipError_t launch_combine(const float* yw, const int32_t* tok_slots, int slots_per_tok,
+                          const float* residual, float* y, int64_t T, int H, hipStream_t s);
+
+// Re-lay raw GGML blocks [rows, k] (device, standard layout) into the tiled device layout.
+hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t rows, int64_t k, hipStream_t s);
+// to_float from the tiled layout back to row-major f32 (layout check).
+hipError_t launch_dequant_tiled(int dt, const uint8_t* tiled, float* out, int64_t rows, int64_t k, hipStream_t s);
+// to_float on standard blocks.
+hipError_t launch_dequant_std(int dt, const uint8_t* blocks, float* out, int64_t n, hipStream_t s);
+// Activation quantiser on plain rows [rows, k] into an ActBuf (same device code the front kernel uses).
+hipError_t launch_quantize_rows(int vdt, const float* x, int64_t rows, int k, const ActBuf& out, hipStream_t s);
+// ActBuf -> standard BlockQ8K / BlockQ8_0 bytes.
+hipError_t launch_actbuf_to_std(int vdt, const ActBuf& in, int64_t rows, int k, uint8_t* out, hipStream_t s);
+// Identity routing for a dense product over `rows` rows: one group, slot i = row i, weight 1.
+hipError_t launch_identity_routing(const RouteBufs& rb, int64_t rows, hipStream_t s);
+
+// bytes of the ActBuf members for `rows` rows of length k
+inline size_t act_qs_bytes(int64_t rows, int64_t k) { return (size_t)rows * k; }
+inline size_t act_d_bytes(int vdt, int64_t rows, int64_t k) { return (size_t)rows * (k / block_elems(vdt)) * 4; }
+inline size_t act_bsum_bytes(int vdt, int64_t rows, int64_t k) {
+    return vdt == MOE_GGML_Q8K ? (size_t)rows * (k / 256) * 16 * 2 : (size_t)rows * (k / 32) * 4;
+}
+
+}  // namespace moe

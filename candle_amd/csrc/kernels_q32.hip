@@ -1,0 +1,276 @@
+// Grouped expert products over Q4_0 / Q8_0 weights with Q8_0 activations (gfx950, int8 MFMA).
+//
+// Arithmetic restated from candle-core/src/quantized/k_quants.rs:241-258 (Q4_0 . Q8_0) and
+// :650-668 (Q8_0 . Q8_0): per 32-element block  sumf += (sum_i as f32) * d_w * d_x.  One
+// v_mfma_i32_16x16x32_i8 yields the exact integer dot of a block for 16 rows x 16 slots, and every
+// lane adds its (row, slot) blocks in ascending block order with separately rounded products, so
+// the f32 result is bit-identical to the scalar reference loop.
+//
+// Q4_0 stores nibble - 8; the kernel multiplies the raw nibbles (0..15) and subtracts
+// 8 * sum(q8) of the block, which is the same integer.
+#include "act_quant.hpp"
+#include "kernels.hpp"
+
+namespace moe {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+template <int DT>
+struct Q32Tile {
+    uint2 q;
+    float d;
+};
+
+template <int DT>
+__device__ inline Q32Tile<DT> load_q32_tile(const uint8_t* tile, int lane) {
+    Q32Tile<DT> t;
+    const int r = lane & 15, g = lane >> 4;
+    if (DT == MOE_GGML_Q8_0) {
+        t.q = *reinterpret_cast<const uint2*>(tile + lane * 8);
+        t.d = __half2float(*reinterpret_cast<const __half*>(tile + 512 + 2 * r));
+    } else {
+        uint2 w = *reinterpret_cast<const uint2*>(tile + r * 16 + 8 * (g >> 1));
+        if (g & 1) { w.x >>= 4; w.y >>= 4; }
+        t.q.x = w.x & 0x0f0f0f0fu;
+        t.q.y = w.y & 0x0f0f0f0fu;
+        t.d = __half2float(*reinterpret_cast<const __half*>(tile + 256 + 2 * r));
+    }
+    return t;
+}
+
+struct Q8_0Operand {
+    uint2 a;
+    float yd[4];
+    int bs[4];
+};
+
+// element offset inside a block of this lane's 8-element MFMA chunk
+template <int DT>
+__device__ inline int chunk_start(int g) {
+    return DT == MOE_GGML_Q8_0 ? 8 * g : (g & 1) * 16 + (g >> 1) * 8;
+}
+
+template <int DT>
+__device__ inline Q8_0Operand load_q8_0_operand(const ActBuf& ab, int K, int nkb, int kb, int rowA, const int rowD[4], int g) {
+    Q8_0Operand o;
+    o.a = *reinterpret_cast<const uint2*>(ab.qs + (int64_t)rowA * K + kb * 32 + chunk_start<DT>(g));
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        o.yd[i] = ab.d[(int64_t)rowD[i] * nkb + kb];
+        o.bs[i] = (DT == MOE_GGML_Q4_0) ? reinterpret_cast<const int32_t*>(ab.bsum)[(int64_t)rowD[i] * nkb + kb] : 0;
+    }
+    return o;
+}
+
+template <int DT>
+__device__ inline void q32_mac(const Q32Tile<DT>& w, const Q8_0Operand& A, float acc[4]) {
+    const v4i zero = {0, 0, 0, 0};
+    const long a = (long)(((uint64_t)A.a.y << 32) | A.a.x);
+    const long b = (long)(((uint64_t)w.q.y << 32) | w.q.x);
+    v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, zero, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int isum = D[i];
+        if (DT == MOE_GGML_Q4_0) isum -= 8 * A.bs[i];
+        float t = (float)isum * w.d;
+        t = t * A.yd[i];
+        acc[i] += t;
+    }
+}
+
+__device__ inline float silu_ref32(float v) { return v / (1.0f + expf_glibc(-v)); }
+
+constexpr int Q32_THREADS = 256;
+
+template <int DT, int TT>
+__global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    const int grp = blockIdx.y;
+    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
+    const int tg0 = blockIdx.z * (TT * 16);
+    if (s_begin + tg0 >= s_end) return;
+    const int H = p.H, F = p.F, nkb = H / 32;
+    const int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
+    if (rt0 >= F / 16) return;
+    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+
+    int rowA[TT], rowD[TT][4];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        int s = s_begin + tg0 + tt * 16 + r;
+        rowA[tt] = p.rb.perm_token[s < s_end ? s : s_end - 1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
+            rowD[tt][i] = p.rb.perm_token[sd < s_end ? sd : s_end - 1];
+        }
+    }
+    const GroupWeights gw = p.groups[grp];
+    const uint8_t* tp[4] = {gw.w1 + (size_t)rt0 * nkb * TB, gw.w1 + (size_t)(rt0 + 1) * nkb * TB,
+                            gw.w3 + (size_t)rt0 * nkb * TB, gw.w3 + (size_t)(rt0 + 1) * nkb * TB};
+    float acc[4][TT][4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
+
+    Q32Tile<DT> cur[4], nxt[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) cur[j] = load_q32_tile<DT>(tp[j], lane);
+    for (int kb = 0; kb < nkb; kb++) {
+        if (kb + 1 < nkb) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) nxt[j] = load_q32_tile<DT>(tp[j] + (size_t)(kb + 1) * TB, lane);
+        }
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) {
+            Q8_0Operand A = load_q8_0_operand<DT>(p.xq, H, nkb, kb, rowA[tt], rowD[tt], g);
+#pragma unroll
+            for (int j = 0; j < 4; j++) q32_mac<DT>(cur[j], A, acc[j][tt]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) cur[j] = nxt[j];
+    }
+
+    // epilogue: h = silu(w1 x) * (w3 x); the wave's 32 rows are exactly one Q8_0 block per slot
+    const int nfb = F / 32;
+    const int fb = rt0 / 2;
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float h0 = silu_ref32(acc[0][tt][i]) * acc[2][tt][i];
+            float h1 = silu_ref32(acc[1][tt][i]) * acc[3][tt][i];
+            float amax = fmaxf(fabsf(h0), fabsf(h1));
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            float d = amax / 127.0f;
+            float id = (d != 0.f) ? 1.0f / d : 0.f;
+            int q0 = sat_i8(roundf(h0 * id)), q1 = sat_i8(roundf(h1 * id));
+            int sum = q0 + q1;
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+            int slot = s_begin + tg0 + tt * 16 + 4 * g + i;
+            if (slot < s_end) {
+                int64_t hrow = slot - p.slot_origin;
+                p.hq.qs[hrow * F + rt0 * 16 + r] = (int8_t)q0;
+                p.hq.qs[hrow * F + rt0 * 16 + 16 + r] = (int8_t)q1;
+                if (r == 0) {
+                    p.hq.d[hrow * nfb + fb] = __half2float(__float2half_rn(d));
+                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + fb] = sum;
+                }
+            }
+        }
+}
+
+constexpr int Q32_DOWN_STEP = 4;
+
+template <int DT, int TT>
+__global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    const int grp = blockIdx.y;
+    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
+    const int tg0 = blockIdx.z * (TT * 16);
+    if (s_begin + tg0 >= s_end) return;
+    const int H = p.H, F = p.F, nkb = F / 32;
+    const int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
+    if (rt >= H / 16) return;
+    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+
+    int rowA[TT], rowD[TT][4];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        int s = s_begin + tg0 + tt * 16 + r;
+        rowA[tt] = (s < s_end ? s : s_end - 1) - p.slot_origin;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
+            rowD[tt][i] = (sd < s_end ? sd : s_end - 1) - p.slot_origin;
+        }
+    }
+    const uint8_t* tp = p.groups[grp].w2 + (size_t)rt * nkb * TB;
+    float acc[TT][4];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[tt][i] = 0.f;
+
+    Q32Tile<DT> cur[Q32_DOWN_STEP], nxt[Q32_DOWN_STEP];
+#pragma unroll
+    for (int j = 0; j < Q32_DOWN_STEP; j++)
+        if (j < nkb) cur[j] = load_q32_tile<DT>(tp + (size_t)j * TB, lane);
+    for (int kb0 = 0; kb0 < nkb; kb0 += Q32_DOWN_STEP) {
+#pragma unroll
+        for (int j = 0; j < Q32_DOWN_STEP; j++)
+            if (kb0 + Q32_DOWN_STEP + j < nkb) nxt[j] = load_q32_tile<DT>(tp + (size_t)(kb0 + Q32_DOWN_STEP + j) * TB, lane);
+#pragma unroll
+        for (int j = 0; j < Q32_DOWN_STEP; j++) {
+            if (kb0 + j < nkb) {
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) {
+                    Q8_0Operand A = load_q8_0_operand<DT>(p.hq, F, nkb, kb0 + j, rowA[tt], rowD[tt], g);
+                    q32_mac<DT>(cur[j], A, acc[tt]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < Q32_DOWN_STEP; j++) cur[j] = nxt[j];
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int slot = s_begin + tg0 + tt * 16 + 4 * g + i;
+            if (slot < s_end) p.yw[(int64_t)slot * H + rt * 16 + r] = acc[tt][i] * p.rb.perm_w[slot];
+        }
+}
+
+template <int DT>
+static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
+    const int tt = p.slot_tiles >= 2 ? 2 : 1;
+    const int wpb = Q32_THREADS / 64;
+    const int n_pairs = p.F / 32;
+    dim3 grid((unsigned)((n_pairs + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (tt == 1)
+        hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+    return hipGetLastError();
+}
+template <int DT>
+static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
+    const int tt = p.slot_tiles >= 2 ? 2 : 1;
+    const int wpb = Q32_THREADS / 64;
+    dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (tt == 1)
+        hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+    else
+        hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s);
+hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s);
+
+hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s) {
+    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
+    switch (p.dt) {
+        case MOE_GGML_Q4K: return launch_q4k_up(p, s);
+        case MOE_GGML_Q8_0: return launch_q32_up_t<MOE_GGML_Q8_0>(p, s);
+        case MOE_GGML_Q4_0: return launch_q32_up_t<MOE_GGML_Q4_0>(p, s);
+    }
+    return hipErrorInvalidValue;
+}
+hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s) {
+    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
+    switch (p.dt) {
+        case MOE_GGML_Q4K: return launch_q4k_down(p, s);
+        case MOE_GGML_Q8_0: return launch_q32_down_t<MOE_GGML_Q8_0>(p, s);
+        case MOE_GGML_Q4_0: return launch_q32_down_t<MOE_GGML_Q4_0>(p, s);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace moe

@@ -1,0 +1,242 @@
+// Layout and format kernels: re-laying GGML blocks into the tiled device layout, `to_float`
+// from either layout, and the stand-alone activation quantiser used by the parity hooks.
+//
+// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0),
+// 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60) and 1858-1870 (Q8K).  The library is
+// built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
+#include "act_quant.hpp"
+#include "kernels.hpp"
+
+namespace moe {
+
+__device__ inline float f16_bits_to_f32(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
+__device__ inline void scale_min_k4(int j, const uint8_t* q, int* sc, int* m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4);
+        *m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+
+// value of element `i` (0..255) of a Q4K block given its header (16 B) and the byte holding it
+__device__ inline float q4k_value(const uint8_t* hdr, int i, uint8_t qbyte) {
+    float d = f16_bits_to_f32((uint16_t)(hdr[0] | (hdr[1] << 8)));
+    float mn = f16_bits_to_f32((uint16_t)(hdr[2] | (hdr[3] << 8)));
+    int sc, m;
+    scale_min_k4(i / 32, hdr + 4, &sc, &m);
+    float d1 = d * (float)sc;
+    float m1 = mn * (float)m;
+    int q = ((i / 32) & 1) ? (qbyte >> 4) : (qbyte & 0xF);
+    return d1 * (float)q - m1;
+}
+
+// ------------------------------------------------------------------ standard layout to_float
+__global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    if (dt == MOE_GGML_Q4K) {
+        const uint8_t* b = blocks + (i / 256) * 144;
+        int e = (int)(i % 256);
+        out[i] = q4k_value(b, e, b[16 + (e / 64) * 32 + (e % 32)]);
+    } else if (dt == MOE_GGML_Q4_0) {
+        const uint8_t* b = blocks + (i / 32) * 18;
+        int e = (int)(i % 32);
+        float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
+        uint8_t q = b[2 + (e % 16)];
+        int v = (e < 16 ? (q & 0xF) : (q >> 4)) - 8;
+        out[i] = (float)v * d;
+    } else if (dt == MOE_GGML_Q8_0) {
+        const uint8_t* b = blocks + (i / 32) * 34;
+        float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
+        out[i] = (float)(int8_t)b[2 + (i % 32)] * d;
+    } else {  // Q8K
+        const uint8_t* b = blocks + (i / 256) * 292;
+        float d;
+        __builtin_memcpy(&d, b, 4);
+        out[i] = d * (float)(int8_t)b[4 + (i % 256)];
+    }
+}
+
+// ------------------------------------------------------------------ re-lay (one thread per 16/8/2-byte piece)
+__global__ void relayout_q4k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
+    // one thread per 16-byte destination chunk: 144 chunks per tile
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    int64_t total = n_rt * nsb * 144;
+    if (c >= total) return;
+    int64_t tile = c / 144;
+    int ch = (int)(c % 144);
+    int64_t rt = tile / nsb;
+    int sb = (int)(tile % nsb);
+    uint8_t* dst = tiled + tile * Q4K_TILE_BYTES + ch * 16;
+    if (ch < 128) {
+        int half = ch / 64, l = ch % 64, r = l % 16, g = l / 16;
+        const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144 + 16;
+        const uint8_t* s0 = blk + (2 * half) * 32 + 8 * g;
+        const uint8_t* s1 = blk + (2 * half + 1) * 32 + 8 * g;
+        for (int i = 0; i < 8; i++) { dst[i] = s0[i]; dst[8 + i] = s1[i]; }
+    } else {
+        int r = ch - 128;
+        const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
+        for (int i = 0; i < 16; i++) dst[i] = blk[i];
+    }
+}
+
+__global__ void relayout_q8_0_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nkb) {
+    // one thread per (tile, lane): 8 quant bytes; lanes < 16 also move the scale
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nkb * 64) return;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int64_t rt = tile / nkb;
+    int kb = (int)(tile % nkb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nkb + kb) * 34;
+    uint8_t* dst = tiled + tile * Q8_0_TILE_BYTES;
+    for (int i = 0; i < 8; i++) dst[l * 8 + i] = blk[2 + 8 * g + i];
+    if (g == 0) { dst[512 + 2 * r] = blk[0]; dst[512 + 2 * r + 1] = blk[1]; }
+}
+
+__global__ void relayout_q4_0_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nkb) {
+    // one thread per (tile, row)
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nkb * 16) return;
+    int64_t tile = c / 16;
+    int r = (int)(c % 16);
+    int64_t rt = tile / nkb;
+    int kb = (int)(tile % nkb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nkb + kb) * 18;
+    uint8_t* dst = tiled + tile * Q4_0_TILE_BYTES;
+    for (int i = 0; i < 16; i++) dst[r * 16 + i] = blk[2 + i];
+    dst[256 + 2 * r] = blk[0];
+    dst[256 + 2 * r + 1] = blk[1];
+}
+
+// ------------------------------------------------------------------ to_float from the tiled layout
+__global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, int64_t rows, int64_t k) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * k) return;
+    int64_t row = i / k;
+    int col = (int)(i % k);
+    int64_t rt = row / 16;
+    int r = (int)(row % 16);
+    if (dt == MOE_GGML_Q4K) {
+        int nsb = (int)(k / 256), sb = col / 256, e = col % 256;
+        const uint8_t* tile = tiled + (rt * nsb + sb) * Q4K_TILE_BYTES;
+        // original qs byte index of element e: (e/64)*32 + e%32 ; that byte sits in pair P = byte/32,
+        // chunk g = (byte%32)/8, position byte%8
+        int byte = (e / 64) * 32 + (e % 32);
+        int P = byte / 32, g = (byte % 32) / 8, pos = byte % 8;
+        int l = g * 16 + r;
+        uint8_t q = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
+        out[i] = q4k_value(tile + 2048 + r * 16, e, q);
+    } else if (dt == MOE_GGML_Q8_0) {
+        int nkb = (int)(k / 32), kb = col / 32, e = col % 32;
+        const uint8_t* tile = tiled + (rt * nkb + kb) * Q8_0_TILE_BYTES;
+        float d = f16_bits_to_f32((uint16_t)(tile[512 + 2 * r] | (tile[512 + 2 * r + 1] << 8)));
+        int l = (e / 8) * 16 + r;
+        out[i] = (float)(int8_t)tile[l * 8 + e % 8] * d;
+    } else {  // Q4_0
+        int nkb = (int)(k / 32), kb = col / 32, e = col % 32;
+        const uint8_t* tile = tiled + (rt * nkb + kb) * Q4_0_TILE_BYTES;
+        float d = f16_bits_to_f32((uint16_t)(tile[256 + 2 * r] | (tile[256 + 2 * r + 1] << 8)));
+        uint8_t q = tile[r * 16 + e % 16];
+        int v = (e < 16 ? (q & 0xF) : (q >> 4)) - 8;
+        out[i] = (float)v * d;
+    }
+}
+
+// ------------------------------------------------------------------ activation quantiser on plain rows
+template <int VDT>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int64_t rows, int k, ActBuf out) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row = blockIdx.x;
+    const float* xr = x + row * k;
+    if (VDT == MOE_GGML_Q8K) {
+        const int nb = k / 256;
+        for (int b = wave; b < nb; b += 4) {
+            float4 v = *reinterpret_cast<const float4*>(xr + b * 256 + lane * 4);
+            quantize_q8k_block(v, lane, out.qs + row * k + b * 256, out.d + row * nb + b,
+                               reinterpret_cast<__half*>(out.bsum) + (row * nb + b) * 16);
+        }
+    } else {
+        const int nb = k / 32;
+        for (int h = tid; h < k; h += 256)
+            quantize_q8_0_block(xr[h], lane, out.qs + row * k + h, out.d + row * nb + h / 32,
+                                reinterpret_cast<int32_t*>(out.bsum) + row * nb + h / 32);
+    }
+}
+
+// ActBuf -> the reference's block structs (BlockQ8K 292 B: d f32, qs[256], bsums i16[16];
+// BlockQ8_0 34 B: d f16, qs[32])
+__global__ void actbuf_to_std_kernel(int vdt, ActBuf in, int64_t rows, int k, uint8_t* out) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * k) return;
+    int64_t row = i / k;
+    int col = (int)(i % k);
+    if (vdt == MOE_GGML_Q8K) {
+        int nb = k / 256, b = col / 256, e = col % 256;
+        uint8_t* blk = out + (row * nb + b) * 292;
+        blk[4 + e] = (uint8_t)in.qs[row * k + b * 256 + q8k_act_offset(e)];
+        if (e == 0) __builtin_memcpy(blk, &in.d[row * nb + b], 4);
+        if (e < 16) {
+            int16_t s = (int16_t)__half2int_rn(reinterpret_cast<const __half*>(in.bsum)[(row * nb + b) * 16 + e]);
+            __builtin_memcpy(blk + 260 + 2 * e, &s, 2);
+        }
+    } else {
+        int nb = k / 32, b = col / 32, e = col % 32;
+        uint8_t* blk = out + (row * nb + b) * 34;
+        blk[2 + e] = (uint8_t)in.qs[row * k + col];
+        if (e == 0) {
+            // the stored f32 is an exactly widened f16
+            uint16_t h = __half_as_ushort(__float2half_rn(in.d[row * nb + b]));
+            __builtin_memcpy(blk, &h, 2);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launchers
+static inline unsigned nblk(int64_t n, int bs) { return (unsigned)((n + bs - 1) / bs); }
+
+hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t rows, int64_t k, hipStream_t s) {
+    int64_t n_rt = rows / 16;
+    int nkb = (int)(k / block_elems(dt));
+    if (n_rt == 0 || nkb == 0) return hipSuccess;
+    if (dt == MOE_GGML_Q4K)
+        hipLaunchKernelGGL(relayout_q4k_kernel, dim3(nblk(n_rt * nkb * 144, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (dt == MOE_GGML_Q8_0)
+        hipLaunchKernelGGL(relayout_q8_0_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else
+        hipLaunchKernelGGL(relayout_q4_0_kernel, dim3(nblk(n_rt * nkb * 16, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_tiled(int dt, const uint8_t* tiled, float* out, int64_t rows, int64_t k, hipStream_t s) {
+    if (rows * k == 0) return hipSuccess;
+    hipLaunchKernelGGL(dequant_tiled_kernel, dim3(nblk(rows * k, 256)), dim3(256), 0, s, dt, tiled, out, rows, k);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_std(int dt, const uint8_t* blocks, float* out, int64_t n, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(dequant_std_kernel, dim3(nblk(n, 256)), dim3(256), 0, s, dt, blocks, out, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_rows(int vdt, const float* x, int64_t rows, int k, const ActBuf& out, hipStream_t s) {
+    if (rows == 0) return hipSuccess;
+    if (vdt == MOE_GGML_Q8K)
+        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8K>, dim3((unsigned)rows), dim3(256), 0, s, x, rows, k, out);
+    else
+        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8_0>, dim3((unsigned)rows), dim3(256), 0, s, x, rows, k, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_actbuf_to_std(int vdt, const ActBuf& in, int64_t rows, int k, uint8_t* out, hipStream_t s) {
+    if (rows == 0) return hipSuccess;
+    hipLaunchKernelGGL(actbuf_to_std_kernel, dim3(nblk(rows * k, 256)), dim3(256), 0, s, vdt, in, rows, k, out);
+    return hipGetLastError();
+}
+
+}  // namespace moe

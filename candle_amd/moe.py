@@ -1,0 +1,253 @@
+"""ctypes binding of libcandle_amd_moe.so.
+
+`SparseMoeBlock.forward(xs)` takes the same `[b, seq, hidden]` (or `[tokens, hidden]`) f32
+activations as `MlpOrMoe::forward` (candle-transformers/src/models/quantized_llama.rs:143-211)
+and returns the same shape.  numpy arrays go through the host entry point (as candle's
+`CustomOp1::cpu_fwd` would); torch CUDA tensors go through the device entry point on torch's
+current stream.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+GGML_Q4_0, GGML_Q8_0, GGML_Q4K, GGML_Q8K = 2, 8, 12, 15
+_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4K: (256, 144), GGML_Q8K: (256, 292)}
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "lib", "libcandle_amd_moe.so")
+_lib = None
+
+
+class MoeError(RuntimeError):
+    """Mirrors candle::Error::Msg: carries the library's message."""
+
+
+class _Desc(C.Structure):
+    _fields_ = [
+        ("hidden", C.c_int64), ("ffn", C.c_int64), ("n_experts", C.c_int64), ("top_k", C.c_int64),
+        ("ggml_dtype", C.c_int32), ("norm_topk", C.c_int32),
+        ("gate", C.c_void_p), ("gate_bias", C.c_void_p),
+        ("w1", C.POINTER(C.c_void_p)), ("w3", C.POINTER(C.c_void_p)), ("w2", C.POINTER(C.c_void_p)),
+        ("shared_ffn", C.c_int64), ("shared_w1", C.c_void_p), ("shared_w3", C.c_void_p), ("shared_w2", C.c_void_p),
+        ("shared_gate", C.c_void_p), ("rms_alpha", C.c_void_p), ("rms_eps", C.c_float),
+    ]
+
+
+def lib_path():
+    return _LIB_PATH
+
+
+def load_library():
+    """Loads the built library; raises if it has not been built (no fallback path exists)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise MoeError("%s is missing: build it with `python -m candle_amd.build` "
+                       "(there is no CPU fallback)" % _LIB_PATH)
+    L = C.CDLL(_LIB_PATH)
+    vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
+    L.moe_layer_create.argtypes = [C.POINTER(_Desc), C.POINTER(vp)]
+    L.moe_layer_destroy.argtypes = [vp]
+    L.moe_layer_destroy.restype = None
+    L.moe_layer_forward.argtypes = [vp, vp, i64, vp]
+    L.moe_layer_forward_device.argtypes = [vp, vp, i64, vp, vp]
+    L.moe_layer_last_logits.argtypes = [vp, vp, i64]
+    L.moe_layer_last_routing.argtypes = [vp, i64, vp, vp, vp, vp, vp]
+    L.moe_layer_dequantize_weight.argtypes = [vp, i64, C.c_int, vp, i64]
+    L.moe_route.argtypes = [vp, i64, i64, i64, i32, vp, vp, vp, vp, vp]
+    L.moe_dequantize.argtypes = [i32, vp, i64, vp]
+    L.moe_quantize_act.argtypes = [i32, vp, i64, i64, vp]
+    L.moe_qmatmul.argtypes = [i32, vp, i64, i64, vp, i64, vp]
+    L.moe_last_error.restype = C.c_char_p
+    L.moe_device_arch.restype = C.c_char_p
+    L.moe_debug_expf.restype = C.c_float
+    L.moe_debug_expf.argtypes = [C.c_float]
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise MoeError(load_library().moe_last_error().decode())
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    a = np.asarray(a)
+    if a.dtype != np.float32:
+        raise MoeError("expected f32 activations, got %s" % a.dtype)  # the reference bails on other dtypes
+    return np.ascontiguousarray(a)
+
+
+def _blocks(a, dtype, n_elems, what):
+    a = np.ascontiguousarray(np.asarray(a).view(np.uint8).reshape(-1))
+    be, bb = _BLOCK[dtype]
+    if n_elems % be or a.size != n_elems // be * bb:
+        raise MoeError("%s: expected %d bytes of dtype %d blocks, got %d" % (what, n_elems // be * bb, dtype, a.size))
+    return a
+
+
+def device_arch():
+    r = load_library().moe_device_arch()
+    if r is None:
+        raise MoeError(load_library().moe_last_error().decode())
+    return r.decode()
+
+
+def debug_expf(x):
+    return float(load_library().moe_debug_expf(float(x)))
+
+
+def dequantize(dtype, blocks, n_elems):
+    """GgmlType::to_float on the GPU (parity hook)."""
+    blocks = _blocks(blocks, dtype, n_elems, "dequantize")
+    out = np.empty(n_elems, dtype=np.float32)
+    _check(load_library().moe_dequantize(dtype, _p(blocks), n_elems, _p(out)))
+    return out
+
+
+def quantize_act(vecdot_dtype, x):
+    """The activation quantiser of k_quants::matmul on the GPU; returns raw BlockQ8_0 / BlockQ8K bytes."""
+    x = _f32(x)
+    rows, k = (1, x.size) if x.ndim == 1 else (x.shape[0], x.shape[1])
+    be, bb = _BLOCK[vecdot_dtype]
+    out = np.zeros(rows * k // be * bb, dtype=np.uint8)
+    _check(load_library().moe_quantize_act(vecdot_dtype, _p(x), rows, k, _p(out)))
+    return out
+
+
+def route(logits, top_k, norm_topk=True):
+    """softmax + top-k + per-expert lists on the GPU given router logits (parity hook)."""
+    logits = _f32(logits)
+    T, E = logits.shape
+    idx = np.zeros((T, top_k), dtype=np.int32)
+    w = np.zeros((T, top_k), dtype=np.float32)
+    offsets = np.zeros(E + 1, dtype=np.int32)
+    perm = np.zeros(T * top_k, dtype=np.int32)
+    perm_w = np.zeros(T * top_k, dtype=np.float32)
+    _check(load_library().moe_route(_p(logits), T, E, top_k, int(norm_topk), _p(idx), _p(w), _p(offsets), _p(perm), _p(perm_w)))
+    return idx, w, offsets, perm, perm_w
+
+
+def qmatmul(dtype, w_blocks, n, k, x):
+    """QMatMul::forward of one quantized [n, k] matrix on the GPU: x [m, k] -> [m, n]."""
+    x = _f32(x)
+    m = x.shape[0]
+    w_blocks = _blocks(w_blocks, dtype, n * k, "qmatmul")
+    y = np.empty((m, n), dtype=np.float32)
+    _check(load_library().moe_qmatmul(dtype, _p(w_blocks), n, k, _p(x), m, _p(y)))
+    return y
+
+
+class SparseMoeBlock:
+    """The MoE arm of `MlpOrMoe` with quantized experts resident on the GPU.
+
+    gate: f32 [E, H]; w1/w3: E raw block arrays of [F, H]; w2: E raw block arrays of [H, F]
+    (the bytes of candle's `QTensor::data()`).
+    """
+
+    def __init__(self, hidden, ffn, n_experts, top_k, ggml_dtype, gate, w1, w3, w2, norm_topk=True,
+                 gate_bias=None, shared_ffn=0, shared_w1=None, shared_w3=None, shared_w2=None,
+                 shared_gate=None, rms_alpha=None, rms_eps=1e-5):
+        L = load_library()
+        if ggml_dtype not in (GGML_Q4_0, GGML_Q8_0, GGML_Q4K):
+            raise MoeError("unsupported ggml_dtype %r" % (ggml_dtype,))
+        if len(w1) != n_experts or len(w2) != n_experts or len(w3) != n_experts:
+            raise MoeError("need one w1/w2/w3 per expert")
+        self.hidden, self.ffn, self.n_experts, self.top_k, self.dtype = hidden, ffn, n_experts, top_k, ggml_dtype
+        self.shared_ffn = shared_ffn
+        gate = _f32(gate).reshape(n_experts, hidden)
+        keep = [gate]
+        mats = {}
+        for name, ws in (("w1", w1), ("w3", w3), ("w2", w2)):
+            arrs = [_blocks(w, ggml_dtype, hidden * ffn, name) for w in ws]
+            keep += arrs
+            mats[name] = (C.c_void_p * n_experts)(*[a.ctypes.data for a in arrs])
+        opt = {}
+        for name, a, n in (("gate_bias", gate_bias, n_experts), ("shared_gate", shared_gate, hidden), ("rms_alpha", rms_alpha, hidden)):
+            if a is not None:
+                a = _f32(a).reshape(n)
+                keep.append(a)
+            opt[name] = a
+        sh = {}
+        for name, a in (("shared_w1", shared_w1), ("shared_w3", shared_w3), ("shared_w2", shared_w2)):
+            if shared_ffn:
+                a = _blocks(a, ggml_dtype, hidden * shared_ffn, name)
+                keep.append(a)
+            else:
+                a = None
+            sh[name] = a
+        ptr = lambda a: None if a is None else a.ctypes.data
+        desc = _Desc(hidden, ffn, n_experts, top_k, ggml_dtype, int(norm_topk), ptr(gate), ptr(opt["gate_bias"]),
+                     C.cast(mats["w1"], C.POINTER(C.c_void_p)), C.cast(mats["w3"], C.POINTER(C.c_void_p)),
+                     C.cast(mats["w2"], C.POINTER(C.c_void_p)), shared_ffn, ptr(sh["shared_w1"]), ptr(sh["shared_w3"]),
+                     ptr(sh["shared_w2"]), ptr(opt["shared_gate"]), ptr(opt["rms_alpha"]), float(rms_eps))
+        handle = C.c_void_p()
+        self._h = None
+        _check(L.moe_layer_create(C.byref(desc), C.byref(handle)))
+        self._h = handle
+        del keep  # host copies are only borrowed during create
+
+    def close(self):
+        if getattr(self, "_h", None) is not None:
+            load_library().moe_layer_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def forward(self, xs, out=None):
+        L = load_library()
+        if self._h is None:
+            raise MoeError("layer is closed")
+        if isinstance(xs, np.ndarray):
+            x = _f32(xs)
+            if x.ndim not in (2, 3) or x.shape[-1] != self.hidden:
+                raise MoeError("expected [b, seq, %d] or [tokens, %d], got %s" % (self.hidden, self.hidden, x.shape))
+            T = x.size // self.hidden
+            y = np.empty_like(x)
+            _check(L.moe_layer_forward(self._h, _p(x), T, _p(y)))
+            return y
+        import torch  # device tensors: plumbing only
+        if not (isinstance(xs, torch.Tensor) and xs.is_cuda):
+            raise MoeError("forward takes a numpy array or a torch CUDA tensor")
+        if xs.dtype != torch.float32 or not xs.is_contiguous():
+            raise MoeError("input has to be contiguous f32")
+        if xs.dim() not in (2, 3) or xs.shape[-1] != self.hidden:
+            raise MoeError("expected [b, seq, %d] or [tokens, %d], got %s" % (self.hidden, self.hidden, tuple(xs.shape)))
+        T = xs.numel() // self.hidden
+        y = torch.empty_like(xs) if out is None else out
+        stream = torch.cuda.current_stream(xs.device).cuda_stream
+        _check(L.moe_layer_forward_device(self._h, xs.data_ptr(), T, y.data_ptr(), stream))
+        return y
+
+    __call__ = forward
+
+    def last_logits(self, n_tokens):
+        out = np.empty((n_tokens, self.n_experts), dtype=np.float32)
+        _check(load_library().moe_layer_last_logits(self._h, _p(out), n_tokens))
+        return out
+
+    def last_routing(self, n_tokens):
+        k, E = self.top_k, self.n_experts
+        idx = np.zeros((n_tokens, k), dtype=np.int32)
+        w = np.zeros((n_tokens, k), dtype=np.float32)
+        offsets = np.zeros(E + 1, dtype=np.int32)
+        perm = np.zeros(n_tokens * k, dtype=np.int32)
+        perm_w = np.zeros(n_tokens * k, dtype=np.float32)
+        _check(load_library().moe_layer_last_routing(self._h, n_tokens, _p(idx), _p(w), _p(offsets), _p(perm), _p(perm_w)))
+        return idx, w, offsets, perm, perm_w
+
+    def dequantize_weight(self, expert, which):
+        """to_float of matrix `which` (1, 2, 3) of `expert` (E = shared expert) read back from the device layout."""
+        F = self.shared_ffn if expert == self.n_experts else self.ffn
+        out = np.empty(self.hidden * F, dtype=np.float32)
+        _check(load_library().moe_layer_dequantize_weight(self._h, expert, which, _p(out), out.size))
+        return out.reshape((self.hidden, F) if which == 2 else (F, self.hidden))
+
+
+MlpOrMoe = SparseMoeBlock  # the reference's name for the enum that holds the MoE arm

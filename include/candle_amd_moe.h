@@ -1,0 +1,139 @@
+/*
+ * candle_amd_moe.h -- C ABI of the MI355X (gfx950) quantized sparse-MoE block.
+ *
+ * The library replaces ONE path of candle: the `MlpOrMoe::MoE` arm of
+ * candle-transformers/src/models/quantized_llama.rs:143-211 together with the per-expert
+ * `QMatMul::forward` calls it makes (candle-core/src/quantized/mod.rs:533-556 ->
+ * k_quants::matmul, candle-core/src/quantized/k_quants.rs:1873-1920).  candle has no C FFI
+ * for this path; its interface is the Rust trait
+ *     candle::Module { fn forward(&self, xs: &Tensor) -> Result<Tensor> }   (candle-core/src/lib.rs:148-150)
+ * and, for user ops, `CustomOp1::cpu_fwd` (candle-core/src/custom_op.rs:7-41).  candle's `Device`
+ * has no HIP variant (candle-core/src/device.rs:16-20), so a drop-in op receives and returns HOST
+ * f32 storage; the quantized weights live on the GPU inside the layer object.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a non-zero MOE_E_* code on failure;
+ *     moe_last_error() returns the message of the calling thread's last failure
+ *     (the Rust side maps it to candle::Error::Msg, candle-core/src/error.rs:233).
+ *   - host pointers passed to moe_layer_create are BORROWED for the duration of the call only;
+ *     the library copies and re-lays the blocks on the device and owns that memory.
+ *   - activations are contiguous row-major f32 [n_tokens, hidden]; the reference bails on
+ *     anything else (candle-core/src/quantized/mod.rs:480-482,501).
+ *   - a layer may be used from several threads (QuantizedType: Send + Sync,
+ *     candle-core/src/quantized/mod.rs:256); calls on one layer are serialised internally.
+ *   - there is no CPU fallback: without a usable HIP device every entry point fails.
+ */
+#ifndef CANDLE_AMD_MOE_H
+#define CANDLE_AMD_MOE_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgmlDType numbering, candle-core/src/quantized/mod.rs:153-174 (also the GGUF on-disk ids). */
+#define MOE_GGML_Q4_0 2
+#define MOE_GGML_Q8_0 8
+#define MOE_GGML_Q4K 12
+#define MOE_GGML_Q8K 15
+
+#define MOE_OK 0
+#define MOE_E_INVALID 1   /* bad argument / unsupported shape or dtype */
+#define MOE_E_HIP 2       /* HIP runtime error (message carries hipGetErrorString) */
+#define MOE_E_NODEVICE 3  /* no gfx950 device visible */
+#define MOE_E_NOMEM 4
+
+typedef struct moe_layer moe_layer;
+
+/* One MoE layer.  Replaces the fields of `MlpOrMoe::MoE` (quantized_llama.rs:133-141):
+ * `feed_forward_gate_inp` -> gate, `experts[e].feed_forward_w{1,2,3}` -> w1/w2/w3,
+ * `n_expert_used` -> top_k.  Weight matrices are the raw bytes of a CPU QTensor
+ * (`QTensor::data()`, candle-core/src/quantized/mod.rs:394-396): rows of GGML blocks,
+ * w1 and w3 are [ffn, hidden], w2 is [hidden, ffn]. */
+typedef struct {
+    int64_t hidden;              /* H */
+    int64_t ffn;                 /* F: per-expert intermediate size */
+    int64_t n_experts;           /* E (1..256) */
+    int64_t top_k;               /* n_expert_used (1..min(E,16)) */
+    int32_t ggml_dtype;          /* MOE_GGML_Q4_0 | Q8_0 | Q4K, same for all expert matrices */
+    int32_t norm_topk;           /* 1: weights renormalised over the selected experts (Mixtral,
+                                    quantized_llama.rs:175-178); 0: raw softmax probability
+                                    (qwen2_moe.rs:287 with norm_topk_prob=false) */
+    const float* gate;           /* [E, H] f32: the router is dequantised at load (mod.rs:430-436) */
+    const float* gate_bias;      /* optional [E], added to the logits; NULL for the reference's models */
+    const void* const* w1;       /* E pointers */
+    const void* const* w3;       /* E pointers */
+    const void* const* w2;       /* E pointers */
+    /* always-on shared expert, qwen2_moe.rs:315-319; shared_ffn == 0 disables it */
+    int64_t shared_ffn;
+    const void* shared_w1;       /* [shared_ffn, H] */
+    const void* shared_w3;       /* [shared_ffn, H] */
+    const void* shared_w2;       /* [H, shared_ffn] */
+    const float* shared_gate;    /* [H] f32, sigmoid gate */
+    /* optional fused pre-norm + residual, quantized_llama.rs:888-892: y = x + moe(rms_norm(x)) */
+    const float* rms_alpha;      /* [H] or NULL */
+    float rms_eps;
+} moe_desc;
+
+/* Uploads and re-lays the weights.  Replaces the construction at quantized_llama.rs:553-578. */
+int moe_layer_create(const moe_desc* desc, moe_layer** out);
+void moe_layer_destroy(moe_layer* layer);
+
+/* `MlpOrMoe::forward`, quantized_llama.rs:143-211 (== CustomOp1::cpu_fwd for the drop-in op):
+ * x and y are HOST f32 [n_tokens, hidden]; synchronous. */
+int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float* y);
+
+/* Same computation on DEVICE pointers, enqueued on `hip_stream` (a hipStream_t, NULL = default
+ * stream) without synchronising.  d_x and d_y must not alias.  This is the entry a caller that
+ * already keeps activations on the GPU uses (no PCIe in the path). */
+int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
+
+/* Router logits [n_tokens, E] (after the optional bias) that the last forward on this layer
+ * computed, copied to the host.  Debug / parity hook: candle computes these with the `gemm`
+ * crate whose f32 summation order is not part of the reference tree. */
+int moe_layer_last_logits(moe_layer* layer, float* logits, int64_t n_tokens);
+
+/* Routing that the last forward produced (host copies): topk_idx/topk_w [n_tokens, k] in rank
+ * order, expert_offsets [E+1], perm_token / perm_w [n_tokens*k] (per-expert token lists).
+ * Any pointer may be NULL. */
+int moe_layer_last_routing(moe_layer* layer, int64_t n_tokens, int32_t* topk_idx, float* topk_w,
+                           int32_t* expert_offsets, int32_t* perm_token, float* perm_w);
+
+/* Device-layout check: dequantises expert `expert` (0..E-1, or E for the shared expert), matrix
+ * `which` (1, 2 or 3) from the re-laid device copy into host f32 [rows*cols] in the ORIGINAL
+ * row-major order.  Must equal `to_float` of the bytes passed at create. */
+int moe_layer_dequantize_weight(moe_layer* layer, int64_t expert, int which, float* out, int64_t n_elems);
+
+/* Parity hook: router + dispatch given logits (host pointers).  Restates softmax_last_dim
+ * (candle-nn/src/ops.rs:313-351) + the host top-k loop (quantized_llama.rs:158-179) on the GPU.
+ * Outputs as for moe_layer_last_routing. */
+int moe_route(const float* logits, int64_t n_tokens, int64_t n_experts, int64_t top_k, int32_t norm_topk,
+              int32_t* topk_idx, float* topk_w, int32_t* expert_offsets, int32_t* perm_token, float* perm_w);
+
+/* Parity hook: GgmlType::to_float on raw blocks (host pointers), k_quants.rs:166-186 (Q4_0),
+ * 587-603 (Q8_0), 1347-1374 (Q4K), 1858-1870 (Q8K). */
+int moe_dequantize(int32_t ggml_dtype, const void* blocks, int64_t n_elems, float* out);
+
+/* Parity hook: the activation quantiser k_quants::matmul applies to every lhs row
+ * (k_quants.rs:1893-1903): vecdot_dtype MOE_GGML_Q8_0 (k_quants.rs:605-634) or MOE_GGML_Q8K
+ * (k_quants.rs:1819-1856).  x is host f32 [rows, k]; out receives rows*k/block standard blocks. */
+int moe_quantize_act(int32_t vecdot_dtype, const float* x, int64_t rows, int64_t k, void* out);
+
+/* Parity hook: QMatMul::forward on one quantized matrix (quantized/mod.rs:533-537 ->
+ * k_quants.rs:1873-1920): y[m, n] = x[m, k] . W[n, k]^T, host pointers, W as raw blocks. */
+int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y);
+
+/* Message of the calling thread's last error ("" if none). */
+const char* moe_last_error(void);
+
+/* Name of the device the library runs on, e.g. "gfx950"; NULL (and an error message) if none. */
+const char* moe_device_arch(void);
+
+/* Host restatement of the exp used by the device router (same source, compiled for the CPU), so
+ * that its agreement with the platform's expf can be checked without a GPU. */
+float moe_debug_expf(float x);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

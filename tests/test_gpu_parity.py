@@ -1,0 +1,220 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle.
+
+Bars: bit-exact for to_float, the activation quantisers, top-k indices, routing weights and the
+per-expert token lists; max-abs error <= 2e-3 * rms(output) for block outputs (f32).
+"""
+import numpy as np
+import pytest
+
+import candle_amd
+import pyoracle as O
+from helpers import CONFIGS, activations, make_pair, rms
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3  # max-abs error relative to rms(output)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def test_device_is_gfx950():
+    assert candle_amd.device_arch().startswith("gfx950")
+
+
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q4K, O.Q8K])
+def test_to_float_bit_exact(dt):
+    n = 256 * 96
+    x = O.fill_normal(dt, n, 0.0, 0.02)
+    x[:256] = 0.0  # an all-zero block
+    x[256:512] *= 1e-3  # tiny values: f16 subnormal scales
+    x[512] = 3.0  # outlier
+    blocks = O.quantize(dt, x)
+    assert np.array_equal(bits(candle_amd.dequantize(dt, blocks, n)), bits(O.dequantize(dt, blocks, n)))
+    # arbitrary bit patterns in the quant payload (scale fields kept finite)
+    rng = np.random.default_rng(dt)
+    raw = blocks.copy().reshape(-1, O.BLOCK_BYTES[dt])
+    lo = {O.Q4_0: 2, O.Q8_0: 2, O.Q4K: 4, O.Q8K: 4}[dt]
+    raw[:, lo:] = rng.integers(0, 256, raw[:, lo:].shape, dtype=np.uint8)
+    raw = raw.reshape(-1)
+    assert np.array_equal(bits(candle_amd.dequantize(dt, raw, n)), bits(O.dequantize(dt, raw, n)))
+    assert candle_amd.dequantize(dt, raw[:0], 0).size == 0
+
+
+@pytest.mark.parametrize("vdt", [O.Q8_0, O.Q8K])
+def test_activation_quantiser_bit_exact(vdt):
+    rows, k = 37, 2048
+    x = O.fill_normal(5 + vdt, rows * k).reshape(rows, k)
+    x[0] = 0.0                      # all-zero row
+    x[1, :256] = 0.0                # zero block inside a row
+    x[2, 7] = -9.5                  # negative maximum
+    x[3, 300] = 9.5                 # positive maximum (maps to -128)
+    x[4, 10] = 4.25; x[4, 20] = -4.25  # equal magnitudes: the first one decides the sign
+    x[5] *= 1e-20
+    x[6] *= 1e20
+    x[7, ::2] = 0.5                 # exact .5 ties after scaling
+    got = candle_amd.quantize_act(vdt, x)
+    want = O.quantize(vdt, x)
+    assert np.array_equal(got, want)
+    assert candle_amd.quantize_act(vdt, x[:0]).size == 0
+
+
+@pytest.mark.parametrize("T,E,k,norm", [(16, 8, 2, True), (1, 8, 2, True), (333, 60, 4, True), (4096, 8, 2, True),
+                                         (65, 64, 6, False), (7, 3, 3, True), (50, 160, 8, True), (9, 1, 1, True)])
+def test_route_bit_exact_given_logits(T, E, k, norm):
+    logits = O.fill_normal(T * 31 + E, T * E, 0.0, 1.5).reshape(T, E)
+    if T > 4:
+        logits[1] = 0.25            # all tied: experts 0..k-1 must win
+        logits[2, E // 2:] = logits[2, : E - E // 2][::-1]  # pairwise ties
+        logits[3] = -80.0 * np.arange(E)  # probabilities underflow to zero past the first few
+    gi, gw, goff, gperm, gpw = candle_amd.route(logits, k, norm)
+    ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), k, norm)
+    assert np.array_equal(gi, ri)
+    assert np.array_equal(bits(gw), bits(rw))
+    assert np.array_equal(goff, roff)
+    assert np.array_equal(gperm, rperm)
+    assert np.array_equal(bits(gpw), bits(rpw))
+
+
+def test_route_zipf_bias_lists():
+    # prefill-like: 4096 tokens, heavy skew
+    T, E, k = 4096, 8, 2
+    logits = O.fill_normal(99, T * E, 0.0, 1.0).reshape(T, E) + np.log(1.0 / np.arange(1, E + 1)).astype(np.float32) * 2
+    gi, gw, goff, gperm, gpw = candle_amd.route(logits, k)
+    ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), k)
+    assert np.array_equal(gi, ri) and np.array_equal(goff, roff) and np.array_equal(gperm, rperm)
+    assert goff[1] - goff[0] > 2 * (goff[-1] - goff[-2])
+
+
+@pytest.mark.parametrize("dt,n,k,m", [(O.Q4K, 64, 512, 5), (O.Q4K, 4096, 1024, 33), (O.Q8_0, 48, 96, 3),
+                                       (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70)])
+def test_qmatmul_against_oracle(dt, n, k, m):
+    w = O.fill_normal_quantized(n + k, dt, n, k, 0.02)
+    x = activations(m, k, seed=n)
+    got = candle_amd.qmatmul(dt, w, n, k, x)
+    want = O.matmul(dt, x, w, n)
+    if dt in (O.Q4_0, O.Q8_0):
+        # same per-block values added in the same order as the scalar reference loop
+        assert np.array_equal(bits(got), bits(want))
+    else:
+        assert np.abs(got - want).max() <= 1e-5 * rms(want) * 10
+
+
+def test_q4_0_matmul_known_answers(golden):
+    # candle-core/tests/quantized_tests.rs:89-104; four weight rows padded to a 16-row tile
+    m, k, n = 3, 64, 4
+    lhs = np.arange(m * k, dtype=np.float32).reshape(m, k)
+    rhs = np.zeros((16, k), dtype=np.float32)
+    rhs[:n] = np.arange(k * n, dtype=np.float32).reshape(n, k)
+    got = candle_amd.qmatmul(O.Q4_0, O.quantize(O.Q4_0, rhs), 16, k, lhs)[:, :n]
+    assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_3_64_4"]["expected_rounded"]
+
+
+def test_batch_invariance():
+    # qmm_batch, candle-core/tests/quantized_tests.rs:221-256
+    n, k = 256, 512
+    w = O.fill_normal_quantized(4, O.Q4K, n, k, 0.02)
+    x = activations(2, k, seed=8)
+    base = candle_amd.qmatmul(O.Q4K, w, n, k, x)
+    for reps in (2, 3, 6, 20):
+        big = candle_amd.qmatmul(O.Q4K, w, n, k, np.concatenate([x] * reps))
+        for r in range(reps):
+            assert np.array_equal(bits(big[2 * r: 2 * r + 2]), bits(base))
+
+
+def check_block(ref, gpu, T, seed=2, tol=TOL):
+    xs = activations(T, ref.H, seed)
+    ys = gpu.forward(xs)
+    logits = gpu.last_logits(T)
+    # the gate product itself: f32 accumulation order is implementation-defined, values must agree
+    _, ref_logits = ref.forward(xs[: min(T, 4)], return_logits=True)
+    assert np.abs(logits[: min(T, 4)] - ref_logits).max() < 1e-4
+    # routing is bit-exact given the same logits
+    gi, gw, goff, gperm, gpw = gpu.last_routing(T)
+    ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), ref.k, bool(ref.c.norm_topk))
+    assert np.array_equal(gi, ri) and np.array_equal(bits(gw), bits(rw))
+    assert np.array_equal(goff, roff) and np.array_equal(gperm, rperm) and np.array_equal(bits(gpw), bits(rpw))
+    want = ref.forward(xs, logits=logits)
+    moe = want - xs if ref.rms_alpha is not None else want
+    err = np.abs(ys - want).max()
+    assert err <= tol * rms(moe), (err, rms(moe))
+    return ys, want
+
+
+def test_weight_layout_roundtrip():
+    for dt, H, F in ((O.Q4K, 512, 768), (O.Q8_0, 256, 96), (O.Q4_0, 128, 160)):
+        ref, gpu = make_pair(H, F, 3, 2, dt, seed=dt, Fs=(64 if dt != O.Q4K else 256))
+        for e in range(3):
+            for which, src, shape in ((1, ref.w1[e], (F, H)), (3, ref.w3[e], (F, H)), (2, ref.w2[e], (H, F))):
+                got = gpu.dequantize_weight(e, which)
+                assert np.array_equal(bits(got).reshape(-1), bits(O.dequantize(dt, src, H * F)))
+        got = gpu.dequantize_weight(3, 2)
+        assert np.array_equal(bits(got).reshape(-1), bits(O.dequantize(dt, ref.sw[2], got.size)))
+        gpu.close()
+
+
+@pytest.mark.parametrize("T", [16, 1, 5])
+def test_block_cfg1_q4_0(T):
+    c = CONFIGS["cfg1"]
+    ref, gpu = make_pair(c["H"], c["F"], c["E"], c["k"], c["dt"], seed=0)
+    check_block(ref, gpu, T)
+    gpu.close()
+
+
+@pytest.mark.parametrize("T", [1, 8, 33, 200])
+def test_block_q4k_small(T):
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
+    check_block(ref, gpu, T)
+    gpu.close()
+
+
+def test_block_q8_0_shared_expert_top4():
+    ref, gpu = make_pair(256, 352, 12, 4, O.Q8_0, seed=3, Fs=704)
+    check_block(ref, gpu, 40)
+    gpu.close()
+
+
+def test_block_no_renorm_and_bias():
+    bias = np.log(1.0 / np.arange(1, 9)).astype(np.float32)
+    ref, gpu = make_pair(256, 512, 8, 2, O.Q4K, seed=4, norm_topk=False, gate_bias=bias)
+    check_block(ref, gpu, 64)
+    gpu.close()
+
+
+def test_block_rms_residual_chain():
+    ref, gpu = make_pair(512, 512, 4, 2, O.Q4K, seed=5, rms=True)
+    xs = activations(6, 512, 9)
+    for _ in range(3):
+        ys = gpu.forward(xs)
+        want = ref.forward(xs, logits=gpu.last_logits(6))
+        assert np.abs(ys - want).max() <= TOL * rms(want - xs)
+        xs = ys
+    gpu.close()
+
+
+def test_empty_and_shape_errors():
+    ref, gpu = make_pair(256, 256, 4, 2, O.Q4_0, seed=6)
+    assert gpu.forward(np.zeros((0, 256), np.float32)).shape == (0, 256)
+    assert gpu.forward(np.zeros((2, 3, 256), np.float32)).shape == (2, 3, 256)
+    with pytest.raises(candle_amd.MoeError):
+        gpu.forward(np.zeros((2, 255), np.float32))
+    with pytest.raises(candle_amd.MoeError):
+        gpu.forward(np.zeros((2, 256), np.float64))
+    gpu.close()
+    with pytest.raises(candle_amd.MoeError):
+        candle_amd.SparseMoeBlock(256, 256, 4, 5, O.Q4_0, np.zeros((4, 256), np.float32), ref.w1, ref.w3, ref.w2)
+    with pytest.raises(candle_amd.MoeError):
+        candle_amd.SparseMoeBlock(256, 256, 4, 2, 14, np.zeros((4, 256), np.float32), ref.w1, ref.w3, ref.w2)
+
+
+def test_device_entry_point_matches_host_entry_point():
+    import torch
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=7)
+    xs = activations(24, 512, 3)
+    y_host = gpu.forward(xs)
+    xd = torch.from_numpy(xs).cuda()
+    yd = gpu.forward(xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(yd.cpu().numpy()), bits(y_host))
+    gpu.close()
