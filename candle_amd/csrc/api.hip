@@ -500,6 +500,34 @@ extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t 
     return d2h(y, dy.p, (size_t)m * n * 4);
 }
 
+extern "C" int moe_quantize_weights_device(int32_t dt, const void* d_x, int64_t n, void* d_out, void* hip_stream) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
+    if (n < 0 || n % block_elems(dt)) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
+    if (n == 0) return MOE_OK;
+    if (!d_x || !d_out) return fail(MOE_E_INVALID, "NULL pointer");
+    MOE_HIP_CHECK(launch_quantize_weights(dt, static_cast<const float*>(d_x), n, static_cast<uint8_t*>(d_out), static_cast<hipStream_t>(hip_stream)));
+    return MOE_OK;
+}
+
+extern "C" int moe_quantize_weights(int32_t dt, const float* x, int64_t n, void* out) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
+    if (n < 0 || n % block_elems(dt)) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
+    if (n == 0) return MOE_OK;
+    if (!x || !out) return fail(MOE_E_INVALID, "NULL pointer");
+    DevBuf dx, dout;
+    const size_t out_bytes = (size_t)(n / block_elems(dt) * block_bytes(dt));
+    if ((rc = dx.reserve((size_t)n * 4))) return rc;
+    if ((rc = dout.reserve(out_bytes))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_quantize_weights(dt, dx.as<float>(), n, dout.as<uint8_t>(), nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(out, dout.p, out_bytes);
+}
+
 extern "C" const char* moe_last_error(void) { return g_err.c_str(); }
 
 extern "C" const char* moe_device_arch(void) {

@@ -80,6 +80,9 @@ hipError_t launch_actbuf_to_std(int vdt, const ActBuf& in, int64_t rows, int k, 
 // Identity routing for a dense product over `rows` rows: one group, slot i = row i, weight 1.
 hipError_t launch_identity_routing(const RouteBufs& rb, int64_t rows, hipStream_t s);
 
+// QTensor::quantize on the GPU: f32 [n] (device) -> standard GGML blocks (device).
+hipError_t launch_quantize_weights(int dt, const float* x, int64_t n, uint8_t* out, hipStream_t s);
+
 // bytes of the ActBuf members for `rows` rows of length k
 inline size_t act_qs_bytes(int64_t rows, int64_t k) { return (size_t)rows * k; }
 inline size_t act_d_bytes(int vdt, int64_t rows, int64_t k) { return (size_t)rows * (k / block_elems(vdt)) * 4; }

@@ -46,6 +46,13 @@ def load_library():
     if not os.path.exists(_LIB_PATH):
         raise MoeError("%s is missing: build it with `python -m candle_amd.build` "
                        "(there is no CPU fallback)" % _LIB_PATH)
+    # A process must hold ONE HIP runtime.  PyTorch ships its own libamdhip64; if this library
+    # pulled in the system copy first, torch would later fail with "No HIP GPUs are available".
+    # Importing torch first makes the loader resolve our dependency to the copy torch uses.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(_LIB_PATH)
     vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int32
     L.moe_layer_create.argtypes = [C.POINTER(_Desc), C.POINTER(vp)]
@@ -60,6 +67,8 @@ def load_library():
     L.moe_dequantize.argtypes = [i32, vp, i64, vp]
     L.moe_quantize_act.argtypes = [i32, vp, i64, i64, vp]
     L.moe_qmatmul.argtypes = [i32, vp, i64, i64, vp, i64, vp]
+    L.moe_quantize_weights.argtypes = [i32, vp, i64, vp]
+    L.moe_quantize_weights_device.argtypes = [i32, vp, i64, vp, vp]
     L.moe_last_error.restype = C.c_char_p
     L.moe_device_arch.restype = C.c_char_p
     L.moe_debug_expf.restype = C.c_float
@@ -142,6 +151,29 @@ def qmatmul(dtype, w_blocks, n, k, x):
     y = np.empty((m, n), dtype=np.float32)
     _check(load_library().moe_qmatmul(dtype, _p(w_blocks), n, k, _p(x), m, _p(y)))
     return y
+
+
+def quantize_weights(dtype, x):
+    """QTensor::quantize on the GPU.  numpy f32 in -> numpy uint8 blocks out; a torch CUDA f32
+    tensor in -> a torch CUDA uint8 tensor out (enqueued on torch's current stream)."""
+    L = load_library()
+    be, bb = _BLOCK[dtype]
+    if isinstance(x, np.ndarray):
+        x = _f32(x)
+        if x.size % be or (x.ndim > 1 and x.shape[-1] % be):
+            raise MoeError("last dimension must be a multiple of the block size %d" % be)
+        out = np.zeros(x.size // be * bb, dtype=np.uint8)
+        _check(L.moe_quantize_weights(dtype, _p(x), x.size, _p(out)))
+        return out
+    import torch
+    if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()):
+        raise MoeError("quantize_weights takes a numpy f32 array or a contiguous f32 torch CUDA tensor")
+    if x.shape[-1] % be:
+        raise MoeError("last dimension must be a multiple of the block size %d" % be)
+    out = torch.empty(x.numel() // be * bb, dtype=torch.uint8, device=x.device)
+    _check(L.moe_quantize_weights_device(dtype, x.data_ptr(), x.numel(), out.data_ptr(),
+                                         torch.cuda.current_stream(x.device).cuda_stream))
+    return out
 
 
 class SparseMoeBlock:

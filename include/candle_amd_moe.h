@@ -123,6 +123,12 @@ int moe_quantize_act(int32_t vecdot_dtype, const float* x, int64_t rows, int64_t
  * k_quants.rs:1873-1920): y[m, n] = x[m, k] . W[n, k]^T, host pointers, W as raw blocks. */
 int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y);
 
+/* QTensor::quantize (candle-core/src/quantized/mod.rs:331-349) on the GPU: f32 [n_elems] -> raw
+ * GGML blocks, bit-identical to GgmlType::from_float of k_quants.rs:188-224 (Q4_0), 605-634 (Q8_0)
+ * and 1287-1345 (Q4K).  Host pointers / device pointers (the latter enqueued on hip_stream). */
+int moe_quantize_weights(int32_t ggml_dtype, const float* x, int64_t n_elems, void* out_blocks);
+int moe_quantize_weights_device(int32_t ggml_dtype, const void* d_x, int64_t n_elems, void* d_out_blocks, void* hip_stream);
+
 /* Message of the calling thread's last error ("" if none). */
 const char* moe_last_error(void);
 

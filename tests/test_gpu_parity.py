@@ -12,7 +12,23 @@ from helpers import CONFIGS, activations, make_pair, rms
 
 pytestmark = pytest.mark.gpu
 
-TOL = 2e-3  # max-abs error relative to rms(output)
+TOL = 2e-3  # max-abs error relative to rms(output), the bar at the benchmark shapes
+
+
+def block_tol(dt, F):
+    """Max-abs tolerance relative to rms(output) for a block of intermediate width F.
+
+    Q4_0 / Q8_0: the first product is bit-identical to the scalar reference, so the re-quantised
+    intermediate is too and only the f32 order of the second product differs -> 2e-3 everywhere.
+    Q4K: the reference adds eight interleaved partial sums per super-block, the MFMA path one; the
+    two differ in the last ulp, which now and then flips one rounding of the re-quantised
+    intermediate.  One flipped quant moves an output by (amax/127)*|w2|, i.e. about
+    (5/127)/sqrt(F) of rms(output): 3e-4 at F = 14336 (inside 2e-3) but 1.2e-3 at F = 1024, so
+    the bar is widened by sqrt(14336/F) for the reduced shapes used here.
+    """
+    if dt != O.Q4K:
+        return TOL
+    return TOL * max(1.0, float(np.sqrt(14336.0 / F)))
 
 
 def bits(a):
@@ -40,6 +56,27 @@ def test_to_float_bit_exact(dt):
     raw = raw.reshape(-1)
     assert np.array_equal(bits(candle_amd.dequantize(dt, raw, n)), bits(O.dequantize(dt, raw, n)))
     assert candle_amd.dequantize(dt, raw[:0], 0).size == 0
+
+
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q4K])
+def test_weight_quantiser_bit_exact(dt, golden):
+    n = 256 * 2048
+    x = O.fill_normal(40 + dt, n, 0.0, 0.02)
+    x[:256] = 0.0                  # all-zero super-block
+    x[256:288] = 0.0125            # constant sub-block (max == min)
+    x[512:768] = np.abs(x[512:768])  # all positive: min clamps to zero
+    x[1024:1280] *= 1e-4           # f16-subnormal scales
+    x[2048] = 1.0                  # outlier
+    assert np.array_equal(candle_amd.quantize_weights(dt, x), O.quantize(dt, x))
+    ramp = np.arange(128, dtype=np.float32)
+    if dt == O.Q4_0:  # candle-core/tests/quantized_tests.rs:262-291
+        got = candle_amd.dequantize(dt, candle_amd.quantize_weights(dt, ramp), 128)
+        assert np.array_equal(bits(got), bits(np.array(golden["q4_0_roundtrip_0_127"]["expected"], dtype=np.float32)))
+    import torch
+    xd = torch.from_numpy(x).cuda()
+    out = candle_amd.quantize_weights(dt, xd)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), O.quantize(dt, x))
 
 
 @pytest.mark.parametrize("vdt", [O.Q8_0, O.Q8K])
@@ -123,7 +160,8 @@ def test_batch_invariance():
             assert np.array_equal(bits(big[2 * r: 2 * r + 2]), bits(base))
 
 
-def check_block(ref, gpu, T, seed=2, tol=TOL):
+def check_block(ref, gpu, T, seed=2, tol=None):
+    tol = block_tol(ref.dtype, ref.F) if tol is None else tol
     xs = activations(T, ref.H, seed)
     ys = gpu.forward(xs)
     logits = gpu.last_logits(T)
@@ -139,6 +177,7 @@ def check_block(ref, gpu, T, seed=2, tol=TOL):
     moe = want - xs if ref.rms_alpha is not None else want
     err = np.abs(ys - want).max()
     assert err <= tol * rms(moe), (err, rms(moe))
+    assert rms(ys - want) <= 2e-4 * rms(moe)  # a wrong term or index moves the whole result, not one element
     return ys, want
 
 
@@ -188,7 +227,7 @@ def test_block_rms_residual_chain():
     for _ in range(3):
         ys = gpu.forward(xs)
         want = ref.forward(xs, logits=gpu.last_logits(6))
-        assert np.abs(ys - want).max() <= TOL * rms(want - xs)
+        assert np.abs(ys - want).max() <= block_tol(O.Q4K, 512) * rms(want - xs)
         xs = ys
     gpu.close()
 
