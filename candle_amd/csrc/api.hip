@@ -98,7 +98,7 @@ struct ActStore {
 };
 
 struct RouteStore {
-    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots, counter;
+    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots;
     int reserve(int64_t T, int E, int k, bool shared) {
         int rc;
         const int64_t S = T * k + (shared ? T : 0);
@@ -110,10 +110,6 @@ struct RouteStore {
         if ((rc = perm_token.reserve((size_t)S * 4))) return rc;
         if ((rc = perm_w.reserve((size_t)S * 4))) return rc;
         if ((rc = tok_slots.reserve((size_t)T * (k + 1) * 4))) return rc;
-        if (!counter.p) {
-            if ((rc = counter.reserve(256))) return rc;
-            MOE_HIP_CHECK(hipMemset(counter.p, 0, 256));
-        }
         return MOE_OK;
     }
     RouteBufs view() const {
@@ -126,7 +122,6 @@ struct RouteStore {
         r.perm_token = perm_token.as<int32_t>();
         r.perm_w = perm_w.as<float>();
         r.tok_slots = tok_slots.as<int32_t>();
-        r.counter = counter.as<uint32_t>();
         return r;
     }
 };
@@ -152,6 +147,7 @@ struct moe_layer {
     hipStream_t stream = nullptr;   // used by the host-pointer entry
     hipEvent_t done = nullptr;      // end of the last enqueued forward
     int64_t last_T = 0;
+    bool last_direct = false;       // the last forward skipped the dispatch pass
 };
 
 static int reserve_workspace(moe_layer* L, int64_t T) {
@@ -300,7 +296,12 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.vdt = L->vdt;
     fp.xq = L->xq.view();
     fp.rb = L->route.view();
+    fp.rb.T = (int)T; fp.rb.k = (int)L->k;
+    // small batches: slots are numbered t*k + r and no dispatch pass runs
+    const bool direct = T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
+    fp.rb.direct = direct ? 1 : 0;
     MOE_HIP_CHECK(launch_front(fp, s));
+    if (!direct) MOE_HIP_CHECK(launch_dispatch(fp.rb, T, (int)L->E, (int)L->k, shared, s));
 
     ExpertParams ep;
     ep.dt = L->dt; ep.H = (int)L->H; ep.F = (int)L->F;
@@ -314,15 +315,15 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     MOE_HIP_CHECK(launch_expert_down(ep, s));
     if (shared) {
         ExpertParams sp = ep;
-        sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E;
+        sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
         sp.groups = L->groups.as<GroupWeights>() + L->E;
         sp.hq = L->hq_shared.view(); sp.slot_origin = (int)(T * L->k);
         sp.max_rows = T; sp.slot_tiles = T > 16 ? 2 : 1;
         MOE_HIP_CHECK(launch_expert_up(sp, s));
         MOE_HIP_CHECK(launch_expert_down(sp, s));
     }
-    MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb.tok_slots, (int)L->k + (shared ? 1 : 0),
-                                 L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    L->last_direct = direct;
     MOE_HIP_CHECK(hipEventRecord(L->done, s));
     L->last_T = T;
     return MOE_OK;
@@ -375,6 +376,13 @@ extern "C" int moe_layer_last_routing(moe_layer* L, int64_t T, int32_t* topk_idx
     MOE_HIP_CHECK(hipEventSynchronize(L->done));
     int rc;
     const size_t A = (size_t)T * L->k;
+    if (L->last_direct && T > 0) {  // the forward needed no lists; build them now for the caller
+        RouteBufs rb = L->route.view();
+        rb.T = (int)T; rb.k = (int)L->k;
+        MOE_HIP_CHECK(launch_dispatch(rb, T, (int)L->E, (int)L->k, L->Fs > 0, nullptr));
+        MOE_HIP_CHECK(hipDeviceSynchronize());
+        L->last_direct = false;
+    }
     if ((rc = d2h(topk_idx, L->route.topk_idx.p, A * 4))) return rc;
     if ((rc = d2h(topk_w, L->route.topk_w.p, A * 4))) return rc;
     if ((rc = d2h(offsets, L->route.offsets.p, (size_t)(L->E + 1) * 4))) return rc;
@@ -415,6 +423,7 @@ extern "C" int moe_route(const float* logits, int64_t T, int64_t E, int64_t k, i
     if ((rc = dl.reserve((size_t)T * E * 4))) return rc;
     MOE_HIP_CHECK(hipMemcpy(dl.p, logits, (size_t)T * E * 4, hipMemcpyHostToDevice));
     MOE_HIP_CHECK(launch_route_from_logits(dl.as<float>(), T, (int)E, (int)k, norm_topk ? 1 : 0, rs.view(), nullptr));
+    MOE_HIP_CHECK(launch_dispatch(rs.view(), T, (int)E, (int)k, false, nullptr));
     MOE_HIP_CHECK(hipDeviceSynchronize());
     const size_t A = (size_t)T * k;
     if ((rc = d2h(topk_idx, rs.topk_idx.p, A * 4))) return rc;

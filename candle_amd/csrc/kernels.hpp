@@ -15,8 +15,14 @@ struct RouteBufs {
     int32_t* perm_token = nullptr;  // [S] token row of every slot
     float* perm_w = nullptr;        // [S] routing weight of every slot
     int32_t* tok_slots = nullptr;   // [T, k(+1)] slots of a token, ascending expert index
-    uint32_t* counter = nullptr;    // one word, zero between launches
+    // Slot numbering.  direct == 0: slots are grouped by expert (offsets / perm_* built by the
+    // dispatch kernel).  direct == 1 (small batches): slot of assignment (token t, rank r) is
+    // simply t*k + r, the shared expert's slots are T*k + t, and every consumer derives its
+    // expert's ascending list from topk_idx itself -- no dispatch pass on the critical path.
+    int direct = 0;
+    int T = 0, k = 0;
 };
+constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a dispatch pass
 
 struct FrontParams {
     const float* x = nullptr;       // [T, H]
@@ -31,12 +37,13 @@ struct FrontParams {
     ActBuf xq;                          // token-indexed quantised activations (output)
     RouteBufs rb;
 };
-// rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token; the
-// last workgroup to finish builds the per-expert lists.
+// rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token.
 hipError_t launch_front(const FrontParams& p, hipStream_t s);
-// softmax + top-k + lists from given logits (parity hook).
+// softmax + top-k from given logits (parity hook).
 hipError_t launch_route_from_logits(const float* logits, int64_t T, int E, int k, int norm_topk,
                                     const RouteBufs& rb, hipStream_t s);
+// Per-expert lists from topk_idx / topk_w: histogram, prefix scan, stable permutation (one workgroup).
+hipError_t launch_dispatch(const RouteBufs& rb, int64_t T, int E, int k, bool shared, hipStream_t s);
 
 struct GroupWeights {
     const uint8_t* w1;
@@ -57,15 +64,16 @@ struct ExpertParams {
     float* yw = nullptr;            // [S, H] weighted expert outputs, slot-indexed (absolute)
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
     int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1 or 2)
+    int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)
 };
 // h = silu(W1 x) * (W3 x), quantised to the activation format, for every slot of every group.
 hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s);
 // yw[slot] = (W2 h[slot]) * perm_w[slot]
 hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
 
-// y[t] = sum over the token's slots (ascending expert index) of yw[slot] (+ residual[t]).
-hipError_t launch_combine(const float* yw, const int32_t* tok_slots, int slots_per_tok,
-                          const float* residual, float* y, int64_t T, int H, hipStream_t s);
+// y[t] = sum over the token's slots (ascending expert index, shared expert last) of yw[slot] (+ residual[t]).
+hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,
+                          int64_t T, int H, hipStream_t s);
 
 // Re-lay raw GGML blocks [rows, k] (device, standard layout) into the tiled device layout.
 hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t rows, int64_t k, hipStream_t s);

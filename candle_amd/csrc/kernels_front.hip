@@ -1,9 +1,11 @@
 // Router, dispatch and combine kernels.
 //
-//   front_kernel            per token: optional rms-norm, gate product, softmax, top-k with
-//                           renormalised weights, activation quantisation; the last workgroup to
-//                           retire builds the per-expert token lists (histogram, prefix scan and a
-//                           stable permutation from wavefront ballots).
+//   front_kernel(s)         per token: optional rms-norm, gate product, softmax, top-k with
+//                           renormalised weights, activation quantisation.
+//   dispatch_kernel         per-expert token lists: histogram, prefix scan and a stable permutation
+//                           from wavefront ballots, in one workgroup.  Small batches skip it: there
+//                           the slot of (token t, rank r) is t*k + r and the expert kernels derive
+//                           their lists from topk_idx themselves.
 //   route_from_logits       the same routing starting from given logits (parity hook).
 //   combine_kernel          routing-weighted sum of the expert outputs back in token order.
 //
@@ -13,6 +15,8 @@
 //   top-k + lists     candle-transformers/src/models/quantized_llama.rs:158-179
 //   combine           quantized_llama.rs:200-202 (index_add in ascending expert order)
 //   rms_norm          candle-nn/src/ops.rs:504-515;  sigmoid candle-nn/src/ops.rs:59-61
+#include <cstdlib>
+
 #include "act_quant.hpp"
 #include "kernels.hpp"
 
@@ -25,6 +29,12 @@ constexpr int MAX_K = 16;
 __device__ inline float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ inline float wave_max_f(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
 
@@ -90,8 +100,9 @@ struct DispatchShared {
     int off[MAX_E + 2];
 };
 
-__device__ inline int ld_i32(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ inline float ld_f32(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// tok_slots is written and re-read inside one workgroup: bypass the vector cache on the re-read
+__device__ inline int ld_i32(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+__device__ inline float ld_f32(const float* p) { return *p; }
 
 __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, bool shared, DispatchShared& sh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -188,28 +199,12 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
     }
 }
 
-// Returns true in every thread of the last workgroup of the grid to get here.
-__device__ inline bool last_block_done(uint32_t* counter, int* flag_lds) {
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned ticket = atomicAdd(counter, 1u);
-        *flag_lds = (ticket == gridDim.x - 1);
-    }
-    __syncthreads();
-    bool last = *flag_lds != 0;
-    if (last) __threadfence();
-    return last;
-}
-
 // ---------------------------------------------------------------------------------------------
 template <int VDT>
 __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     extern __shared__ float xrow[];  // [H]
     __shared__ float probs[MAX_E];
     __shared__ float red[FRONT_THREADS / 64];
-    __shared__ int last_flag;
-    __shared__ DispatchShared dsh;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t t = blockIdx.x;
     const int H = p.H, E = p.E;
@@ -281,18 +276,201 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
         }
     }
 
-    // ---- the last workgroup builds the expert lists
-    if (last_block_done(p.rb.counter, &last_flag)) {
-        dispatch_block(p.rb, p.T, E, p.k, p.shared_gate != nullptr, dsh);
-        if (tid == 0) *p.rb.counter = 0u;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wave-parallel routing for E <= 64: lane e holds expert e.  Same arithmetic, in the same order,
+// as route_one_token: the exp values are summed left to right (E < 32) or in the 4 x 8
+// accumulator order followed by the serial tail (E >= 32); the rank of an expert is the number of
+// experts that precede it in the (total_cmp key descending, index ascending) order.  Cross-lane
+// traffic goes through v_readlane (scalar broadcast), not LDS.  Call with all 64 lanes active.
+__device__ inline float lane_bcast(float v, int i) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), i));
+}
+__device__ inline void route_one_token_wave(float logit, int lane, int E, int k, int norm_topk,
+                                            int32_t* idx_out, float* w_out) {
+    const bool valid = lane < E;
+    float mx = -__builtin_inff();
+    for (int i = 0; i < E; i++) mx = fmaxf(mx, lane_bcast(logit, i));
+    const float ex = valid ? expf_glibc(logit - mx) : 0.f;
+    float s;
+    if (E < 32) {
+        s = 0.f;
+        for (int i = 0; i < E; i++) s += lane_bcast(ex, i);
+    } else {
+        // acc[j] (lane j < 32) = sum over complete blocks of 32 of ex[32*b + j]
+        const int np = E & ~31;
+        float a = ex;                                  // block 0 (0 + ex, exact)
+        float hi = __shfl(ex, (lane & 31) + 32, 64);   // block 1
+        if (np >= 64) a = a + hi;
+        const int l = lane & 7;
+        float x0 = (__shfl(a, l, 64) + __shfl(a, 8 + l, 64)) + (__shfl(a, 16 + l, 64) + __shfl(a, 24 + l, 64));
+        float t0 = lane_bcast(x0, 0) + lane_bcast(x0, 4);
+        float t1 = lane_bcast(x0, 1) + lane_bcast(x0, 5);
+        float t2 = lane_bcast(x0, 2) + lane_bcast(x0, 6);
+        float t3 = lane_bcast(x0, 3) + lane_bcast(x0, 7);
+        s = (t0 + t1) + (t2 + t3);
+        for (int i = np; i < E; i++) s += lane_bcast(ex, i);
     }
+    const float pr = ex / s;
+    const int key = total_key(pr);
+    int rank = 0;
+    for (int i = 0; i < E; i++) {
+        const int ki = __builtin_amdgcn_readlane(key, i);
+        rank += (ki > key || (ki == key && i < lane)) ? 1 : 0;
+    }
+    if (!valid) rank = 0x7fffffff;
+    // probabilities in rank order: sum, then the (renormalised) weights
+    float sum = 0.f;
+    float my_p = 0.f;
+    int my_e = 0;
+    for (int r = 0; r < k; r++) {
+        const unsigned long long m = __ballot(rank == r);
+        const int e = __ffsll((long long)m) - 1;
+        const float pe = lane_bcast(pr, e);
+        sum += pe;
+        if (lane == r) { my_p = pe; my_e = e; }
+    }
+    if (lane < k) {
+        idx_out[lane] = my_e;
+        w_out[lane] = norm_topk ? my_p / sum : my_p;
+    }
+}
+
+// Low-latency front end for H = NCH * 256 (NCH <= 32) and E <= 64.  512 threads per token: waves
+// 0-3 compute the gate products (two experts at a time, all loads issued up front), waves 4-7
+// quantise the row, then one barrier and wave 0 routes.  Every wave keeps the activation row in
+// registers (lane l holds elements 256*i + 4l .. +3); with the pre-norm every wave evaluates the
+// same sum of squares in the same order, so all of them normalise with the same divisor.
+// Plain float arrays with compile-time indices only: nothing here may end up in scratch memory.
+constexpr int FAST_THREADS = 512;
+
+// Quantises chunk `chunk` (256 elements, this lane holds 4) of token row t; phases are written so
+// that a caller looping over several chunks gets independent dependency chains.
+template <int VDT>
+__device__ inline void quantize_chunk(const FrontParams& p, int64_t t, int H, int chunk, const float e[4], int lane) {
+    if (VDT == MOE_GGML_Q8K) {
+        const int nb = H / 256;
+        float4 v = make_float4(e[0], e[1], e[2], e[3]);
+        quantize_q8k_block(v, lane, p.xq.qs + t * H + chunk * 256, p.xq.d + t * nb + chunk,
+                           reinterpret_cast<__half*>(p.xq.bsum) + (t * nb + chunk) * 16);
+    } else {
+        const int nb = H / 32;
+        float amax = fmaxf(fmaxf(fabsf(e[0]), fabsf(e[1])), fmaxf(fabsf(e[2]), fabsf(e[3])));
+#pragma unroll
+        for (int o = 4; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));  // eight lanes share a block
+        const float d = amax / 127.0f;
+        const float id = (d != 0.f) ? 1.0f / d : 0.f;
+        uint32_t packed = 0;
+        int sum = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int qv = sat_i8(roundf(e[j] * id));
+            sum += qv;
+            packed |= (uint32_t)(uint8_t)qv << (8 * j);
+        }
+#pragma unroll
+        for (int o = 4; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        *reinterpret_cast<uint32_t*>(p.xq.qs + t * H + chunk * 256 + lane * 4) = packed;
+        if ((lane & 7) == 0) {
+            const int b = chunk * 8 + (lane >> 3);
+            p.xq.d[t * nb + b] = __half2float(__float2half_rn(d));
+            reinterpret_cast<int32_t*>(p.xq.bsum)[t * nb + b] = sum;
+        }
+    }
+}
+
+template <int VDT, int NCH>
+__global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p) {
+    __shared__ float logit_lds[64];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t t = blockIdx.x;
+    constexpr int H = NCH * 256;
+    const int E = p.E;
+    const float* x = p.x + t * H;
+    float xr[NCH * 4];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const float4 v = *reinterpret_cast<const float4*>(x + i * 256 + lane * 4);
+        xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+    }
+    if (p.rms_alpha) {
+        float sum2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH * 4; i++) sum2 += xr[i] * xr[i];
+        sum2 = wave_sum(sum2);
+        const float m = sqrtf(sum2 / (float)H + p.rms_eps);
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const float4 a = *reinterpret_cast<const float4*>(p.rms_alpha + i * 256 + lane * 4);
+            xr[4 * i] = xr[4 * i] / m * a.x; xr[4 * i + 1] = xr[4 * i + 1] / m * a.y;
+            xr[4 * i + 2] = xr[4 * i + 2] / m * a.z; xr[4 * i + 3] = xr[4 * i + 3] / m * a.w;
+        }
+    }
+    if (wave < 4) {
+        // gate products; the shared-expert gate counts as expert E
+        const int n_dot = E + (p.shared_gate ? 1 : 0);
+        for (int e0 = wave; e0 < n_dot; e0 += 8) {
+            const int e1 = e0 + 4 < n_dot ? e0 + 4 : e0;
+            const float* w0 = (e0 < E) ? p.gate + (int64_t)e0 * H : p.shared_gate;
+            const float* w1 = (e1 < E) ? p.gate + (int64_t)e1 * H : p.shared_gate;
+            float4 wa[NCH], wb[NCH];
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                wa[i] = *reinterpret_cast<const float4*>(w0 + i * 256 + lane * 4);
+                wb[i] = *reinterpret_cast<const float4*>(w1 + i * 256 + lane * 4);
+            }
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NCH; i++) {
+                acc0 = __builtin_fmaf(wa[i].x, xr[4 * i], acc0);     acc1 = __builtin_fmaf(wb[i].x, xr[4 * i], acc1);
+                acc0 = __builtin_fmaf(wa[i].y, xr[4 * i + 1], acc0); acc1 = __builtin_fmaf(wb[i].y, xr[4 * i + 1], acc1);
+                acc0 = __builtin_fmaf(wa[i].z, xr[4 * i + 2], acc0); acc1 = __builtin_fmaf(wb[i].z, xr[4 * i + 2], acc1);
+                acc0 = __builtin_fmaf(wa[i].w, xr[4 * i + 3], acc0); acc1 = __builtin_fmaf(wb[i].w, xr[4 * i + 3], acc1);
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                acc0 += __shfl_xor(acc0, o, 64);
+                acc1 += __shfl_xor(acc1, o, 64);
+            }
+            if (lane == 0) {
+                if (e0 < E) {
+                    if (p.gate_bias) acc0 += p.gate_bias[e0];
+                    logit_lds[e0] = acc0;
+                    p.rb.logits[t * E + e0] = acc0;
+                } else {
+                    p.rb.shared_w[t] = 1.0f / (expf_glibc(-acc0) + 1.0f);
+                }
+                if (e1 != e0) {
+                    if (e1 < E) {
+                        if (p.gate_bias) acc1 += p.gate_bias[e1];
+                        logit_lds[e1] = acc1;
+                        p.rb.logits[t * E + e1] = acc1;
+                    } else {
+                        p.rb.shared_w[t] = 1.0f / (expf_glibc(-acc1) + 1.0f);
+                    }
+                }
+            }
+        }
+    } else {
+        // quantise: wave 4+q owns chunks q, q+4, ...; the branches are wave-uniform
+        const int q = wave - 4;
+#pragma unroll
+        for (int i = 0; i < NCH; i++)
+            if ((i & 3) == q) {
+                const float e4[4] = {xr[4 * i], xr[4 * i + 1], xr[4 * i + 2], xr[4 * i + 3]};
+                quantize_chunk<VDT>(p, t, H, i, e4, lane);
+            }
+    }
+    __syncthreads();
+    if (wave == 0) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk,
+                                        p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
 }
 
 __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const float* logits, int64_t T, int E, int k,
                                                                          int norm_topk, RouteBufs rb) {
     __shared__ float probs[FRONT_THREADS / 64][MAX_E];
-    __shared__ int last_flag;
-    __shared__ DispatchShared dsh;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // one wave per token (4 tokens per workgroup); lane 0 routes
     int64_t t = (int64_t)blockIdx.x * (FRONT_THREADS / 64) + wave;
@@ -304,11 +482,16 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
         }
     }
     __syncthreads();
-    if (t < T && lane == 0) route_one_token(probs[wave], E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
-    if (last_block_done(rb.counter, &last_flag)) {
-        dispatch_block(rb, T, E, k, false, dsh);
-        if (tid == 0) *rb.counter = 0u;
+    if (E <= 64) {
+        if (t < T) route_one_token_wave(lane < E ? probs[wave][lane] : 0.f, lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
+    } else if (t < T && lane == 0) {
+        route_one_token(probs[wave], E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
     }
+}
+
+__global__ __launch_bounds__(FRONT_THREADS) void dispatch_kernel(RouteBufs rb, int64_t T, int E, int k, int shared) {
+    __shared__ DispatchShared dsh;
+    dispatch_block(rb, T, E, k, shared != 0, dsh);
 }
 
 __global__ void identity_routing_kernel(RouteBufs rb, int64_t rows) {
@@ -317,17 +500,32 @@ __global__ void identity_routing_kernel(RouteBufs rb, int64_t rows) {
     if (i < rows) { rb.perm_token[i] = (int)i; rb.perm_w[i] = 1.0f; rb.tok_slots[i] = (int)i; }
 }
 
-// y[t, :] = sum_j yw[slot_j, :] in ascending expert order, starting from zero as `zeros_like`
-// does, each term already rounded (broadcast_mul happens before index_add in the reference).
-__global__ __launch_bounds__(256) void combine_kernel(const float* yw, const int32_t* tok_slots, int spt,
-                                                      const float* residual, float* y, int64_t T, int H) {
-    int64_t t = blockIdx.x;
-    int h = (blockIdx.y * 256 + threadIdx.x) * 4;
+// y[t, :] = sum_j yw[slot_j, :] in ascending expert order (shared expert last), starting from
+// zero as `zeros_like` does, each term already rounded (broadcast_mul happens before index_add in
+// the reference).
+__global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs rb, int shared, const float* residual,
+                                                      float* y, int64_t T, int H) {
+    const int64_t t = blockIdx.x;
+    const int h = (blockIdx.y * 256 + threadIdx.x) * 4;
     if (h >= H) return;
+    const int k = rb.k;
+    int slots[MAX_K + 1];
+    int n = k + (shared ? 1 : 0);
+    if (rb.direct) {
+        int es[MAX_K];
+        for (int r = 0; r < k; r++) { es[r] = rb.topk_idx[t * k + r]; slots[r] = (int)(t * k + r); }
+        for (int i = 1; i < k; i++) {
+            int ev = es[i], sv = slots[i], j = i - 1;
+            while (j >= 0 && es[j] > ev) { es[j + 1] = es[j]; slots[j + 1] = slots[j]; j--; }
+            es[j + 1] = ev; slots[j + 1] = sv;
+        }
+        if (shared) slots[k] = (int)(T * k + t);
+    } else {
+        for (int j = 0; j < n; j++) slots[j] = rb.tok_slots[t * n + j];
+    }
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int j = 0; j < spt; j++) {
-        int slot = tok_slots[t * spt + j];
-        float4 v = *reinterpret_cast<const float4*>(yw + (int64_t)slot * H + h);
+    for (int j = 0; j < n; j++) {
+        float4 v = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h);
         acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
     }
     if (residual) {
@@ -338,10 +536,29 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, const int
 }
 
 // ---------------------------------------------------------------------------------------------
-hipError_t launch_front(const FrontParams& p, hipStream_t s) {
-    if (p.T == 0) return hipSuccess;
+template <int VDT>
+static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
+    if (p.E > 64 || p.H % 256) return false;
+    dim3 grid((unsigned)p.T), block(FAST_THREADS);
+    switch (p.H / 256) {
+        case 1: hipLaunchKernelGGL((front_fast_kernel<VDT, 1>), grid, block, 0, s, p); return true;
+        case 2: hipLaunchKernelGGL((front_fast_kernel<VDT, 2>), grid, block, 0, s, p); return true;
+        case 4: hipLaunchKernelGGL((front_fast_kernel<VDT, 4>), grid, block, 0, s, p); return true;
+        case 8: hipLaunchKernelGGL((front_fast_kernel<VDT, 8>), grid, block, 0, s, p); return true;
+        case 16: hipLaunchKernelGGL((front_fast_kernel<VDT, 16>), grid, block, 0, s, p); return true;
+        case 32: hipLaunchKernelGGL((front_fast_kernel<VDT, 32>), grid, block, 0, s, p); return true;
+    }
+    return false;
+}
+
+hipError_t launch_front(const FrontParams& p_in, hipStream_t s) {
+    if (p_in.T == 0) return hipSuccess;
+    const FrontParams& p = p_in;
+    static const bool no_fast = getenv("MOE_FRONT_GENERIC") != nullptr;
+    const bool q8k = p.vdt == MOE_GGML_Q8K;
+    if (!no_fast && (q8k ? launch_front_fast<MOE_GGML_Q8K>(p, s) : launch_front_fast<MOE_GGML_Q8_0>(p, s))) return hipGetLastError();
     size_t lds = (size_t)p.H * sizeof(float);
-    if (p.vdt == MOE_GGML_Q8K)
+    if (q8k)
         hipLaunchKernelGGL(front_kernel<MOE_GGML_Q8K>, dim3((unsigned)p.T), dim3(FRONT_THREADS), lds, s, p);
     else
         hipLaunchKernelGGL(front_kernel<MOE_GGML_Q8_0>, dim3((unsigned)p.T), dim3(FRONT_THREADS), lds, s, p);
@@ -363,11 +580,17 @@ hipError_t launch_identity_routing(const RouteBufs& rb, int64_t rows, hipStream_
     return hipGetLastError();
 }
 
-hipError_t launch_combine(const float* yw, const int32_t* tok_slots, int spt, const float* residual, float* y,
+hipError_t launch_dispatch(const RouteBufs& rb, int64_t T, int E, int k, bool shared, hipStream_t s) {
+    if (T == 0) return hipSuccess;
+    hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(FRONT_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,
                           int64_t T, int H, hipStream_t s) {
     if (T == 0) return hipSuccess;
     dim3 grid((unsigned)T, (unsigned)((H / 4 + 255) / 256));
-    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, s, yw, tok_slots, spt, residual, y, T, H);
+    hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, s, yw, rb, shared ? 1 : 0, residual, y, T, H);
     return hipGetLastError();
 }
 

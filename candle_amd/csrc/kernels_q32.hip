@@ -10,6 +10,7 @@
 // 8 * sum(q8) of the block, which is the same integer.
 #include "act_quant.hpp"
 #include "kernels.hpp"
+#include "slots.hpp"
 
 namespace moe {
 
@@ -84,11 +85,13 @@ constexpr int Q32_THREADS = 256;
 
 template <int DT, int TT>
 __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
+    __shared__ int list_lds[DIRECT_MAX_SLOTS];
+    __shared__ int wtot_lds[Q32_THREADS / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
     const int grp = blockIdx.y;
-    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
+    const GroupSlots gs = group_slots<Q32_THREADS>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
-    if (s_begin + tg0 >= s_end) return;
+    if (tg0 >= gs.n) return;
     const int H = p.H, F = p.F, nkb = H / 32;
     const int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
     if (rt0 >= F / 16) return;
@@ -97,12 +100,12 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
     int rowA[TT], rowD[TT][4];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        int s = s_begin + tg0 + tt * 16 + r;
-        rowA[tt] = p.rb.perm_token[s < s_end ? s : s_end - 1];
+        int ia = tg0 + tt * 16 + r;
+        rowA[tt] = slot_token(p, gs.slot(ia < gs.n ? ia : gs.n - 1));
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = p.rb.perm_token[sd < s_end ? sd : s_end - 1];
+            int id = tg0 + tt * 16 + 4 * g + i;
+            rowD[tt][i] = slot_token(p, gs.slot(id < gs.n ? id : gs.n - 1));
         }
     }
     const GroupWeights gw = p.groups[grp];
@@ -152,9 +155,9 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
             int sum = q0 + q1;
 #pragma unroll
             for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-            int slot = s_begin + tg0 + tt * 16 + 4 * g + i;
-            if (slot < s_end) {
-                int64_t hrow = slot - p.slot_origin;
+            const int pos = tg0 + tt * 16 + 4 * g + i;
+            if (pos < gs.n) {
+                int64_t hrow = gs.slot(pos) - p.slot_origin;
                 p.hq.qs[hrow * F + rt0 * 16 + r] = (int8_t)q0;
                 p.hq.qs[hrow * F + rt0 * 16 + 16 + r] = (int8_t)q1;
                 if (r == 0) {
@@ -169,11 +172,13 @@ constexpr int Q32_DOWN_STEP = 4;
 
 template <int DT, int TT>
 __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
+    __shared__ int list_lds[DIRECT_MAX_SLOTS];
+    __shared__ int wtot_lds[Q32_THREADS / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
     const int grp = blockIdx.y;
-    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
+    const GroupSlots gs = group_slots<Q32_THREADS>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
-    if (s_begin + tg0 >= s_end) return;
+    if (tg0 >= gs.n) return;
     const int H = p.H, F = p.F, nkb = F / 32;
     const int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
     if (rt >= H / 16) return;
@@ -182,12 +187,12 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
     int rowA[TT], rowD[TT][4];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        int s = s_begin + tg0 + tt * 16 + r;
-        rowA[tt] = (s < s_end ? s : s_end - 1) - p.slot_origin;
+        int ia = tg0 + tt * 16 + r;
+        rowA[tt] = gs.slot(ia < gs.n ? ia : gs.n - 1) - p.slot_origin;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = (sd < s_end ? sd : s_end - 1) - p.slot_origin;
+            int id = tg0 + tt * 16 + 4 * g + i;
+            rowD[tt][i] = gs.slot(id < gs.n ? id : gs.n - 1) - p.slot_origin;
         }
     }
     const uint8_t* tp = p.groups[grp].w2 + (size_t)rt * nkb * TB;
@@ -222,8 +227,11 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
     for (int tt = 0; tt < TT; tt++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            int slot = s_begin + tg0 + tt * 16 + 4 * g + i;
-            if (slot < s_end) p.yw[(int64_t)slot * H + rt * 16 + r] = acc[tt][i] * p.rb.perm_w[slot];
+            const int pos = tg0 + tt * 16 + 4 * g + i;
+            if (pos < gs.n) {
+                const int slot = gs.slot(pos);
+                p.yw[(int64_t)slot * H + rt * 16 + r] = acc[tt][i] * slot_weight(p, slot);
+            }
         }
 }
 

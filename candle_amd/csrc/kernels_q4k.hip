@@ -16,8 +16,11 @@
 //                    quantised to Q8K in the epilogue (Mlp::forward, quantized_llama.rs:124-131;
 //                    the re-quantisation is what k_quants::matmul does to the lhs of w2).
 //   q4k_down_kernel  yw[slot, :] = (W2 h[slot]) * routing weight (quantized_llama.rs:199-201).
+#include <cstdlib>
+
 #include "act_quant.hpp"
 #include "kernels.hpp"
+#include "slots.hpp"
 
 namespace moe {
 
@@ -29,11 +32,26 @@ struct Q4KTile {
     uint4 q0, q1, sc;
 };
 
+// Loads go through explicit global-address-space pointers made of a wave-uniform base and a 32-bit
+// per-lane offset: the base then lives in scalar registers and the instruction is a global (not
+// flat) load, which keeps 64-bit addresses out of the vector register file.
+typedef const __attribute__((address_space(1))) uint8_t* gbytes;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <typename T>
+__device__ inline T gload(const void* uniform_base, uint32_t off) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) T*>((gbytes)uniform_base + off);
+}
+template <>
+__device__ inline uint4 gload<uint4>(const void* uniform_base, uint32_t off) {
+    u32x4 v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4*>((gbytes)uniform_base + off);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ inline Q4KTile load_q4k_tile(const uint8_t* tile, int lane) {
     Q4KTile t;
-    t.q0 = *reinterpret_cast<const uint4*>(tile + lane * 16);
-    t.q1 = *reinterpret_cast<const uint4*>(tile + 1024 + lane * 16);
-    t.sc = *reinterpret_cast<const uint4*>(tile + 2048 + (lane & 15) * 16);
+    t.q0 = gload<uint4>(tile, (uint32_t)lane * 16u);
+    t.q1 = gload<uint4>(tile, 1024u + (uint32_t)lane * 16u);
+    t.sc = gload<uint4>(tile, 2048u + (uint32_t)(lane & 15) * 16u);
     return t;
 }
 
@@ -41,24 +59,26 @@ __device__ inline Q4KTile load_q4k_tile(const uint8_t* tile, int lane) {
 struct Q8KOperand {
     uint4 a[4];   // pair P: sub-block 2P (x,y) and 2P+1 (z,w), this lane's 8-element chunk
     v4h bs;       // bsums 4g..4g+3 of the lane's slot (l%16)
-    float yd[4];  // Q8K scale of the lane's four output slots (4g+i)
+    float yd;     // Q8K scale of the lane's own slot (l%16)
 };
 
-__device__ inline Q8KOperand load_q8k_operand(const ActBuf& ab, int K, int nsb, int sb, int rowA, const int rowD[4], int g) {
+__device__ inline Q8KOperand load_q8k_operand(const ActBuf& ab, int K, int nsb, int sb, int rowA, int g) {
     Q8KOperand o;
-    const int8_t* base = ab.qs + (int64_t)rowA * K + sb * 256 + g * 16;
+    // uniform base pointers + 32-bit per-lane offsets (rows * K < 2^31 is checked on the host)
+    const uint32_t qoff = (uint32_t)rowA * (uint32_t)K + (uint32_t)(sb * 256 + g * 16);
+    const uint32_t boff = ((uint32_t)rowA * (uint32_t)nsb + (uint32_t)sb);
 #pragma unroll
-    for (int P = 0; P < 4; P++) o.a[P] = *reinterpret_cast<const uint4*>(base + P * 64);
-    o.bs = *reinterpret_cast<const v4h*>(reinterpret_cast<const __half*>(ab.bsum) + ((int64_t)rowA * nsb + sb) * 16 + 4 * g);
-#pragma unroll
-    for (int i = 0; i < 4; i++) o.yd[i] = ab.d[(int64_t)rowD[i] * nsb + sb];
+    for (int P = 0; P < 4; P++) o.a[P] = gload<uint4>(ab.qs, qoff + P * 64);
+    o.bs = gload<v4h>(ab.bsum, (boff * 16 + 4 * g) * 2);
+    o.yd = gload<float>(ab.d, boff * 4);
     return o;
 }
 
 __device__ inline long pack64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
 
 // acc[i] += contribution of one (16 rows x 256 k) weight tile against one 16-slot operand.
-__device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, int g, float acc[4]) {
+// yd[i] is the activation scale of output slot 4g+i.
+__device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
     const uint32_t M4 = 0x0f0f0f0fu;
     const uint32_t hdr = w.sc.x, u0 = w.sc.y, u1 = w.sc.z, u2 = w.sc.w;
     const float d = __half2float(__ushort_as_half((unsigned short)(hdr & 0xffffu)));
@@ -96,46 +116,146 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, int g, flo
     v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, mB, zf, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const float dd = d * A.yd[i];
-        const float dm = dmin * A.yd[i];
+        const float dd = d * yd[i];
+        const float dm = dmin * yd[i];
         acc[i] += dd * (float)isum[i];
         acc[i] -= dm * Dm[i];
+    }
+}
+
+// One wave, NT weight tiles per super-block (tp[0..NT), each walking along K), TT 16-slot operand
+// tiles shared by all of them.  RING tile buffers rotate over the item sequence (sb, j): a buffer
+// is refilled with the item RING places ahead as soon as it has been consumed, so RING tiles
+// (2304 B each per wave) are in flight while one is being multiplied.
+template <int TT, int NT, int RING>
+__device__ inline void q4k_engine(const uint8_t* const tp[NT], const ActBuf& ab, int K, int nsb, int sb_lo, int sb_hi,
+                                  const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
+    static_assert(NT % RING == 0, "ring must divide the tiles per super-block");
+    if (sb_lo >= sb_hi) return;
+    Q4KTile t[RING];
+#pragma unroll
+    for (int j = 0; j < RING; j++) t[j] = load_q4k_tile(tp[j] + (size_t)sb_lo * Q4K_TILE_BYTES, lane);
+    Q8KOperand A[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_lo, rowA[tt], g);
+    // The loop body is one basic block: prefetches past the end are redirected to the last
+    // super-block (a harmless repeated load) instead of being branched around, so that the
+    // scheduling fences below really bound the live ranges.
+    for (int sb = sb_lo; sb < sb_hi; sb++) {
+        float yd[TT][4];
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) yd[tt][i] = __shfl(A[tt].yd, 4 * g + i, 64);
+        const int sb_next = (sb + 1 < sb_hi) ? sb + 1 : sb;
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const Q4KTile w = t[j % RING];
+            const int jn = (j + RING) % NT;
+            const int sbn = (j + RING) / NT ? sb_next : sb;
+            t[j % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * Q4K_TILE_BYTES, lane);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
     }
 }
 
 __device__ inline float silu_ref(float v) { return v / (1.0f + expf_glibc(-v)); }  // op.rs:646-648
 
 // ---------------------------------------------------------------------------------------------
-constexpr int UP_THREADS = 512;
-constexpr int UP_ROWS = 256;     // rows of F per workgroup = one Q8K block of h per slot
+// Up projection.  A workgroup owns 256 rows of F of one expert (= one Q8K block of h per slot);
+// wave w carries rows [w*256/NW, (w+1)*256/NW) of both w1 and w3 over the whole of K.
+constexpr int UP_ROWS = 256;
 constexpr int HBUF_STRIDE = 260;
 
-template <int TT>
-__global__ __launch_bounds__(UP_THREADS) void q4k_up_kernel(ExpertParams p) {
-    __shared__ float hbuf[TT * 16][HBUF_STRIDE];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+template <int TT, int NW, int RING>
+__device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STRIDE], int* list_lds, int* wtot_lds) {
+    constexpr int RTW = (UP_ROWS / 16) / NW;  // row tiles per wave and matrix
+    constexpr int NT = 2 * RTW;
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
     const int grp = blockIdx.y;
-    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
+    const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
-    if (s_begin + tg0 >= s_end) return;
+    if (tg0 >= gs.n) return;
     const int H = p.H, F = p.F, nsb = H / 256;
     const int rb = blockIdx.x;
 
-    int rowA[TT], rowD[TT][4];
+    int rowA[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        int s = s_begin + tg0 + tt * 16 + r;
-        rowA[tt] = p.rb.perm_token[s < s_end ? s : s_end - 1];
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = p.rb.perm_token[sd < s_end ? sd : s_end - 1];
-        }
+        int i = tg0 + tt * 16 + r;
+        rowA[tt] = slot_token(p, gs.slot(i < gs.n ? i : gs.n - 1));
     }
     const GroupWeights gw = p.groups[grp];
-    const int rt0 = rb * (UP_ROWS / 16) + wave * 2;
-    const uint8_t* tp[4] = {gw.w1 + (size_t)rt0 * nsb * Q4K_TILE_BYTES, gw.w1 + (size_t)(rt0 + 1) * nsb * Q4K_TILE_BYTES,
-                            gw.w3 + (size_t)rt0 * nsb * Q4K_TILE_BYTES, gw.w3 + (size_t)(rt0 + 1) * nsb * Q4K_TILE_BYTES};
+    const int rt0 = rb * (UP_ROWS / 16) + wave * RTW;
+    const uint8_t* tp[NT];
+#pragma unroll
+    for (int j = 0; j < RTW; j++) {
+        tp[j] = gw.w1 + (size_t)(rt0 + j) * nsb * Q4K_TILE_BYTES;
+        tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * nsb * Q4K_TILE_BYTES;
+    }
+    float acc[NT][TT][4];
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
+
+    q4k_engine<TT, NT, RING>(tp, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
+
+    // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+        for (int j = 0; j < RTW; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_ref(acc[j][tt][i]) * acc[RTW + j][tt][i];
+    __syncthreads();
+    const int nfb = F / 256;
+    for (int tok = wave; tok < TT * 16; tok += NW) {
+        if (tg0 + tok >= gs.n) break;
+        float4 v = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
+        int64_t hrow = gs.slot(tg0 + tok) - p.slot_origin;
+        quantize_q8k_block(v, lane, p.hq.qs + hrow * F + rb * 256, p.hq.d + hrow * nfb + rb,
+                           reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Down projection: a workgroup owns 64 weight rows (four row tiles) of one expert; its NW waves
+// split K, every wave carrying the four tiles over its K range, and the partial sums meet in LDS.
+template <int TT, int NW, int RING>
+__device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT * 4][64], int* list_lds, int* wtot_lds) {
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
+    const int grp = blockIdx.y;
+    const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
+    const int tg0 = blockIdx.z * (TT * 16);
+    if (tg0 >= gs.n) return;
+    const int H = p.H, F = p.F, nsb = F / 256;
+    const int n_rt = H / 16;
+    const int rt0 = blockIdx.x * 4;
+
+    int rowA[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        int i = tg0 + tt * 16 + r;
+        rowA[tt] = gs.slot(i < gs.n ? i : gs.n - 1) - p.slot_origin;
+    }
+    const uint8_t* w2 = p.groups[grp].w2;
+    const uint8_t* tp[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
+        tp[j] = w2 + (size_t)rt * nsb * Q4K_TILE_BYTES;
+    }
     float acc[4][TT][4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -144,138 +264,96 @@ __global__ __launch_bounds__(UP_THREADS) void q4k_up_kernel(ExpertParams p) {
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    Q4KTile cur[4], nxt[4];
-    Q8KOperand Acur[TT], Anxt[TT];
-#pragma unroll
-    for (int j = 0; j < 4; j++) cur[j] = load_q4k_tile(tp[j], lane);
-#pragma unroll
-    for (int tt = 0; tt < TT; tt++) Acur[tt] = load_q8k_operand(p.xq, H, nsb, 0, rowA[tt], rowD[tt], g);
+    const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
+    q4k_engine<TT, 4, RING>(tp, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
 
-    for (int sb = 0; sb < nsb; sb++) {
-        if (sb + 1 < nsb) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) nxt[j] = load_q4k_tile(tp[j] + (size_t)(sb + 1) * Q4K_TILE_BYTES, lane);
-#pragma unroll
-            for (int tt = 0; tt < TT; tt++) Anxt[tt] = load_q8k_operand(p.xq, H, nsb, sb + 1, rowA[tt], rowD[tt], g);
-        }
+    for (int j = 0; j < 4; j++)
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) q4k_mac(cur[j], Acur[tt], g, acc[j][tt]);
-#pragma unroll
-        for (int j = 0; j < 4; j++) cur[j] = nxt[j];
-#pragma unroll
-        for (int tt = 0; tt < TT; tt++) Acur[tt] = Anxt[tt];
-    }
-
-    // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
-#pragma unroll
-    for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                hbuf[tt * 16 + 4 * g + i][wave * 32 + j * 16 + r] = silu_ref(acc[j][tt][i]) * acc[2 + j][tt][i];
+            for (int i = 0; i < 4; i++) part[wave][(j * TT + tt) * 4 + i][lane] = acc[j][tt][i];
     __syncthreads();
-    const int nfb = F / 256;
-    for (int tok = wave; tok < TT * 16; tok += UP_THREADS / 64) {
-        int slot = s_begin + tg0 + tok;
-        if (slot >= s_end) break;
-        float4 v = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
-        int64_t hrow = slot - p.slot_origin;
-        quantize_q8k_block(v, lane, p.hq.qs + hrow * F + rb * 256, p.hq.d + hrow * nfb + rb,
-                           reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16);
+    // 4*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ...
+    for (int v = wave; v < 4 * TT * 4; v += NW) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) sum += part[w][v][lane];
+        const int j = v / (TT * 4), tt = (v / 4) % TT, i = v % 4;
+        const int pos = tg0 + tt * 16 + 4 * g + i;
+        if (pos < gs.n && rt0 + j < n_rt) {
+            const int slot = gs.slot(pos);
+            p.yw[(int64_t)slot * H + (rt0 + j) * 16 + r] = sum * slot_weight(p, slot);
+        }
     }
 }
 
+#define DEF_UP(NAME, TT, NW, RING, WPE)                                                                     \
+    __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
+        __shared__ float hbuf[TT * 16][HBUF_STRIDE];                                                        \
+        __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
+        __shared__ int wtot_lds[NW];                                                                        \
+        q4k_up_body<TT, NW, RING>(p, hbuf, list_lds, wtot_lds);                                             \
+    }
+#define DEF_DOWN(NAME, TT, NW, RING, WPE)                                                                   \
+    __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
+        __shared__ float part[NW][4 * TT * 4][64];                                                          \
+        __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
+        __shared__ int wtot_lds[NW];                                                                        \
+        q4k_down_body<TT, NW, RING>(p, part, list_lds, wtot_lds);                                           \
+    }
+
+// variant 0: 8 waves, 128 VGPRs (two workgroups per CU); variant 1: 4 waves, 168 VGPRs (three per CU)
+DEF_UP(q4k_up_t1_v0, 1, 8, 2, 4)
+DEF_UP(q4k_up_t2_v0, 2, 8, 2, 4)
+DEF_UP(q4k_up_t1_v1, 1, 4, 2, 3)
+DEF_UP(q4k_up_t2_v1, 2, 4, 2, 3)
+DEF_UP(q4k_up_t1_v2, 1, 4, 4, 3)
+DEF_UP(q4k_up_t1_v3, 1, 8, 4, 2)
+DEF_DOWN(q4k_down_t1_v0, 1, 8, 2, 4)
+DEF_DOWN(q4k_down_t2_v0, 2, 8, 2, 4)
+DEF_DOWN(q4k_down_t1_v1, 1, 4, 2, 3)
+DEF_DOWN(q4k_down_t2_v1, 2, 4, 2, 3)
+DEF_DOWN(q4k_down_t1_v2, 1, 4, 4, 3)
+DEF_DOWN(q4k_down_t1_v3, 1, 8, 4, 2)
+
 // ---------------------------------------------------------------------------------------------
-constexpr int DOWN_THREADS = 256;
-constexpr int DOWN_STEP = 4;  // super-blocks in flight per wave
-
-template <int TT>
-__global__ __launch_bounds__(DOWN_THREADS) void q4k_down_kernel(ExpertParams p) {
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
-    const int grp = blockIdx.y;
-    const int s_begin = p.rb.offsets[p.group0 + grp], s_end = p.rb.offsets[p.group0 + grp + 1];
-    const int tg0 = blockIdx.z * (TT * 16);
-    if (s_begin + tg0 >= s_end) return;
-    const int H = p.H, F = p.F, nsb = F / 256;
-    const int rt = blockIdx.x * (DOWN_THREADS / 64) + wave;
-    if (rt >= H / 16) return;
-
-    int rowA[TT], rowD[TT][4];
-#pragma unroll
-    for (int tt = 0; tt < TT; tt++) {
-        int s = s_begin + tg0 + tt * 16 + r;
-        rowA[tt] = (s < s_end ? s : s_end - 1) - p.slot_origin;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int sd = s_begin + tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = (sd < s_end ? sd : s_end - 1) - p.slot_origin;
-        }
-    }
-    const uint8_t* tp = p.groups[grp].w2 + (size_t)rt * nsb * Q4K_TILE_BYTES;
-    float acc[TT][4];
-#pragma unroll
-    for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[tt][i] = 0.f;
-
-    Q4KTile cur[DOWN_STEP], nxt[DOWN_STEP];
-#pragma unroll
-    for (int j = 0; j < DOWN_STEP; j++)
-        if (j < nsb) cur[j] = load_q4k_tile(tp + (size_t)j * Q4K_TILE_BYTES, lane);
-
-    for (int sb0 = 0; sb0 < nsb; sb0 += DOWN_STEP) {
-#pragma unroll
-        for (int j = 0; j < DOWN_STEP; j++)
-            if (sb0 + DOWN_STEP + j < nsb) nxt[j] = load_q4k_tile(tp + (size_t)(sb0 + DOWN_STEP + j) * Q4K_TILE_BYTES, lane);
-#pragma unroll
-        for (int j = 0; j < DOWN_STEP; j++) {
-            if (sb0 + j < nsb) {
-#pragma unroll
-                for (int tt = 0; tt < TT; tt++) {
-                    Q8KOperand A = load_q8k_operand(p.hq, F, nsb, sb0 + j, rowA[tt], rowD[tt], g);
-                    q4k_mac(cur[j], A, g, acc[tt]);
-                }
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < DOWN_STEP; j++) cur[j] = nxt[j];
-    }
-
-#pragma unroll
-    for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int slot = s_begin + tg0 + tt * 16 + 4 * g + i;
-            if (slot < s_end) p.yw[(int64_t)slot * H + rt * 16 + r] = acc[tt][i] * p.rb.perm_w[slot];
-        }
+static int variant(const char* name, int dflt) {
+    const char* e = getenv(name);
+    return e ? atoi(e) : dflt;
 }
-
-// ---------------------------------------------------------------------------------------------
-static inline int pick_tt(const ExpertParams& p) { return p.slot_tiles >= 2 ? 2 : 1; }
 
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    const int tt = pick_tt(p);
+    static const int v = variant("MOE_UP_VARIANT", 0);
+    const int tt = p.slot_tiles >= 2 ? 2 : 1;
     dim3 grid((unsigned)(p.F / UP_ROWS), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (tt == 1)
-        hipLaunchKernelGGL(q4k_up_kernel<1>, grid, dim3(UP_THREADS), 0, s, p);
-    else
-        hipLaunchKernelGGL(q4k_up_kernel<2>, grid, dim3(UP_THREADS), 0, s, p);
+    if (tt == 2) {
+        if (v == 1 || v == 2) hipLaunchKernelGGL(q4k_up_t2_v1, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q4k_up_t2_v0, grid, dim3(512), 0, s, p);
+    } else {
+        if (v == 1) hipLaunchKernelGGL(q4k_up_t1_v1, grid, dim3(256), 0, s, p);
+        else if (v == 2) hipLaunchKernelGGL(q4k_up_t1_v2, grid, dim3(256), 0, s, p);
+        else if (v == 3) hipLaunchKernelGGL(q4k_up_t1_v3, grid, dim3(512), 0, s, p);
+        else hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
+    }
     return hipGetLastError();
 }
 
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    const int tt = pick_tt(p);
-    const int wpb = DOWN_THREADS / 64;
-    dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (tt == 1)
-        hipLaunchKernelGGL(q4k_down_kernel<1>, grid, dim3(DOWN_THREADS), 0, s, p);
-    else
-        hipLaunchKernelGGL(q4k_down_kernel<2>, grid, dim3(DOWN_THREADS), 0, s, p);
+    static const int v = variant("MOE_DOWN_VARIANT", 0);
+    const int tt = p.slot_tiles >= 2 ? 2 : 1;
+    dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (tt == 2) {
+        if (v == 1 || v == 2) hipLaunchKernelGGL(q4k_down_t2_v1, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q4k_down_t2_v0, grid, dim3(512), 0, s, p);
+    } else {
+        if (v == 1) hipLaunchKernelGGL(q4k_down_t1_v1, grid, dim3(256), 0, s, p);
+        else if (v == 2) hipLaunchKernelGGL(q4k_down_t1_v2, grid, dim3(256), 0, s, p);
+        else if (v == 3) hipLaunchKernelGGL(q4k_down_t1_v3, grid, dim3(512), 0, s, p);
+        else hipLaunchKernelGGL(q4k_down_t1_v0, grid, dim3(512), 0, s, p);
+    }
     return hipGetLastError();
 }
 

@@ -1,0 +1,70 @@
+// How an expert kernel finds the slots (token, expert assignments) of its group.
+#pragma once
+#include "kernels.hpp"
+
+namespace moe {
+
+// View of one group's slots for one workgroup.
+struct GroupSlots {
+    int n;            // slots in the group
+    int s_begin;      // dispatched mode: first slot
+    const int* list;  // direct mode: LDS list of slot ids (ascending); nullptr when dispatched
+    __device__ inline int slot(int i) const { return list ? list[i] : s_begin + i; }
+};
+
+// Builds the view.  All threads of the workgroup must call it (it contains barriers in direct
+// mode).  `list_lds` holds DIRECT_MAX_SLOTS ints, `wtot_lds` one int per wave.
+template <int NTHREADS>
+__device__ inline GroupSlots group_slots(const ExpertParams& p, int grp, int* list_lds, int* wtot_lds) {
+    GroupSlots gs;
+    if (!p.rb.direct) {
+        gs.s_begin = p.rb.offsets[p.group0 + grp];
+        gs.n = p.rb.offsets[p.group0 + grp + 1] - gs.s_begin;
+        gs.list = nullptr;
+        return gs;
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int A = p.rb.T * p.rb.k;
+    gs.s_begin = 0;
+    gs.list = list_lds;
+    if (p.is_shared) {  // every token, in order
+        for (int i = tid; i < p.rb.T; i += NTHREADS) list_lds[i] = A + i;
+        __syncthreads();
+        gs.n = p.rb.T;
+        return gs;
+    }
+    const int e = p.group0 + grp;
+    int base = 0;
+    const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int c0 = 0; c0 < A; c0 += NTHREADS) {
+        const int a = c0 + tid;
+        const bool m = a < A && p.rb.topk_idx[a] == e;
+        const unsigned long long b = __ballot(m);
+        if (lane == 0) wtot_lds[wave] = __popcll(b);
+        __syncthreads();
+        int off = base, tot = 0;
+#pragma unroll
+        for (int w = 0; w < NTHREADS / 64; w++) {
+            const int c = wtot_lds[w];
+            off += (w < wave) ? c : 0;
+            tot += c;
+        }
+        if (m) list_lds[off + __popcll(b & lt)] = a;
+        base += tot;
+        __syncthreads();
+    }
+    gs.n = base;
+    return gs;
+}
+
+// token row / routing weight of a slot
+__device__ inline int slot_token(const ExpertParams& p, int slot) {
+    if (!p.rb.direct) return p.rb.perm_token[slot];
+    return p.is_shared ? slot - p.rb.T * p.rb.k : slot / p.rb.k;
+}
+__device__ inline float slot_weight(const ExpertParams& p, int slot) {
+    if (!p.rb.direct) return p.rb.perm_w[slot];
+    return p.is_shared ? p.rb.shared_w[slot - p.rb.T * p.rb.k] : p.rb.topk_w[slot];
+}
+
+}  // namespace moe
