@@ -280,7 +280,11 @@ extern "C" void moe_layer_destroy(moe_layer* L) {
 }
 
 // Enqueue one forward on `s`.  Caller holds L->mu.
-static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s) {
+// Stage marks for moe_layer_forward_timed: events recorded between the launches.
+enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_DOWN, ST_SHARED, ST_COMBINE, ST_COUNT };
+
+static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
+#define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
     int rc = reserve_workspace(L, T);
     if (rc) return rc;
     // a previous call may still be running on another stream and shares the workspace
@@ -300,8 +304,11 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     const bool direct = T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     fp.rb.direct = direct ? 1 : 0;
+    MOE_MARK(ST_BEGIN);
     MOE_HIP_CHECK(launch_front(fp, s));
+    MOE_MARK(ST_FRONT);
     if (!direct) MOE_HIP_CHECK(launch_dispatch(fp.rb, T, (int)L->E, (int)L->k, shared, s));
+    MOE_MARK(ST_DISPATCH);
 
     ExpertParams ep;
     ep.dt = L->dt; ep.H = (int)L->H; ep.F = (int)L->F;
@@ -312,7 +319,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.max_rows = T;
     ep.slot_tiles = (T * L->k > 9 * L->E) ? 2 : 1;   // expected rows per expert above ~9: carry 32 slots per pass
     MOE_HIP_CHECK(launch_expert_up(ep, s));
+    MOE_MARK(ST_UP);
     MOE_HIP_CHECK(launch_expert_down(ep, s));
+    MOE_MARK(ST_DOWN);
     if (shared) {
         ExpertParams sp = ep;
         sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
@@ -322,7 +331,10 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         MOE_HIP_CHECK(launch_expert_up(sp, s));
         MOE_HIP_CHECK(launch_expert_down(sp, s));
     }
+    MOE_MARK(ST_SHARED);
     MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    MOE_MARK(ST_COMBINE);
+#undef MOE_MARK
     L->last_direct = direct;
     MOE_HIP_CHECK(hipEventRecord(L->done, s));
     L->last_T = T;
@@ -336,6 +348,24 @@ extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T
     std::lock_guard<std::mutex> lk(L->mu);
     if (T == 0) { L->last_T = 0; return MOE_OK; }
     return enqueue_forward(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int moe_layer_forward_timed(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream, float* stage_ms) {
+    if (!L || T <= 0 || !d_x || !d_y || !stage_ms || d_x == d_y) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_timed");
+    if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
+    std::lock_guard<std::mutex> lk(L->mu);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    hipEvent_t marks[ST_COUNT] = {};
+    int rc = MOE_OK;
+    for (int i = 0; i < ST_COUNT && !rc; i++)
+        if (hipEventCreate(&marks[i]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventCreate failed");
+    if (!rc) rc = enqueue_forward(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s, marks);
+    if (!rc && hipEventSynchronize(marks[ST_COMBINE]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventSynchronize failed");
+    for (int i = 0; i + 1 < ST_COUNT && !rc; i++)
+        if (hipEventElapsedTime(&stage_ms[i], marks[i], marks[i + 1]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventElapsedTime failed");
+    for (int i = 0; i < ST_COUNT; i++)
+        if (marks[i]) (void)hipEventDestroy(marks[i]);
+    return rc;
 }
 
 extern "C" int moe_layer_forward(moe_layer* L, const float* x, int64_t T, float* y) {

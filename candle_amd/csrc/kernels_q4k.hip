@@ -127,14 +127,22 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
 // tiles shared by all of them.  RING tile buffers rotate over the item sequence (sb, j): a buffer
 // is refilled with the item RING places ahead as soon as it has been consumed, so RING tiles
 // (2304 B each per wave) are in flight while one is being multiplied.
-template <int TT, int NT, int RING>
-__device__ inline void q4k_engine(const uint8_t* const tp[NT], const ActBuf& ab, int K, int nsb, int sb_lo, int sb_hi,
-                                  const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
+// Tiles of one matrix are ordered [super-block][row tile] (sb-major): all the waves of the grid that
+// are at the same step of their K walk then read one contiguous region, which spreads the requests
+// evenly over the HBM channels.  `sb_stride` = row tiles of the matrix * Q4K_TILE_BYTES.
+template <int NT, int RING>
+__device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t sb_stride, int sb_lo, int lane, Q4KTile t[RING]) {
+#pragma unroll
+    for (int j = 0; j < RING; j++) t[j] = load_q4k_tile(tp[j] + (size_t)sb_lo * sb_stride, lane);
+}
+
+// `t` must have been filled by q4k_engine_prefetch for sb_lo (callers issue it before they know
+// their slot list, so the first weight tiles are already on their way while the list is built).
+template <int TT, int NT, int RING, int DBG = 0>
+__device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride, Q4KTile t[RING], const ActBuf& ab, int K, int nsb,
+                                  int sb_lo, int sb_hi, const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
     static_assert(NT % RING == 0, "ring must divide the tiles per super-block");
     if (sb_lo >= sb_hi) return;
-    Q4KTile t[RING];
-#pragma unroll
-    for (int j = 0; j < RING; j++) t[j] = load_q4k_tile(tp[j] + (size_t)sb_lo * Q4K_TILE_BYTES, lane);
     Q8KOperand A[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_lo, rowA[tt], g);
@@ -153,17 +161,28 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], const ActBuf& ab,
             const Q4KTile w = t[j % RING];
             const int jn = (j + RING) % NT;
             const int sbn = (j + RING) / NT ? sb_next : sb;
-            t[j % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * Q4K_TILE_BYTES, lane);
+            t[j % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * sb_stride, lane);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
+            for (int tt = 0; tt < TT; tt++) {
+                if (DBG == 1)  // timing experiment: consume the loads without the arithmetic
+                    acc[j][tt][0] += __uint_as_float((w.q0.x ^ w.q0.w ^ w.q1.y ^ w.q1.z ^ w.sc.z ^ A[tt].a[0].x ^ A[tt].a[3].w) & 0x007fffffu);
+                else
+                    q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (DBG != 2) {  // DBG 2: timing experiment without the per-super-block operand reload
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
+            for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
+        }
     }
 }
 
+// silu for the Q4K path: v / (1 + exp(-v)) with the hardware exp2.  The first product is not
+// bit-identical to the CPU's anyway (f32 order), so the last-ulp accuracy of exp buys nothing here,
+// while the double-precision exp costs microseconds in every workgroup's epilogue.
+__device__ inline float silu_fast(float v) { return v / (1.0f + __expf(-v)); }
 __device__ inline float silu_ref(float v) { return v / (1.0f + expf_glibc(-v)); }  // op.rs:646-648
 
 // ---------------------------------------------------------------------------------------------
@@ -172,32 +191,37 @@ __device__ inline float silu_ref(float v) { return v / (1.0f + expf_glibc(-v)); 
 constexpr int UP_ROWS = 256;
 constexpr int HBUF_STRIDE = 260;
 
-template <int TT, int NW, int RING>
+template <int TT, int NW, int RING, int DBG = 0>
 __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STRIDE], int* list_lds, int* wtot_lds) {
     constexpr int RTW = (UP_ROWS / 16) / NW;  // row tiles per wave and matrix
     constexpr int NT = 2 * RTW;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
     const int grp = blockIdx.y;
+    const int H = p.H, F = p.F, nsb = H / 256;
+    const int rb = blockIdx.x;
+    const GroupWeights gw = p.groups[grp];
+    const int rt0 = rb * (UP_ROWS / 16) + wave * RTW;
+    const uint8_t* tp[NT];
+#pragma unroll
+    for (int j = 0; j < RTW; j++) {
+        tp[j] = gw.w1 + (size_t)(rt0 + j) * Q4K_TILE_BYTES;
+        tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * Q4K_TILE_BYTES;
+    }
+    const size_t sb_stride = (size_t)(F / 16) * Q4K_TILE_BYTES;
+    // first weight tiles go out before anything else; an expert without tokens wastes them
+    Q4KTile ring[RING];
+    q4k_engine_prefetch<NT, RING>(tp, sb_stride, 0, lane, ring);
+
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
     if (tg0 >= gs.n) return;
-    const int H = p.H, F = p.F, nsb = H / 256;
-    const int rb = blockIdx.x;
 
     int rowA[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
         int i = tg0 + tt * 16 + r;
         rowA[tt] = slot_token(p, gs.slot(i < gs.n ? i : gs.n - 1));
-    }
-    const GroupWeights gw = p.groups[grp];
-    const int rt0 = rb * (UP_ROWS / 16) + wave * RTW;
-    const uint8_t* tp[NT];
-#pragma unroll
-    for (int j = 0; j < RTW; j++) {
-        tp[j] = gw.w1 + (size_t)(rt0 + j) * nsb * Q4K_TILE_BYTES;
-        tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * nsb * Q4K_TILE_BYTES;
     }
     float acc[NT][TT][4];
 #pragma unroll
@@ -207,7 +231,7 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<TT, NT, RING>(tp, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
+    q4k_engine<TT, NT, RING, DBG>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
 
     // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
 #pragma unroll
@@ -216,7 +240,7 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
         for (int j = 0; j < RTW; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_ref(acc[j][tt][i]) * acc[RTW + j][tt][i];
+                hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
     __syncthreads();
     const int nfb = F / 256;
     for (int tok = wave; tok < TT * 16; tok += NW) {
@@ -236,25 +260,30 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
     const int grp = blockIdx.y;
-    const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
-    const int tg0 = blockIdx.z * (TT * 16);
-    if (tg0 >= gs.n) return;
     const int H = p.H, F = p.F, nsb = F / 256;
     const int n_rt = H / 16;
     const int rt0 = blockIdx.x * 4;
+    const uint8_t* w2 = p.groups[grp].w2;
+    const uint8_t* tp[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
+        tp[j] = w2 + (size_t)rt * Q4K_TILE_BYTES;
+    }
+    const size_t sb_stride = (size_t)n_rt * Q4K_TILE_BYTES;
+    const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
+    Q4KTile ring[RING];
+    q4k_engine_prefetch<4, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, lane, ring);
+
+    const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
+    const int tg0 = blockIdx.z * (TT * 16);
+    if (tg0 >= gs.n) return;
 
     int rowA[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
         int i = tg0 + tt * 16 + r;
         rowA[tt] = gs.slot(i < gs.n ? i : gs.n - 1) - p.slot_origin;
-    }
-    const uint8_t* w2 = p.groups[grp].w2;
-    const uint8_t* tp[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
-        tp[j] = w2 + (size_t)rt * nsb * Q4K_TILE_BYTES;
     }
     float acc[4][TT][4];
 #pragma unroll
@@ -264,8 +293,7 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
-    q4k_engine<TT, 4, RING>(tp, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
+    q4k_engine<TT, 4, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
 
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -288,12 +316,13 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
     }
 }
 
-#define DEF_UP(NAME, TT, NW, RING, WPE)                                                                     \
+#define DEF_UP(NAME, TT, NW, RING, WPE) DEF_UP_D(NAME, TT, NW, RING, WPE, 0)
+#define DEF_UP_D(NAME, TT, NW, RING, WPE, DBG)                                                                   \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ float hbuf[TT * 16][HBUF_STRIDE];                                                        \
         __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
         __shared__ int wtot_lds[NW];                                                                        \
-        q4k_up_body<TT, NW, RING>(p, hbuf, list_lds, wtot_lds);                                             \
+        q4k_up_body<TT, NW, RING, DBG>(p, hbuf, list_lds, wtot_lds);                                             \
     }
 #define DEF_DOWN(NAME, TT, NW, RING, WPE)                                                                   \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
@@ -310,6 +339,13 @@ DEF_UP(q4k_up_t1_v1, 1, 4, 2, 3)
 DEF_UP(q4k_up_t2_v1, 2, 4, 2, 3)
 DEF_UP(q4k_up_t1_v2, 1, 4, 4, 3)
 DEF_UP(q4k_up_t1_v3, 1, 8, 4, 2)
+DEF_UP_D(q4k_up_t1_v8, 1, 4, 2, 3, 1)
+DEF_UP_D(q4k_up_t1_v9, 1, 4, 2, 3, 2)
+DEF_UP_D(q4k_up_t1_v10, 1, 4, 4, 3, 1)
+DEF_UP_D(q4k_up_t1_v11, 1, 8, 2, 4, 1)
+DEF_UP_D(q4k_up_t1_v12, 1, 8, 4, 4, 1)
+DEF_UP_D(q4k_up_t1_v13, 1, 4, 8, 3, 1)
+DEF_UP_D(q4k_up_t1_v14, 1, 16, 2, 4, 1)
 DEF_DOWN(q4k_down_t1_v0, 1, 8, 2, 4)
 DEF_DOWN(q4k_down_t2_v0, 2, 8, 2, 4)
 DEF_DOWN(q4k_down_t1_v1, 1, 4, 2, 3)
@@ -325,7 +361,7 @@ static int variant(const char* name, int dflt) {
 
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    static const int v = variant("MOE_UP_VARIANT", 0);
+    static const int v = variant("MOE_UP_VARIANT", 1);
     const int tt = p.slot_tiles >= 2 ? 2 : 1;
     dim3 grid((unsigned)(p.F / UP_ROWS), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     if (tt == 2) {
@@ -335,6 +371,13 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
         if (v == 1) hipLaunchKernelGGL(q4k_up_t1_v1, grid, dim3(256), 0, s, p);
         else if (v == 2) hipLaunchKernelGGL(q4k_up_t1_v2, grid, dim3(256), 0, s, p);
         else if (v == 3) hipLaunchKernelGGL(q4k_up_t1_v3, grid, dim3(512), 0, s, p);
+        else if (v == 8) hipLaunchKernelGGL(q4k_up_t1_v8, grid, dim3(256), 0, s, p);
+        else if (v == 9) hipLaunchKernelGGL(q4k_up_t1_v9, grid, dim3(256), 0, s, p);
+        else if (v == 10) hipLaunchKernelGGL(q4k_up_t1_v10, grid, dim3(256), 0, s, p);
+        else if (v == 11) hipLaunchKernelGGL(q4k_up_t1_v11, grid, dim3(512), 0, s, p);
+        else if (v == 12) hipLaunchKernelGGL(q4k_up_t1_v12, grid, dim3(512), 0, s, p);
+        else if (v == 13) hipLaunchKernelGGL(q4k_up_t1_v13, grid, dim3(256), 0, s, p);
+        else if (v == 14) hipLaunchKernelGGL(q4k_up_t1_v14, grid, dim3(1024), 0, s, p);
         else hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
     }
     return hipGetLastError();
@@ -342,7 +385,7 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
 
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    static const int v = variant("MOE_DOWN_VARIANT", 0);
+    static const int v = variant("MOE_DOWN_VARIANT", 1);
     const int tt = p.slot_tiles >= 2 ? 2 : 1;
     dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     if (tt == 2) {

@@ -70,7 +70,7 @@ __global__ void relayout_q4k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t 
     int ch = (int)(c % 144);
     int64_t rt = tile / nsb;
     int sb = (int)(tile % nsb);
-    uint8_t* dst = tiled + tile * Q4K_TILE_BYTES + ch * 16;
+    uint8_t* dst = tiled + (sb * n_rt + rt) * Q4K_TILE_BYTES + ch * 16;  // tiles ordered [sb][rt]
     if (ch < 128) {
         int half = ch / 64, l = ch % 64, r = l % 16, g = l / 16;
         const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144 + 16;
@@ -123,7 +123,7 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
     int r = (int)(row % 16);
     if (dt == MOE_GGML_Q4K) {
         int nsb = (int)(k / 256), sb = col / 256, e = col % 256;
-        const uint8_t* tile = tiled + (rt * nsb + sb) * Q4K_TILE_BYTES;
+        const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q4K_TILE_BYTES;
         // original qs byte index of element e: (e/64)*32 + e%32 ; that byte sits in pair P = byte/32,
         // chunk g = (byte%32)/8, position byte%8
         int byte = (e / 64) * 32 + (e % 32);

@@ -58,7 +58,8 @@ inline int vecdot_dtype(int dt) {  // GgmlType::VecDotType, k_quants.rs:163,584,
 //         [0,1024)    lane l: qs[row l%16][ 0+8g .. 0+8g+8) | qs[row][32+8g .. +8)   (g = l/16)
 //         [1024,2048) lane l: qs[row l%16][64+8g ..       ) | qs[row][96+8g .. +8)
 //         [2048,2304) row r : the block's first 16 bytes (d, dmin, 12 packed scale bytes)
-//       tiles ordered [rt][sb]: a wave walking along K reads contiguous memory.
+//       tiles ordered [sb][rt]: the waves of a launch that are at the same step of their walk along
+//       K read one contiguous region, which keeps the HBM channels evenly loaded.
 //  Q8_0 tile(rt, kb) = 544 B for 16 rows x one 32-element block:
 //         [0,512)   lane l: qs[row l%16][8g .. 8g+8)
 //         [512,544) row r : d (f16)

@@ -60,6 +60,7 @@ def load_library():
     L.moe_layer_destroy.restype = None
     L.moe_layer_forward.argtypes = [vp, vp, i64, vp]
     L.moe_layer_forward_device.argtypes = [vp, vp, i64, vp, vp]
+    L.moe_layer_forward_timed.argtypes = [vp, vp, i64, vp, vp, vp]
     L.moe_layer_last_logits.argtypes = [vp, vp, i64]
     L.moe_layer_last_routing.argtypes = [vp, i64, vp, vp, vp, vp, vp]
     L.moe_layer_dequantize_weight.argtypes = [vp, i64, C.c_int, vp, i64]
@@ -258,6 +259,18 @@ class SparseMoeBlock:
         return y
 
     __call__ = forward
+
+    STAGES = ("front", "dispatch", "up", "down", "shared", "combine")
+
+    def forward_timed(self, xs, out):
+        """One forward on torch CUDA tensors with HIP events between the launches (on torch's
+        current stream); returns {stage: milliseconds}.  Synchronises."""
+        import torch
+        T = xs.numel() // self.hidden
+        ms = (C.c_float * 6)()
+        stream = torch.cuda.current_stream(xs.device).cuda_stream
+        _check(load_library().moe_layer_forward_timed(self._h, xs.data_ptr(), T, out.data_ptr(), stream, ms))
+        return dict(zip(self.STAGES, [float(v) for v in ms]))
 
     def last_logits(self, n_tokens):
         out = np.empty((n_tokens, self.n_experts), dtype=np.float32)

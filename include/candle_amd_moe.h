@@ -88,6 +88,12 @@ int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float*
  * already keeps activations on the GPU uses (no PCIe in the path). */
 int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
 
+/* Measurement aid (no counterpart in the reference): one forward as moe_layer_forward_device with
+ * HIP events recorded on `hip_stream` between the launches; waits for completion and returns the
+ * elapsed milliseconds of the six stages in stage_ms[0..5]: front (router + activation quantiser),
+ * dispatch (0 for small batches), up (w1/w3 + SiLU), down (w2), shared expert, combine. */
+int moe_layer_forward_timed(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream, float* stage_ms);
+
 /* Router logits [n_tokens, E] (after the optional bias) that the last forward on this layer
  * computed, copied to the host.  Debug / parity hook: candle computes these with the `gemm`
  * crate whose f32 summation order is not part of the reference tree. */
