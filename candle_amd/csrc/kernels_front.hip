@@ -221,12 +221,16 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
         sum2 += v.w * v.w;
     }
     if (p.rms_alpha) {
-        sum2 = wave_sum(sum2);
-        if (lane == 0) red[wave] = sum2;
+        // sum of squares left to right, as the reference does (see front_fast_kernel)
         __syncthreads();
-        float tot = 0.f;
-        for (int w = 0; w < FRONT_THREADS / 64; w++) tot += red[w];
-        float m = sqrtf(tot / (float)H + p.rms_eps);
+        if (tid == 0) {
+            float tot = 0.f;
+            for (int h = 0; h < H; h++) tot += xrow[h] * xrow[h];
+            red[0] = sqrtf(tot / (float)H + p.rms_eps);
+        }
+        __syncthreads();
+        const float m = red[0];
+        __syncthreads();
         for (int h = tid; h < H; h += FRONT_THREADS) xrow[h] = xrow[h] / m * p.rms_alpha[h];
     }
     __syncthreads();
@@ -396,11 +400,29 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
         xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
     }
     if (p.rms_alpha) {
-        float sum2 = 0.f;
+        // rms_norm (candle-nn/src/ops.rs:504-515) sums the squares left to right in f32.  A different
+        // order changes the divisor in the last ulp, which flips quantised activations now and then
+        // and moves a whole output row by 1e-3 of its rms, so the sum is taken serially by one lane
+        // (H dependent adds, a few microseconds) to keep the normalised row bit-identical.
+        __shared__ float sq[H];
+        __shared__ float m_lds;
+        if (wave == 0) {
 #pragma unroll
-        for (int i = 0; i < NCH * 4; i++) sum2 += xr[i] * xr[i];
-        sum2 = wave_sum(sum2);
-        const float m = sqrtf(sum2 / (float)H + p.rms_eps);
+            for (int i = 0; i < NCH; i++)
+                *reinterpret_cast<float4*>(&sq[i * 256 + lane * 4]) =
+                    make_float4(xr[4 * i] * xr[4 * i], xr[4 * i + 1] * xr[4 * i + 1], xr[4 * i + 2] * xr[4 * i + 2], xr[4 * i + 3] * xr[4 * i + 3]);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float sum2 = 0.f;
+            for (int h = 0; h < H; h += 4) {
+                const float4 v = *reinterpret_cast<const float4*>(&sq[h]);
+                sum2 += v.x; sum2 += v.y; sum2 += v.z; sum2 += v.w;
+            }
+            m_lds = sqrtf(sum2 / (float)H + p.rms_eps);
+        }
+        __syncthreads();
+        const float m = m_lds;
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const float4 a = *reinterpret_cast<const float4*>(p.rms_alpha + i * 256 + lane * 4);
