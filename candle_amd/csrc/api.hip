@@ -1,6 +1,7 @@
 // C ABI of the library (see include/candle_amd_moe.h): layer objects, device memory and the
 // sequence of kernel launches of one forward pass.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -98,7 +99,7 @@ struct ActStore {
 };
 
 struct RouteStore {
-    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots;
+    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots, tile_tab;
     int reserve(int64_t T, int E, int k, bool shared) {
         int rc;
         const int64_t S = T * k + (shared ? T : 0);
@@ -110,6 +111,7 @@ struct RouteStore {
         if ((rc = perm_token.reserve((size_t)S * 4))) return rc;
         if ((rc = perm_w.reserve((size_t)S * 4))) return rc;
         if ((rc = tok_slots.reserve((size_t)T * (k + 1) * 4))) return rc;
+        if ((rc = tile_tab.reserve((size_t)(1 + 2 * max_gemm_tiles(S, E + 1)) * 4))) return rc;
         return MOE_OK;
     }
     RouteBufs view() const {
@@ -122,6 +124,7 @@ struct RouteStore {
         r.perm_token = perm_token.as<int32_t>();
         r.perm_w = perm_w.as<float>();
         r.tok_slots = tok_slots.as<int32_t>();
+        r.tile_tab = tile_tab.as<int32_t>();
         return r;
     }
 };
@@ -143,7 +146,7 @@ struct moe_layer {
     int64_t cap_T = -1;
     RouteStore route;
     ActStore xq, hq, hq_shared;
-    DevBuf yw, x_dev, y_dev;
+    DevBuf yw, x_dev, y_dev, hbuf;
     hipStream_t stream = nullptr;   // used by the host-pointer entry
     hipEvent_t done = nullptr;      // end of the last enqueued forward
     int64_t last_T = 0;
@@ -318,10 +321,25 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.yw = L->yw.as<float>();
     ep.max_rows = T;
     ep.slot_tiles = (T * L->k > 9 * L->E) ? 2 : 1;   // expected rows per expert above ~9: carry 32 slots per pass
-    MOE_HIP_CHECK(launch_expert_up(ep, s));
-    MOE_MARK(ST_UP);
-    MOE_HIP_CHECK(launch_expert_down(ep, s));
-    MOE_MARK(ST_DOWN);
+    // large Q4K batches take the tiled MFMA path: F a multiple of 64, H of 128, many rows per expert
+    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    const bool tiled = !no_gemm && !direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
+                       T * L->k >= 32 * L->E;
+    if (tiled) {
+        if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
+        ep.hbuf = L->hbuf.as<float>();
+        ep.n_slots = T * L->k;
+        MOE_HIP_CHECK(launch_q4k_gemm_up(ep, s));
+        MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
+        MOE_MARK(ST_UP);
+        MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
+        MOE_MARK(ST_DOWN);
+    } else {
+        MOE_HIP_CHECK(launch_expert_up(ep, s));
+        MOE_MARK(ST_UP);
+        MOE_HIP_CHECK(launch_expert_down(ep, s));
+        MOE_MARK(ST_DOWN);
+    }
     if (shared) {
         ExpertParams sp = ep;
         sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;

@@ -15,6 +15,10 @@ struct RouteBufs {
     int32_t* perm_token = nullptr;  // [S] token row of every slot
     float* perm_w = nullptr;        // [S] routing weight of every slot
     int32_t* tok_slots = nullptr;   // [T, k(+1)] slots of a token, ascending expert index
+    // Work list of the tiled (prefill) expert kernels, written by the dispatch kernel: [0] = number
+    // of 64-slot tiles, then (group, first position inside the group) per tile.  Built from the
+    // real list lengths, so a skewed routing yields tiles in proportion to each expert's load.
+    int32_t* tile_tab = nullptr;
     // Slot numbering.  direct == 0: slots are grouped by expert (offsets / perm_* built by the
     // dispatch kernel).  direct == 1 (small batches): slot of assignment (token t, rank r) is
     // simply t*k + r, the shared expert's slots are T*k + t, and every consumer derives its
@@ -23,6 +27,8 @@ struct RouteBufs {
     int T = 0, k = 0;
 };
 constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a dispatch pass
+constexpr int GEMM_TILE_SLOTS = 64;     // slots per tile of the tiled expert kernels
+inline int64_t max_gemm_tiles(int64_t slots, int64_t groups) { return slots / GEMM_TILE_SLOTS + groups + 1; }
 
 struct FrontParams {
     const float* x = nullptr;       // [T, H]
@@ -65,11 +71,19 @@ struct ExpertParams {
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
     int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1 or 2)
     int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)
+    float* hbuf = nullptr;          // tiled path only: f32 intermediate [slots, F] before re-quantisation
+    int64_t n_slots = 0;            // tiled path only: total slots (bounds the tile grid)
 };
 // h = silu(W1 x) * (W3 x), quantised to the activation format, for every slot of every group.
 hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s);
 // yw[slot] = (W2 h[slot]) * perm_w[slot]
 hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
+
+// Tiled (prefill) variants for Q4K in dispatched mode: activations staged through LDS, weights
+// unpacked and pre-scaled per wave, v_mfma_i32_32x32x32_i8.  up writes f32 h into p.hbuf (the
+// caller re-quantises it), down writes yw.
+hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
+hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 
 // y[t] = sum over the token's slots (ascending expert index, shared expert last) of yw[slot] (+ residual[t]).
 hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,

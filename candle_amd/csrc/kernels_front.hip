@@ -147,6 +147,19 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         }
     }
     for (int e = tid; e <= E + (shared ? 1 : 0); e += FRONT_THREADS) rb.offsets[e] = sh.off[e];
+    if (tid == 0 && rb.tile_tab) {  // work list of the tiled expert kernels
+        int n = 0;
+        const int G = E + (shared ? 1 : 0);
+        for (int gi = 0; gi < G; gi++) {
+            const int len = sh.off[gi + 1] - sh.off[gi];
+            for (int pos = 0; pos < len; pos += GEMM_TILE_SLOTS) {
+                rb.tile_tab[1 + 2 * n] = gi;
+                rb.tile_tab[2 + 2 * n] = pos;
+                n++;
+            }
+        }
+        rb.tile_tab[0] = n;
+    }
     __syncthreads();
     // phase 3: stable placement
     const int kk = k + (shared ? 1 : 0);
