@@ -323,8 +323,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.slot_tiles = (T * L->k > 9 * L->E) ? 2 : 1;   // expected rows per expert above ~9: carry 32 slots per pass
     // large Q4K batches take the tiled MFMA path: F a multiple of 64, H of 128, many rows per expert
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    // (the tiled kernels address activation rows with 32-bit byte offsets)
     const bool tiled = !no_gemm && !direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k >= 32 * L->E;
+                       T * L->k >= 32 * L->E && T * L->k * std::max(L->H, L->F) < (int64_t)1 << 32;
     if (tiled) {
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();

@@ -27,7 +27,7 @@ struct RouteBufs {
     int T = 0, k = 0;
 };
 constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a dispatch pass
-constexpr int GEMM_TILE_SLOTS = 64;     // slots per tile of the tiled expert kernels
+constexpr int GEMM_TILE_SLOTS = 128;    // slots per tile of the tiled expert kernels
 inline int64_t max_gemm_tiles(int64_t slots, int64_t groups) { return slots / GEMM_TILE_SLOTS + groups + 1; }
 
 struct FrontParams {

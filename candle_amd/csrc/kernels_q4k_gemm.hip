@@ -10,10 +10,13 @@
 // accumulate over the whole 256-element super-block.  8*acc_hi + acc_lo is then the exact integer
 // the reference computes; the mins term is an exact f16 MFMA over the 16 block sums.
 //
-// Work split: a workgroup owns one tile of 64 slots of one expert (from the dispatch kernel's tile
-// list, so a skewed routing is balanced by tiles, not by experts) and four 32-row operands; the 64
-// activation rows of a super-block are staged once in LDS (double-buffered) and every wave reads them
-// as MFMA A operands, while each wave unpacks and pre-scales its own 32 weight rows in registers.
+// Work split: a workgroup owns one tile of 128 slots of one expert (from the dispatch kernel's tile
+// list, so a skewed routing is balanced by tiles, not by experts) and four 32-row weight operands,
+// one per wave.  The 128 activation rows of a super-block go straight from global memory into LDS
+// (double-buffered, no staging registers) and every wave reads them as MFMA A operands.  A wave unpacks and pre-scales its 32 weight rows of
+// the super-block once, keeps the two planes in registers (64 VGPRs) and runs them against the four
+// 32-slot operands one after the other, so the unpacking cost is spread over 128 slots while only
+// one operand's integer accumulators are live at a time.
 #include "act_quant.hpp"
 #include "kernels.hpp"
 
@@ -41,52 +44,60 @@ __device__ __forceinline__ uint32_t scale_bytes(uint32_t q, uint32_t s) {
     return __builtin_bit_cast(uint32_t, (u16x2)(a * b));
 }
 
-constexpr int GT = GEMM_TILE_SLOTS;   // 64 slots per tile = two 32-row MFMA operands
-constexpr int QSTRIDE = 272;          // LDS row stride of the quants (256 + 16: conflict-free b128 reads)
+constexpr int GT = GEMM_TILE_SLOTS;   // 128 slots per tile = four 32-row MFMA operands
+constexpr int MT = GT / 32;
 constexpr int G_THREADS = 256;
+// Activation quants in LDS: the tile's rows go in chunks of four; a chunk is 1 KiB, written by ONE
+// direct global->LDS load of a wave (lane i lands at byte 16 i), and holds [16-byte piece c][row r%4].
+// Chunks are 1088 bytes apart, so the 16 rows that one phase of a 16-byte LDS read touches (four
+// chunks x four rows, same piece) fall into 16 different 16-byte bank groups.
+constexpr int CHUNK = 1088;
+constexpr int QBUF = (GT / 4) * CHUNK;
 
 struct alignas(16) GemmLds {
-    alignas(16) uint8_t q[2][GT * QSTRIDE];   // activation quants, natural k order inside a row
+    alignas(16) uint8_t q[2][QBUF];           // activation quants (device order of the row: pieces (pair P, chunk g))
     alignas(16) _Float16 bs[2][GT][16];       // block sums
     alignas(16) float yd[2][GT];              // activation scales
 };
 
-// registers holding one thread's share of an activation tile on its way from global memory to LDS
-struct AStage {
-    u32x4 q[4];
-    u32x4 bs;
-    float yd;
-};
-
-// Thread t moves quant chunks c = t + 256*j (row c/16, piece c%16 = pair*4 + chunk), the block sums
-// (row (t%128)/2, half t%2) and the scales (row t%64).  Every thread issues every load -- the upper
-// threads repeat the lower ones' addresses and drop the result -- so that the loop body has no
-// divergent branch around a load: with branches the compiler can no longer count the loads in flight
-// and falls back to waiting for all of them at the top of the next iteration.
-__device__ __forceinline__ AStage a_stage_load(const ActBuf& ab, int K, int nsb, int sb, const int rows4[4], int row_bs, int row_yd, int tid) {
-    AStage st;
-    const int piece = tid & 15;
-#pragma unroll
-    for (int j = 0; j < 4; j++)
-        st.q[j] = gld<u32x4>(ab.qs, (uint32_t)rows4[j] * (uint32_t)K + (uint32_t)(sb * 256 + piece * 16));
-    st.bs = gld<u32x4>(ab.bsum, (((uint32_t)row_bs * (uint32_t)nsb + (uint32_t)sb) * 16 + (tid & 1) * 8) * 2);
-    st.yd = gld<float>(ab.d, ((uint32_t)row_yd * (uint32_t)nsb + (uint32_t)sb) * 4);
-    return st;
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
+// Direct global->LDS loads: lane i of the wave writes SIZE bytes at lds + SIZE*i; nothing passes through
+// registers, so a whole super-block of activations can be in flight while the wave computes.  The
+// compiler does not see these loads: the issuing wave waits for them (vmcnt) before the barrier that
+// publishes the buffer.
+__device__ __forceinline__ void dma16(const void* gbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbase), "s"(lds));
+}
+__device__ __forceinline__ void dma4(const void* gbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(gbase), "s"(lds));
+}
+__device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
-__device__ __forceinline__ void a_stage_store(const AStage& st, GemmLds& L, int buf, int tid) {
-    const int piece = tid & 15, P = piece >> 2, g = piece & 3;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int row = (tid >> 4) + 16 * j;
-        uint8_t* base = L.q[buf] + row * QSTRIDE;
-        // the 16 bytes are [sub-block 2P, chunk g | sub-block 2P+1, chunk g]
-        *reinterpret_cast<u32x2*>(base + (2 * P) * 32 + g * 8) = u32x2{st.q[j].x, st.q[j].y};
-        *reinterpret_cast<u32x2*>(base + (2 * P + 1) * 32 + g * 8) = u32x2{st.q[j].z, st.q[j].w};
-    }
-    // duplicates write the same value to the same place
-    *reinterpret_cast<u32x4*>(&L.bs[buf][(tid & 127) >> 1][(tid & 1) * 8]) = st.bs;
-    L.yd[buf][tid & 63] = st.yd;
+// What a lane fetches for the tile: quants of rows 4*(8 wave + j) + lane%4 (piece lane/4), block sums of
+// row 32 wave + lane/2, scale of row 64 (wave%2) + lane (waves 2,3 repeat waves 0,1: same bytes to the
+// same place, and no branch around a load).
+struct StageRows {
+    uint32_t q[8];     // byte offset of the row's quants
+    uint32_t bs, yd;   // row index
+};
+// transfer number i (0..9) of a wave's share of the tile: eight quant chunks, the block sums, the scales
+template <int I>
+__device__ __forceinline__ void stage_piece(const ActBuf& ab, const StageRows& r, int nsb, int sb, GemmLds& L, int buf, int wave, int lane) {
+    if (I < 8)
+        dma16(ab.qs, r.q[I] + (uint32_t)(sb * 256 + (lane >> 2) * 16), lds_address(L.q[buf]) + (uint32_t)((wave * 8 + I) * CHUNK));
+    else if (I == 8)
+        dma16(ab.bsum, ((r.bs * (uint32_t)nsb + (uint32_t)sb) * 16 + (lane & 1) * 8) * 2, lds_address(&L.bs[buf][0][0]) + (uint32_t)(wave * 1024));
+    else
+        dma4(ab.d, (r.yd * (uint32_t)nsb + (uint32_t)sb) * 4, lds_address(&L.yd[buf][0]) + (uint32_t)((wave & 1) * 256));
+}
+__device__ __forceinline__ void stage_tile(const ActBuf& ab, const StageRows& r, int nsb, int sb, GemmLds& L, int buf, int wave, int lane) {
+    stage_piece<0>(ab, r, nsb, sb, L, buf, wave, lane); stage_piece<1>(ab, r, nsb, sb, L, buf, wave, lane);
+    stage_piece<2>(ab, r, nsb, sb, L, buf, wave, lane); stage_piece<3>(ab, r, nsb, sb, L, buf, wave, lane);
+    stage_piece<4>(ab, r, nsb, sb, L, buf, wave, lane); stage_piece<5>(ab, r, nsb, sb, L, buf, wave, lane);
+    stage_piece<6>(ab, r, nsb, sb, L, buf, wave, lane); stage_piece<7>(ab, r, nsb, sb, L, buf, wave, lane);
+    stage_piece<8>(ab, r, nsb, sb, L, buf, wave, lane); stage_piece<9>(ab, r, nsb, sb, L, buf, wave, lane);
 }
 
 // One wave's weights for one super-block: 32 rows = row tiles rt, rt+1 of the 16-row tile layout.
@@ -110,14 +121,23 @@ __device__ __forceinline__ BRegs b_load(const uint8_t* tile_pair /* tile of row-
     return b;
 }
 
-// accumulate one super-block of one 32-row weight operand against MT 32-slot activation operands
-template <int MT>
-__device__ __forceinline__ void gemm_superblock(const BRegs& b, const GemmLds& L, int buf, int lane, v16f facc[MT]) {
-    const int m = lane & 31, half = lane >> 5;
+// The unpacked, pre-scaled operand of one super-block.  MFMA number 2P+e of the super-block multiplies
+// activation piece (pair P, chunk 2*half+e) = [8 values of sub-block 2P | 8 values of sub-block 2P+1]
+// by the low and the high nibbles of the same 8 weight bytes, each half scaled by its own sub-block's
+// digit (the planes are accumulated over the whole super-block, so an MFMA may mix sub-blocks).
+struct BPlanes {
+    v4i lo[8], hi[8];
+    v8h mB;
+    float d, dmin;
+};
+
+__device__ __forceinline__ BPlanes b_prepare(const BRegs& b, int lane) {
+    const int half = lane >> 5;
     const uint32_t M4 = 0x0f0f0f0fu;
     const uint32_t u0 = b.hdr.y, u1 = b.hdr.z, u2 = b.hdr.w;
-    const float d = __half2float(__ushort_as_half((unsigned short)(b.hdr.x & 0xffffu)));
-    const float dmin = __half2float(__ushort_as_half((unsigned short)(b.hdr.x >> 16)));
+    BPlanes o;
+    o.d = __half2float(__ushort_as_half((unsigned short)(b.hdr.x & 0xffffu)));
+    o.dmin = __half2float(__ushort_as_half((unsigned short)(b.hdr.x >> 16)));
     const uint32_t sc03 = u0 & 0x3f3f3f3fu;
     const uint32_t sc47 = (u2 & M4) | (((u0 >> 6) & 0x03030303u) << 4);
     const uint32_t m03 = u1 & 0x3f3f3f3fu;
@@ -125,62 +145,84 @@ __device__ __forceinline__ void gemm_superblock(const BRegs& b, const GemmLds& L
     // scales split into two 3-bit digits, still one byte per sub-block
     const uint32_t lo03 = sc03 & 0x07070707u, hi03 = (sc03 >> 3) & 0x07070707u;
     const uint32_t lo47 = sc47 & 0x07070707u, hi47 = (sc47 >> 3) & 0x07070707u;
-
-    v16i acc_hi[MT], acc_lo[MT];
-    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};  // first MFMA of a chain takes the constant 0 as C
-
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        // sub-block s = pair P (s/2), low (s even) or high (s odd) nibbles; pair P lives in plane P/2,
-        // bytes (x,y) for P even and (z,w) for P odd of both chunk registers
-        const int P = s >> 1, pl = P >> 1;
-        const uint32_t w0 = (P & 1) ? b.c0[pl].z : b.c0[pl].x, w1 = (P & 1) ? b.c0[pl].w : b.c0[pl].y;
-        const uint32_t w2 = (P & 1) ? b.c1[pl].z : b.c1[pl].x, w3 = (P & 1) ? b.c1[pl].w : b.c1[pl].y;
-        const int sh = (s & 1) ? 4 : 0;
-        const uint32_t q0 = (w0 >> sh) & M4, q1 = (w1 >> sh) & M4, q2 = (w2 >> sh) & M4, q3 = (w3 >> sh) & M4;
-        const uint32_t lw = (s < 4) ? lo03 : lo47, hw = (s < 4) ? hi03 : hi47;
-        const uint32_t slo = (lw >> (8 * (s & 3))) & 0xffu, shi = (hw >> (8 * (s & 3))) & 0xffu;
-        const v4i blo = {(int)scale_bytes(q0, slo), (int)scale_bytes(q1, slo), (int)scale_bytes(q2, slo), (int)scale_bytes(q3, slo)};
-        const v4i bhi = {(int)scale_bytes(q0, shi), (int)scale_bytes(q1, shi), (int)scale_bytes(q2, shi), (int)scale_bytes(q3, shi)};
+    for (int P = 0; P < 4; P++) {
+        // pair P lives in plane P/2 of the tile, dwords (x,y) for P even and (z,w) for P odd
+        const int pl = P >> 1;
+        const uint32_t lw = (P < 2) ? lo03 : lo47, hw = (P < 2) ? hi03 : hi47;
+        const uint32_t slo_a = (lw >> (16 * (P & 1))) & 0xffu, slo_b = (lw >> (16 * (P & 1) + 8)) & 0xffu;
+        const uint32_t shi_a = (hw >> (16 * (P & 1))) & 0xffu, shi_b = (hw >> (16 * (P & 1) + 8)) & 0xffu;
 #pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const v4i a = *reinterpret_cast<const v4i*>(L.q[buf] + (t * 32 + m) * QSTRIDE + s * 32 + half * 16);
-            acc_lo[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, blo, s == 0 ? zero16 : acc_lo[t], 0, 0, 0);
-            acc_hi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bhi, s == 0 ? zero16 : acc_hi[t], 0, 0, 0);
+        for (int e = 0; e < 2; e++) {
+            const u32x4 c = e ? b.c1[pl] : b.c0[pl];
+            const uint32_t w0 = (P & 1) ? c.z : c.x, w1 = (P & 1) ? c.w : c.y;
+            const uint32_t a0 = w0 & M4, a1 = w1 & M4, b0 = (w0 >> 4) & M4, b1 = (w1 >> 4) & M4;
+            o.lo[P * 2 + e] = v4i{(int)scale_bytes(a0, slo_a), (int)scale_bytes(a1, slo_a), (int)scale_bytes(b0, slo_b), (int)scale_bytes(b1, slo_b)};
+            o.hi[P * 2 + e] = v4i{(int)scale_bytes(a0, shi_a), (int)scale_bytes(a1, shi_a), (int)scale_bytes(b0, shi_b), (int)scale_bytes(b1, shi_b)};
         }
     }
     // mins: k = 8*half + j is block sum j of this half; it belongs to sub-block 4*half + j/2
     const uint32_t mw = half ? m47 : m03;
-    v8h mB;
 #pragma unroll
-    for (int j = 0; j < 8; j++) mB[j] = (_Float16)(int)((mw >> (8 * (j >> 1))) & 0xffu);
-#pragma unroll
-    for (int t = 0; t < MT; t++) {
-        const v8h mA = *reinterpret_cast<const v8h*>(&L.bs[buf][t * 32 + m][half * 8]);
-        const v16f zf = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-        const v16f Dm = __builtin_amdgcn_mfma_f32_32x32x16_f16(mA, mB, zf, 0, 0, 0);
-        // D[i] belongs to slot (i/4)*8 + half*4 + i%4 of operand t, weight row n = lane%32
-#pragma unroll
-        for (int i4 = 0; i4 < 4; i4++) {
-            typedef float v4fl __attribute__((ext_vector_type(4)));
-            const v4fl yd = *reinterpret_cast<const v4fl*>(&L.yd[buf][t * 32 + i4 * 8 + half * 4]);
-            const float ydv[4] = {yd.x, yd.y, yd.z, yd.w};
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const int i = i4 * 4 + c;
-                const int isum = (acc_hi[t][i] << 3) + acc_lo[t][i];
-                const float v = __builtin_fmaf(d, (float)isum, -(dmin * Dm[i]));
-                facc[t][i] = __builtin_fmaf(ydv[c], v, facc[t][i]);
-            }
-        }
-    }
+    for (int j = 0; j < 8; j++) o.mB[j] = (_Float16)(int)((mw >> (8 * (j >> 1))) & 0xffu);
+    return o;
 }
+
+// one super-block of the wave's 32 weight rows against 32-slot operand t of the staged tile
+// `while_busy` runs right after the MFMAs are issued: the wave would otherwise idle until they drain,
+// so this is where the next super-block's loads are issued.
+template <typename Fill>
+__device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds& L, int buf, int t, int lane, v16f& facc, Fill while_busy) {
+    const int m = lane & 31, half = lane >> 5;
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};  // first MFMA of a chain takes the constant 0 as C
+    v16i acc_lo, acc_hi;
+    // row t*32+m: chunk t*8 + m/4, slot m%4 of every piece; pieces 4P + 2*half + e
+    const uint8_t* arow = L.q[buf] + (t * 8 + (m >> 2)) * CHUNK + (m & 3) * 16 + half * 128;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        const v4i a = *reinterpret_cast<const v4i*>(arow + (u >> 1) * 256 + (u & 1) * 64);
+        acc_lo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, B.lo[u], u == 0 ? zero16 : acc_lo, 0, 0, 0);
+        acc_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, B.hi[u], u == 0 ? zero16 : acc_hi, 0, 0, 0);
+    }
+    const v8h mA = *reinterpret_cast<const v8h*>(&L.bs[buf][t * 32 + m][half * 8]);
+    const v16f zf = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const v16f Dm = __builtin_amdgcn_mfma_f32_32x32x16_f16(mA, B.mB, zf, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    while_busy();
+    __builtin_amdgcn_sched_barrier(0);
+    // D[i] belongs to slot (i/4)*8 + half*4 + i%4 of operand t, weight row n = lane%32.
+    // The 16 values go through each step together (the fences keep the compiler from re-serialising
+    // them into 16 dependent chains: a lone dependent VALU chain issues at half rate).
+    typedef float v4fl __attribute__((ext_vector_type(4)));
+    float ydv[16];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; i4++) {
+        const v4fl yd = *reinterpret_cast<const v4fl*>(&L.yd[buf][t * 32 + i4 * 8 + half * 4]);
+        ydv[i4 * 4 + 0] = yd.x; ydv[i4 * 4 + 1] = yd.y; ydv[i4 * 4 + 2] = yd.z; ydv[i4 * 4 + 3] = yd.w;
+    }
+    int isum[16];
+    float fs[16], mm[16], v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) isum[i] = (acc_hi[i] << 3) + acc_lo[i];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) fs[i] = (float)isum[i];
+#pragma unroll
+    for (int i = 0; i < 16; i++) mm[i] = B.dmin * Dm[i];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = __builtin_fmaf(B.d, fs[i], -mm[i]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) facc[i] = __builtin_fmaf(ydv[i], v[i], facc[i]);
+}
+
 
 __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(-v)); }
 
 // ---------------------------------------------------------------------------------------------
-// One 32-row weight operand per wave (keeps the accumulators in architectural registers and two
-// waves per SIMD, so one wave's integer/float work overlaps the other's MFMAs).
+// One 32-row weight operand per wave, two workgroups per CU (two waves per SIMD from different
+// workgroups, so one wave's integer/float work overlaps the other's MFMAs).
 // MODE 0: up   -- a workgroup owns 64 rows of F: waves 0,1 carry those rows of w1, waves 2,3 the same
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
@@ -212,16 +254,17 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)
     const size_t sb_stride = (size_t)(N / 16) * Q4K_TILE_BYTES;
     const ActBuf& ab = MODE == 0 ? p.xq : p.hq;
 
-    // which activation rows this thread stages: rows tid/16 + 16 j (quants), tid/2 (sums), tid-128 (scales)
+    // activation row behind position r of the tile (positions past the expert's list repeat its last row)
     auto act_row = [&](int r) {
         const int pos = pos0 + r;
         const int slot = s_begin + (pos < n_g ? pos : n_g - 1);
         return MODE == 0 ? p.rb.perm_token[slot] : slot - p.slot_origin;
     };
-    int rows4[4];
+    StageRows rows;
 #pragma unroll
-    for (int j = 0; j < 4; j++) rows4[j] = act_row((tid >> 4) + 16 * j);
-    const int row_bs = act_row((tid & 127) >> 1), row_yd = act_row(tid & 63);
+    for (int j = 0; j < 8; j++) rows.q[j] = (uint32_t)act_row(4 * (wave * 8 + j) + (lane & 3)) * (uint32_t)K;
+    rows.bs = (uint32_t)act_row(32 * wave + (lane >> 1));
+    rows.yd = (uint32_t)act_row(64 * (wave & 1) + lane);
 
     // weight operand of this wave
     const GroupWeights gw = p.groups[grp];
@@ -234,28 +277,36 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)
         row0 = rblk * 128 + wave * 32;
         wp = gw.w2 + (size_t)(row0 / 16) * Q4K_TILE_BYTES;
     }
-    v16f facc[2];
+    v16f facc[MT];
 #pragma unroll
-    for (int t = 0; t < 2; t++)
+    for (int t = 0; t < MT; t++)
 #pragma unroll
         for (int i = 0; i < 16; i++) facc[t][i] = 0.f;
 
-    {
-        AStage st = a_stage_load(ab, K, nsb, 0, rows4, row_bs, row_yd, tid);
-        a_stage_store(st, L, 0, tid);
-    }
-    BRegs b0 = b_load(wp, lane);
+    stage_tile(ab, rows, nsb, 0, L, 0, wave, lane);
+    BRegs raw = b_load(wp, lane);
+    wait_all_loads();
     __syncthreads();
     for (int sb = 0; sb < nsb; sb++) {
         const int buf = sb & 1;
         const int sbn = sb + 1 < nsb ? sb + 1 : sb;
-        const BRegs n0 = b_load(wp + (size_t)sbn * sb_stride, lane);
-        AStage st = a_stage_load(ab, K, nsb, sbn, rows4, row_bs, row_yd, tid);
-        __builtin_amdgcn_sched_barrier(0);   // the prefetches must be in flight before the MFMA work, not after it
-        gemm_superblock<2>(b0, L, buf, lane, facc);
+        const BPlanes B = b_prepare(raw, lane);
+        const int nb = buf ^ 1;
+        gemm_operand(B, L, buf, 0, lane, facc[0], [&] {
+            stage_piece<0>(ab, rows, nsb, sbn, L, nb, wave, lane); stage_piece<1>(ab, rows, nsb, sbn, L, nb, wave, lane);
+            stage_piece<2>(ab, rows, nsb, sbn, L, nb, wave, lane); });
         __builtin_amdgcn_sched_barrier(0);
-        a_stage_store(st, L, buf ^ 1, tid);
-        b0 = n0;
+        gemm_operand(B, L, buf, 1, lane, facc[1], [&] {
+            stage_piece<3>(ab, rows, nsb, sbn, L, nb, wave, lane); stage_piece<4>(ab, rows, nsb, sbn, L, nb, wave, lane);
+            stage_piece<5>(ab, rows, nsb, sbn, L, nb, wave, lane); });
+        __builtin_amdgcn_sched_barrier(0);
+        gemm_operand(B, L, buf, 2, lane, facc[2], [&] {
+            stage_piece<6>(ab, rows, nsb, sbn, L, nb, wave, lane); stage_piece<7>(ab, rows, nsb, sbn, L, nb, wave, lane);
+            stage_piece<8>(ab, rows, nsb, sbn, L, nb, wave, lane); stage_piece<9>(ab, rows, nsb, sbn, L, nb, wave, lane); });
+        __builtin_amdgcn_sched_barrier(0);
+        gemm_operand(B, L, buf, 3, lane, facc[3], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
+        __builtin_amdgcn_sched_barrier(0);
+        wait_all_loads();
         __syncthreads();
     }
 
@@ -263,28 +314,29 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)
     const int n = lane & 31, half = lane >> 5;
     if (MODE == 0) {
         // w3 waves (2,3) park their sums in LDS (the activation buffers are free now), w1 waves combine
-        float* xch = reinterpret_cast<float*>(L.q[0]);   // [2 waves][2 t][16 i][64 lanes] = 16 KB <= sizeof(L.q[0])
+        float* xch = reinterpret_cast<float*>(L.q[0]);   // [2 waves][MT][16 i][64 lanes] floats
+        static_assert(2 * MT * 16 * 64 * 4 <= sizeof(L.q[0]), "exchange area");
         if (wave >= 2) {
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < MT; t++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) xch[(((wave - 2) * 2 + t) * 16 + i) * 64 + lane] = facc[t][i];
+                for (int i = 0; i < 16; i++) xch[(((wave - 2) * MT + t) * 16 + i) * 64 + lane] = facc[t][i];
         }
         __syncthreads();
         if (wave < 2) {
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int t = 0; t < MT; t++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int pos = pos0 + t * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
                     if (pos >= n_g) continue;
-                    const float bsum = xch[((wave * 2 + t) * 16 + i) * 64 + lane];
+                    const float bsum = xch[((wave * MT + t) * 16 + i) * 64 + lane];
                     p.hbuf[(int64_t)(s_begin + pos - p.slot_origin) * p.F + row0 + n] = silu_gemm(facc[t][i]) * bsum;
                 }
         }
     } else {
 #pragma unroll
-        for (int t = 0; t < 2; t++)
+        for (int t = 0; t < MT; t++)
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int pos = pos0 + t * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
