@@ -7,8 +7,12 @@ decode batch of 32 tokens of N(0, 1) activations.  A "step" is one forward of th
 activations already resident in HBM.  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 32] [--no-cpu-baseline]
+
+`--workload prefill` measures BASELINE config 3 instead (same layer, 4096 tokens, router bias that makes
+the expert load follow Zipf(1)); its roofline object is the int8-MFMA one of the tiled up kernel.
 """
 import argparse
+import re
 import ctypes as C
 import json
 import os
@@ -22,9 +26,12 @@ H, F, E, TOPK = 4096, 14336, 8, 2
 Q4K = 12
 EXPERT_BYTES = 3 * H * F * 144 // 256          # 99,090,432 B of Q4_K blocks per expert
 HBM_PEAK_GBS = 8000.0                          # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5000.0                        # MI355X dense int8 MFMA, published
+# per-expert logit biases under which top-2 routing of N(0, 1.28^2) logits gives Zipf(1) loads (shares 1/i)
+ZIPF_BIAS = [0.0, -1.158, -1.581, -1.845, -2.033, -2.186, -2.299, -2.398]
 
 
-def build_layer(torch, candle_amd, seed=0):
+def build_layer(torch, candle_amd, seed=0, gate_bias=None):
     """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel
     (bit-identical to candle's CPU quantiser), kept as host bytes for the CPU baseline too."""
     g = torch.Generator(device="cuda")
@@ -37,7 +44,7 @@ def build_layer(torch, candle_amd, seed=0):
             del x
     g.manual_seed(seed + 1)
     gate = (torch.randn((E, H), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
-    layer = candle_amd.SparseMoeBlock(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"])
+    layer = candle_amd.SparseMoeBlock(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
     return layer, gate, w
 
 
@@ -51,7 +58,7 @@ def hip_events():
     return hip
 
 
-def cpu_baseline(gate, w, xs_host, logits_host, min_seconds):
+def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None):
     """candle's CPU path restated (the oracle: serial rows, columns threaded, AVX2 inner loops of
     candle's x86 build) on all host cores: the same batch, same weight bytes, same routing,
     repeated until `min_seconds` of wall time have passed."""
@@ -60,7 +67,7 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds):
 
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
-    layer = O.Layer(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"])
+    layer = O.Layer(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
     layer.forward(xs_host[:1], logits=logits_host[:1], simd=True, threads=cores)  # warm the pages
     reps, t0 = 0, time.perf_counter()
     while True:
@@ -74,15 +81,33 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds):
                       "(AVX2 vec_dot, %d threads over output columns)" % (reps, xs_host.shape[0], dt, cores)}
 
 
+def measured_traffic(batch):
+    """HBM bytes per launch of the up kernel from the committed rocprofv3 counter summary (FETCH_SIZE +
+    WRITE_SIZE, scaled by the copy kernel), or None when the summary does not cover this batch size."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "q4k_up_decode_hbm_traffic.md")
+    try:
+        for line in open(path):
+            m = re.match(r"traffic_bytes_per_launch\[batch=(\d+)\]:\s*(\d+)", line.strip())
+            if m and int(m.group(1)) == batch:
+                return int(m.group(2))
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill)")
+    ap.add_argument("--workload", choices=("decode", "prefill"), default="decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 1 GiB device copy (the known-size kernel that scales rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); --gpus %d is not supported" % args.gpus)
@@ -93,8 +118,18 @@ def main():
 
     candle_amd.load_library()  # fails loudly if the HIP extension is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    B = args.batch
-    layer, gate, w = build_layer(torch, candle_amd)
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
+        return
+    prefill = args.workload == "prefill"
+    B = args.batch or (4096 if prefill else 32)
+    bias = np.array(ZIPF_BIAS, dtype=np.float32) if prefill else None
+    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias)
     g = torch.Generator(device="cuda")
     g.manual_seed(2)
     # several distinct activation batches, rotated, so that no step repeats the previous one's input
@@ -107,7 +142,8 @@ def main():
         for i in range(args.warmup):
             layer.forward(xs[i % 4], out=ys[i % 4])
         stream.synchronize()
-        n_active = int((np.diff(layer.last_routing(B)[2]) > 0).sum())
+        loads = np.diff(layer.last_routing(B)[2])[:E]
+        n_active = int((loads > 0).sum())
         ev = [C.c_void_p() for _ in range(2)]
         for e in ev:
             hip.hipEventCreate(C.byref(e))
@@ -133,29 +169,49 @@ def main():
                 stage[k] += v / args.stage_iters
     stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
 
-    # Roofline of the dominant kernel, the up projection (w1, w3 + SiLU): it streams w1 and w3 of
-    # every active expert exactly once per launch; algorithmic bytes = Q4_K bytes of those matrices
-    # plus the quantised activations it reads and the quantised intermediate it writes.
-    up_bytes = n_active * (2 * H * F * 144 // 256) + B * (H + H // 256 * 36) + B * TOPK * (F + F // 256 * 36)
-    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
     step_bytes = n_active * EXPERT_BYTES + E * H * 4 + 2 * B * H * 4
+    if prefill:
+        # Roofline of the dominant kernel, the tiled up projection: 2 * slots * 2 * H * F integer
+        # multiply-adds (w1 and w3) per launch against the dense int8 MFMA peak.
+        up_ops = 2.0 * B * TOPK * 2 * H * F
+        achieved = up_ops / (stage["up"] * 1e-3) / 1e12
+        step_ops = 2.0 * B * TOPK * 3 * H * F
+        roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, two scale planes)",
+                    "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": achieved / INT8_PEAK_TOPS,
+                    "traffic": None, "algorithmic_ops_per_launch": up_ops, "launch_us": stage_us["up"]}
+        workload = ("BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, prefill of %d tokens, "
+                    "Zipf(1) expert load" % B)
+        extra = {"expert_loads": [int(v) for v in loads], "step_int8_ops": step_ops,
+                 "step_mfma_frac": step_ops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS}
+    else:
+        # Roofline of the dominant kernel, the up projection (w1, w3 + SiLU): it streams w1 and w3 of
+        # every active expert exactly once per launch; algorithmic bytes = Q4_K bytes of those matrices
+        # plus the quantised activations it reads and the quantised intermediate it writes.
+        up_bytes = n_active * (2 * H * F * 144 // 256) + B * (H + H // 256 * 36) + B * TOPK * (F + F // 256 * 36)
+        achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)", "achieved": achieved,
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": measured_traffic(B),
+                    "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+        workload = "BASELINE config 2: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, decode batch %d" % B
+        extra = {"step_algorithmic_bytes": step_bytes,
+                 "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
     out = {
-        "metric": "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, decode)", "value": tokens_per_s, "unit": "tokens/s",
+        "metric": "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, %s)" % args.workload, "value": tokens_per_s, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, decode batch %d" % B,
-                   "active_experts": n_active, "wall_ms_per_step": wall * 1e3 / args.steps, "stage_us": stage_us,
-                   "step_algorithmic_bytes": step_bytes,
-                   "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        "roofline": {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]},
+        "config": dict({"workload": workload, "active_experts": n_active,
+                        "wall_ms_per_step": wall * 1e3 / args.steps, "stage_us": stage_us}, **extra),
+        "roofline": roofline,
     }
     if not args.no_cpu_baseline:
         layer.forward(xs[0], out=ys[0])
         torch.cuda.synchronize()
-        out["cpu_baseline"] = cpu_baseline(gate, w, xs[0].cpu().numpy(), layer.last_logits(B), args.cpu_seconds)
+        # a bounded sample: the CPU path does ~1 k tokens/s, so a prefill batch is cut to its first 64 tokens
+        n_cpu = min(B, 64)
+        out["cpu_baseline"] = cpu_baseline(gate, w, xs[0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu],
+                                           args.cpu_seconds, gate_bias=bias)
     print(json.dumps(out))
 
 

@@ -284,7 +284,7 @@ extern "C" void moe_layer_destroy(moe_layer* L) {
 
 // Enqueue one forward on `s`.  Caller holds L->mu.
 // Stage marks for moe_layer_forward_timed: events recorded between the launches.
-enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_DOWN, ST_SHARED, ST_COMBINE, ST_COUNT };
+enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_REQUANT, ST_DOWN, ST_SHARED, ST_COMBINE, ST_COUNT };
 
 static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
 #define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
@@ -331,13 +331,15 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         ep.hbuf = L->hbuf.as<float>();
         ep.n_slots = T * L->k;
         MOE_HIP_CHECK(launch_q4k_gemm_up(ep, s));
-        MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_UP);
+        MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
+        MOE_MARK(ST_REQUANT);
         MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
         MOE_MARK(ST_DOWN);
     } else {
-        MOE_HIP_CHECK(launch_expert_up(ep, s));
+        MOE_HIP_CHECK(launch_expert_up(ep, s));   // re-quantises the intermediate in its epilogue
         MOE_MARK(ST_UP);
+        MOE_MARK(ST_REQUANT);
         MOE_HIP_CHECK(launch_expert_down(ep, s));
         MOE_MARK(ST_DOWN);
     }

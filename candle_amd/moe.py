@@ -260,14 +260,14 @@ class SparseMoeBlock:
 
     __call__ = forward
 
-    STAGES = ("front", "dispatch", "up", "down", "shared", "combine")
+    STAGES = ("front", "dispatch", "up", "requant", "down", "shared", "combine")
 
     def forward_timed(self, xs, out):
         """One forward on torch CUDA tensors with HIP events between the launches (on torch's
         current stream); returns {stage: milliseconds}.  Synchronises."""
         import torch
         T = xs.numel() // self.hidden
-        ms = (C.c_float * 6)()
+        ms = (C.c_float * len(self.STAGES))()
         stream = torch.cuda.current_stream(xs.device).cuda_stream
         _check(load_library().moe_layer_forward_timed(self._h, xs.data_ptr(), T, out.data_ptr(), stream, ms))
         return dict(zip(self.STAGES, [float(v) for v in ms]))

@@ -90,8 +90,10 @@ int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens
 
 /* Measurement aid (no counterpart in the reference): one forward as moe_layer_forward_device with
  * HIP events recorded on `hip_stream` between the launches; waits for completion and returns the
- * elapsed milliseconds of the six stages in stage_ms[0..5]: front (router + activation quantiser),
- * dispatch (0 for small batches), up (w1/w3 + SiLU), down (w2), shared expert, combine. */
+ * elapsed milliseconds of the seven stages in stage_ms[0..6]: front (router + activation quantiser),
+ * dispatch (0 for small batches), up (w1/w3 + SiLU), requant (Q8K/Q8_0 quantisation of the
+ * intermediate as a pass of its own: large Q4_K batches only, otherwise part of up), down (w2),
+ * shared expert, combine. */
 int moe_layer_forward_timed(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream, float* stage_ms);
 
 /* Router logits [n_tokens, E] (after the optional bias) that the last forward on this layer

@@ -119,17 +119,23 @@ def test_cfg2_device_entry_and_repeatability(mixtral_layer):
     assert np.array_equal(bits(y0), bits(y1)) and np.array_equal(bits(y1), bits(y2))
 
 
+ZIPF_BIAS = np.array([0.0, -1.158, -1.581, -1.845, -2.033, -2.186, -2.299, -2.398], dtype=np.float32)
+
+
 def test_cfg3_prefill_zipf(mixtral_layer):
-    # 4096 tokens; a per-expert bias on the logits makes the load follow Zipf(s=1)
+    # 4096 tokens; a per-expert bias on the logits makes the top-2 load follow Zipf(s=1): shares 1/i,
+    # heaviest expert ~37 %.  The biases were fitted once on N(0, 1.28^2) logits (what an N(0, 0.02) gate
+    # gives on N(0, 1) activations of width 4096).
     ref, gpu0 = mixtral_layer
-    bias = (2.2 * np.log(1.0 / np.arange(1, 9))).astype(np.float32)
+    bias = ZIPF_BIAS
     gate = ref.gate
     gpu = candle_amd.SparseMoeBlock(4096, 14336, 8, 2, O.Q4K, gate, ref.w1, ref.w3, ref.w2, gate_bias=bias)
     ref_b = O.Layer(4096, 14336, 8, 2, O.Q4K, gate, ref.w1, ref.w3, ref.w2, gate_bias=bias)
     xs = acts(4096, 4096, 11)
     _, off = check(ref_b, gpu, xs, flip_allowance=True)
     load = np.diff(off) / off[-1]
-    assert load[0] > 0.3 and load[-1] < 0.08  # heavy skew really happened
+    zipf = 1.0 / np.arange(1, 9)
+    assert np.abs(load - zipf / zipf.sum()).max() < 0.03, load  # the skew really is Zipf(1)
     gpu.close()
 
 
