@@ -304,9 +304,17 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.xq = L->xq.view();
     fp.rb = L->route.view();
     fp.rb.T = (int)T; fp.rb.k = (int)L->k;
+    // Q4K batches with more than ~24 rows per expert take the tiled MFMA kernels (F a multiple of 64,
+    // H of 128; those kernels address activation rows with 32-bit byte offsets).  Their tiles hold 64
+    // slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
+    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
+                       T * L->k > 24 * L->E && T * L->k * std::max(L->H, L->F) < (int64_t)1 << 32;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
-    const bool direct = T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
+    const bool direct = !tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     fp.rb.direct = direct ? 1 : 0;
+    static const int force_tile = getenv("MOE_TILE_SLOTS") ? atoi(getenv("MOE_TILE_SLOTS")) : 0;
+    fp.rb.tile_slots = force_tile == 64 || force_tile == 128 ? force_tile : T * L->k >= 96 * L->E ? 128 : 64;
     MOE_MARK(ST_BEGIN);
     MOE_HIP_CHECK(launch_front(fp, s));
     MOE_MARK(ST_FRONT);
@@ -320,12 +328,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = L->hq.view(); ep.slot_origin = 0;
     ep.yw = L->yw.as<float>();
     ep.max_rows = T;
-    ep.slot_tiles = (T * L->k > 9 * L->E) ? 2 : 1;   // expected rows per expert above ~9: carry 32 slots per pass
-    // large Q4K batches take the tiled MFMA path: F a multiple of 64, H of 128, many rows per expert
-    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
-    // (the tiled kernels address activation rows with 32-bit byte offsets)
-    const bool tiled = !no_gemm && !direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k >= 32 * L->E && T * L->k * std::max(L->H, L->F) < (int64_t)1 << 32;
+    // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
+    // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
+    ep.slot_tiles = (T * L->k > 24 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
     if (tiled) {
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();
@@ -348,7 +353,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
         sp.groups = L->groups.as<GroupWeights>() + L->E;
         sp.hq = L->hq_shared.view(); sp.slot_origin = (int)(T * L->k);
-        sp.max_rows = T; sp.slot_tiles = T > 16 ? 2 : 1;
+        sp.max_rows = T; sp.slot_tiles = T > 32 ? 4 : T > 16 ? 2 : 1;
         MOE_HIP_CHECK(launch_expert_up(sp, s));
         MOE_HIP_CHECK(launch_expert_down(sp, s));
     }
@@ -554,7 +559,7 @@ extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t 
     ep.dt = dt; ep.H = (int)n; ep.F = (int)k; ep.n_groups = 1; ep.group0 = 0;
     ep.groups = grp.as<GroupWeights>();
     ep.rb = rs.view(); ep.hq = as.view(); ep.slot_origin = 0; ep.yw = dy.as<float>();
-    ep.max_rows = m; ep.slot_tiles = m > 16 ? 2 : 1;
+    ep.max_rows = m; ep.slot_tiles = m > 32 ? 4 : m > 16 ? 2 : 1;
     MOE_HIP_CHECK(launch_expert_down(ep, nullptr));
     MOE_HIP_CHECK(hipDeviceSynchronize());
     return d2h(y, dy.p, (size_t)m * n * 4);

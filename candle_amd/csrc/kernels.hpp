@@ -16,9 +16,10 @@ struct RouteBufs {
     float* perm_w = nullptr;        // [S] routing weight of every slot
     int32_t* tok_slots = nullptr;   // [T, k(+1)] slots of a token, ascending expert index
     // Work list of the tiled (prefill) expert kernels, written by the dispatch kernel: [0] = number
-    // of 64-slot tiles, then (group, first position inside the group) per tile.  Built from the
-    // real list lengths, so a skewed routing yields tiles in proportion to each expert's load.
+    // of tiles of `tile_slots` slots, then (group, first position inside the group) per tile.  Built
+    // from the real list lengths, so a skewed routing yields tiles in proportion to each expert's load.
     int32_t* tile_tab = nullptr;
+    int tile_slots = 128;           // 128, or 64 when the lists are short
     // Slot numbering.  direct == 0: slots are grouped by expert (offsets / perm_* built by the
     // dispatch kernel).  direct == 1 (small batches): slot of assignment (token t, rank r) is
     // simply t*k + r, the shared expert's slots are T*k + t, and every consumer derives its
@@ -27,8 +28,8 @@ struct RouteBufs {
     int T = 0, k = 0;
 };
 constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a dispatch pass
-constexpr int GEMM_TILE_SLOTS = 128;    // slots per tile of the tiled expert kernels
-inline int64_t max_gemm_tiles(int64_t slots, int64_t groups) { return slots / GEMM_TILE_SLOTS + groups + 1; }
+constexpr int GEMM_MIN_TILE_SLOTS = 64;  // smallest tile of the tiled expert kernels
+inline int64_t max_gemm_tiles(int64_t slots, int64_t groups, int tile_slots = GEMM_MIN_TILE_SLOTS) { return slots / tile_slots + groups + 1; }
 
 struct FrontParams {
     const float* x = nullptr;       // [T, H]
@@ -69,7 +70,7 @@ struct ExpertParams {
     int slot_origin = 0;
     float* yw = nullptr;            // [S, H] weighted expert outputs, slot-indexed (absolute)
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
-    int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1 or 2)
+    int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1, 2 or, Q4K only, 4)
     int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)
     float* hbuf = nullptr;          // tiled path only: f32 intermediate [slots, F] before re-quantisation
     int64_t n_slots = 0;            // tiled path only: total slots (bounds the tile grid)

@@ -152,7 +152,7 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         const int G = E + (shared ? 1 : 0);
         for (int gi = 0; gi < G; gi++) {
             const int len = sh.off[gi + 1] - sh.off[gi];
-            for (int pos = 0; pos < len; pos += GEMM_TILE_SLOTS) {
+            for (int pos = 0; pos < len; pos += rb.tile_slots) {
                 rb.tile_tab[1 + 2 * n] = gi;
                 rb.tile_tab[2 + 2 * n] = pos;
                 n++;

@@ -332,26 +332,17 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
         q4k_down_body<TT, NW, RING>(p, part, list_lds, wtot_lds);                                           \
     }
 
-// variant 0: 8 waves, 128 VGPRs (two workgroups per CU); variant 1: 4 waves, 168 VGPRs (three per CU)
+// One 16-slot tile per pass (small batches): variant 1 (default) 4 waves, 168 VGPRs, three workgroups
+// per CU; variant 0 8 waves, 128 VGPRs.  Two and four tiles per pass (up to 32 / 64 rows per expert
+// without streaming its weights twice) need the registers of a two-waves-per-SIMD launch.
 DEF_UP(q4k_up_t1_v0, 1, 8, 2, 4)
-DEF_UP(q4k_up_t2_v0, 2, 8, 2, 4)
 DEF_UP(q4k_up_t1_v1, 1, 4, 2, 3)
-DEF_UP(q4k_up_t2_v1, 2, 4, 2, 3)
-DEF_UP(q4k_up_t1_v2, 1, 4, 4, 3)
-DEF_UP(q4k_up_t1_v3, 1, 8, 4, 2)
-DEF_UP_D(q4k_up_t1_v8, 1, 4, 2, 3, 1)
-DEF_UP_D(q4k_up_t1_v9, 1, 4, 2, 3, 2)
-DEF_UP_D(q4k_up_t1_v10, 1, 4, 4, 3, 1)
-DEF_UP_D(q4k_up_t1_v11, 1, 8, 2, 4, 1)
-DEF_UP_D(q4k_up_t1_v12, 1, 8, 4, 4, 1)
-DEF_UP_D(q4k_up_t1_v13, 1, 4, 8, 3, 1)
-DEF_UP_D(q4k_up_t1_v14, 1, 16, 2, 4, 1)
+DEF_UP(q4k_up_t2, 2, 4, 2, 2)
+DEF_UP(q4k_up_t4, 4, 8, 2, 2)
 DEF_DOWN(q4k_down_t1_v0, 1, 8, 2, 4)
-DEF_DOWN(q4k_down_t2_v0, 2, 8, 2, 4)
 DEF_DOWN(q4k_down_t1_v1, 1, 4, 2, 3)
-DEF_DOWN(q4k_down_t2_v1, 2, 4, 2, 3)
-DEF_DOWN(q4k_down_t1_v2, 1, 4, 4, 3)
-DEF_DOWN(q4k_down_t1_v3, 1, 8, 4, 2)
+DEF_DOWN(q4k_down_t2, 2, 4, 2, 2)
+DEF_DOWN(q4k_down_t4, 4, 8, 2, 2)
 
 // ---------------------------------------------------------------------------------------------
 static int variant(const char* name, int dflt) {
@@ -362,41 +353,24 @@ static int variant(const char* name, int dflt) {
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_UP_VARIANT", 1);
-    const int tt = p.slot_tiles >= 2 ? 2 : 1;
+    const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     dim3 grid((unsigned)(p.F / UP_ROWS), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (tt == 2) {
-        if (v == 1 || v == 2) hipLaunchKernelGGL(q4k_up_t2_v1, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q4k_up_t2_v0, grid, dim3(512), 0, s, p);
-    } else {
-        if (v == 1) hipLaunchKernelGGL(q4k_up_t1_v1, grid, dim3(256), 0, s, p);
-        else if (v == 2) hipLaunchKernelGGL(q4k_up_t1_v2, grid, dim3(256), 0, s, p);
-        else if (v == 3) hipLaunchKernelGGL(q4k_up_t1_v3, grid, dim3(512), 0, s, p);
-        else if (v == 8) hipLaunchKernelGGL(q4k_up_t1_v8, grid, dim3(256), 0, s, p);
-        else if (v == 9) hipLaunchKernelGGL(q4k_up_t1_v9, grid, dim3(256), 0, s, p);
-        else if (v == 10) hipLaunchKernelGGL(q4k_up_t1_v10, grid, dim3(256), 0, s, p);
-        else if (v == 11) hipLaunchKernelGGL(q4k_up_t1_v11, grid, dim3(512), 0, s, p);
-        else if (v == 12) hipLaunchKernelGGL(q4k_up_t1_v12, grid, dim3(512), 0, s, p);
-        else if (v == 13) hipLaunchKernelGGL(q4k_up_t1_v13, grid, dim3(256), 0, s, p);
-        else if (v == 14) hipLaunchKernelGGL(q4k_up_t1_v14, grid, dim3(1024), 0, s, p);
-        else hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
-    }
+    if (tt == 4) hipLaunchKernelGGL(q4k_up_t4, grid, dim3(512), 0, s, p);
+    else if (tt == 2) hipLaunchKernelGGL(q4k_up_t2, grid, dim3(256), 0, s, p);
+    else if (v == 0) hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
+    else hipLaunchKernelGGL(q4k_up_t1_v1, grid, dim3(256), 0, s, p);
     return hipGetLastError();
 }
 
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_DOWN_VARIANT", 1);
-    const int tt = p.slot_tiles >= 2 ? 2 : 1;
+    const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (tt == 2) {
-        if (v == 1 || v == 2) hipLaunchKernelGGL(q4k_down_t2_v1, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q4k_down_t2_v0, grid, dim3(512), 0, s, p);
-    } else {
-        if (v == 1) hipLaunchKernelGGL(q4k_down_t1_v1, grid, dim3(256), 0, s, p);
-        else if (v == 2) hipLaunchKernelGGL(q4k_down_t1_v2, grid, dim3(256), 0, s, p);
-        else if (v == 3) hipLaunchKernelGGL(q4k_down_t1_v3, grid, dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(q4k_down_t1_v0, grid, dim3(512), 0, s, p);
-    }
+    if (tt == 4) hipLaunchKernelGGL(q4k_down_t4, grid, dim3(512), 0, s, p);
+    else if (tt == 2) hipLaunchKernelGGL(q4k_down_t2, grid, dim3(256), 0, s, p);
+    else if (v == 0) hipLaunchKernelGGL(q4k_down_t1_v0, grid, dim3(512), 0, s, p);
+    else hipLaunchKernelGGL(q4k_down_t1_v1, grid, dim3(256), 0, s, p);
     return hipGetLastError();
 }
 

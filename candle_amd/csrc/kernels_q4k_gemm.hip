@@ -19,6 +19,7 @@
 // The 16-row operand keeps a wave below 128 VGPRs, so four waves share a SIMD: a single wave issues
 // at most one vector instruction every ~5 cycles and stalls on every MFMA result, and it takes that
 // many waves to keep the MFMA pipe and the vector ALU busy at the same time.
+#include <type_traits>
 #include "act_quant.hpp"
 #include "kernels.hpp"
 
@@ -45,8 +46,8 @@ __device__ __forceinline__ uint32_t scale_bytes(uint32_t q, uint32_t s) {
     return __builtin_bit_cast(uint32_t, (u16x2)(a * b));
 }
 
-constexpr int GT = GEMM_TILE_SLOTS;   // 128 slots per tile
-constexpr int NOP = GT / 16;          // eight 16-slot MFMA operands
+// A tile is NOP 16-slot MFMA operands: 8 (128 slots) for big batches, 4 (64 slots) when the experts'
+// lists are short, so that less of a tile is padding.
 constexpr int G_WAVES = 8;
 constexpr int G_THREADS = 64 * G_WAVES;
 // Activations in LDS, laid out so that what one MFMA reads is one contiguous stretch in lane order
@@ -57,12 +58,11 @@ constexpr int G_THREADS = 64 * G_WAVES;
 //   block sums [operand o][half h][row m] 16-byte pieces (8 sums): lane (m, g) reads 8 bytes at
 //          piece (g/2, m), offset 8 (g%2);
 //   scales [slot].
-constexpr int QBUF = GT * 256;
-
+template <int NOP>
 struct alignas(16) GemmLds {
-    alignas(16) uint8_t q[2][QBUF];
+    alignas(16) uint8_t q[2][NOP * 16 * 256];
     alignas(16) _Float16 bs[2][NOP][2][16][8];
-    alignas(16) float yd[2][GT];
+    alignas(16) float yd[2][NOP * 16];
 };
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
@@ -80,24 +80,28 @@ __device__ __forceinline__ void dma4(const void* gbase, uint32_t voff, uint32_t 
 }
 __device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
-// What a lane fetches for the tile.  Quants: wave w stages operand w, transfer P moves pair P: lane
-// (m = l%16, g = l/16) fetches piece (P, g) of row 16 w + m.  Block sums: wave w%4 stages operands
-// 2(w%4), 2(w%4)+1: lane fetches half (l/16)%2 of row 32 (w%4) + 16 (l/32) + l%16.  Scales: row
-// 64 (w%2) + l.  The upper waves repeat the lower ones for sums and scales: same bytes to the same
-// place, and no branch around a load.
+// What a lane fetches for the tile.  Quants: the NOP*4 (operand, pair) stretches of 1 KiB are dealt to
+// the eight waves, NOP/2 each: lane (m = l%16, g = l/16) fetches piece (P, g) of row 16 o + m.  Block
+// sums: one transfer covers two operands: lane fetches half (l/16)%2 of row 32 x + 16 (l/32) + l%16.
+// Scales: row 64 x + l.  Waves without a share of the sums and scales repeat another wave's transfer:
+// same bytes to the same place, and no branch around a load.
 struct StageRows {
     uint32_t q;        // byte offset of the row's quants
     uint32_t bs, yd;   // row index
 };
-// transfer number I (0..5) of a wave's share of the tile: four quant pairs, block sums, scales
-template <int I>
-__device__ __forceinline__ void stage_piece(const ActBuf& ab, const StageRows& r, int nsb, int sb, GemmLds& L, int buf, int wave, int lane) {
-    if (I < 4)
-        dma16(ab.qs, r.q + (uint32_t)(sb * 256 + (I * 4 + (lane >> 4)) * 16), lds_address(L.q[buf]) + (uint32_t)((wave * 4 + I) * 1024));
-    else if (I == 4)
-        dma16(ab.bsum, ((r.bs * (uint32_t)nsb + (uint32_t)sb) * 16 + ((lane >> 4) & 1) * 8) * 2, lds_address(&L.bs[buf][0][0][0][0]) + (uint32_t)((wave & 3) * 1024));
-    else
-        dma4(ab.d, (r.yd * (uint32_t)nsb + (uint32_t)sb) * 4, lds_address(&L.yd[buf][0]) + (uint32_t)((wave & 1) * 256));
+// transfer number I (0 .. NOP/2+1) of a wave's share of the tile: NOP/2 quant stretches, block sums, scales
+template <int I, int NOP>
+__device__ __forceinline__ void stage_piece(const ActBuf& ab, const StageRows& r, int nsb, int sb, GemmLds<NOP>& L, int buf, int wave, int lane) {
+    constexpr int NB = NOP / 2;
+    if (I < NB) {
+        const int blk = wave * NB + I;            // = 4 o + P with o the wave's operand (r.q is its row)
+        dma16(ab.qs, r.q + (uint32_t)(sb * 256 + ((blk & 3) * 4 + (lane >> 4)) * 16), lds_address(L.q[buf]) + (uint32_t)(blk * 1024));
+    } else if (I == NB) {
+        dma16(ab.bsum, ((r.bs * (uint32_t)nsb + (uint32_t)sb) * 16 + ((lane >> 4) & 1) * 8) * 2,
+              lds_address(&L.bs[buf][0][0][0][0]) + (uint32_t)((wave % (NOP / 2)) * 1024));
+    } else {
+        dma4(ab.d, (r.yd * (uint32_t)nsb + (uint32_t)sb) * 4, lds_address(&L.yd[buf][0]) + (uint32_t)((wave % (NOP / 4)) * 256));
+    }
 }
 
 // One wave's weights for one super-block: the 16 rows of one tile of the device layout.  Lane
@@ -158,8 +162,8 @@ __device__ __forceinline__ BPlanes b_prepare(const BRegs& b, int lane) {
 
 // one super-block of the wave's 16 weight rows against 16-slot operand o of the staged tile
 // `while_busy` runs right after the MFMAs are issued: this is where the next super-block's loads go.
-template <typename Fill>
-__device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds& L, int buf, int o, int lane, v4f& facc, Fill while_busy) {
+template <int NOP, typename Fill>
+__device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP>& L, int buf, int o, int lane, v4f& facc, Fill while_busy) {
     const int m = lane & 15, g = lane >> 4;
     const v4i zero4 = {0, 0, 0, 0};
     v4i acc_lo, acc_hi;
@@ -187,14 +191,16 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds& L,
 __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(-v)); }
 
 // ---------------------------------------------------------------------------------------------
-// One 16-row weight operand per wave, eight waves per workgroup, two workgroups per CU.
+// One 16-row weight operand per wave, eight waves per workgroup, two workgroups per CU; a tile of
+// NOP*16 slots.
 // MODE 0: up   -- a workgroup owns 64 rows of F: waves 0-3 carry those rows of w1, waves 4-7 the same
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-template <int MODE>
+template <int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
-    __shared__ GemmLds L;
+    constexpr int NB = NOP / 2;
+    __shared__ GemmLds<NOP> L;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_tiles = p.rb.tile_tab[0];
@@ -226,9 +232,9 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
         return MODE == 0 ? p.rb.perm_token[slot] : slot - p.slot_origin;
     };
     StageRows rows;
-    rows.q = (uint32_t)act_row(16 * wave + (lane & 15)) * (uint32_t)K;
-    rows.bs = (uint32_t)act_row(32 * (wave & 3) + 16 * (lane >> 5) + (lane & 15));
-    rows.yd = (uint32_t)act_row(64 * (wave & 1) + lane);
+    rows.q = (uint32_t)act_row(16 * ((wave * NB) >> 2) + (lane & 15)) * (uint32_t)K;
+    rows.bs = (uint32_t)act_row(32 * (wave % (NOP / 2)) + 16 * (lane >> 5) + (lane & 15));
+    rows.yd = (uint32_t)act_row(64 * (wave % (NOP / 4)) + lane);
 
     // weight operand of this wave
     const GroupWeights gw = p.groups[grp];
@@ -245,9 +251,14 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
 #pragma unroll
     for (int o = 0; o < NOP; o++) facc[o] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    stage_piece<0>(ab, rows, nsb, 0, L, 0, wave, lane); stage_piece<1>(ab, rows, nsb, 0, L, 0, wave, lane);
-    stage_piece<2>(ab, rows, nsb, 0, L, 0, wave, lane); stage_piece<3>(ab, rows, nsb, 0, L, 0, wave, lane);
-    stage_piece<4>(ab, rows, nsb, 0, L, 0, wave, lane); stage_piece<5>(ab, rows, nsb, 0, L, 0, wave, lane);
+    // transfer t of the wave's share (quant stretches, sums, scales), then the weight tile
+    auto stage = [&](auto I, int sb, int buf) { stage_piece<decltype(I)::value, NOP>(ab, rows, nsb, sb, L, buf, wave, lane); };
+    using std::integral_constant;
+    stage(integral_constant<int, 0>{}, 0, 0);
+    stage(integral_constant<int, 1>{}, 0, 0);
+    stage(integral_constant<int, NB>{}, 0, 0);
+    stage(integral_constant<int, NB + 1>{}, 0, 0);
+    if constexpr (NB == 4) { stage(integral_constant<int, 2>{}, 0, 0); stage(integral_constant<int, 3>{}, 0, 0); }
     BRegs raw = b_load(wp, lane);
     wait_all_loads();
     __syncthreads();
@@ -255,15 +266,22 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
         const int buf = sb & 1, nb = buf ^ 1;
         const int sbn = sb + 1 < nsb ? sb + 1 : sb;
         const BPlanes B = b_prepare(raw, lane);
-        // the next super-block's activations and weights are requested one transfer per operand
-        gemm_operand(B, L, buf, 0, lane, facc[0], [&] { stage_piece<0>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 1, lane, facc[1], [&] { stage_piece<1>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 2, lane, facc[2], [&] { stage_piece<2>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 3, lane, facc[3], [&] { stage_piece<3>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 4, lane, facc[4], [&] { stage_piece<4>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 5, lane, facc[5], [&] { stage_piece<5>(ab, rows, nsb, sbn, L, nb, wave, lane); });
-        gemm_operand(B, L, buf, 6, lane, facc[6], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
-        gemm_operand(B, L, buf, 7, lane, facc[7], [&] {});
+        // the next super-block's activations and weights are requested while the operands' MFMAs drain
+        if constexpr (NOP == 8) {
+            gemm_operand(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, 1>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 2, lane, facc[2], [&] { stage(integral_constant<int, 2>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 3, lane, facc[3], [&] { stage(integral_constant<int, 3>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 4, lane, facc[4], [&] { stage(integral_constant<int, 4>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 5, lane, facc[5], [&] { stage(integral_constant<int, 5>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 6, lane, facc[6], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
+            gemm_operand(B, L, buf, 7, lane, facc[7], [&] {});
+        } else {
+            gemm_operand(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); stage(integral_constant<int, 1>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, NB>{}, sbn, nb); stage(integral_constant<int, NB + 1>{}, sbn, nb); });
+            gemm_operand(B, L, buf, 2, lane, facc[2], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
+            gemm_operand(B, L, buf, 3, lane, facc[3], [&] {});
+        }
         wait_all_loads();
         __syncthreads();
     }
@@ -273,7 +291,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     if (MODE == 0) {
         // w3 waves (4-7) park their sums in LDS (the activation buffers are free now), w1 waves combine
         float* xch = reinterpret_cast<float*>(L.q[0]);   // [4 waves][NOP][4 i][64 lanes] floats
-        static_assert(4 * NOP * 4 * 64 * 4 <= sizeof(L.q[0]), "exchange area");
+        static_assert(4 * NOP * 4 * 64 * 4 <= sizeof(L.q), "exchange area");
         if (wave >= 4) {
 #pragma unroll
             for (int o = 0; o < NOP; o++)
@@ -306,17 +324,20 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
 }
 
 static unsigned gemm_grid(int n_rb, int64_t max_tiles) {
+    // patches of 8 row blocks x 8 tiles, dealt round-robin to the eight XCDs: a whole number of rounds
     const int64_t RG = (n_rb + 7) / 8, TG = (max_tiles + 7) / 8;
-    return (unsigned)(RG * TG * 64);
+    return (unsigned)((RG * TG + 7) / 8 * 8 * 64);
 }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s) {
-    dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1)));
-    hipLaunchKernelGGL(q4k_gemm_kernel<0>, grid, dim3(G_THREADS), 0, s, p);
+    dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
+    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<0, 4>), grid, dim3(G_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q4k_gemm_kernel<0, 8>), grid, dim3(G_THREADS), 0, s, p);
     return hipGetLastError();
 }
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s) {
-    dim3 grid(gemm_grid(p.H / 128, max_gemm_tiles(p.n_slots, p.n_groups + 1)));
-    hipLaunchKernelGGL(q4k_gemm_kernel<1>, grid, dim3(G_THREADS), 0, s, p);
+    dim3 grid(gemm_grid(p.H / 128, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
+    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<1, 4>), grid, dim3(G_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q4k_gemm_kernel<1, 8>), grid, dim3(G_THREADS), 0, s, p);
     return hipGetLastError();
 }
 
