@@ -331,6 +331,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
     ep.slot_tiles = (T * L->k > 24 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;
+    const bool narrow = direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
+                        (force_narrow >= 0 ? force_narrow > 0 : T * L->k <= L->E);
     if (tiled) {
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();
@@ -340,6 +343,17 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_REQUANT);
         MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
+        MOE_MARK(ST_DOWN);
+    } else if (narrow) {
+        // very small Q4K batches: at most half of the experts can be active, so the weights are cut
+        // into four times as many workgroups; those write f32 h and a small pass quantises it
+        if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
+        ep.hbuf = L->hbuf.as<float>();
+        MOE_HIP_CHECK(launch_expert_up(ep, s));
+        MOE_MARK(ST_UP);
+        MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
+        MOE_MARK(ST_REQUANT);
+        MOE_HIP_CHECK(launch_expert_down(ep, s));
         MOE_MARK(ST_DOWN);
     } else {
         MOE_HIP_CHECK(launch_expert_up(ep, s));   // re-quantises the intermediate in its epilogue

@@ -131,17 +131,25 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
 // are at the same step of their K walk then read one contiguous region, which spreads the requests
 // evenly over the HBM channels.  `sb_stride` = row tiles of the matrix * Q4K_TILE_BYTES.
 template <int NT, int RING>
-__device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t sb_stride, int sb_lo, int lane, Q4KTile t[RING]) {
+__device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t sb_stride, int sb_lo, int sb_last, int lane, Q4KTile t[RING]) {
 #pragma unroll
-    for (int j = 0; j < RING; j++) t[j] = load_q4k_tile(tp[j] + (size_t)sb_lo * sb_stride, lane);
+    for (int j = 0; j < RING; j++) {
+        const int sb = sb_lo + j / NT < sb_last ? sb_lo + j / NT : sb_last;
+        t[j] = load_q4k_tile(tp[j % NT] + (size_t)sb * sb_stride, lane);
+    }
 }
 
 // `t` must have been filled by q4k_engine_prefetch for sb_lo (callers issue it before they know
 // their slot list, so the first weight tiles are already on their way while the list is built).
+// RING <= NT: the ring rotates inside a super-block.  RING a multiple of NT (few tiles per wave):
+// the ring spans RING/NT super-blocks, so that a wave with little work per super-block still keeps
+// RING tiles in flight; the loop then advances RING/NT super-blocks per trip, and a trip that runs
+// past the end multiplies its surplus super-blocks by a zero activation scale.
 template <int TT, int NT, int RING, int DBG = 0>
 __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride, Q4KTile t[RING], const ActBuf& ab, int K, int nsb,
                                   int sb_lo, int sb_hi, const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
-    static_assert(NT % RING == 0, "ring must divide the tiles per super-block");
+    static_assert(NT % RING == 0 || RING % NT == 0, "ring must divide, or be a multiple of, the tiles per super-block");
+    constexpr int U = RING > NT ? RING / NT : 1;   // super-blocks per trip
     if (sb_lo >= sb_hi) return;
     Q8KOperand A[TT];
 #pragma unroll
@@ -149,32 +157,43 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride,
     // The loop body is one basic block: prefetches past the end are redirected to the last
     // super-block (a harmless repeated load) instead of being branched around, so that the
     // scheduling fences below really bound the live ranges.
-    for (int sb = sb_lo; sb < sb_hi; sb++) {
-        float yd[TT][4];
+    for (int sb0 = sb_lo; sb0 < sb_hi; sb0 += U) {
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++)
+        for (int u = 0; u < U; u++) {
+            const int sb = sb0 + u;
+            const bool live = U == 1 || sb < sb_hi;
+            float yd[TT][4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) yd[tt][i] = __shfl(A[tt].yd, 4 * g + i, 64);
-        const int sb_next = (sb + 1 < sb_hi) ? sb + 1 : sb;
+            for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-        for (int j = 0; j < NT; j++) {
-            const Q4KTile w = t[j % RING];
-            const int jn = (j + RING) % NT;
-            const int sbn = (j + RING) / NT ? sb_next : sb;
-            t[j % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * sb_stride, lane);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int i = 0; i < 4; i++) {
+                    const float v = __shfl(A[tt].yd, 4 * g + i, 64);
+                    yd[tt][i] = live ? v : 0.f;
+                }
+            const int sb_next = (sb + 1 < sb_hi) ? sb + 1 : sb_hi - 1;
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) {
-                if (DBG == 1)  // timing experiment: consume the loads without the arithmetic
-                    acc[j][tt][0] += __uint_as_float((w.q0.x ^ w.q0.w ^ w.q1.y ^ w.q1.z ^ w.sc.z ^ A[tt].a[0].x ^ A[tt].a[3].w) & 0x007fffffu);
-                else
-                    q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
+            for (int j = 0; j < NT; j++) {
+                const int idx = u * NT + j;            // position in the trip
+                const Q4KTile w = t[idx % RING];
+                const int ahead = idx + RING;          // the item that takes this ring place
+                const int jn = ahead % NT;
+                int sbn = sb0 + ahead / NT;
+                sbn = sbn < sb_hi ? sbn : sb_hi - 1;
+                t[idx % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * sb_stride, lane);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) {
+                    if (DBG == 1)  // timing experiment: consume the loads without the arithmetic
+                        acc[j][tt][0] += __uint_as_float((w.q0.x ^ w.q0.w ^ w.q1.y ^ w.q1.z ^ w.sc.z ^ A[tt].a[0].x ^ A[tt].a[3].w) & 0x007fffffu);
+                    else
+                        q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (DBG != 2) {  // DBG 2: timing experiment without the per-super-block operand reload
+            if (DBG != 2) {  // DBG 2: timing experiment without the per-super-block operand reload
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
+                for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
+            }
         }
     }
 }
@@ -186,12 +205,14 @@ __device__ inline float silu_fast(float v) { return v / (1.0f + __expf(-v)); }
 __device__ inline float silu_ref(float v) { return v / (1.0f + expf_glibc(-v)); }  // op.rs:646-648
 
 // ---------------------------------------------------------------------------------------------
-// Up projection.  A workgroup owns 256 rows of F of one expert (= one Q8K block of h per slot);
-// wave w carries rows [w*256/NW, (w+1)*256/NW) of both w1 and w3 over the whole of K.
-constexpr int UP_ROWS = 256;
+// Up projection.  A workgroup owns UP_ROWS rows of F of one expert; wave w carries rows
+// [w*UP_ROWS/NW, (w+1)*UP_ROWS/NW) of both w1 and w3 over the whole of K.  UP_ROWS = 256 is one Q8K
+// block of h per slot, quantised in the epilogue.  UP_ROWS = 64 (very small batches, where only a
+// few experts are active and 256-row workgroups would leave most CUs without work) writes f32 h to
+// p.hbuf instead and leaves the quantisation to a pass of its own.
 constexpr int HBUF_STRIDE = 260;
 
-template <int TT, int NW, int RING, int DBG = 0>
+template <int TT, int NW, int RING, int DBG = 0, int UP_ROWS = 256>
 __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STRIDE], int* list_lds, int* wtot_lds) {
     constexpr int RTW = (UP_ROWS / 16) / NW;  // row tiles per wave and matrix
     constexpr int NT = 2 * RTW;
@@ -211,7 +232,7 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
     const size_t sb_stride = (size_t)(F / 16) * Q4K_TILE_BYTES;
     // first weight tiles go out before anything else; an expert without tokens wastes them
     Q4KTile ring[RING];
-    q4k_engine_prefetch<NT, RING>(tp, sb_stride, 0, lane, ring);
+    q4k_engine_prefetch<NT, RING>(tp, sb_stride, 0, nsb - 1, lane, ring);
 
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
@@ -233,6 +254,20 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
 
     q4k_engine<TT, NT, RING, DBG>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
 
+    if (UP_ROWS != 256) {   // h = silu(w1 x) * (w3 x) straight to memory
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int pos = tg0 + tt * 16 + 4 * g + i;
+                if (pos >= gs.n) continue;
+                const int64_t hrow = gs.slot(pos) - p.slot_origin;
+#pragma unroll
+                for (int j = 0; j < RTW; j++)
+                    p.hbuf[hrow * F + rb * UP_ROWS + (wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
+            }
+        return;
+    }
     // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
 #pragma unroll
     for (int tt = 0; tt < TT; tt++)
@@ -253,27 +288,28 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
 }
 
 // ---------------------------------------------------------------------------------------------
-// Down projection: a workgroup owns 64 weight rows (four row tiles) of one expert; its NW waves
-// split K, every wave carrying the four tiles over its K range, and the partial sums meet in LDS.
-template <int TT, int NW, int RING>
-__device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT * 4][64], int* list_lds, int* wtot_lds) {
+// Down projection: a workgroup owns NTD row tiles (64 weight rows; 32 for very small batches) of one
+// expert; its NW waves split K, every wave carrying the tiles over its K range, and the partial sums
+// meet in LDS.
+template <int TT, int NW, int RING, int NTD = 4>
+__device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * TT * 4][64], int* list_lds, int* wtot_lds) {
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
     const int grp = blockIdx.y;
     const int H = p.H, F = p.F, nsb = F / 256;
     const int n_rt = H / 16;
-    const int rt0 = blockIdx.x * 4;
+    const int rt0 = blockIdx.x * NTD;
     const uint8_t* w2 = p.groups[grp].w2;
-    const uint8_t* tp[4];
+    const uint8_t* tp[NTD];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NTD; j++) {
         int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
         tp[j] = w2 + (size_t)rt * Q4K_TILE_BYTES;
     }
     const size_t sb_stride = (size_t)n_rt * Q4K_TILE_BYTES;
     const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
     Q4KTile ring[RING];
-    q4k_engine_prefetch<4, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, lane, ring);
+    q4k_engine_prefetch<NTD, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, sb_hi > sb_lo ? sb_hi - 1 : (sb_lo < nsb ? sb_lo : nsb - 1), lane, ring);
 
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
@@ -285,25 +321,25 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
         int i = tg0 + tt * 16 + r;
         rowA[tt] = gs.slot(i < gs.n ? i : gs.n - 1) - p.slot_origin;
     }
-    float acc[4][TT][4];
+    float acc[NTD][TT][4];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NTD; j++)
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<TT, 4, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
+    q4k_engine<TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
 
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NTD; j++)
 #pragma unroll
         for (int tt = 0; tt < TT; tt++)
 #pragma unroll
             for (int i = 0; i < 4; i++) part[wave][(j * TT + tt) * 4 + i][lane] = acc[j][tt][i];
     __syncthreads();
-    // 4*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ...
-    for (int v = wave; v < 4 * TT * 4; v += NW) {
+    // NTD*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ...
+    for (int v = wave; v < NTD * TT * 4; v += NW) {
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; w++) sum += part[w][v][lane];
@@ -317,6 +353,19 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
 }
 
 #define DEF_UP(NAME, TT, NW, RING, WPE) DEF_UP_D(NAME, TT, NW, RING, WPE, 0)
+#define DEF_UP_NARROW(NAME, NW, RING, WPE)                                                                    \
+    __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
+        __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
+        __shared__ int wtot_lds[NW];                                                                        \
+        q4k_up_body<1, NW, RING, 0, 64>(p, nullptr, list_lds, wtot_lds);                                    \
+    }
+#define DEF_DOWN_NARROW(NAME, NW, RING, WPE)                                                                  \
+    __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
+        __shared__ float part[NW][2 * 4][64];                                                               \
+        __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
+        __shared__ int wtot_lds[NW];                                                                        \
+        q4k_down_body<1, NW, RING, 2>(p, part, list_lds, wtot_lds);                                         \
+    }
 #define DEF_UP_D(NAME, TT, NW, RING, WPE, DBG)                                                                   \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ float hbuf[TT * 16][HBUF_STRIDE];                                                        \
@@ -337,10 +386,12 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[4 * TT
 // without streaming its weights twice) need the registers of a two-waves-per-SIMD launch.
 DEF_UP(q4k_up_t1_v0, 1, 8, 2, 4)
 DEF_UP(q4k_up_t1_v1, 1, 4, 2, 3)
+DEF_UP_NARROW(q4k_up_t1_narrow, 4, 2, 3)
 DEF_UP(q4k_up_t2, 2, 4, 2, 2)
 DEF_UP(q4k_up_t4, 4, 8, 2, 2)
 DEF_DOWN(q4k_down_t1_v0, 1, 8, 2, 4)
 DEF_DOWN(q4k_down_t1_v1, 1, 4, 2, 3)
+DEF_DOWN_NARROW(q4k_down_t1_narrow, 8, 2, 4)
 DEF_DOWN(q4k_down_t2, 2, 4, 2, 2)
 DEF_DOWN(q4k_down_t4, 4, 8, 2, 2)
 
@@ -354,7 +405,12 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_UP_VARIANT", 1);
     const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
-    dim3 grid((unsigned)(p.F / UP_ROWS), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (p.hbuf && tt == 1) {   // narrow workgroups (64 rows), f32 h to p.hbuf
+        dim3 ngrid((unsigned)(p.F / 64), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
+        hipLaunchKernelGGL(q4k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
+    dim3 grid((unsigned)(p.F / 256), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     if (tt == 4) hipLaunchKernelGGL(q4k_up_t4, grid, dim3(512), 0, s, p);
     else if (tt == 2) hipLaunchKernelGGL(q4k_up_t2, grid, dim3(256), 0, s, p);
     else if (v == 0) hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
@@ -366,6 +422,11 @@ hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_DOWN_VARIANT", 1);
     const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    if (p.hbuf && tt == 1) {   // narrow workgroups (32 rows), eight waves split K
+        dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
+        hipLaunchKernelGGL(q4k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
+        return hipGetLastError();
+    }
     dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     if (tt == 4) hipLaunchKernelGGL(q4k_down_t4, grid, dim3(512), 0, s, p);
     else if (tt == 2) hipLaunchKernelGGL(q4k_down_t2, grid, dim3(256), 0, s, p);

@@ -4,6 +4,7 @@
 // to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0),
 // 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
+#include <algorithm>
 #include "act_quant.hpp"
 #include "kernels.hpp"
 
@@ -154,15 +155,16 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int6
     const int64_t row = blockIdx.x;
     const float* xr = x + row * k;
     if (VDT == MOE_GGML_Q8K) {
+        // blocks of a row are dealt to the waves of gridDim.y workgroups (few rows: many workgroups per row)
         const int nb = k / 256;
-        for (int b = wave; b < nb; b += 4) {
+        for (int b = blockIdx.y * 4 + wave; b < nb; b += 4 * gridDim.y) {
             float4 v = *reinterpret_cast<const float4*>(xr + b * 256 + lane * 4);
             quantize_q8k_block(v, lane, out.qs + row * k + b * 256, out.d + row * nb + b,
                                reinterpret_cast<__half*>(out.bsum) + (row * nb + b) * 16);
         }
     } else {
         const int nb = k / 32;
-        for (int h = tid; h < k; h += 256)
+        for (int h = blockIdx.y * 256 + tid; h < k; h += 256 * gridDim.y)
             quantize_q8_0_block(xr[h], lane, out.qs + row * k + h, out.d + row * nb + h / 32,
                                 reinterpret_cast<int32_t*>(out.bsum) + row * nb + h / 32);
     }
@@ -226,10 +228,12 @@ hipError_t launch_dequant_std(int dt, const uint8_t* blocks, float* out, int64_t
 
 hipError_t launch_quantize_rows(int vdt, const float* x, int64_t rows, int k, const ActBuf& out, hipStream_t s) {
     if (rows == 0) return hipSuccess;
+    const int64_t per_row = vdt == MOE_GGML_Q8K ? (k / 256 + 3) / 4 : (k + 255) / 256;   // workgroups that have a share of a row
+    const unsigned split = (unsigned)std::max<int64_t>(1, std::min<int64_t>(per_row, 2048 / rows));
     if (vdt == MOE_GGML_Q8K)
-        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8K>, dim3((unsigned)rows), dim3(256), 0, s, x, rows, k, out);
+        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8K>, dim3((unsigned)rows, split), dim3(256), 0, s, x, rows, k, out);
     else
-        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8_0>, dim3((unsigned)rows), dim3(256), 0, s, x, rows, k, out);
+        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8_0>, dim3((unsigned)rows, split), dim3(256), 0, s, x, rows, k, out);
     return hipGetLastError();
 }
 
