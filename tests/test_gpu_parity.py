@@ -214,6 +214,23 @@ def test_block_q8_0_shared_expert_top4():
     gpu.close()
 
 
+@pytest.mark.parametrize("T", [20, 40, 70])
+def test_block_q4k_shared_expert_slot_tiles(T):
+    # the always-on expert sees every token: its streaming kernels carry 2 (T = 20) or 4 (T = 40) 16-slot
+    # tiles per pass over the weights, and need a second pass at T = 70
+    ref, gpu = make_pair(512, 512, 8, 2, O.Q4K, seed=6, Fs=1024)
+    check_block(ref, gpu, T)
+    gpu.close()
+
+
+def test_block_q4k_tile_sizes_and_paths():
+    # 25 rows per expert and more go to the tiled kernels: 64-slot tiles up to ~96 rows per expert, 128 beyond
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
+    for T in (104, 130, 400, 600):
+        check_block(ref, gpu, T)
+    gpu.close()
+
+
 def test_block_no_renorm_and_bias():
     bias = np.log(1.0 / np.arange(1, 9)).astype(np.float32)
     ref, gpu = make_pair(256, 512, 8, 2, O.Q4K, seed=4, norm_topk=False, gate_bias=bias)
