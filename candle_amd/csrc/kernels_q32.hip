@@ -22,19 +22,31 @@ struct Q32Tile {
     float d;
 };
 
+// weight tiles are read once per launch: non-temporal loads keep them from displacing the activations
+// and routing lists in the caches
+typedef uint32_t u32x2_q32 __attribute__((ext_vector_type(2)));
+__device__ inline uint2 load_stream8(const uint8_t* p) {
+    const u32x2_q32 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_q32*>(p));
+    return make_uint2(v.x, v.y);
+}
+__device__ inline float load_stream_half(const uint8_t* p) {
+    const unsigned short h = __builtin_nontemporal_load(reinterpret_cast<const unsigned short*>(p));
+    return __half2float(__ushort_as_half(h));
+}
+
 template <int DT>
 __device__ inline Q32Tile<DT> load_q32_tile(const uint8_t* tile, int lane) {
     Q32Tile<DT> t;
     const int r = lane & 15, g = lane >> 4;
     if (DT == MOE_GGML_Q8_0) {
-        t.q = *reinterpret_cast<const uint2*>(tile + lane * 8);
-        t.d = __half2float(*reinterpret_cast<const __half*>(tile + 512 + 2 * r));
+        t.q = load_stream8(tile + lane * 8);
+        t.d = load_stream_half(tile + 512 + 2 * r);
     } else {
-        uint2 w = *reinterpret_cast<const uint2*>(tile + r * 16 + 8 * (g >> 1));
+        uint2 w = load_stream8(tile + r * 16 + 8 * (g >> 1));
         if (g & 1) { w.x >>= 4; w.y >>= 4; }
         t.q.x = w.x & 0x0f0f0f0fu;
         t.q.y = w.y & 0x0f0f0f0fu;
-        t.d = __half2float(*reinterpret_cast<const __half*>(tile + 256 + 2 * r));
+        t.d = load_stream_half(tile + 256 + 2 * r);
     }
     return t;
 }

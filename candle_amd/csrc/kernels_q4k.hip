@@ -47,11 +47,17 @@ __device__ inline uint4 gload<uint4>(const void* uniform_base, uint32_t off) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// weight tiles are read once per launch: non-temporal loads keep them from displacing the activations
+// and routing lists in the caches
+__device__ inline uint4 gload_stream(const void* uniform_base, uint32_t off) {
+    u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x4*>((gbytes)uniform_base + off));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 __device__ inline Q4KTile load_q4k_tile(const uint8_t* tile, int lane) {
     Q4KTile t;
-    t.q0 = gload<uint4>(tile, (uint32_t)lane * 16u);
-    t.q1 = gload<uint4>(tile, 1024u + (uint32_t)lane * 16u);
-    t.sc = gload<uint4>(tile, 2048u + (uint32_t)(lane & 15) * 16u);
+    t.q0 = gload_stream(tile, (uint32_t)lane * 16u);
+    t.q1 = gload_stream(tile, 1024u + (uint32_t)lane * 16u);
+    t.sc = gload_stream(tile, 2048u + (uint32_t)(lane & 15) * 16u);
     return t;
 }
 
