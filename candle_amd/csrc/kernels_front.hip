@@ -92,53 +92,76 @@ __device__ inline void route_one_token(float* p /*[E] logits in, probs out*/, in
 }
 
 // ---------------------------------------------------------------------------------------------
-// Per-expert lists.  Runs in ONE workgroup of FRONT_THREADS threads.  Assignments are taken in
-// (token, rank) order; within an expert the slots keep that order, i.e. ascending token index,
-// exactly as the Vec pushes of the reference produce them.
+// Per-expert lists.  Runs in ONE workgroup of DISPATCH_THREADS threads (16 waves).  Assignments are
+// taken in (token, rank) order; within an expert the slots keep that order, i.e. ascending token
+// index, exactly as the Vec pushes of the reference produce them.
+constexpr int DISPATCH_THREADS = 1024;
 struct DispatchShared {
-    int cnt[FRONT_THREADS / 64][MAX_E];
+    int cnt[DISPATCH_THREADS / 64][MAX_E];
     int off[MAX_E + 2];
+    int tot[MAX_E];
 };
 
 // tok_slots is written and re-read inside one workgroup: bypass the vector cache on the re-read
 __device__ inline int ld_i32(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-__device__ inline float ld_f32(const float* p) { return *p; }
 
 __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, bool shared, DispatchShared& sh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    constexpr int NW = FRONT_THREADS / 64;
+    constexpr int NW = DISPATCH_THREADS / 64;
     const int64_t A = T * k;
     const int64_t chunk = ((A + NW - 1) / NW + 63) / 64 * 64;
     const int64_t lo = wave * chunk, hi = (lo + chunk < A) ? lo + chunk : A;
-    for (int i = tid; i < NW * MAX_E; i += FRONT_THREADS) (&sh.cnt[0][0])[i] = 0;
+    for (int i = tid; i < NW * MAX_E; i += DISPATCH_THREADS) (&sh.cnt[0][0])[i] = 0;
     __syncthreads();
-    // phase 1: per-wave histogram from ballots
-    for (int64_t base = lo; base < hi; base += 64) {
-        int64_t a = base + lane;
-        bool valid = a < hi;
-        int e = valid ? ld_i32(rb.topk_idx + a) : -1;
-        unsigned long long rem = __ballot(valid);
-        while (rem) {
-            int leader = __ffsll((long long)rem) - 1;
-            int e0 = __shfl(e, leader, 64);
-            unsigned long long m = __ballot(valid && e == e0);
-            if (lane == leader) sh.cnt[wave][e0] += __popcll(m);
-            rem &= ~m;
+    // phase 1: per-wave histogram from ballots (topk_idx comes from the previous kernel: plain loads,
+    // the next 64 assignments requested while these are counted)
+    {
+        int e_next = (lo + lane < hi) ? rb.topk_idx[lo + lane] : -1;
+        for (int64_t base = lo; base < hi; base += 64) {
+            const int e = e_next;
+            const bool valid = base + lane < hi;
+            e_next = (base + 64 + lane < hi) ? rb.topk_idx[base + 64 + lane] : -1;
+            unsigned long long rem = __ballot(valid);
+            while (rem) {
+                int leader = __ffsll((long long)rem) - 1;
+                int e0 = __shfl(e, leader, 64);
+                unsigned long long m = __ballot(valid && e == e0);
+                if (lane == leader) sh.cnt[wave][e0] += __popcll(m);
+                rem &= ~m;
+            }
         }
     }
     __syncthreads();
-    // phase 2: exclusive scan over experts, then per-wave bases
-    if (tid == 0) {
-        int run = 0;
-        for (int e = 0; e < E; e++) {
-            sh.off[e] = run;
-            for (int w = 0; w < NW; w++) run += sh.cnt[w][e];
-        }
-        sh.off[E] = run;
-        sh.off[E + 1] = run + (shared ? (int)T : 0);
+    // phase 2: totals per expert, exclusive scan over experts (one wave, four experts per lane), per-wave bases
+    for (int e = tid; e < MAX_E; e += DISPATCH_THREADS) {
+        int t = 0;
+        if (e < E)
+            for (int w = 0; w < NW; w++) t += sh.cnt[w][e];
+        sh.tot[e] = t;
     }
     __syncthreads();
-    for (int e = tid; e < E; e += FRONT_THREADS) {
+    if (wave == 0) {
+        static_assert(MAX_E == 256, "four experts per lane");
+        const int t0 = sh.tot[4 * lane], t1 = sh.tot[4 * lane + 1], t2 = sh.tot[4 * lane + 2], t3 = sh.tot[4 * lane + 3];
+        int incl = t0 + t1 + t2 + t3;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += v;
+        }
+        const int base = incl - (t0 + t1 + t2 + t3);
+        sh.off[4 * lane] = base;
+        sh.off[4 * lane + 1] = base + t0;
+        sh.off[4 * lane + 2] = base + t0 + t1;
+        sh.off[4 * lane + 3] = base + t0 + t1 + t2;
+        if (lane == 63) sh.off[MAX_E] = incl;   // = A
+    }
+    __syncthreads();
+    if (tid == 0) {   // experts past E have no assignments: off[E] == A already; the shared expert follows
+        sh.off[E] = (int)A;
+        sh.off[E + 1] = (int)A + (shared ? (int)T : 0);
+    }
+    for (int e = tid; e < E; e += DISPATCH_THREADS) {
         int run = sh.off[e];
         for (int w = 0; w < NW; w++) {
             int c = sh.cnt[w][e];
@@ -146,7 +169,8 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
             run += c;
         }
     }
-    for (int e = tid; e <= E + (shared ? 1 : 0); e += FRONT_THREADS) rb.offsets[e] = sh.off[e];
+    __syncthreads();
+    for (int e = tid; e <= E + (shared ? 1 : 0); e += DISPATCH_THREADS) rb.offsets[e] = sh.off[e];
     if (tid == 0 && rb.tile_tab) {  // work list of the tiled expert kernels
         int n = 0;
         const int G = E + (shared ? 1 : 0);
@@ -160,41 +184,46 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         }
         rb.tile_tab[0] = n;
     }
-    __syncthreads();
     // phase 3: stable placement
     const int kk = k + (shared ? 1 : 0);
-    for (int64_t base = lo; base < hi; base += 64) {
-        int64_t a = base + lane;
-        bool valid = a < hi;
-        int e = valid ? ld_i32(rb.topk_idx + a) : -1;
-        float w = valid ? ld_f32(rb.topk_w + a) : 0.f;
-        unsigned long long rem = __ballot(valid);
-        unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-        int slot = -1;
-        while (rem) {
-            int leader = __ffsll((long long)rem) - 1;
-            int e0 = __shfl(e, leader, 64);
-            unsigned long long m = __ballot(valid && e == e0);
-            int cur = sh.cnt[wave][e0];
-            if (valid && e == e0) slot = cur + __popcll(m & lt);
-            // all lanes have read `cur` before the leader updates it (same wave, program order)
-            if (lane == leader) sh.cnt[wave][e0] = cur + __popcll(m);
-            rem &= ~m;
-        }
-        if (valid) {
-            int t = (int)(a / k);
-            rb.perm_token[slot] = t;
-            rb.perm_w[slot] = w;
-            // stash (slot) per assignment in tok_slots, unsorted for now
-            rb.tok_slots[(int64_t)t * kk + (int)(a % k)] = slot;
+    {
+        int e_next = (lo + lane < hi) ? rb.topk_idx[lo + lane] : -1;
+        float w_next = (lo + lane < hi) ? rb.topk_w[lo + lane] : 0.f;
+        const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+        for (int64_t base = lo; base < hi; base += 64) {
+            const int64_t a = base + lane;
+            const bool valid = a < hi;
+            const int e = e_next;
+            const float w = w_next;
+            e_next = (a + 64 < hi) ? rb.topk_idx[a + 64] : -1;
+            w_next = (a + 64 < hi) ? rb.topk_w[a + 64] : 0.f;
+            unsigned long long rem = __ballot(valid);
+            int slot = -1;
+            while (rem) {
+                int leader = __ffsll((long long)rem) - 1;
+                int e0 = __shfl(e, leader, 64);
+                unsigned long long m = __ballot(valid && e == e0);
+                int cur = sh.cnt[wave][e0];
+                if (valid && e == e0) slot = cur + __popcll(m & lt);
+                // all lanes have read `cur` before the leader updates it (same wave, program order)
+                if (lane == leader) sh.cnt[wave][e0] = cur + __popcll(m);
+                rem &= ~m;
+            }
+            if (valid) {
+                int t = (int)(a / k);
+                rb.perm_token[slot] = t;
+                rb.perm_w[slot] = w;
+                // stash (slot) per assignment in tok_slots, unsorted for now
+                rb.tok_slots[(int64_t)t * kk + (int)(a % k)] = slot;
+            }
         }
     }
     __syncthreads();
     // phase 4: per token, order its slots by ascending expert index (combine order); append shared
-    for (int64_t t = tid; t < T; t += FRONT_THREADS) {
+    for (int64_t t = tid; t < T; t += DISPATCH_THREADS) {
         int es[MAX_K], ss[MAX_K];
         for (int r = 0; r < k; r++) {
-            es[r] = ld_i32(rb.topk_idx + t * k + r);
+            es[r] = rb.topk_idx[t * k + r];
             ss[r] = ld_i32(rb.tok_slots + t * kk + r);
         }
         for (int i = 1; i < k; i++) {
@@ -207,7 +236,7 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
             int slot = (int)(A + t);
             rb.tok_slots[t * kk + k] = slot;
             rb.perm_token[slot] = (int)t;
-            rb.perm_w[slot] = ld_f32(rb.shared_w + t);
+            rb.perm_w[slot] = rb.shared_w[t];
         }
     }
 }
@@ -524,7 +553,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
     }
 }
 
-__global__ __launch_bounds__(FRONT_THREADS) void dispatch_kernel(RouteBufs rb, int64_t T, int E, int k, int shared) {
+__global__ __launch_bounds__(DISPATCH_THREADS) void dispatch_kernel(RouteBufs rb, int64_t T, int E, int k, int shared) {
     __shared__ DispatchShared dsh;
     dispatch_block(rb, T, E, k, shared != 0, dsh);
 }
@@ -617,7 +646,7 @@ hipError_t launch_identity_routing(const RouteBufs& rb, int64_t rows, hipStream_
 
 hipError_t launch_dispatch(const RouteBufs& rb, int64_t T, int E, int k, bool shared, hipStream_t s) {
     if (T == 0) return hipSuccess;
-    hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(FRONT_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0);
+    hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(DISPATCH_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0);
     return hipGetLastError();
 }
 
