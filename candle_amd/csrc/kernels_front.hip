@@ -456,10 +456,20 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
         }
         __syncthreads();
         if (tid == 0) {
+            // the chain of H dependent adds is the cost; the operands are fetched 32 at a time ahead of it
             float sum2 = 0.f;
-            for (int h = 0; h < H; h += 4) {
-                const float4 v = *reinterpret_cast<const float4*>(&sq[h]);
-                sum2 += v.x; sum2 += v.y; sum2 += v.z; sum2 += v.w;
+            float4 nxt[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) nxt[j] = *reinterpret_cast<const float4*>(&sq[4 * j]);
+            for (int h = 0; h < H; h += 32) {
+                float4 cur[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) cur[j] = nxt[j];
+                const int hn = h + 32 < H ? h + 32 : h;
+#pragma unroll
+                for (int j = 0; j < 8; j++) nxt[j] = *reinterpret_cast<const float4*>(&sq[hn + 4 * j]);
+#pragma unroll
+                for (int j = 0; j < 8; j++) { sum2 += cur[j].x; sum2 += cur[j].y; sum2 += cur[j].z; sum2 += cur[j].w; }
             }
             m_lds = sqrtf(sum2 / (float)H + p.rms_eps);
         }
