@@ -8,7 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(OUT_DIR, "libcandle_amd_moe.so")
-SOURCES = ["api.hip", "kernels_front.hip", "kernels_util.hip", "kernels_q4k.hip", "kernels_q32.hip", "kernels_wquant.hip", "kernels_q4k_gemm.hip"]
+SOURCES = ["api.hip", "kernels_front.hip", "kernels_util.hip", "kernels_q4k.hip", "kernels_q32.hip", "kernels_wquant.hip", "kernels_q4k_gemm.hip", "gguf.cpp"]
 
 # -ffp-contract=off: candle's Rust never fuses a*b+c, and `to_float` / combine must round the
 # product first to stay bit-exact.  Packed-FP32 instructions are switched off for the whole build.

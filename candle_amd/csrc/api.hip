@@ -331,6 +331,8 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
     ep.slot_tiles = (T * L->k > 24 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
+    if (force_st) ep.slot_tiles = force_st;
     static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;
     const bool narrow = direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
                         (force_narrow >= 0 ? force_narrow > 0 : T * L->k <= L->E);

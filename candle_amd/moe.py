@@ -70,6 +70,24 @@ def load_library():
     L.moe_qmatmul.argtypes = [i32, vp, i64, i64, vp, i64, vp]
     L.moe_quantize_weights.argtypes = [i32, vp, i64, vp]
     L.moe_quantize_weights_device.argtypes = [i32, vp, i64, vp, vp]
+    L.moe_gguf_open.argtypes = [C.c_char_p, C.POINTER(vp)]
+    L.moe_gguf_close.argtypes = [vp]
+    L.moe_gguf_close.restype = None
+    L.moe_gguf_version.argtypes = [vp]
+    L.moe_gguf_tensor_count.argtypes = [vp]
+    L.moe_gguf_tensor_count.restype = i64
+    L.moe_gguf_tensor_data_offset.argtypes = [vp]
+    L.moe_gguf_tensor_data_offset.restype = C.c_uint64
+    L.moe_gguf_tensor_name.argtypes = [vp, i64]
+    L.moe_gguf_tensor_name.restype = C.c_char_p
+    L.moe_gguf_metadata_type.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int)]
+    L.moe_gguf_metadata_u64.argtypes = [vp, C.c_char_p, C.POINTER(C.c_uint64)]
+    L.moe_gguf_metadata_i64.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int64)]
+    L.moe_gguf_metadata_f64.argtypes = [vp, C.c_char_p, C.POINTER(C.c_double)]
+    L.moe_gguf_metadata_str.argtypes = [vp, C.c_char_p, C.c_char_p, C.c_uint64]
+    L.moe_gguf_metadata_array_len.argtypes = [vp, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_int)]
+    L.moe_gguf_tensor.argtypes = [vp, C.c_char_p, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(i64), C.POINTER(vp), C.POINTER(C.c_uint64)]
+    L.moe_layer_create_from_gguf.argtypes = [vp, C.c_int, C.c_int, C.POINTER(vp)]
     L.moe_last_error.restype = C.c_char_p
     L.moe_device_arch.restype = C.c_char_p
     L.moe_debug_expf.restype = C.c_float
@@ -177,6 +195,75 @@ def quantize_weights(dtype, x):
     return out
 
 
+class GgufFile:
+    """A memory-mapped GGUF file (`gguf_file::Content`): metadata, tensor table, tensor bytes."""
+
+    def __init__(self, path):
+        self._h = None
+        h = C.c_void_p()
+        _check(load_library().moe_gguf_open(os.fsencode(path), C.byref(h)))
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None) is not None:
+            load_library().moe_gguf_close(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    @property
+    def version(self):
+        return load_library().moe_gguf_version(self._h)
+
+    @property
+    def tensor_data_offset(self):
+        return load_library().moe_gguf_tensor_data_offset(self._h)
+
+    def tensor_names(self):
+        L = load_library()
+        return [L.moe_gguf_tensor_name(self._h, i).decode() for i in range(L.moe_gguf_tensor_count(self._h))]
+
+    def metadata(self, key):
+        """The value of a metadata key as int / float / bool / str, or ("array", length, element type id)."""
+        L = load_library()
+        k = key.encode()
+        vt = C.c_int()
+        _check(L.moe_gguf_metadata_type(self._h, k, C.byref(vt)))
+        if vt.value in (0, 2, 4, 7, 10):
+            v = C.c_uint64()
+            _check(L.moe_gguf_metadata_u64(self._h, k, C.byref(v)))
+            return bool(v.value) if vt.value == 7 else v.value
+        if vt.value in (1, 3, 5, 11):
+            v = C.c_int64()
+            _check(L.moe_gguf_metadata_i64(self._h, k, C.byref(v)))
+            return v.value
+        if vt.value in (6, 12):
+            v = C.c_double()
+            _check(L.moe_gguf_metadata_f64(self._h, k, C.byref(v)))
+            return v.value
+        if vt.value == 8:
+            buf = C.create_string_buffer(1 << 16)
+            _check(L.moe_gguf_metadata_str(self._h, k, buf, len(buf)))
+            return buf.value.decode(errors="replace")
+        n, et = C.c_uint64(), C.c_int()
+        _check(L.moe_gguf_metadata_array_len(self._h, k, C.byref(n), C.byref(et)))
+        return ("array", n.value, et.value)
+
+    def tensor(self, name):
+        """(ggml dtype id, shape, bytes as a numpy uint8 view of the mapping)."""
+        L = load_library()
+        dt, nd, dims, data, nbytes = C.c_int(), C.c_int(), (C.c_int64 * 8)(), C.c_void_p(), C.c_uint64()
+        _check(L.moe_gguf_tensor(self._h, name.encode(), C.byref(dt), C.byref(nd), dims, C.byref(data), C.byref(nbytes)))
+        raw = np.ctypeslib.as_array(C.cast(data, C.POINTER(C.c_uint8)), shape=(nbytes.value,)) if nbytes.value else np.zeros(0, np.uint8)
+        return dt.value, tuple(dims[i] for i in range(nd.value)), raw
+
+
 class SparseMoeBlock:
     """The MoE arm of `MlpOrMoe` with quantized experts resident on the GPU.
 
@@ -225,6 +312,28 @@ class SparseMoeBlock:
         _check(L.moe_layer_create(C.byref(desc), C.byref(handle)))
         self._h = handle
         del keep  # host copies are only borrowed during create
+
+    @classmethod
+    def from_gguf(cls, gguf, layer_index, norm_topk=True):
+        """The MoE block of layer `layer_index` of a GGUF file (a path or an open GgufFile), as
+        `ModelWeights::from_gguf` builds it (quantized_llama.rs:506-512, 553-578)."""
+        own = not isinstance(gguf, GgufFile)
+        g = GgufFile(gguf) if own else gguf
+        try:
+            h = C.c_void_p()
+            _check(load_library().moe_layer_create_from_gguf(g._h, int(layer_index), int(norm_topk), C.byref(h)))
+            prefix = "blk.%d" % layer_index
+            dt, (f, hdim), _ = g.tensor(prefix + ".ffn_gate.0.weight")
+            self = cls.__new__(cls)
+            self._h = h
+            self.hidden, self.ffn, self.dtype = hdim, f, dt
+            self.n_experts = g.metadata("llama.expert_count")
+            self.top_k = g.metadata("llama.expert_used_count")
+            self.shared_ffn = 0
+            return self
+        finally:
+            if own:
+                g.close()
 
     def close(self):
         if getattr(self, "_h", None) is not None:

@@ -137,6 +137,35 @@ int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, 
 int moe_quantize_weights(int32_t ggml_dtype, const float* x, int64_t n_elems, void* out_blocks);
 int moe_quantize_weights_device(int32_t ggml_dtype, const void* d_x, int64_t n_elems, void* d_out_blocks, void* hip_stream);
 
+/* ---- GGUF expert loader -------------------------------------------------------------------
+ * `Content::read` (candle-core/src/quantized/gguf_file.rs:439-511) on a memory-mapped file: magic and
+ * version 1-3, metadata table, tensor table (dimensions reversed to outermost-first), tensor data
+ * start rounded up to `general.alignment` (default 32).  Host code only: usable without a GPU. */
+typedef struct moe_gguf moe_gguf;
+int moe_gguf_open(const char* path, moe_gguf** out);
+void moe_gguf_close(moe_gguf* file);
+int moe_gguf_version(const moe_gguf* file);
+int64_t moe_gguf_tensor_count(const moe_gguf* file);
+uint64_t moe_gguf_tensor_data_offset(const moe_gguf* file);          /* Content::tensor_data_offset */
+const char* moe_gguf_tensor_name(const moe_gguf* file, int64_t index); /* file order; NULL past the end */
+/* Metadata accessors, `Value::to_*` (gguf_file.rs:226-294): value_type is the on-disk ValueType id
+ * (gguf_file.rs:402-420); u64 upcasts u8/u16/u32/bool as Value::to_u64 does. */
+int moe_gguf_metadata_type(const moe_gguf* file, const char* key, int* value_type);
+int moe_gguf_metadata_u64(const moe_gguf* file, const char* key, uint64_t* out);
+int moe_gguf_metadata_i64(const moe_gguf* file, const char* key, int64_t* out);
+int moe_gguf_metadata_f64(const moe_gguf* file, const char* key, double* out);
+int moe_gguf_metadata_str(const moe_gguf* file, const char* key, char* buf, uint64_t cap);
+int moe_gguf_metadata_array_len(const moe_gguf* file, const char* key, uint64_t* len, int* elem_type);
+/* `TensorInfo::read_from_mmap` (gguf_file.rs:91-126): dtype id, shape (outermost first, up to 8 dims)
+ * and a pointer into the mapping, valid until moe_gguf_close; same divisibility and bounds checks. */
+int moe_gguf_tensor(const moe_gguf* file, const char* name, int* ggml_dtype, int* n_dims, int64_t dims[8], const void** data,
+                    uint64_t* nbytes);
+/* The MoE arm of `ModelWeights::from_gguf` for ONE layer (quantized_llama.rs:506-512, 553-578):
+ * `llama.expert_count`, `llama.expert_used_count`, `blk.{l}.ffn_gate_inp.weight` (F32, F16 or a
+ * supported quantized dtype) and `blk.{l}.ffn_{gate,down,up}.{i}.weight` as w1 / w2 / w3.  All expert
+ * matrices of the layer must share one supported dtype.  Needs the GPU. */
+int moe_layer_create_from_gguf(const moe_gguf* file, int layer_index, int norm_topk, moe_layer** out);
+
 /* Message of the calling thread's last error ("" if none). */
 const char* moe_last_error(void);
 

@@ -1,0 +1,121 @@
+"""GGUF container reader (host code of the library, no GPU needed) against files written the way the
+reference's own writer does (gguf_file.rs:534-582), and against the reference's error behaviour."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import candle_amd
+import gguf_writer as W
+
+
+def rnd(n, seed=0):
+    return np.random.default_rng(seed).integers(0, 256, n, dtype=np.uint8)
+
+
+@pytest.mark.parametrize("version", [1, 2, 3])
+def test_round_trip_all_value_types_and_tensors(tmp_path, version):
+    md = [("a.u8", W.U8, 200), ("a.i8", W.I8, -100), ("a.u16", W.U16, 60000), ("a.i16", W.I16, -30000),
+          ("a.u32", W.U32, 4000000000), ("a.i32", W.I32, -2000000000), ("a.u64", W.U64, 1 << 40), ("a.i64", W.I64, -(1 << 40)),
+          ("a.f32", W.F32, 1.5), ("a.f64", W.F64, -2.25), ("a.true", W.BOOL, 1), ("a.false", W.BOOL, 0),
+          ("a.str", W.STRING, b"hello\0\0"),  # trailing NULs are dropped (gguf_file.rs:145-148)
+          ("a.arr", W.ARRAY, (W.U32, [1, 2, 3])), ("a.strs", W.ARRAY, (W.STRING, ["x", "yy"])),
+          ("a.nested", W.ARRAY, (W.ARRAY, [(W.U8, [1, 2]), (W.U8, [])])), ("a.empty", W.ARRAY, (W.U32, []))]
+    tensors = [("t.f32", 0, (3, 5), rnd(60, 1)), ("t.f16", 1, (7,), rnd(14, 2)), ("t.q4_0", 2, (4, 64), rnd(4 * 2 * 18, 3)),
+               ("t.q8_0", 8, (2, 3, 32), rnd(6 * 34, 4)), ("t.q4k", 12, (2, 512), rnd(4 * 144, 5)), ("t.q6k", 14, (256,), rnd(210, 6))]
+    path = tmp_path / "f.gguf"
+    data_start = W.write_gguf(path, md, tensors, version=version)
+    with candle_amd.GgufFile(str(path)) as g:
+        assert g.version == version
+        assert g.tensor_data_offset == data_start and data_start % 32 == 0
+        assert g.tensor_names() == [t[0] for t in tensors]
+        assert g.metadata("a.u8") == 200 and g.metadata("a.i8") == -100
+        assert g.metadata("a.u16") == 60000 and g.metadata("a.i16") == -30000
+        assert g.metadata("a.u32") == 4000000000 and g.metadata("a.i32") == -2000000000
+        assert g.metadata("a.u64") == 1 << 40 and g.metadata("a.i64") == -(1 << 40)
+        assert g.metadata("a.f32") == 1.5 and g.metadata("a.f64") == -2.25
+        assert g.metadata("a.true") is True and g.metadata("a.false") is False
+        assert g.metadata("a.str") == "hello"
+        assert g.metadata("a.arr") == ("array", 3, W.U32) and g.metadata("a.strs") == ("array", 2, W.STRING)
+        assert g.metadata("a.nested") == ("array", 2, W.ARRAY) and g.metadata("a.empty")[1] == 0
+        raw = open(path, "rb").read()
+        off = data_start
+        for name, dt, shape, data in tensors:
+            gdt, gshape, gbytes = g.tensor(name)
+            assert (gdt, gshape) == (dt, shape)          # dimensions come back outermost first
+            assert bytes(gbytes) == bytes(data) == raw[off: off + len(bytes(data))]
+            off += (len(bytes(data)) + 31) // 32 * 32    # every tensor starts on a 32-byte boundary
+        with pytest.raises(candle_amd.MoeError, match="cannot find tensor info for nope"):
+            g.tensor("nope")
+        with pytest.raises(candle_amd.MoeError, match="cannot find nope in metadata"):
+            g.metadata("nope")
+
+
+def test_alignment_key_moves_the_tensor_data(tmp_path):
+    path = tmp_path / "a.gguf"
+    start = W.write_gguf(path, [("general.alignment", W.U32, 256), ("k", W.STRING, "v" * 70)], [("t", 0, (4,), rnd(16))], alignment=256)
+    with candle_amd.GgufFile(str(path)) as g:
+        assert g.tensor_data_offset == start and start % 256 == 0
+        assert bytes(g.tensor("t")[2]) == bytes(rnd(16))
+    # a negative signed alignment is ignored (gguf_file.rs:497-504): the default 32 applies
+    path2 = tmp_path / "b.gguf"
+    start2 = W.write_gguf(path2, [("general.alignment", W.I32, -8)], [("t", 0, (4,), rnd(16))])
+    with candle_amd.GgufFile(str(path2)) as g:
+        assert g.tensor_data_offset == start2 and start2 % 32 == 0
+
+
+def test_both_magics_are_accepted(tmp_path):
+    for magic in (0x46554747, 0x47475546):  # gguf_file.rs:19
+        path = tmp_path / ("m%x.gguf" % magic)
+        W.write_gguf(path, [], [], magic=magic)
+        with candle_amd.GgufFile(str(path)) as g:
+            assert g.tensor_names() == []
+
+
+def test_malformed_files_are_rejected(tmp_path):
+    good = tmp_path / "good.gguf"
+    W.write_gguf(good, [("k", W.U32, 1)], [("t", 12, (256,), rnd(144))])
+    raw = open(good, "rb").read()
+
+    def expect(blob, pattern, name):
+        p = tmp_path / name
+        open(p, "wb").write(blob)
+        with pytest.raises(candle_amd.MoeError, match=pattern):
+            candle_amd.GgufFile(str(p))
+
+    expect(b"GGML" + raw[4:], "unknown magic 0x4c4d4747", "magic.gguf")
+    expect(raw[:4] + struct.pack("<I", 4) + raw[8:], "unsupported version 4", "version.gguf")
+    expect(raw[:30], "end of file|truncated", "short.gguf")
+    expect(raw[:3], "too short", "tiny.gguf")
+    # value type 13 does not exist (gguf_file.rs:402-420)
+    bad_vt = bytearray(raw)
+    bad_vt[24 + 8 + 1: 24 + 8 + 1 + 4] = struct.pack("<I", 13)
+    expect(bytes(bad_vt), "unrecognized value-type", "vt.gguf")
+    with pytest.raises(candle_amd.MoeError, match="cannot open"):
+        candle_amd.GgufFile(str(tmp_path / "missing.gguf"))
+    # dtype id 5 is not a GgmlDType (quantized/mod.rs:153-174)
+    p = tmp_path / "dtype.gguf"
+    W.write_gguf(p, [], [("t", 12, (256,), rnd(144))])
+    blob = bytearray(open(p, "rb").read())
+    i = blob.index(b"t", 24) + 1 + 4 + 8           # name, n_dims, one u64 dimension
+    assert struct.unpack_from("<I", blob, i)[0] == 12
+    struct.pack_into("<I", blob, i, 5)
+    expect(bytes(blob), "unknown dtype for tensor 5", "dtype2.gguf")
+
+
+def test_tensor_size_and_bounds_checks(tmp_path):
+    # 100 elements are not a whole number of Q4K blocks (gguf_file.rs:66-70)
+    p = tmp_path / "div.gguf"
+    W.write_gguf(p, [], [("t", 12, (100,), rnd(144))])
+    with candle_amd.GgufFile(str(p)) as g:
+        with pytest.raises(candle_amd.MoeError, match="the number of elements 100 is not divisible by the block size 256"):
+            g.tensor("t")
+    # the table promises more bytes than the file holds (gguf_file.rs:103-110)
+    p2 = tmp_path / "cut.gguf"
+    W.write_gguf(p2, [], [("t", 0, (1024,), rnd(4096))])
+    raw = open(p2, "rb").read()
+    open(p2, "wb").write(raw[:-2048])
+    with candle_amd.GgufFile(str(p2)) as g:
+        with pytest.raises(candle_amd.MoeError, match="tensor data extends beyond file boundary"):
+            g.tensor("t")

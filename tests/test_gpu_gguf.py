@@ -1,0 +1,80 @@
+"""The GGUF expert loader on the GPU: a layer built from a file must behave exactly like the layer built
+from the same bytes through moe_layer_create (names and metadata as quantized_llama.rs:506-512, 553-578)."""
+import numpy as np
+import pytest
+
+import candle_amd
+import gguf_writer as W
+import pyoracle as O
+from helpers import activations, make_weights
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def build(dt, H=512, F=1024, E=8, seed=11):
+    w1, w3, w2, _ = make_weights(H, F, E, dt, seed)
+    gate = O.fill_normal(seed * 1000003 + 777, E * H, 0.0, 0.02).reshape(E, H)
+    return gate, w1, w3, w2
+
+
+@pytest.mark.parametrize("dt", [O.Q4K, O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("version", [2, 3])
+def test_layer_from_gguf_equals_layer_from_arrays(tmp_path, dt, version):
+    H, F, E, k = 512, 1024, 8, 2
+    gate, w1, w3, w2 = build(dt)
+    path = tmp_path / "moe.gguf"
+    W.moe_layer_file(path, 3, gate, w1, w3, w2, dt, k, version=version)
+    direct = candle_amd.SparseMoeBlock(H, F, E, k, dt, gate, w1, w3, w2)
+    loaded = candle_amd.SparseMoeBlock.from_gguf(str(path), 3)
+    assert (loaded.hidden, loaded.ffn, loaded.n_experts, loaded.top_k, loaded.dtype) == (H, F, E, k, dt)
+    for T in (1, 9, 70):
+        xs = activations(T, H, 40 + T)
+        assert np.array_equal(bits(direct.forward(xs)), bits(loaded.forward(xs)))
+    want = O.dequantize(dt, w2[5], H * F)
+    assert np.array_equal(bits(loaded.dequantize_weight(5, 2)).reshape(-1), bits(want).reshape(-1))
+    direct.close(); loaded.close()
+
+
+def test_router_stored_as_f16_or_quantised(tmp_path):
+    H, F, E, k = 512, 1024, 8, 2
+    gate, w1, w3, w2 = build(O.Q4K)
+    # F16 router: candle widens it (QMatMul::from_qtensor dequantises F16 tensors, quantized/mod.rs:430-436)
+    p16 = tmp_path / "f16.gguf"
+    W.moe_layer_file(p16, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=1)
+    a = candle_amd.SparseMoeBlock.from_gguf(str(p16), 0)
+    b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, gate.astype(np.float16).astype(np.float32), w1, w3, w2)
+    xs = activations(12, H, 5)
+    assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
+    a.close(); b.close()
+    # Q8_0 router: the layer uses to_float of the blocks
+    gq = O.quantize(O.Q8_0, gate.reshape(-1))
+    pq = tmp_path / "q8.gguf"
+    W.moe_layer_file(pq, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=O.Q8_0, gate_blocks=gq)
+    a = candle_amd.SparseMoeBlock.from_gguf(str(pq), 0)
+    b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, O.dequantize(O.Q8_0, gq, E * H).reshape(E, H), w1, w3, w2)
+    assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
+    a.close(); b.close()
+
+
+def test_loader_errors(tmp_path):
+    H, F, E, k = 512, 1024, 8, 2
+    gate, w1, w3, w2 = build(O.Q4K)
+    p = tmp_path / "ok.gguf"
+    W.moe_layer_file(p, 0, gate, w1, w3, w2, O.Q4K, k)
+    with pytest.raises(candle_amd.MoeError, match=r"cannot find tensor info for blk\.1\.ffn_gate_inp\.weight"):
+        candle_amd.SparseMoeBlock.from_gguf(str(p), 1)
+    # no expert keys: the reference defaults both counts to 0 (quantized_llama.rs:507-512) and takes the dense arm
+    p0 = tmp_path / "dense.gguf"
+    W.moe_layer_file(p0, 0, gate, w1, w3, w2, O.Q4K, k, expert_keys=False)
+    with pytest.raises(candle_amd.MoeError, match="expert_count is 0"):
+        candle_amd.SparseMoeBlock.from_gguf(str(p0), 0)
+    # ffn_down stored with another dtype (what Q4_K_M files do with Q6K): refused, not silently converted
+    pm = tmp_path / "mixed.gguf"
+    w2_q8 = [np.zeros(H * F // 32 * 34, np.uint8) for _ in range(E)]
+    W.moe_layer_file(pm, 0, gate, w1, w3, w2_q8, O.Q4K, k, down_dtype=O.Q8_0)
+    with pytest.raises(candle_amd.MoeError, match="differs from the layer's other expert matrices"):
+        candle_amd.SparseMoeBlock.from_gguf(str(pm), 0)
