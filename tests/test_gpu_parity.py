@@ -274,3 +274,34 @@ def test_device_entry_point_matches_host_entry_point():
     torch.cuda.synchronize()
     assert np.array_equal(bits(yd.cpu().numpy()), bits(y_host))
     gpu.close()
+
+
+def test_concurrent_forward_from_several_threads():
+    # QuantizedType is Send + Sync (candle-core/src/quantized/mod.rs:256): candle calls a layer from any thread.
+    # Four threads share two layers (calls on one layer are serialised inside the library) and use their own inputs.
+    import threading
+    ref_a, gpu_a = make_pair(512, 1024, 8, 2, O.Q4K, seed=21)
+    ref_b, gpu_b = make_pair(256, 512, 8, 2, O.Q8_0, seed=22)
+    jobs = [(gpu_a, activations(7, 512, 50)), (gpu_b, activations(33, 256, 51)), (gpu_a, activations(40, 512, 52)), (gpu_b, activations(3, 256, 53))]
+    want = [g.forward(x).copy() for g, x in jobs]
+    errors, got = [], [None] * len(jobs)
+
+    def work(i):
+        try:
+            g, x = jobs[i]
+            for _ in range(20):
+                y = g.forward(x)
+                if not np.array_equal(bits(y), bits(want[i])):
+                    errors.append("thread %d: result differs from the single-threaded one" % i)
+                    return
+            got[i] = y
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (i, e))
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(len(jobs))]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errors, errors
+    gpu_a.close(); gpu_b.close()
