@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -544,41 +545,140 @@ extern "C" int moe_quantize_act(int32_t vdt, const float* x, int64_t rows, int64
     return d2h(out, dout.p, out_bytes);
 }
 
-extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y) {
+// ------------------------------------------------------------------ dense quantized linear
+// One quantized matrix kept resident in the tiled layout, applied to f32 rows: the attention and
+// output projections around the MoE block use the same matmul as the experts.
+struct moe_qlinear {
+    int64_t n = 0, k = 0;
+    int dt = 0, vdt = 0;
+    DevBuf weights, group;
+    std::mutex mu;
+    RouteStore route;
+    ActStore xq;
+    int64_t cap_m = -1;
+    DevBuf x_dev, y_dev;
+    hipStream_t stream = nullptr;
+};
+
+extern "C" void moe_qlinear_destroy(moe_qlinear* Q) {
+    if (!Q) return;
+    if (Q->stream) { (void)hipStreamSynchronize(Q->stream); (void)hipStreamDestroy(Q->stream); }
+    delete Q;
+}
+
+extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, int64_t k, moe_qlinear** out) {
+    if (out) *out = nullptr;
     int rc = ensure_device();
     if (rc) return rc;
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_qmatmul: unsupported dtype");
+    if (!out || !w_blocks) return fail(MOE_E_INVALID, "moe_qlinear_create: NULL pointer");
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
+        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q4K=12)");
     const int64_t be = block_elems(dt);
-    if (n <= 0 || n % 16 || k <= 0 || k % be || m < 0) return fail(MOE_E_INVALID, "moe_qmatmul: need n % 16 == 0 and k a multiple of the block size");
-    if (m == 0) return MOE_OK;
-    if (!w_blocks || !x || !y) return fail(MOE_E_INVALID, "NULL pointer");
-    const int vdt = vecdot_dtype(dt);
-    DevBuf raw, tiled, dx, dy, grp;
-    ActStore as;
-    RouteStore rs;
+    if (n <= 0 || n % 16 || k <= 0 || k % be || k > (1 << 24))
+        return fail(MOE_E_INVALID, "moe_qlinear_create: need n % 16 == 0 and k a multiple of the block size (" + std::to_string(be) + ")");
+    std::unique_ptr<moe_qlinear, void (*)(moe_qlinear*)> Q(new moe_qlinear, moe_qlinear_destroy);
+    Q->n = n; Q->k = k; Q->dt = dt; Q->vdt = vecdot_dtype(dt);
+    DevBuf raw;
     const size_t raw_bytes = (size_t)(n * k / be * block_bytes(dt));
     if ((rc = raw.reserve(raw_bytes))) return rc;
-    if ((rc = tiled.reserve((size_t)relaid_bytes(dt, n, k)))) return rc;
-    if ((rc = dx.reserve((size_t)m * k * 4))) return rc;
-    if ((rc = dy.reserve((size_t)m * n * 4))) return rc;
-    if ((rc = grp.reserve(sizeof(GroupWeights)))) return rc;
-    if ((rc = as.reserve(vdt, m, k))) return rc;
-    if ((rc = rs.reserve(m, 1, 1, false))) return rc;
+    if ((rc = Q->weights.reserve((size_t)relaid_bytes(dt, n, k)))) return rc;
+    if ((rc = Q->group.reserve(sizeof(GroupWeights)))) return rc;
     MOE_HIP_CHECK(hipMemcpy(raw.p, w_blocks, raw_bytes, hipMemcpyHostToDevice));
-    MOE_HIP_CHECK(hipMemcpy(dx.p, x, (size_t)m * k * 4, hipMemcpyHostToDevice));
-    MOE_HIP_CHECK(launch_relayout(dt, raw.as<uint8_t>(), tiled.as<uint8_t>(), n, k, nullptr));
-    GroupWeights g{nullptr, nullptr, tiled.as<uint8_t>()};
-    MOE_HIP_CHECK(hipMemcpy(grp.p, &g, sizeof g, hipMemcpyHostToDevice));
-    MOE_HIP_CHECK(launch_quantize_rows(vdt, dx.as<float>(), m, (int)k, as.view(), nullptr));
-    MOE_HIP_CHECK(launch_identity_routing(rs.view(), m, nullptr));
-    ExpertParams ep;
-    ep.dt = dt; ep.H = (int)n; ep.F = (int)k; ep.n_groups = 1; ep.group0 = 0;
-    ep.groups = grp.as<GroupWeights>();
-    ep.rb = rs.view(); ep.hq = as.view(); ep.slot_origin = 0; ep.yw = dy.as<float>();
-    ep.max_rows = m; ep.slot_tiles = m > 32 ? 4 : m > 16 ? 2 : 1;
-    MOE_HIP_CHECK(launch_expert_down(ep, nullptr));
+    MOE_HIP_CHECK(launch_relayout(dt, raw.as<uint8_t>(), Q->weights.as<uint8_t>(), n, k, nullptr));
+    GroupWeights g{nullptr, nullptr, Q->weights.as<uint8_t>()};
+    MOE_HIP_CHECK(hipMemcpy(Q->group.p, &g, sizeof g, hipMemcpyHostToDevice));
     MOE_HIP_CHECK(hipDeviceSynchronize());
-    return d2h(y, dy.p, (size_t)m * n * 4);
+    MOE_HIP_CHECK(hipStreamCreateWithFlags(&Q->stream, hipStreamNonBlocking));
+    *out = Q.release();
+    return MOE_OK;
+}
+
+// quantise the rows, then one pass over the matrix: streamed for short batches, tiled MFMA beyond
+static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d_y, hipStream_t s) {
+    int rc;
+    if (m > Q->cap_m) {
+        if ((rc = Q->route.reserve(m, 1, 1, false))) return rc;
+        if ((rc = Q->xq.reserve(Q->vdt, m, Q->k))) return rc;
+        Q->cap_m = m;
+    }
+    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    // The tiled MFMA kernel runs one workgroup per (128 weight rows, tile of 64 or 128 x rows): it pays
+    // once that grid fills most of the 256 CUs; below, the streamed kernels split the matrix finer.
+    const int64_t row_blocks = Q->n / 128;
+    const int tile_slots = row_blocks * ((m + 127) / 128) >= 512 ? 128 : 64;
+    const bool tiled = !no_gemm && Q->dt == MOE_GGML_Q4K && Q->n % 128 == 0 && m >= 96 &&
+                       row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192 && m * Q->k < (int64_t)1 << 32;
+    RouteBufs rb = Q->route.view();
+    rb.T = (int)m; rb.k = 1;
+    rb.tile_slots = tile_slots;
+    if (!tiled) rb.tile_tab = nullptr;
+    MOE_HIP_CHECK(launch_quantize_rows(Q->vdt, d_x, m, (int)Q->k, Q->xq.view(), s));
+    MOE_HIP_CHECK(launch_identity_routing(rb, m, s));
+    ExpertParams ep;
+    ep.dt = Q->dt; ep.H = (int)Q->n; ep.F = (int)Q->k; ep.n_groups = 1; ep.group0 = 0;
+    ep.groups = Q->group.as<GroupWeights>();
+    ep.rb = rb; ep.hq = Q->xq.view(); ep.slot_origin = 0; ep.yw = d_y;
+    ep.max_rows = m; ep.n_slots = m; ep.slot_tiles = m > 32 ? 4 : m > 16 ? 2 : 1;
+    if (tiled) MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
+    else MOE_HIP_CHECK(launch_expert_down(ep, s));
+    return MOE_OK;
+}
+
+static int check_qlinear_call(moe_qlinear* Q, const void* x, int64_t m, const void* y, const char* who) {
+    if (!Q || m < 0 || (m > 0 && (!x || !y))) return fail(MOE_E_INVALID, std::string("bad argument to ") + who);
+    if (m > (1 << 20)) return fail(MOE_E_INVALID, std::string(who) + ": more than 2^20 rows is not supported");
+    return MOE_OK;
+}
+
+extern "C" int moe_qlinear_forward_device(moe_qlinear* Q, const void* d_x, int64_t m, void* d_y, void* hip_stream) {
+    int rc = check_qlinear_call(Q, d_x, m, d_y, "moe_qlinear_forward_device");
+    if (rc || m == 0) return rc;
+    if (d_x == d_y) return fail(MOE_E_INVALID, "d_x and d_y must not alias");
+    std::lock_guard<std::mutex> lk(Q->mu);
+    return enqueue_qlinear(Q, static_cast<const float*>(d_x), m, static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream));
+}
+
+extern "C" int moe_qlinear_forward(moe_qlinear* Q, const float* x, int64_t m, float* y) {
+    int rc = check_qlinear_call(Q, x, m, y, "moe_qlinear_forward");
+    if (rc || m == 0) return rc;
+    std::lock_guard<std::mutex> lk(Q->mu);
+    const size_t xb = (size_t)m * Q->k * 4, yb = (size_t)m * Q->n * 4;
+    if ((rc = Q->x_dev.reserve(xb))) return rc;
+    if ((rc = Q->y_dev.reserve(yb))) return rc;
+    MOE_HIP_CHECK(hipMemcpyAsync(Q->x_dev.p, x, xb, hipMemcpyHostToDevice, Q->stream));
+    if ((rc = enqueue_qlinear(Q, Q->x_dev.as<float>(), m, Q->y_dev.as<float>(), Q->stream))) return rc;
+    MOE_HIP_CHECK(hipMemcpyAsync(y, Q->y_dev.p, yb, hipMemcpyDeviceToHost, Q->stream));
+    MOE_HIP_CHECK(hipStreamSynchronize(Q->stream));
+    return MOE_OK;
+}
+
+extern "C" int moe_qlinear_dequantize(moe_qlinear* Q, float* out, int64_t n_elems) {
+    if (!Q || !out) return fail(MOE_E_INVALID, "bad argument to moe_qlinear_dequantize");
+    if (n_elems != Q->n * Q->k) return fail(MOE_E_INVALID, "n_elems must be n*k = " + std::to_string(Q->n * Q->k));
+    DevBuf tmp;
+    int rc = tmp.reserve((size_t)n_elems * 4);
+    if (rc) return rc;
+    MOE_HIP_CHECK(launch_dequant_tiled(Q->dt, Q->weights.as<uint8_t>(), tmp.as<float>(), Q->n, Q->k, nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(out, tmp.p, (size_t)n_elems * 4);
+}
+
+extern "C" int moe_qlinear_shape(const moe_qlinear* Q, int64_t* n, int64_t* k, int32_t* dt) {
+    if (!Q) return fail(MOE_E_INVALID, "qlinear is NULL");
+    if (n) *n = Q->n;
+    if (k) *k = Q->k;
+    if (dt) *dt = Q->dt;
+    return MOE_OK;
+}
+
+extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y) {
+    if (m < 0) return fail(MOE_E_INVALID, "moe_qmatmul: negative row count");
+    moe_qlinear* Q = nullptr;
+    int rc = moe_qlinear_create(dt, w_blocks, n, k, &Q);
+    if (rc) return rc;
+    rc = moe_qlinear_forward(Q, x, m, y);
+    moe_qlinear_destroy(Q);
+    return rc;
 }
 
 extern "C" int moe_quantize_weights_device(int32_t dt, const void* d_x, int64_t n, void* d_out, void* hip_stream) {

@@ -373,3 +373,21 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     d.w1 = w1.data(); d.w3 = w3.data(); d.w2 = w2.data();
     return moe_layer_create(&d, out);
 }
+
+// One named matrix of the file as a resident dense projection: what `QMatMul::from_qtensor(ct.tensor(
+// reader, name, device)?)` builds for `blk.{l}.attn_q.weight` ... `output.weight`
+// (quantized_llama.rs:533-547, 590-593, 608).
+extern "C" int moe_qlinear_create_from_gguf(const moe_gguf* g, const char* tensor_name, moe_qlinear** out) {
+    if (out) *out = nullptr;
+    if (!g || !tensor_name || !out) return fail(MOE_E_INVALID, "moe_qlinear_create_from_gguf: bad argument");
+    int dt = 0, nd = 0;
+    int64_t dims[8];
+    const void* data = nullptr;
+    uint64_t nbytes = 0;
+    int rc = moe_gguf_tensor(g, tensor_name, &dt, &nd, dims, &data, &nbytes);
+    if (rc) return rc;
+    if (nd != 2) return fail(MOE_E_INVALID, std::string(tensor_name) + ": a projection matrix has two dimensions, this tensor has " + std::to_string(nd));
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
+        return fail(MOE_E_INVALID, std::string(tensor_name) + ": unsupported dtype " + std::to_string(dt) + " (supported: Q4_0, Q8_0, Q4K)");
+    return moe_qlinear_create(dt, data, dims[0], dims[1], out);
+}

@@ -572,6 +572,11 @@ __global__ void identity_routing_kernel(RouteBufs rb, int64_t rows) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i == 0) { rb.offsets[0] = 0; rb.offsets[1] = (int)rows; }
     if (i < rows) { rb.perm_token[i] = (int)i; rb.perm_w[i] = 1.0f; rb.tok_slots[i] = (int)i; }
+    if (rb.tile_tab) {  // work list of the tiled kernels: one group cut into tiles of tile_slots rows
+        const int64_t n_tiles = (rows + rb.tile_slots - 1) / rb.tile_slots;
+        if (i == 0) rb.tile_tab[0] = (int)n_tiles;
+        if (i < n_tiles) { rb.tile_tab[1 + 2 * i] = 0; rb.tile_tab[2 + 2 * i] = (int)(i * rb.tile_slots); }
+    }
 }
 
 // y[t, :] = sum_j yw[slot_j, :] in ascending expert order (shared expert last), starting from

@@ -68,6 +68,14 @@ def load_library():
     L.moe_dequantize.argtypes = [i32, vp, i64, vp]
     L.moe_quantize_act.argtypes = [i32, vp, i64, i64, vp]
     L.moe_qmatmul.argtypes = [i32, vp, i64, i64, vp, i64, vp]
+    L.moe_qlinear_create.argtypes = [i32, vp, i64, i64, C.POINTER(vp)]
+    L.moe_qlinear_destroy.argtypes = [vp]
+    L.moe_qlinear_destroy.restype = None
+    L.moe_qlinear_forward.argtypes = [vp, vp, i64, vp]
+    L.moe_qlinear_forward_device.argtypes = [vp, vp, i64, vp, vp]
+    L.moe_qlinear_dequantize.argtypes = [vp, vp, i64]
+    L.moe_qlinear_shape.argtypes = [vp, C.POINTER(i64), C.POINTER(i64), C.POINTER(i32)]
+    L.moe_qlinear_create_from_gguf.argtypes = [vp, C.c_char_p, C.POINTER(vp)]
     L.moe_quantize_weights.argtypes = [i32, vp, i64, vp]
     L.moe_quantize_weights_device.argtypes = [i32, vp, i64, vp, vp]
     L.moe_gguf_open.argtypes = [C.c_char_p, C.POINTER(vp)]
@@ -405,3 +413,82 @@ class SparseMoeBlock:
 
 
 MlpOrMoe = SparseMoeBlock  # the reference's name for the enum that holds the MoE arm
+
+
+class QMatMul:
+    """The `QMatMul::QTensor` arm (candle-core/src/quantized/mod.rs:428-447, 533-537): one quantized
+    [n, k] matrix resident on the GPU, applied as xs . W^T (the attention and output projections
+    of quantized_llama.rs:590-593, 608)."""
+
+    def __init__(self, ggml_dtype, w_blocks, n, k):
+        if ggml_dtype not in (GGML_Q4_0, GGML_Q8_0, GGML_Q4K):
+            raise MoeError("unsupported ggml_dtype %r" % (ggml_dtype,))
+        w_blocks = _blocks(w_blocks, ggml_dtype, n * k, "QMatMul")
+        h = C.c_void_p()
+        self._h = None
+        _check(load_library().moe_qlinear_create(ggml_dtype, _p(w_blocks), n, k, C.byref(h)))
+        self._h, self.n, self.k, self.dtype = h, n, k, ggml_dtype
+
+    from_qtensor = classmethod(lambda cls, ggml_dtype, w_blocks, n, k: cls(ggml_dtype, w_blocks, n, k))
+
+    @classmethod
+    def from_gguf(cls, gguf, tensor_name):
+        """`QMatMul::from_qtensor(ct.tensor(reader, name, device)?)` (quantized_llama.rs:533-547)."""
+        own = not isinstance(gguf, GgufFile)
+        g = GgufFile(gguf) if own else gguf
+        try:
+            L = load_library()
+            h = C.c_void_p()
+            _check(L.moe_qlinear_create_from_gguf(g._h, tensor_name.encode(), C.byref(h)))
+            n, k, dt = C.c_int64(), C.c_int64(), C.c_int32()
+            self = cls.__new__(cls)
+            self._h = h
+            _check(L.moe_qlinear_shape(h, C.byref(n), C.byref(k), C.byref(dt)))
+            self.n, self.k, self.dtype = n.value, k.value, dt.value
+            return self
+        finally:
+            if own:
+                g.close()
+
+    def close(self):
+        if getattr(self, "_h", None) is not None:
+            load_library().moe_qlinear_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def forward(self, xs, out=None):
+        """xs [..., k] f32 (numpy, or a contiguous torch CUDA tensor on torch's current stream) -> [..., n]."""
+        L = load_library()
+        if self._h is None:
+            raise MoeError("QMatMul is closed")
+        if isinstance(xs, np.ndarray):
+            x = _f32(xs)
+            if x.ndim < 1 or x.shape[-1] != self.k:
+                raise MoeError("expected [..., %d], got %s" % (self.k, x.shape))
+            m = x.size // self.k
+            y = np.empty(x.shape[:-1] + (self.n,), dtype=np.float32)
+            _check(L.moe_qlinear_forward(self._h, _p(x), m, _p(y)))
+            return y
+        import torch  # device tensors: plumbing only
+        if not (isinstance(xs, torch.Tensor) and xs.is_cuda):
+            raise MoeError("forward takes a numpy array or a torch CUDA tensor")
+        if xs.dtype != torch.float32 or not xs.is_contiguous():
+            raise MoeError("input has to be contiguous f32")
+        if xs.dim() < 1 or xs.shape[-1] != self.k:
+            raise MoeError("expected [..., %d], got %s" % (self.k, tuple(xs.shape)))
+        m = xs.numel() // self.k
+        y = torch.empty(tuple(xs.shape[:-1]) + (self.n,), dtype=torch.float32, device=xs.device) if out is None else out
+        if y.numel() != m * self.n or y.dtype != torch.float32 or not y.is_contiguous() or not y.is_cuda:
+            raise MoeError("out has to be a contiguous f32 CUDA tensor of %d elements" % (m * self.n))
+        stream = torch.cuda.current_stream(xs.device).cuda_stream
+        _check(L.moe_qlinear_forward_device(self._h, xs.data_ptr(), m, y.data_ptr(), stream))
+        return y
+
+    __call__ = forward
+
+    def dequantize(self):
+        """`QMatMul::dequantize` of the resident copy: f32 [n, k]."""
+        out = np.empty((self.n, self.k), dtype=np.float32)
+        _check(load_library().moe_qlinear_dequantize(self._h, _p(out), out.size))
+        return out

@@ -128,8 +128,27 @@ int moe_dequantize(int32_t ggml_dtype, const void* blocks, int64_t n_elems, floa
 int moe_quantize_act(int32_t vecdot_dtype, const float* x, int64_t rows, int64_t k, void* out);
 
 /* Parity hook: QMatMul::forward on one quantized matrix (quantized/mod.rs:533-537 ->
- * k_quants.rs:1873-1920): y[m, n] = x[m, k] . W[n, k]^T, host pointers, W as raw blocks. */
+ * k_quants.rs:1873-1920): y[m, n] = x[m, k] . W[n, k]^T, host pointers, W as raw blocks.
+ * (moe_qlinear_create + moe_qlinear_forward + moe_qlinear_destroy in one call.) */
 int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, const float* x, int64_t m, float* y);
+
+/* ---- dense quantized projection --------------------------------------------------------------
+ * The QMatMul::QTensor arm of candle-core/src/quantized/mod.rs:428-447 (from_arc / from_qtensor) and
+ * 533-537 (forward): the attention projections and the output head around the MoE block
+ * (quantized_llama.rs:590-593 attention_wq/wk/wv/wo, :608 output; applied at :275-277, :345, :897).
+ * create uploads the [n, k] matrix of raw GGML blocks once (n % 16 == 0, k a multiple of the block
+ * size; Q4_0, Q8_0, Q4K) and keeps it resident in the kernels' layout; forward quantises the m rows
+ * of x as k_quants::matmul does (k_quants.rs:1893-1903) and writes y[m, n] = x . W^T.
+ * forward takes host pointers and returns when y is filled; forward_device takes device pointers and
+ * enqueues on hip_stream.  Calls on one object serialise; dequantize is QMatMul::dequantize
+ * (QTensor::dequantize, mod.rs:367-371) of the resident copy: [n, k] f32. */
+typedef struct moe_qlinear moe_qlinear;
+int moe_qlinear_create(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, moe_qlinear** out);
+void moe_qlinear_destroy(moe_qlinear* q);
+int moe_qlinear_forward(moe_qlinear* q, const float* x, int64_t m, float* y);
+int moe_qlinear_forward_device(moe_qlinear* q, const void* d_x, int64_t m, void* d_y, void* hip_stream);
+int moe_qlinear_dequantize(moe_qlinear* q, float* out, int64_t n_elems);
+int moe_qlinear_shape(const moe_qlinear* q, int64_t* n, int64_t* k, int32_t* ggml_dtype);
 
 /* QTensor::quantize (candle-core/src/quantized/mod.rs:331-349) on the GPU: f32 [n_elems] -> raw
  * GGML blocks, bit-identical to GgmlType::from_float of k_quants.rs:188-224 (Q4_0), 605-634 (Q8_0)
@@ -165,6 +184,10 @@ int moe_gguf_tensor(const moe_gguf* file, const char* name, int* ggml_dtype, int
  * supported quantized dtype) and `blk.{l}.ffn_{gate,down,up}.{i}.weight` as w1 / w2 / w3.  All expert
  * matrices of the layer must share one supported dtype.  Needs the GPU. */
 int moe_layer_create_from_gguf(const moe_gguf* file, int layer_index, int norm_topk, moe_layer** out);
+/* One named two-dimensional quantized tensor of the file as a resident projection: what
+ * `QMatMul::from_qtensor(ct.tensor(reader, name, device)?)` builds for `blk.{l}.attn_q.weight`,
+ * `blk.{l}.attn_output.weight`, `output.weight` ... (quantized_llama.rs:533-547, 590-593, 608).  Needs the GPU. */
+int moe_qlinear_create_from_gguf(const moe_gguf* file, const char* tensor_name, moe_qlinear** out);
 
 /* Message of the calling thread's last error ("" if none). */
 const char* moe_last_error(void);
