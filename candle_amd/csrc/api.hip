@@ -136,7 +136,7 @@ using namespace moe;
 
 struct moe_layer {
     int64_t H = 0, F = 0, E = 0, k = 0, Fs = 0;
-    int dt = 0, vdt = 0, norm_topk = 1;
+    int dt = 0, dt_down = 0, vdt = 0, norm_topk = 1;   // dt: w1 / w3, dt_down: w2 (same activation format)
     bool has_bias = false, has_rms = false;
     float rms_eps = 0.f;
     DevBuf weights;                 // all re-laid expert matrices
@@ -170,9 +170,14 @@ static int reserve_workspace(moe_layer* L, int64_t T) {
 
 static int check_desc(const moe_desc* d) {
     if (!d) return fail(MOE_E_INVALID, "desc is NULL");
-    const int dt = d->ggml_dtype;
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
-        return fail(MOE_E_INVALID, "unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q4K=12)");
+    const int dt = d->ggml_dtype, dtd = d->ggml_dtype_down ? d->ggml_dtype_down : dt;
+    if (!weight_dtype_supported(dt) || !weight_dtype_supported(dtd))
+        return fail(MOE_E_INVALID, "unsupported ggml_dtype " + std::to_string(weight_dtype_supported(dt) ? dtd : dt) +
+                                       " (supported: Q4_0=2, Q8_0=8, Q4K=12, Q6K=14)");
+    // w2 consumes the intermediate in the activation format of its own dtype; the up kernels emit the one of dt
+    if (vecdot_dtype(dt) != vecdot_dtype(dtd))
+        return fail(MOE_E_INVALID, "ggml_dtype " + std::to_string(dt) + " and ggml_dtype_down " + std::to_string(dtd) +
+                                       " quantise activations differently (Q8_0 vs Q8K); such a layer is not supported");
     const int64_t be = block_elems(dt);
     if (d->hidden <= 0 || d->ffn <= 0) return fail(MOE_E_INVALID, "hidden and ffn must be positive");
     // the reference rejects a last dimension that is not a multiple of the block size
@@ -217,7 +222,8 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
         return code;
     };
     L->H = d->hidden; L->F = d->ffn; L->E = d->n_experts; L->k = d->top_k; L->Fs = d->shared_ffn;
-    L->dt = d->ggml_dtype; L->vdt = vecdot_dtype(L->dt); L->norm_topk = d->norm_topk ? 1 : 0;
+    L->dt = d->ggml_dtype; L->dt_down = d->ggml_dtype_down ? d->ggml_dtype_down : L->dt;
+    L->vdt = vecdot_dtype(L->dt); L->norm_topk = d->norm_topk ? 1 : 0;
     L->rms_eps = d->rms_eps;
     if ((rc = upload_f32(L->gate, d->gate, (size_t)L->E * L->H))) return bail(rc);
     if (d->gate_bias) {
@@ -230,38 +236,38 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
         if ((rc = upload_f32(L->rms_alpha, d->rms_alpha, (size_t)L->H))) return bail(rc);
     }
     // one allocation for all matrices
-    const size_t mat = (size_t)relaid_bytes(L->dt, L->F, L->H);      // w1/w3: [F,H]; w2: [H,F] has the same size
-    const size_t smat = L->Fs ? (size_t)relaid_bytes(L->dt, L->Fs, L->H) : 0;
-    const size_t total = mat * 3 * L->E + smat * 3;
+    auto raw_bytes_of = [](int dt, int64_t elems) { return (size_t)(elems / block_elems(dt) * block_bytes(dt)); };
+    const size_t total = (size_t)(2 * relaid_bytes(L->dt, L->F, L->H) + relaid_bytes(L->dt_down, L->H, L->F)) * L->E +
+                         (L->Fs ? (size_t)(2 * relaid_bytes(L->dt, L->Fs, L->H) + relaid_bytes(L->dt_down, L->H, L->Fs)) : 0);
     if ((rc = L->weights.reserve(total))) return bail(rc);
-    const size_t raw_mat = (size_t)(L->F * L->H / block_elems(L->dt) * block_bytes(L->dt));
-    const size_t raw_smat = (size_t)(L->Fs * L->H / block_elems(L->dt) * block_bytes(L->dt));
+    const size_t raw_mat = raw_bytes_of(L->dt, L->F * L->H), raw_mat_down = raw_bytes_of(L->dt_down, L->F * L->H);
+    const size_t raw_smat = raw_bytes_of(L->dt, L->Fs * L->H), raw_smat_down = raw_bytes_of(L->dt_down, L->Fs * L->H);
     DevBuf staging;
-    if ((rc = staging.reserve(std::max(raw_mat, raw_smat)))) return bail(rc);
+    if ((rc = staging.reserve(std::max(std::max(raw_mat, raw_smat), std::max(raw_mat_down, raw_smat_down))))) return bail(rc);
     uint8_t* wbase = L->weights.as<uint8_t>();
     size_t off = 0;
-    auto put = [&](const void* src, size_t raw_bytes, int64_t rows, int64_t cols, const uint8_t** dst) -> int {
+    auto put = [&](int dt, const void* src, size_t raw_bytes, int64_t rows, int64_t cols, const uint8_t** dst) -> int {
         hipError_t e = hipMemcpy(staging.p, src, raw_bytes, hipMemcpyHostToDevice);
         if (e != hipSuccess) return fail(MOE_E_HIP, std::string("hipMemcpy(weights): ") + hipGetErrorString(e));
-        e = launch_relayout(L->dt, staging.as<uint8_t>(), wbase + off, rows, cols, nullptr);
+        e = launch_relayout(dt, staging.as<uint8_t>(), wbase + off, rows, cols, nullptr);
         if (e == hipSuccess) e = hipDeviceSynchronize();
         if (e != hipSuccess) return fail(MOE_E_HIP, std::string("relayout: ") + hipGetErrorString(e));
         *dst = wbase + off;
-        off += (size_t)relaid_bytes(L->dt, rows, cols);
+        off += (size_t)relaid_bytes(dt, rows, cols);
         return MOE_OK;
     };
     L->host_groups.resize(L->E + (L->Fs ? 1 : 0));
     for (int64_t e = 0; e < L->E; e++) {
         GroupWeights& g = L->host_groups[e];
-        if ((rc = put(d->w1[e], raw_mat, L->F, L->H, &g.w1))) return bail(rc);
-        if ((rc = put(d->w3[e], raw_mat, L->F, L->H, &g.w3))) return bail(rc);
-        if ((rc = put(d->w2[e], raw_mat, L->H, L->F, &g.w2))) return bail(rc);
+        if ((rc = put(L->dt, d->w1[e], raw_mat, L->F, L->H, &g.w1))) return bail(rc);
+        if ((rc = put(L->dt, d->w3[e], raw_mat, L->F, L->H, &g.w3))) return bail(rc);
+        if ((rc = put(L->dt_down, d->w2[e], raw_mat_down, L->H, L->F, &g.w2))) return bail(rc);
     }
     if (L->Fs) {
         GroupWeights& g = L->host_groups[L->E];
-        if ((rc = put(d->shared_w1, raw_smat, L->Fs, L->H, &g.w1))) return bail(rc);
-        if ((rc = put(d->shared_w3, raw_smat, L->Fs, L->H, &g.w3))) return bail(rc);
-        if ((rc = put(d->shared_w2, raw_smat, L->H, L->Fs, &g.w2))) return bail(rc);
+        if ((rc = put(L->dt, d->shared_w1, raw_smat, L->Fs, L->H, &g.w1))) return bail(rc);
+        if ((rc = put(L->dt, d->shared_w3, raw_smat, L->Fs, L->H, &g.w3))) return bail(rc);
+        if ((rc = put(L->dt_down, d->shared_w2, raw_smat_down, L->H, L->Fs, &g.w2))) return bail(rc);
     }
     if ((rc = L->groups.reserve(L->host_groups.size() * sizeof(GroupWeights)))) return bail(rc);
     hipError_t e = hipMemcpy(L->groups.p, L->host_groups.data(), L->host_groups.size() * sizeof(GroupWeights), hipMemcpyHostToDevice);
@@ -309,6 +315,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // H of 128; those kernels address activation rows with 32-bit byte offsets).  Their tiles hold 64
     // slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
     const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
                        T * L->k > 24 * L->E && T * L->k * std::max(L->H, L->F) < (int64_t)1 << 32;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
@@ -323,7 +330,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     MOE_MARK(ST_DISPATCH);
 
     ExpertParams ep;
-    ep.dt = L->dt; ep.H = (int)L->H; ep.F = (int)L->F;
+    ep.dt = L->dt; ep.dt_down = L->dt_down; ep.H = (int)L->H; ep.F = (int)L->F;
     ep.n_groups = (int)L->E; ep.group0 = 0;
     ep.groups = L->groups.as<GroupWeights>();
     ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = L->hq.view(); ep.slot_origin = 0;
@@ -335,7 +342,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
     if (force_st) ep.slot_tiles = force_st;
     static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;
-    const bool narrow = direct && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
+    const bool narrow = direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
                         (force_narrow >= 0 ? force_narrow > 0 : T * L->k <= L->E);
     if (tiled) {
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
@@ -345,7 +352,13 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         MOE_MARK(ST_UP);
         MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_REQUANT);
-        MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
+        if (L->dt_down == MOE_GGML_Q4K) {
+            MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
+        } else {
+            ExpertParams dp = ep;
+            dp.hbuf = nullptr;
+            MOE_HIP_CHECK(launch_expert_down(dp, s));
+        }
         MOE_MARK(ST_DOWN);
     } else if (narrow) {
         // very small Q4K batches: at most half of the experts can be active, so the weights are cut
@@ -475,7 +488,7 @@ extern "C" int moe_layer_dequantize_weight(moe_layer* L, int64_t expert, int whi
     DevBuf tmp;
     int rc = tmp.reserve((size_t)n_elems * 4);
     if (rc) return rc;
-    MOE_HIP_CHECK(launch_dequant_tiled(L->dt, src, tmp.as<float>(), rows, cols, nullptr));
+    MOE_HIP_CHECK(launch_dequant_tiled(which == 2 ? L->dt_down : L->dt, src, tmp.as<float>(), rows, cols, nullptr));
     MOE_HIP_CHECK(hipDeviceSynchronize());
     return d2h(out, tmp.p, (size_t)n_elems * 4);
 }
@@ -571,8 +584,8 @@ extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, i
     int rc = ensure_device();
     if (rc) return rc;
     if (!out || !w_blocks) return fail(MOE_E_INVALID, "moe_qlinear_create: NULL pointer");
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
-        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q4K=12)");
+    if (!weight_dtype_supported(dt))
+        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q4K=12, Q6K=14)");
     const int64_t be = block_elems(dt);
     if (n <= 0 || n % 16 || k <= 0 || k % be || k > (1 << 24))
         return fail(MOE_E_INVALID, "moe_qlinear_create: need n % 16 == 0 and k a multiple of the block size (" + std::to_string(be) + ")");

@@ -340,24 +340,26 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     else if (dt == 1) {
         const uint16_t* h = static_cast<const uint16_t*>(data);
         for (size_t i = 0; i < gate.size(); i++) gate[i] = half_bits_to_float(h[i]);
-    } else if (dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4K) {
+    } else if (dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q6K) {
         if ((rc = moe_dequantize(dt, data, E * H, gate.data()))) return rc;   // on the GPU
     } else
-        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: unsupported dtype " + std::to_string(dt) + " (supported: F32, F16, Q4_0, Q8_0, Q4K)");
+        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: unsupported dtype " + std::to_string(dt) + " (supported: F32, F16, Q4_0, Q8_0, Q4K, Q6K)");
 
     std::vector<const void*> w1((size_t)E), w2((size_t)E), w3((size_t)E);
-    int expert_dt = -1;
-    int64_t F = 0;
+    int up_dt = -1, down_dt = -1;   // gate / up matrices share one dtype, down matrices one
+    int64_t F = -1;
     for (int64_t e = 0; e < E; e++) {
         struct { const char* stem; std::vector<const void*>* dst; bool up; } parts[3] = {{"ffn_gate", &w1, true}, {"ffn_down", &w2, false}, {"ffn_up", &w3, true}};
         for (auto& part : parts) {
             const std::string name = prefix + "." + part.stem + "." + std::to_string(e) + ".weight";
             if ((rc = moe_gguf_tensor(g, name.c_str(), &dt, &nd, dims, &data, &nbytes))) return rc;
             if (nd != 2) return fail(MOE_E_INVALID, name + ": expected a matrix");
-            if (expert_dt < 0) { expert_dt = dt; F = part.up ? dims[0] : dims[1]; }
-            if (dt != expert_dt)
-                return fail(MOE_E_INVALID, name + ": dtype " + std::to_string(dt) + " differs from the layer's other expert matrices (" + std::to_string(expert_dt) +
-                                               "); mixed-dtype layers (e.g. Q6K ffn_down of Q4_K_M files) are not supported");
+            if (F < 0) F = part.up ? dims[0] : dims[1];
+            int& want = part.up ? up_dt : down_dt;
+            if (want < 0) want = dt;
+            if (dt != want)
+                return fail(MOE_E_INVALID, name + ": dtype " + std::to_string(dt) + " differs from the layer's other " + (part.up ? "gate / up" : "down") +
+                                               " matrices (" + std::to_string(want) + ")");
             const int64_t rows = part.up ? F : H, cols = part.up ? H : F;
             if (dims[0] != rows || dims[1] != cols)
                 return fail(MOE_E_INVALID, name + ": shape [" + std::to_string(dims[0]) + ", " + std::to_string(dims[1]) + "] does not match hidden " + std::to_string(H) +
@@ -368,7 +370,7 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     moe_desc d;
     memset(&d, 0, sizeof d);
     d.hidden = H; d.ffn = F; d.n_experts = E; d.top_k = (int64_t)n_used;
-    d.ggml_dtype = expert_dt; d.norm_topk = norm_topk;
+    d.ggml_dtype = up_dt; d.ggml_dtype_down = down_dt == up_dt ? 0 : down_dt; d.norm_topk = norm_topk;
     d.gate = gate.data();
     d.w1 = w1.data(); d.w3 = w3.data(); d.w2 = w2.data();
     return moe_layer_create(&d, out);
@@ -387,7 +389,7 @@ extern "C" int moe_qlinear_create_from_gguf(const moe_gguf* g, const char* tenso
     int rc = moe_gguf_tensor(g, tensor_name, &dt, &nd, dims, &data, &nbytes);
     if (rc) return rc;
     if (nd != 2) return fail(MOE_E_INVALID, std::string(tensor_name) + ": a projection matrix has two dimensions, this tensor has " + std::to_string(nd));
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K)
-        return fail(MOE_E_INVALID, std::string(tensor_name) + ": unsupported dtype " + std::to_string(dt) + " (supported: Q4_0, Q8_0, Q4K)");
+    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K && dt != MOE_GGML_Q6K)
+        return fail(MOE_E_INVALID, std::string(tensor_name) + ": unsupported dtype " + std::to_string(dt) + " (supported: Q4_0, Q8_0, Q4K, Q6K)");
     return moe_qlinear_create(dt, data, dims[0], dims[1], out);
 }

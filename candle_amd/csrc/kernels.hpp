@@ -59,7 +59,8 @@ struct GroupWeights {
 };
 
 struct ExpertParams {
-    int dt = 0;
+    int dt = 0;                     // dtype of w1 / w3
+    int dt_down = 0;                // dtype of w2 when it differs from dt (same activation format), else 0
     int H = 0, F = 0;
     int n_groups = 0;               // groups handled by this launch
     int group0 = 0;                 // index of the first of them in rb.offsets

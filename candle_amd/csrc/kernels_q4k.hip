@@ -1,4 +1,4 @@
-// Grouped expert products over Q4K weights with Q8K activations (gfx950, wave64, int8 MFMA).
+// Grouped expert products over Q4K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
 //
 // Arithmetic restated from BlockQ4K::vec_dot, candle-core/src/quantized/k_quants.rs:1205-1285:
 // per 256-element super-block
@@ -11,6 +11,13 @@
 //
 // MFMA orientation: A = activations (M = 16 slots), B = weights (N = 16 rows), so lane l ends up
 // with D[slot 4*(l/16)+i][row l%16]: one weight row per lane, hence one set of scales per lane.
+//
+// Q6K (BlockQ6K::vec_dot, k_quants.rs:1613-1671): d * y.d * sum_j sc_j * ((code_j - 32) . q8_j) over
+// the sixteen 16-element sub-blocks, sc_j an i8.  One v_mfma_i32_16x16x32_i8 spans two sub-blocks with
+// different scales, so each is issued twice, with the weight operand of the lane groups that hold the
+// other sub-block zeroed; the codes stay unsigned (0..63) and the -32 is taken out through the
+// activations' 16-element sums: sum_j sc_j * bsum_j is one exact f16 MFMA (|bsum| <= 2032,
+// |sc| <= 128, the sum of sixteen products stays below 2^24).
 //
 //   q4k_up_kernel    h[slot, f] = silu(W1 x) * (W3 x) for a 256-row block of F, then the block is
 //                    quantised to Q8K in the epilogue (Mlp::forward, quantized_llama.rs:124-131;
@@ -129,6 +136,75 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
     }
 }
 
+struct Q6KTile {
+    uint4 q0, q1, qh, sc;
+    uint32_t d;   // f16 bits of the lane's row
+};
+__device__ inline Q6KTile load_q6k_tile(const uint8_t* tile, int lane) {
+    Q6KTile t;
+    t.q0 = gload_stream(tile, (uint32_t)lane * 16u);
+    t.q1 = gload_stream(tile, 1024u + (uint32_t)lane * 16u);
+    t.qh = gload_stream(tile, 2048u + (uint32_t)lane * 16u);
+    t.sc = gload_stream(tile, 3072u + (uint32_t)(lane & 15) * 16u);
+    t.d = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>((gbytes)tile + 3328u + (uint32_t)(lane & 15) * 2u));
+    return t;
+}
+
+// acc[i] += contribution of one (16 rows x 256 k) Q6K tile against one 16-slot operand.
+__device__ inline void q6k_mac(const Q6KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+    const uint32_t M4 = 0x0f0f0f0fu, M2 = 0x03030303u;
+    const float d = __half2float(__ushort_as_half((unsigned short)w.d));
+    // lane groups 0,1 carry elements 0..15 of a 32-element stretch, groups 2,3 elements 16..31
+    const uint32_t first = g < 2 ? 0xffffffffu : 0u, second = ~first;
+    const v4i zero = {0, 0, 0, 0};
+    v4i isum = {0, 0, 0, 0};
+    const uint32_t qw[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+    const uint32_t hw[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
+    const uint32_t sw[4] = {w.sc.x, w.sc.y, w.sc.z, w.sc.w};
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t wx = qw[2 * P], wy = qw[2 * P + 1], h = hw[P];
+        const uint32_t lx = (wx & M4) | ((h & M2) << 4), ly = (wy & M4) | (((h >> 2) & M2) << 4);
+        const uint32_t hx = ((wx >> 4) & M4) | (((h >> 4) & M2) << 4), hy = ((wy >> 4) & M4) | (((h >> 6) & M2) << 4);
+        const long a_lo = pack64(A.a[P].x, A.a[P].y);
+        const long a_hi = pack64(A.a[P].z, A.a[P].w);
+        // sub-blocks 4P .. 4P+3 (16 elements each)
+        v4i D0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & first, ly & first), zero, 0, 0, 0);
+        v4i D1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & second, ly & second), zero, 0, 0, 0);
+        v4i D2 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & first, hy & first), zero, 0, 0, 0);
+        v4i D3 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & second, hy & second), zero, 0, 0, 0);
+        const int s0 = (int)(int8_t)(sw[P] & 0xffu), s1 = (int)(int8_t)((sw[P] >> 8) & 0xffu);
+        const int s2 = (int)(int8_t)((sw[P] >> 16) & 0xffu), s3 = (int)(int8_t)(sw[P] >> 24);
+#pragma unroll
+        for (int i = 0; i < 4; i++) isum[i] += __mul24(s0, D0[i]) + __mul24(s1, D1[i]) + __mul24(s2, D2[i]) + __mul24(s3, D3[i]);
+    }
+    // offset term: sum_j sc_j * bsum_j as an exact f16 MFMA; this lane supplies sub-blocks 4g..4g+3
+    const uint32_t sg = sw[g];
+    const v4h sB = {(_Float16)(int)(int8_t)(sg & 0xffu), (_Float16)(int)(int8_t)((sg >> 8) & 0xffu),
+                    (_Float16)(int)(int8_t)((sg >> 16) & 0xffu), (_Float16)(int)(int8_t)(sg >> 24)};
+    const v4f zf = {0.f, 0.f, 0.f, 0.f};
+    v4f Ds = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, sB, zf, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int tot = isum[i] - 32 * (int)Ds[i];   // exact: |tot| < 2^28
+        acc[i] += (d * yd[i]) * (float)tot;
+    }
+}
+
+// Weight formats of the engine below: tile type, bytes per (16 rows x 256 k) tile, load and multiply.
+struct FmtQ4K {
+    typedef Q4KTile Tile;
+    static constexpr int TILE_BYTES = Q4K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q4k_tile(tile, lane); }
+    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q4k_mac(w, A, yd, g, acc); }
+};
+struct FmtQ6K {
+    typedef Q6KTile Tile;
+    static constexpr int TILE_BYTES = Q6K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q6k_tile(tile, lane); }
+    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q6k_mac(w, A, yd, g, acc); }
+};
+
 // One wave, NT weight tiles per super-block (tp[0..NT), each walking along K), TT 16-slot operand
 // tiles shared by all of them.  RING tile buffers rotate over the item sequence (sb, j): a buffer
 // is refilled with the item RING places ahead as soon as it has been consumed, so RING tiles
@@ -136,12 +212,12 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
 // Tiles of one matrix are ordered [super-block][row tile] (sb-major): all the waves of the grid that
 // are at the same step of their K walk then read one contiguous region, which spreads the requests
 // evenly over the HBM channels.  `sb_stride` = row tiles of the matrix * Q4K_TILE_BYTES.
-template <int NT, int RING>
-__device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t sb_stride, int sb_lo, int sb_last, int lane, Q4KTile t[RING]) {
+template <class FMT, int NT, int RING>
+__device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t sb_stride, int sb_lo, int sb_last, int lane, typename FMT::Tile t[RING]) {
 #pragma unroll
     for (int j = 0; j < RING; j++) {
         const int sb = sb_lo + j / NT < sb_last ? sb_lo + j / NT : sb_last;
-        t[j] = load_q4k_tile(tp[j % NT] + (size_t)sb * sb_stride, lane);
+        t[j] = FMT::load(tp[j % NT] + (size_t)sb * sb_stride, lane);
     }
 }
 
@@ -151,8 +227,8 @@ __device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t s
 // the ring spans RING/NT super-blocks, so that a wave with little work per super-block still keeps
 // RING tiles in flight; the loop then advances RING/NT super-blocks per trip, and a trip that runs
 // past the end multiplies its surplus super-blocks by a zero activation scale.
-template <int TT, int NT, int RING, int DBG = 0>
-__device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride, Q4KTile t[RING], const ActBuf& ab, int K, int nsb,
+template <class FMT, int TT, int NT, int RING>
+__device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride, typename FMT::Tile t[RING], const ActBuf& ab, int K, int nsb,
                                   int sb_lo, int sb_hi, const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
     static_assert(NT % RING == 0 || RING % NT == 0, "ring must divide, or be a multiple of, the tiles per super-block");
     constexpr int U = RING > NT ? RING / NT : 1;   // super-blocks per trip
@@ -180,26 +256,19 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride,
 #pragma unroll
             for (int j = 0; j < NT; j++) {
                 const int idx = u * NT + j;            // position in the trip
-                const Q4KTile w = t[idx % RING];
+                const typename FMT::Tile w = t[idx % RING];
                 const int ahead = idx + RING;          // the item that takes this ring place
                 const int jn = ahead % NT;
                 int sbn = sb0 + ahead / NT;
                 sbn = sbn < sb_hi ? sbn : sb_hi - 1;
-                t[idx % RING] = load_q4k_tile(tp[jn] + (size_t)sbn * sb_stride, lane);
+                t[idx % RING] = FMT::load(tp[jn] + (size_t)sbn * sb_stride, lane);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int tt = 0; tt < TT; tt++) {
-                    if (DBG == 1)  // timing experiment: consume the loads without the arithmetic
-                        acc[j][tt][0] += __uint_as_float((w.q0.x ^ w.q0.w ^ w.q1.y ^ w.q1.z ^ w.sc.z ^ A[tt].a[0].x ^ A[tt].a[3].w) & 0x007fffffu);
-                    else
-                        q4k_mac(w, A[tt], yd[tt], g, acc[j][tt]);
-                }
+                for (int tt = 0; tt < TT; tt++) FMT::mac(w, A[tt], yd[tt], g, acc[j][tt]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (DBG != 2) {  // DBG 2: timing experiment without the per-super-block operand reload
 #pragma unroll
-                for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
-            }
+            for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
         }
     }
 }
@@ -218,7 +287,7 @@ __device__ inline float silu_ref(float v) { return v / (1.0f + expf_glibc(-v)); 
 // p.hbuf instead and leaves the quantisation to a pass of its own.
 constexpr int HBUF_STRIDE = 260;
 
-template <int TT, int NW, int RING, int DBG = 0, int UP_ROWS = 256>
+template <class FMT, int TT, int NW, int RING, int UP_ROWS = 256>
 __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STRIDE], int* list_lds, int* wtot_lds) {
     constexpr int RTW = (UP_ROWS / 16) / NW;  // row tiles per wave and matrix
     constexpr int NT = 2 * RTW;
@@ -232,13 +301,13 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
     const uint8_t* tp[NT];
 #pragma unroll
     for (int j = 0; j < RTW; j++) {
-        tp[j] = gw.w1 + (size_t)(rt0 + j) * Q4K_TILE_BYTES;
-        tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * Q4K_TILE_BYTES;
+        tp[j] = gw.w1 + (size_t)(rt0 + j) * FMT::TILE_BYTES;
+        tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * FMT::TILE_BYTES;
     }
-    const size_t sb_stride = (size_t)(F / 16) * Q4K_TILE_BYTES;
+    const size_t sb_stride = (size_t)(F / 16) * FMT::TILE_BYTES;
     // first weight tiles go out before anything else; an expert without tokens wastes them
-    Q4KTile ring[RING];
-    q4k_engine_prefetch<NT, RING>(tp, sb_stride, 0, nsb - 1, lane, ring);
+    typename FMT::Tile ring[RING];
+    q4k_engine_prefetch<FMT, NT, RING>(tp, sb_stride, 0, nsb - 1, lane, ring);
 
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
@@ -258,7 +327,7 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<TT, NT, RING, DBG>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
+    q4k_engine<FMT, TT, NT, RING>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
 
     if (UP_ROWS != 256) {   // h = silu(w1 x) * (w3 x) straight to memory
 #pragma unroll
@@ -297,7 +366,7 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
 // Down projection: a workgroup owns NTD row tiles (64 weight rows; 32 for very small batches) of one
 // expert; its NW waves split K, every wave carrying the tiles over its K range, and the partial sums
 // meet in LDS.
-template <int TT, int NW, int RING, int NTD = 4>
+template <class FMT, int TT, int NW, int RING, int NTD = 4>
 __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * TT * 4][64], int* list_lds, int* wtot_lds) {
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
@@ -310,12 +379,12 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
 #pragma unroll
     for (int j = 0; j < NTD; j++) {
         int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
-        tp[j] = w2 + (size_t)rt * Q4K_TILE_BYTES;
+        tp[j] = w2 + (size_t)rt * FMT::TILE_BYTES;
     }
-    const size_t sb_stride = (size_t)n_rt * Q4K_TILE_BYTES;
+    const size_t sb_stride = (size_t)n_rt * FMT::TILE_BYTES;
     const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
-    Q4KTile ring[RING];
-    q4k_engine_prefetch<NTD, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, sb_hi > sb_lo ? sb_hi - 1 : (sb_lo < nsb ? sb_lo : nsb - 1), lane, ring);
+    typename FMT::Tile ring[RING];
+    q4k_engine_prefetch<FMT, NTD, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, sb_hi > sb_lo ? sb_hi - 1 : (sb_lo < nsb ? sb_lo : nsb - 1), lane, ring);
 
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
@@ -335,7 +404,7 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
+    q4k_engine<FMT, TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
 
 #pragma unroll
     for (int j = 0; j < NTD; j++)
@@ -358,48 +427,55 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
     }
 }
 
-#define DEF_UP(NAME, TT, NW, RING, WPE) DEF_UP_D(NAME, TT, NW, RING, WPE, 0)
-#define DEF_UP_NARROW(NAME, NW, RING, WPE)                                                                    \
+#define DEF_UP_NARROW(NAME, FMT, NW, RING, WPE)                                                               \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
         __shared__ int wtot_lds[NW];                                                                        \
-        q4k_up_body<1, NW, RING, 0, 64>(p, nullptr, list_lds, wtot_lds);                                    \
+        q4k_up_body<FMT, 1, NW, RING, 64>(p, nullptr, list_lds, wtot_lds);                                  \
     }
-#define DEF_DOWN_NARROW(NAME, NW, RING, WPE)                                                                  \
+#define DEF_DOWN_NARROW(NAME, FMT, NW, RING, WPE)                                                             \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ float part[NW][2 * 4][64];                                                               \
         __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
         __shared__ int wtot_lds[NW];                                                                        \
-        q4k_down_body<1, NW, RING, 2>(p, part, list_lds, wtot_lds);                                         \
+        q4k_down_body<FMT, 1, NW, RING, 2>(p, part, list_lds, wtot_lds);                                    \
     }
-#define DEF_UP_D(NAME, TT, NW, RING, WPE, DBG)                                                                   \
+#define DEF_UP(NAME, FMT, TT, NW, RING, WPE)                                                                  \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ float hbuf[TT * 16][HBUF_STRIDE];                                                        \
         __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
         __shared__ int wtot_lds[NW];                                                                        \
-        q4k_up_body<TT, NW, RING, DBG>(p, hbuf, list_lds, wtot_lds);                                             \
+        q4k_up_body<FMT, TT, NW, RING>(p, hbuf, list_lds, wtot_lds);                                        \
     }
-#define DEF_DOWN(NAME, TT, NW, RING, WPE)                                                                   \
+#define DEF_DOWN(NAME, FMT, TT, NW, RING, WPE)                                                              \
     __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
         __shared__ float part[NW][4 * TT * 4][64];                                                          \
         __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
         __shared__ int wtot_lds[NW];                                                                        \
-        q4k_down_body<TT, NW, RING>(p, part, list_lds, wtot_lds);                                           \
+        q4k_down_body<FMT, TT, NW, RING>(p, part, list_lds, wtot_lds);                                      \
     }
 
 // One 16-slot tile per pass (small batches): variant 1 (default) 4 waves, 168 VGPRs, three workgroups
 // per CU; variant 0 8 waves, 128 VGPRs.  Two and four tiles per pass (up to 32 / 64 rows per expert
 // without streaming its weights twice) need the registers of a two-waves-per-SIMD launch.
-DEF_UP(q4k_up_t1_v0, 1, 8, 2, 4)
-DEF_UP(q4k_up_t1_v1, 1, 4, 2, 3)
-DEF_UP_NARROW(q4k_up_t1_narrow, 4, 2, 3)
-DEF_UP(q4k_up_t2, 2, 4, 2, 2)
-DEF_UP(q4k_up_t4, 4, 8, 2, 2)
-DEF_DOWN(q4k_down_t1_v0, 1, 8, 2, 4)
-DEF_DOWN(q4k_down_t1_v1, 1, 4, 2, 3)
-DEF_DOWN_NARROW(q4k_down_t1_narrow, 8, 2, 4)
-DEF_DOWN(q4k_down_t2, 2, 4, 2, 2)
-DEF_DOWN(q4k_down_t4, 4, 8, 2, 2)
+DEF_UP(q4k_up_t1_v0, FmtQ4K, 1, 8, 2, 4)
+DEF_UP(q4k_up_t1_v1, FmtQ4K, 1, 4, 2, 3)
+DEF_UP_NARROW(q4k_up_t1_narrow, FmtQ4K, 4, 2, 3)
+DEF_UP(q4k_up_t2, FmtQ4K, 2, 4, 2, 2)
+DEF_UP(q4k_up_t4, FmtQ4K, 4, 8, 2, 2)
+DEF_DOWN(q4k_down_t1_v0, FmtQ4K, 1, 8, 2, 4)
+DEF_DOWN(q4k_down_t1_v1, FmtQ4K, 1, 4, 2, 3)
+DEF_DOWN_NARROW(q4k_down_t1_narrow, FmtQ4K, 8, 2, 4)
+DEF_DOWN(q4k_down_t2, FmtQ4K, 2, 4, 2, 2)
+DEF_DOWN(q4k_down_t4, FmtQ4K, 4, 8, 2, 2)
+// Q6K: the same bodies; its tiles take five loads and seventeen registers, so every variant gets the
+// registers of a two-waves-per-SIMD launch, and four slot tiles per pass would spill: two at most
+DEF_UP(q6k_up_t1, FmtQ6K, 1, 4, 2, 2)
+DEF_UP_NARROW(q6k_up_t1_narrow, FmtQ6K, 4, 2, 2)
+DEF_UP(q6k_up_t2, FmtQ6K, 2, 4, 2, 2)
+DEF_DOWN(q6k_down_t1, FmtQ6K, 1, 4, 2, 2)
+DEF_DOWN_NARROW(q6k_down_t1_narrow, FmtQ6K, 8, 2, 2)
+DEF_DOWN(q6k_down_t2, FmtQ6K, 2, 4, 2, 2)
 
 // ---------------------------------------------------------------------------------------------
 static int variant(const char* name, int dflt) {
@@ -410,13 +486,20 @@ static int variant(const char* name, int dflt) {
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_UP_VARIANT", 1);
-    const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const bool q6k = p.dt == MOE_GGML_Q6K;
+    const int tt = p.slot_tiles >= 4 && !q6k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (64 rows), f32 h to p.hbuf
         dim3 ngrid((unsigned)(p.F / 64), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
-        hipLaunchKernelGGL(q4k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
+        if (q6k) hipLaunchKernelGGL(q6k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q4k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
     dim3 grid((unsigned)(p.F / 256), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (q6k) {
+        if (tt == 2) hipLaunchKernelGGL(q6k_up_t2, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q6k_up_t1, grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
     if (tt == 4) hipLaunchKernelGGL(q4k_up_t4, grid, dim3(512), 0, s, p);
     else if (tt == 2) hipLaunchKernelGGL(q4k_up_t2, grid, dim3(256), 0, s, p);
     else if (v == 0) hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
@@ -427,13 +510,20 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_DOWN_VARIANT", 1);
-    const int tt = p.slot_tiles >= 4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const bool q6k = (p.dt_down ? p.dt_down : p.dt) == MOE_GGML_Q6K;
+    const int tt = p.slot_tiles >= 4 && !q6k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (32 rows), eight waves split K
         dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
-        hipLaunchKernelGGL(q4k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
+        if (q6k) hipLaunchKernelGGL(q6k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
+        else hipLaunchKernelGGL(q4k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
         return hipGetLastError();
     }
     dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    if (q6k) {
+        if (tt == 2) hipLaunchKernelGGL(q6k_down_t2, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q6k_down_t1, grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
     if (tt == 4) hipLaunchKernelGGL(q4k_down_t4, grid, dim3(512), 0, s, p);
     else if (tt == 2) hipLaunchKernelGGL(q4k_down_t2, grid, dim3(256), 0, s, p);
     else if (v == 0) hipLaunchKernelGGL(q4k_down_t1_v0, grid, dim3(512), 0, s, p);

@@ -2,7 +2,7 @@
 // from either layout, and the stand-alone activation quantiser used by the parity hooks.
 //
 // to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0),
-// 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60) and 1858-1870 (Q8K).  The library is
+// 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
 #include <algorithm>
 #include "act_quant.hpp"
@@ -34,6 +34,17 @@ __device__ inline float q4k_value(const uint8_t* hdr, int i, uint8_t qbyte) {
     return d1 * (float)q - m1;
 }
 
+// code (0..63) of element e (0..255) of a raw BlockQ6K: the bit fields of k_quants.rs:1772-1778
+__device__ inline int q6k_code(const uint8_t* blk, int e) {
+    const int half = e / 128, q = (e % 128) / 32, l = e % 32;
+    const uint8_t b = blk[64 * half + 32 * (q & 1) + l];
+    const int nib = q >= 2 ? (b >> 4) : (b & 0xF);
+    const int hi = (blk[128 + 32 * half + l] >> (2 * q)) & 3;
+    return nib | (hi << 4);
+}
+// to_float of one Q6K element, k_quants.rs:1779-1782: `d * sc as f32 * q as f32`, left to right
+__device__ inline float q6k_value(float d, int8_t sc, int code) { return d * (float)sc * (float)(int8_t)(code - 32); }
+
 // ------------------------------------------------------------------ standard layout to_float
 __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -42,6 +53,10 @@ __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, in
         const uint8_t* b = blocks + (i / 256) * 144;
         int e = (int)(i % 256);
         out[i] = q4k_value(b, e, b[16 + (e / 64) * 32 + (e % 32)]);
+    } else if (dt == MOE_GGML_Q6K) {
+        const uint8_t* b = blocks + (i / 256) * 210;
+        int e = (int)(i % 256);
+        out[i] = q6k_value(f16_bits_to_f32((uint16_t)(b[208] | (b[209] << 8))), (int8_t)b[192 + e / 16], q6k_code(b, e));
     } else if (dt == MOE_GGML_Q4_0) {
         const uint8_t* b = blocks + (i / 32) * 18;
         int e = (int)(i % 32);
@@ -82,6 +97,34 @@ __global__ void relayout_q4k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t 
         int r = ch - 128;
         const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
         for (int i = 0; i < 16; i++) dst[i] = blk[i];
+    }
+}
+
+__global__ void relayout_q6k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
+    // one thread per (tile, lane): its 32 nibble bytes and 16 high-bit bytes; lanes < 16 also move the
+    // row's scales and d
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nsb * 64) return;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int64_t rt = tile / nsb;
+    int sb = (int)(tile % nsb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 210;
+    uint8_t* dst = tiled + (sb * n_rt + rt) * Q6K_TILE_BYTES;  // tiles ordered [sb][rt]
+    for (int P = 0; P < 4; P++) {
+        int ca[8], cb[8];
+        for (int i = 0; i < 8; i++) {
+            ca[i] = q6k_code(blk, 64 * P + 8 * g + i);
+            cb[i] = q6k_code(blk, 64 * P + 32 + 8 * g + i);
+            dst[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + i] = (uint8_t)((ca[i] & 15) | ((cb[i] & 15) << 4));
+        }
+        for (int i = 0; i < 4; i++)
+            dst[2048 + l * 16 + P * 4 + i] = (uint8_t)((ca[i] >> 4) | ((ca[i + 4] >> 4) << 2) | ((cb[i] >> 4) << 4) | ((cb[i + 4] >> 4) << 6));
+    }
+    if (g == 0) {
+        for (int j = 0; j < 16; j++) dst[3072 + r * 16 + j] = blk[192 + j];
+        dst[3328 + 2 * r] = blk[208];
+        dst[3328 + 2 * r + 1] = blk[209];
     }
 }
 
@@ -132,6 +175,16 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         int l = g * 16 + r;
         uint8_t q = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
         out[i] = q4k_value(tile + 2048 + r * 16, e, q);
+    } else if (dt == MOE_GGML_Q6K) {
+        int sb = col / 256, e = col % 256;
+        const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q6K_TILE_BYTES;
+        int P = e / 64, sub = (e % 64) / 32, g = (e % 32) / 8, pos = e % 8;
+        int l = g * 16 + r;
+        uint8_t nb = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
+        uint8_t hb = tile[2048 + l * 16 + P * 4 + pos % 4];
+        int code = (sub ? (nb >> 4) : (nb & 0xF)) | (((hb >> (2 * (2 * sub + pos / 4))) & 3) << 4);
+        float d = f16_bits_to_f32((uint16_t)(tile[3328 + 2 * r] | (tile[3328 + 2 * r + 1] << 8)));
+        out[i] = q6k_value(d, (int8_t)tile[3072 + r * 16 + e / 16], code);
     } else if (dt == MOE_GGML_Q8_0) {
         int nkb = (int)(k / 32), kb = col / 32, e = col % 32;
         const uint8_t* tile = tiled + (rt * nkb + kb) * Q8_0_TILE_BYTES;
@@ -207,6 +260,8 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
     if (n_rt == 0 || nkb == 0) return hipSuccess;
     if (dt == MOE_GGML_Q4K)
         hipLaunchKernelGGL(relayout_q4k_kernel, dim3(nblk(n_rt * nkb * 144, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (dt == MOE_GGML_Q6K)
+        hipLaunchKernelGGL(relayout_q6k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q8_0)
         hipLaunchKernelGGL(relayout_q8_0_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else

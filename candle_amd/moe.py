@@ -11,8 +11,8 @@ import os
 
 import numpy as np
 
-GGML_Q4_0, GGML_Q8_0, GGML_Q4K, GGML_Q8K = 2, 8, 12, 15
-_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4K: (256, 144), GGML_Q8K: (256, 292)}
+GGML_Q4_0, GGML_Q8_0, GGML_Q4K, GGML_Q6K, GGML_Q8K = 2, 8, 12, 14, 15
+_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q4K: (256, 144), GGML_Q6K: (256, 210), GGML_Q8K: (256, 292)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "lib", "libcandle_amd_moe.so")
@@ -31,6 +31,7 @@ class _Desc(C.Structure):
         ("w1", C.POINTER(C.c_void_p)), ("w3", C.POINTER(C.c_void_p)), ("w2", C.POINTER(C.c_void_p)),
         ("shared_ffn", C.c_int64), ("shared_w1", C.c_void_p), ("shared_w3", C.c_void_p), ("shared_w2", C.c_void_p),
         ("shared_gate", C.c_void_p), ("rms_alpha", C.c_void_p), ("rms_eps", C.c_float),
+        ("ggml_dtype_down", C.c_int32),
     ]
 
 
@@ -281,10 +282,13 @@ class SparseMoeBlock:
 
     def __init__(self, hidden, ffn, n_experts, top_k, ggml_dtype, gate, w1, w3, w2, norm_topk=True,
                  gate_bias=None, shared_ffn=0, shared_w1=None, shared_w3=None, shared_w2=None,
-                 shared_gate=None, rms_alpha=None, rms_eps=1e-5):
+                 shared_gate=None, rms_alpha=None, rms_eps=1e-5, ggml_dtype_down=None):
         L = load_library()
-        if ggml_dtype not in (GGML_Q4_0, GGML_Q8_0, GGML_Q4K):
-            raise MoeError("unsupported ggml_dtype %r" % (ggml_dtype,))
+        dtype_down = ggml_dtype if ggml_dtype_down is None else ggml_dtype_down
+        for dt in (ggml_dtype, dtype_down):
+            if dt not in _BLOCK or dt == GGML_Q8K:
+                raise MoeError("unsupported ggml_dtype %r" % (dt,))
+        self.dtype_down = dtype_down
         if len(w1) != n_experts or len(w2) != n_experts or len(w3) != n_experts:
             raise MoeError("need one w1/w2/w3 per expert")
         self.hidden, self.ffn, self.n_experts, self.top_k, self.dtype = hidden, ffn, n_experts, top_k, ggml_dtype
@@ -293,7 +297,7 @@ class SparseMoeBlock:
         keep = [gate]
         mats = {}
         for name, ws in (("w1", w1), ("w3", w3), ("w2", w2)):
-            arrs = [_blocks(w, ggml_dtype, hidden * ffn, name) for w in ws]
+            arrs = [_blocks(w, dtype_down if name == "w2" else ggml_dtype, hidden * ffn, name) for w in ws]
             keep += arrs
             mats[name] = (C.c_void_p * n_experts)(*[a.ctypes.data for a in arrs])
         opt = {}
@@ -305,7 +309,7 @@ class SparseMoeBlock:
         sh = {}
         for name, a in (("shared_w1", shared_w1), ("shared_w3", shared_w3), ("shared_w2", shared_w2)):
             if shared_ffn:
-                a = _blocks(a, ggml_dtype, hidden * shared_ffn, name)
+                a = _blocks(a, dtype_down if name == "shared_w2" else ggml_dtype, hidden * shared_ffn, name)
                 keep.append(a)
             else:
                 a = None
@@ -314,7 +318,8 @@ class SparseMoeBlock:
         desc = _Desc(hidden, ffn, n_experts, top_k, ggml_dtype, int(norm_topk), ptr(gate), ptr(opt["gate_bias"]),
                      C.cast(mats["w1"], C.POINTER(C.c_void_p)), C.cast(mats["w3"], C.POINTER(C.c_void_p)),
                      C.cast(mats["w2"], C.POINTER(C.c_void_p)), shared_ffn, ptr(sh["shared_w1"]), ptr(sh["shared_w3"]),
-                     ptr(sh["shared_w2"]), ptr(opt["shared_gate"]), ptr(opt["rms_alpha"]), float(rms_eps))
+                     ptr(sh["shared_w2"]), ptr(opt["shared_gate"]), ptr(opt["rms_alpha"]), float(rms_eps),
+                     0 if dtype_down == ggml_dtype else dtype_down)
         handle = C.c_void_p()
         self._h = None
         _check(L.moe_layer_create(C.byref(desc), C.byref(handle)))
@@ -335,6 +340,7 @@ class SparseMoeBlock:
             self = cls.__new__(cls)
             self._h = h
             self.hidden, self.ffn, self.dtype = hdim, f, dt
+            self.dtype_down = g.tensor(prefix + ".ffn_down.0.weight")[0]
             self.n_experts = g.metadata("llama.expert_count")
             self.top_k = g.metadata("llama.expert_used_count")
             self.shared_ffn = 0
@@ -421,7 +427,7 @@ class QMatMul:
     of quantized_llama.rs:590-593, 608)."""
 
     def __init__(self, ggml_dtype, w_blocks, n, k):
-        if ggml_dtype not in (GGML_Q4_0, GGML_Q8_0, GGML_Q4K):
+        if ggml_dtype not in _BLOCK or ggml_dtype == GGML_Q8K:
             raise MoeError("unsupported ggml_dtype %r" % (ggml_dtype,))
         w_blocks = _blocks(w_blocks, ggml_dtype, n * k, "QMatMul")
         h = C.c_void_p()

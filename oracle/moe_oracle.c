@@ -97,7 +97,7 @@ static inline float rmin(float a, float b) { return fminf(a, b); }
 int64_t orc_block_elems(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return 32;
-        case ORC_Q4K: case ORC_Q8K: return 256;
+        case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return 256;
         default: return -1;
     }
 }
@@ -106,6 +106,7 @@ int64_t orc_block_bytes(int dtype) {
         case ORC_Q4_0: return 18;
         case ORC_Q8_0: return 34;
         case ORC_Q4K: return 144;
+        case ORC_Q6K: return 210;
         case ORC_Q8K: return 292;
         default: return -1;
     }
@@ -113,7 +114,7 @@ int64_t orc_block_bytes(int dtype) {
 int orc_vecdot_dtype(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
-        case ORC_Q4K: case ORC_Q8K: return ORC_Q8K;
+        case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
         default: return -1;
     }
 }
@@ -367,6 +368,226 @@ static float vec_dot_q4k_q8k(int64_t n, const orc_block_q4k* xs, const orc_block
     return sumf + tail;
 }
 
+/* ------------------------------------------------------------------ Q6K */
+/* make_qx_quants, utils.rs:62-203 (the caller below uses rmse_type 1: unit weights, early return) */
+static float make_qx_quants(int n, int nmax, const float* x, int8_t* ls, int rmse_type) {
+    float max = 0.f, amax = 0.f;
+    for (int i = 0; i < n; i++) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax == 0.f) {
+        for (int i = 0; i < n; i++) ls[i] = 0;
+        return 0.f;
+    }
+    float iscale = -(float)nmax / max;
+    if (rmse_type == 0) {
+        for (int i = 0; i < n; i++) {
+            int32_t l = nearest_int(iscale * x[i]);
+            l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+            ls[i] = (int8_t)(nmax + l);
+        }
+        return 1.0f / iscale;
+    }
+    const int weight_type = rmse_type % 2;
+    float sumlx = 0.f, suml2 = 0.f;
+    for (int i = 0; i < n; i++) {
+        int32_t l = nearest_int(iscale * x[i]);
+        l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+        ls[i] = (int8_t)(l + nmax);
+        float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+        float lf = (float)l;
+        sumlx += w * x[i] * lf;
+        suml2 += w * lf * lf;
+    }
+    float scale = sumlx / suml2;
+    float best = scale * sumlx;
+    for (int itry = 0; itry < 3; itry++) {
+        float is2 = 1.0f / scale;
+        float slx = 0.f, sl2 = 0.f;
+        int changed = 0;
+        for (int i = 0; i < n; i++) {
+            int32_t l = nearest_int(is2 * x[i]);
+            l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+            if (l + nmax != (int32_t)ls[i]) changed = 1;
+            float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+            float lf = (float)l;
+            slx += w * x[i] * lf;
+            sl2 += w * lf * lf;
+        }
+        if (!changed || sl2 == 0.0f || slx * slx <= best * sl2) break;
+        for (int i = 0; i < n; i++) {
+            int32_t l = nearest_int(is2 * x[i]);
+            l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+            ls[i] = (int8_t)(nmax + l);
+        }
+        sumlx = slx;
+        suml2 = sl2;
+        scale = sumlx / suml2;
+        best = scale * sumlx;
+    }
+    for (int itry = 0; itry < 5; itry++) {
+        int n_changed = 0;
+        for (int i = 0; i < n; i++) {
+            float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+            int32_t l = (int32_t)ls[i] - nmax;
+            float slx = sumlx - w * x[i] * (float)l;
+            if (slx > 0.f) {
+                float sl2 = suml2 - w * (float)l * (float)l;
+                int32_t new_l = nearest_int(x[i] * sl2 / slx);
+                new_l = new_l < -nmax ? -nmax : new_l > nmax - 1 ? nmax - 1 : new_l;
+                if (new_l != l) {
+                    slx += w * x[i] * (float)new_l;
+                    sl2 += w * (float)new_l * (float)new_l;
+                    if (sl2 > 0.f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                        ls[i] = (int8_t)(nmax + new_l);
+                        sumlx = slx;
+                        suml2 = sl2;
+                        scale = sumlx / suml2;
+                        best = scale * sumlx;
+                        n_changed++;
+                    }
+                }
+            }
+        }
+        if (n_changed == 0) break;
+    }
+    if (rmse_type < 3) return scale;
+    for (int is = -4; is < 4; is++) {
+        if (is == 0) continue;
+        iscale = -((float)nmax + 0.1f * (float)is) / max;
+        float slx = 0.f, sl2 = 0.f;
+        for (int i = 0; i < n; i++) {
+            int32_t l = nearest_int(iscale * x[i]);
+            l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+            float w = weight_type == 1 ? x[i] * x[i] : 1.0f;
+            float lf = (float)l;
+            slx += w * x[i] * lf;
+            sl2 += w * lf * lf;
+        }
+        if (sl2 > 0.f && slx * slx > best * sl2) {
+            for (int i = 0; i < n; i++) {
+                int32_t l = nearest_int(iscale * x[i]);
+                l = l < -nmax ? -nmax : l > nmax - 1 ? nmax - 1 : l;
+                ls[i] = (int8_t)(nmax + l);
+            }
+            scale = slx / sl2;
+            best = scale * slx;
+        }
+    }
+    return scale;
+}
+/* k_quants.rs:1673-1751 */
+static void quantize_q6k(const float* xs, int64_t k, orc_block_q6k* ys) {
+    int8_t l[256];
+    float scales[16];
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float* x = xs + b * 256;
+        orc_block_q6k* y = &ys[b];
+        float max_scale = 0.f, max_abs_scale = 0.f;
+        for (int ib = 0; ib < 16; ib++) {
+            float scale = make_qx_quants(16, 32, x + 16 * ib, l + 16 * ib, 1);
+            scales[ib] = scale;
+            float a = fabsf(scale);
+            if (a > max_abs_scale) { max_abs_scale = a; max_scale = scale; }
+        }
+        float iscale = -128.0f / max_scale;
+        y->d = orc_f32_to_f16(1.0f / iscale);
+        for (int j = 0; j < 16; j++) {
+            int32_t v = nearest_int(iscale * scales[j]);
+            y->scales[j] = (int8_t)(v < 127 ? v : 127);   /* `as i8` wraps below -128; cannot occur: |v| <= 128 */
+        }
+        for (int j = 0; j < 16; j++) {
+            float d = orc_f16_to_f32(y->d) * (float)y->scales[j];
+            if (d == 0.f) continue;
+            for (int ii = 0; ii < 16; ii++) {
+                int32_t ll = nearest_int(x[16 * j + ii] / d);
+                ll = ll < -32 ? -32 : ll > 31 ? 31 : ll;
+                l[16 * j + ii] = (int8_t)(ll + 32);
+            }
+        }
+        uint8_t* ql = y->ql;
+        uint8_t* qh = y->qh;
+        for (int j = 0; j < 256; j += 128) {
+            for (int i = 0; i < 32; i++) {
+                uint8_t q1 = (uint8_t)l[j + i] & 0xF, q2 = (uint8_t)l[j + i + 32] & 0xF;
+                uint8_t q3 = (uint8_t)l[j + i + 64] & 0xF, q4 = (uint8_t)l[j + i + 96] & 0xF;
+                ql[i] = (uint8_t)(q1 | (q3 << 4));
+                ql[i + 32] = (uint8_t)(q2 | (q4 << 4));
+                /* arithmetic shifts of i8 values 0..63: same as unsigned here */
+                qh[i] = (uint8_t)((l[j + i] >> 4) | ((l[j + i + 32] >> 4) << 2) | ((l[j + i + 64] >> 4) << 4) |
+                                  ((l[j + i + 96] >> 4) << 6));
+            }
+            ql += 64;
+            qh += 32;
+        }
+    }
+}
+/* k_quants.rs:1753-1790 */
+static void dequantize_q6k(const orc_block_q6k* xs, int64_t k, float* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const orc_block_q6k* x = &xs[b];
+        float d = orc_f16_to_f32(x->d);
+        for (int n = 0; n < 256; n += 128) {
+            int idx = n / 128;
+            float* y = ys + b * 256 + n;
+            const int8_t* sc = x->scales + 8 * idx;
+            const uint8_t* ql = x->ql + 64 * idx;
+            const uint8_t* qh = x->qh + 32 * idx;
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int8_t q1 = (int8_t)((int8_t)((ql[l] & 0xF) | ((qh[l] & 3) << 4)) - 32);
+                int8_t q2 = (int8_t)((int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+                int8_t q3 = (int8_t)((int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+                int8_t q4 = (int8_t)((int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+                y[l] = d * (float)sc[is] * (float)q1;           /* (d * sc) * q, left to right */
+                y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+                y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+                y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+            }
+        }
+    }
+}
+/* k_quants.rs:1613-1671 (vec_dot_unopt) */
+static float vec_dot_q6k_q8k(int64_t n, const orc_block_q6k* xs, const orc_block_q8k* ys) {
+    int8_t aux8[256];
+    int16_t aux16[8];
+    float sums[8] = {0};
+    float aux32[8];
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q6k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        for (int l = 0; l < 8; l++) aux32[l] = 0.f;
+        for (int j = 0; j < 256; j += 128) {
+            int8_t* a = aux8 + j;
+            const uint8_t* q4 = x->ql + j / 2;
+            const uint8_t* qh = x->qh + j / 4;
+            for (int l = 0; l < 32; l++) {
+                a[l] = (int8_t)((int32_t)((q4[l] & 0xF) | ((qh[l] & 3) << 4)) - 32);
+                a[l + 32] = (int8_t)((int32_t)((q4[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32);
+                a[l + 64] = (int8_t)((int32_t)((q4[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32);
+                a[l + 96] = (int8_t)((int32_t)((q4[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32);
+            }
+        }
+        for (int j = 0; j < 16; j++) {
+            float scale = (float)x->scales[j];
+            const int8_t* q8 = y->qs + 16 * j;
+            const int8_t* a = aux8 + 16 * j;
+            for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+            for (int l = 0; l < 8; l++) aux32[l] += scale * (float)aux16[l];
+            q8 += 8;
+            a += 8;
+            for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+            for (int l = 0; l < 8; l++) aux32[l] += scale * (float)aux16[l];
+        }
+        float d = orc_f16_to_f32(x->d) * y->d;
+        for (int l = 0; l < 8; l++) sums[l] += aux32[l] * d;
+    }
+    float total = 0.f;
+    for (int l = 0; l < 8; l++) total += sums[l];
+    return total;
+}
+
 /* ------------------------------------------------------------------ Q8K */
 /* k_quants.rs:1819-1856 */
 static void quantize_q8k(const float* xs, int64_t k, orc_block_q8k* ys) {
@@ -422,6 +643,7 @@ int orc_quantize(int dtype, const float* x, int64_t n, void* blocks) {
         case ORC_Q4_0: quantize_q4_0(x, n, (orc_block_q4_0*)blocks); return 0;
         case ORC_Q8_0: quantize_q8_0(x, n, (orc_block_q8_0*)blocks); return 0;
         case ORC_Q4K: memset(blocks, 0, (size_t)(n / 256) * 144); quantize_q4k(x, n, (orc_block_q4k*)blocks); return 0;
+        case ORC_Q6K: memset(blocks, 0, (size_t)(n / 256) * 210); quantize_q6k(x, n, (orc_block_q6k*)blocks); return 0;
         case ORC_Q8K: quantize_q8k(x, n, (orc_block_q8k*)blocks); return 0;
     }
     return -1;
@@ -433,6 +655,7 @@ int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y) {
         case ORC_Q4_0: dequantize_q4_0((const orc_block_q4_0*)blocks, n, y); return 0;
         case ORC_Q8_0: dequantize_q8_0((const orc_block_q8_0*)blocks, n, y); return 0;
         case ORC_Q4K: dequantize_q4k((const orc_block_q4k*)blocks, n, y); return 0;
+        case ORC_Q6K: dequantize_q6k((const orc_block_q6k*)blocks, n, y); return 0;
         case ORC_Q8K: dequantize_q8k((const orc_block_q8k*)blocks, n, y); return 0;
     }
     return -1;
@@ -442,6 +665,7 @@ float orc_vec_dot(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q4_0: return vec_dot_q4_0_q8_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return vec_dot_q8_0_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return vec_dot_q4k_q8k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q6K: return vec_dot_q6k_q8k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         case ORC_Q8K: return vec_dot_q8k_q8k(n, (const orc_block_q8k*)w, (const orc_block_q8k*)a);
     }
     return NAN;
@@ -587,7 +811,7 @@ int orc_route(const float* probs, int64_t T, int64_t E, int64_t k, int norm_topk
 
 /* ------------------------------------------------------------------ block */
 /* Mlp::forward quantized_llama.rs:124-131 on n rows */
-static int expert_mlp(int dtype, int64_t n, int64_t H, int64_t F, const float* x, const void* w1,
+static int expert_mlp(int dtype, int dtype_down, int64_t n, int64_t H, int64_t F, const float* x, const void* w1,
                       const void* w3, const void* w2, float* out, int simd, int threads) {
     float* a = (float*)malloc(sizeof(float) * (size_t)(n * F));
     float* b = (float*)malloc(sizeof(float) * (size_t)(n * F));
@@ -596,7 +820,7 @@ static int expert_mlp(int dtype, int64_t n, int64_t H, int64_t F, const float* x
     if (!rc) rc = orc_matmul(dtype, n, H, F, x, w3, b, simd, threads);
     if (!rc) {
         for (int64_t i = 0; i < n * F; i++) a[i] = orc_silu(a[i]) * b[i];
-        rc = orc_matmul(dtype, n, F, H, a, w2, out, simd, threads);
+        rc = orc_matmul(dtype_down, n, F, H, a, w2, out, simd, threads);
     }
     free(a); free(b);
     return rc;
@@ -605,6 +829,7 @@ static int expert_mlp(int dtype, int64_t n, int64_t H, int64_t F, const float* x
 int orc_moe_forward(const orc_layer* L, const float* xs_in, int64_t T, const float* logits_in,
                     float* logits_out, float* ys, int simd, int threads) {
     const int64_t H = L->H, E = L->E, k = L->k;
+    const int dtype_down = L->dtype_down ? L->dtype_down : L->dtype;
     int rc = 0;
     float* xn = NULL;
     const float* xs = xs_in;
@@ -641,7 +866,7 @@ int orc_moe_forward(const orc_layer* L, const float* xs_in, int64_t T, const flo
         float* out = (float*)malloc(sizeof(float) * (size_t)(n * H));
         if (!cur || !out) { free(cur); free(out); rc = -1; break; }
         for (int64_t i = 0; i < n; i++) memcpy(cur + i * H, xs + (int64_t)rows[i] * H, sizeof(float) * (size_t)H);
-        rc = expert_mlp(L->dtype, n, H, L->F, cur, L->w1[e], L->w3[e], L->w2[e], out, simd, threads);
+        rc = expert_mlp(L->dtype, dtype_down, n, H, L->F, cur, L->w1[e], L->w3[e], L->w2[e], out, simd, threads);
         if (!rc)
             for (int64_t i = 0; i < n; i++) {
                 float w = perm_w[offsets[e] + i];
@@ -656,7 +881,7 @@ int orc_moe_forward(const orc_layer* L, const float* xs_in, int64_t T, const flo
     if (!rc && L->Fs > 0) { /* qwen2_moe.rs:315-319 */
         float* so = (float*)malloc(sizeof(float) * (size_t)(T * H));
         if (!so) rc = -1;
-        if (!rc) rc = expert_mlp(L->dtype, T, H, L->Fs, xs, L->sw1, L->sw3, L->sw2, so, simd, threads);
+        if (!rc) rc = expert_mlp(L->dtype, dtype_down, T, H, L->Fs, xs, L->sw1, L->sw3, L->sw2, so, simd, threads);
         if (!rc)
             for (int64_t t = 0; t < T; t++) {
                 float g = 0.f;

@@ -6,6 +6,7 @@
  *   vec_dot_q4_0_q8_0  candle-core/src/quantized/avx.rs:50-68
  *   vec_dot_q8_0_q8_0  candle-core/src/quantized/avx.rs:71-87
  *   vec_dot_q4k_q8k    candle-core/src/quantized/avx.rs:443-525
+ *   vec_dot_q6k_q8k    candle-core/src/quantized/avx.rs:131-216
  * The integer parts are exact; the f32 accumulation order differs from the scalar
  * vec_dot_unopt, which the reference's own tests allow up to 1e-6 * k
  * (candle-core/tests/quantized_tests.rs:869-876).  Used for the CPU-baseline timing.
@@ -109,11 +110,61 @@ static float dot_q4k(int64_t n, const orc_block_q4k* xs, const orc_block_q8k* ys
     return hsum_float_8(acc) + _mm_cvtss_f32(acc_m);
 }
 
+static float dot_q6k(int64_t n, const orc_block_q6k* xs, const orc_block_q8k* ys) {
+    const __m256i m4 = _mm256_set1_epi8(0xF), m2 = _mm256_set1_epi8(3), m32s = _mm256_set1_epi8(32);
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q6k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        float d = y->d * orc_f16_to_f32(x->d);
+        const uint8_t* q4 = x->ql;
+        const uint8_t* qh = x->qh;
+        const int8_t* q8 = y->qs;
+        __m128i scales = _mm_loadu_si128((const __m128i*)x->scales);
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < 2; j++) {
+            __m256i sc[4];
+            for (int t = 0; t < 4; t++) {
+                /* scale 2i in the low eight bytes, scale 2i+1 in the high eight (get_scale_shuffle, avx.rs:89-99) */
+                const int i = 4 * j + t;
+                __m128i shuf = _mm_set_epi64x(0x0101010101010101LL * (2 * i + 1), 0x0101010101010101LL * (2 * i));
+                sc[t] = _mm256_cvtepi8_epi16(_mm_shuffle_epi8(scales, shuf));
+            }
+            __m256i q4bits1 = _mm256_loadu_si256((const __m256i*)q4);
+            __m256i q4bits2 = _mm256_loadu_si256((const __m256i*)(q4 + 32));
+            q4 += 64;
+            __m256i q4bits_h = _mm256_loadu_si256((const __m256i*)qh);
+            qh += 32;
+            __m256i qv[4];
+            qv[0] = _mm256_or_si256(_mm256_and_si256(q4bits1, m4), _mm256_slli_epi16(_mm256_and_si256(q4bits_h, m2), 4));
+            qv[1] = _mm256_or_si256(_mm256_and_si256(q4bits2, m4),
+                                    _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bits_h, 2), m2), 4));
+            qv[2] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(q4bits1, 4), m4),
+                                    _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bits_h, 4), m2), 4));
+            qv[3] = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(q4bits2, 4), m4),
+                                    _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bits_h, 6), m2), 4));
+            __m256i p[4];
+            for (int t = 0; t < 4; t++) {
+                __m256i q8v = _mm256_loadu_si256((const __m256i*)q8);
+                q8 += 32;
+                __m256i q8s = _mm256_maddubs_epi16(m32s, q8v);
+                __m256i p16 = _mm256_sub_epi16(_mm256_maddubs_epi16(qv[t], q8v), q8s);
+                p[t] = _mm256_madd_epi16(sc[t], p16);
+            }
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(p[0], p[1]));
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(p[2], p[3]));
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum_float_8(acc);
+}
+
 float orc_vec_dot_avx2(int dtype, int64_t n, const void* w, const void* a) {
     switch (dtype) {
         case ORC_Q4_0: return dot_q4_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return dot_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return dot_q4k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q6K: return dot_q6k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         default: return orc_vec_dot(dtype, n, w, a);
     }
 }

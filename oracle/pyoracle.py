@@ -12,10 +12,10 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmoe_oracle.so")
 
-Q4_0, Q8_0, Q4K, Q8K = 2, 8, 12, 15
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4K: 256, Q8K: 256}
-BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4K: 144, Q8K: 292}
-VECDOT = {Q4_0: Q8_0, Q8_0: Q8_0, Q4K: Q8K, Q8K: Q8K}
+Q4_0, Q8_0, Q4K, Q6K, Q8K = 2, 8, 12, 14, 15
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4K: 256, Q6K: 256, Q8K: 256}
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q4K: 144, Q6K: 210, Q8K: 292}
+VECDOT = {Q4_0: Q8_0, Q8_0: Q8_0, Q4K: Q8K, Q6K: Q8K, Q8K: Q8K}
 
 
 def build(force=False):
@@ -33,6 +33,7 @@ class _Layer(C.Structure):
         ("w1", C.POINTER(C.c_void_p)), ("w3", C.POINTER(C.c_void_p)), ("w2", C.POINTER(C.c_void_p)),
         ("Fs", C.c_int64), ("sw1", C.c_void_p), ("sw3", C.c_void_p), ("sw2", C.c_void_p),
         ("shared_gate", C.c_void_p), ("rms_alpha", C.c_void_p), ("rms_eps", C.c_float),
+        ("dtype_down", C.c_int),
     ]
 
 
@@ -196,8 +197,9 @@ class Layer:
     """Block-level oracle: candle's MlpOrMoe::MoE forward on raw GGUF blocks."""
 
     def __init__(self, H, F, E, k, dtype, gate, w1, w3, w2, norm_topk=True, gate_bias=None,
-                 Fs=0, sw1=None, sw3=None, sw2=None, shared_gate=None, rms_alpha=None, rms_eps=1e-5):
+                 Fs=0, sw1=None, sw3=None, sw2=None, shared_gate=None, rms_alpha=None, rms_eps=1e-5, dtype_down=None):
         self.H, self.F, self.E, self.k, self.dtype = H, F, E, k, dtype
+        self.dtype_down = dtype if dtype_down is None else dtype_down
         self._keep = []
 
         def keep(a, dt):
@@ -212,8 +214,10 @@ class Layer:
         self.w1 = [keep(w, np.uint8) for w in w1]
         self.w3 = [keep(w, np.uint8) for w in w3]
         self.w2 = [keep(w, np.uint8) for w in w2]
-        for w in self.w1 + self.w3 + self.w2:
+        for w in self.w1 + self.w3:
             assert w.size == nbytes(dtype, H * F)
+        for w in self.w2:
+            assert w.size == nbytes(self.dtype_down, H * F)
         self.sw = [keep(w, np.uint8) for w in (sw1, sw3, sw2)]
         self.shared_gate = keep(shared_gate, np.float32)
         self.rms_alpha = keep(rms_alpha, np.float32)
@@ -223,7 +227,8 @@ class Layer:
         self.c = _Layer(H, F, E, k, dtype, int(norm_topk), ptr(self.gate), ptr(self.gate_bias),
                         C.cast(self._a1, C.POINTER(C.c_void_p)), C.cast(self._a3, C.POINTER(C.c_void_p)),
                         C.cast(self._a2, C.POINTER(C.c_void_p)), Fs, ptr(self.sw[0]), ptr(self.sw[1]),
-                        ptr(self.sw[2]), ptr(self.shared_gate), ptr(self.rms_alpha), rms_eps)
+                        ptr(self.sw[2]), ptr(self.shared_gate), ptr(self.rms_alpha), rms_eps,
+                        0 if self.dtype_down == dtype else self.dtype_down)
 
     def forward(self, xs, logits=None, simd=False, threads=1, return_logits=False):
         xs = _f32(xs)

@@ -12,28 +12,30 @@ CONFIGS = {
 }
 
 
-def make_weights(H, F, E, dt, seed=0, Fs=0, std=0.02, threads=8):
-    """Expert weights N(0, std) quantised by the oracle's quantiser (stream order e, then w1, w3, w2)."""
+def make_weights(H, F, E, dt, seed=0, Fs=0, std=0.02, threads=8, dt_down=None):
+    """Expert weights N(0, std) quantised by the oracle's quantiser (stream order e, then w1, w3, w2).
+    dt_down: dtype of the w2 matrices when it differs from dt."""
+    dtd = dt if dt_down is None else dt_down
     w1, w3, w2 = [], [], []
     s = seed * 1000003
     for e in range(E):
         w1.append(O.fill_normal_quantized(s + 3 * e + 0, dt, F, H, std, threads))
         w3.append(O.fill_normal_quantized(s + 3 * e + 1, dt, F, H, std, threads))
-        w2.append(O.fill_normal_quantized(s + 3 * e + 2, dt, H, F, std, threads))
+        w2.append(O.fill_normal_quantized(s + 3 * e + 2, dtd, H, F, std, threads))
     shared = None
     if Fs:
         shared = (O.fill_normal_quantized(s + 3 * E + 0, dt, Fs, H, std, threads),
                   O.fill_normal_quantized(s + 3 * E + 1, dt, Fs, H, std, threads),
-                  O.fill_normal_quantized(s + 3 * E + 2, dt, H, Fs, std, threads))
+                  O.fill_normal_quantized(s + 3 * E + 2, dtd, H, Fs, std, threads))
     return w1, w3, w2, shared
 
 
-def make_pair(H, F, E, k, dt, seed=0, Fs=0, rms=False, norm_topk=True, gate_bias=None, want_gpu=True):
+def make_pair(H, F, E, k, dt, seed=0, Fs=0, rms=False, norm_topk=True, gate_bias=None, want_gpu=True, dt_down=None):
     """Returns (oracle Layer, HIP SparseMoeBlock or None) built from identical bytes."""
-    w1, w3, w2, shared = make_weights(H, F, E, dt, seed, Fs)
+    w1, w3, w2, shared = make_weights(H, F, E, dt, seed, Fs, dt_down=dt_down)
     gate = O.fill_normal(seed * 1000003 + 777, E * H, 0.0, 0.02).reshape(E, H)
     kw = dict(norm_topk=norm_topk, gate_bias=gate_bias)
-    okw, gkw = dict(kw), dict(kw)
+    okw, gkw = dict(kw, dtype_down=dt_down), dict(kw, ggml_dtype_down=dt_down)
     if Fs:
         sg = O.fill_normal(seed * 1000003 + 778, H, 0.0, 0.02)
         okw.update(Fs=Fs, sw1=shared[0], sw3=shared[1], sw2=shared[2], shared_gate=sg)

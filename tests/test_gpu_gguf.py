@@ -72,9 +72,35 @@ def test_loader_errors(tmp_path):
     W.moe_layer_file(p0, 0, gate, w1, w3, w2, O.Q4K, k, expert_keys=False)
     with pytest.raises(candle_amd.MoeError, match="expert_count is 0"):
         candle_amd.SparseMoeBlock.from_gguf(str(p0), 0)
-    # ffn_down stored with another dtype (what Q4_K_M files do with Q6K): refused, not silently converted
+    # ffn_down in a dtype with another activation format: refused, not silently converted
     pm = tmp_path / "mixed.gguf"
     w2_q8 = [np.zeros(H * F // 32 * 34, np.uint8) for _ in range(E)]
     W.moe_layer_file(pm, 0, gate, w1, w3, w2_q8, O.Q4K, k, down_dtype=O.Q8_0)
-    with pytest.raises(candle_amd.MoeError, match="differs from the layer's other expert matrices"):
+    with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):
         candle_amd.SparseMoeBlock.from_gguf(str(pm), 0)
+    # an unsupported dtype among the experts (Q5K = 13)
+    pu = tmp_path / "q5k.gguf"
+    w2_q5 = [np.zeros(H * F // 256 * 176, np.uint8) for _ in range(E)]
+    W.moe_layer_file(pu, 0, gate, w1, w3, w2_q5, O.Q4K, k, down_dtype=13)
+    with pytest.raises(candle_amd.MoeError, match="unsupported ggml_dtype 13"):
+        candle_amd.SparseMoeBlock.from_gguf(str(pu), 0)
+
+
+def test_q4_k_m_layer_with_q6k_down(tmp_path):
+    # what Q4_K_M files hold for part of their layers: Q4K ffn_gate / ffn_up, Q6K ffn_down
+    H, F, E, k = 512, 1024, 8, 2
+    w1, w3, w2, _ = make_weights(H, F, E, O.Q4K, 21, dt_down=O.Q6K)
+    gate = O.fill_normal(4242, E * H, 0.0, 0.02).reshape(E, H)
+    path = tmp_path / "q4_k_m.gguf"
+    W.moe_layer_file(path, 7, gate, w1, w3, w2, O.Q4K, k, down_dtype=O.Q6K)
+    loaded = candle_amd.SparseMoeBlock.from_gguf(str(path), 7)
+    assert (loaded.dtype, loaded.dtype_down) == (O.Q4K, O.Q6K)
+    direct = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, gate, w1, w3, w2, ggml_dtype_down=O.Q6K)
+    ref = O.Layer(H, F, E, k, O.Q4K, gate, w1, w3, w2, dtype_down=O.Q6K)
+    for T in (2, 40):
+        xs = activations(T, H, 50 + T)
+        ys = loaded.forward(xs)
+        assert np.array_equal(bits(ys), bits(direct.forward(xs)))
+        want = ref.forward(xs, logits=loaded.last_logits(T))
+        assert np.abs(ys - want).max() <= 2e-3 * np.sqrt(14336.0 / F) * np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    loaded.close(); direct.close()

@@ -26,7 +26,7 @@ def check(dt, got, want):
         assert np.abs(got - want).max() <= Q4K_TOL * rms(want)
 
 
-@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024)])
+@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q6K, 528, 768), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024)])
 def test_resident_projection_over_batch_sizes(dt, n, k):
     # one object, many calls: decode rows, mid batches, and (Q4K, n % 128 == 0) the tiled kernel
     # at 64- and 128-row tiles with ragged last tiles; shrinking and growing batches reuse the workspace
@@ -79,7 +79,7 @@ def test_argument_checks():
     with pytest.raises(candle_amd.MoeError, match="n % 16"):
         candle_amd.QMatMul(O.Q8_0, w[: 34 * 48], 24, 64)
     with pytest.raises(candle_amd.MoeError):
-        candle_amd.QMatMul(14, w, 32, 64)      # Q6K
+        candle_amd.QMatMul(13, w, 32, 64)      # Q5K
     lin = candle_amd.QMatMul(O.Q8_0, w, 32, 64)
     with pytest.raises(candle_amd.MoeError, match="expected"):
         lin.forward(np.zeros((3, 32), dtype=np.float32))
@@ -88,7 +88,8 @@ def test_argument_checks():
 def test_projection_from_gguf(tmp_path):
     # names of quantized_llama.rs:533-547
     H = 512
-    mats = {"blk.0.attn_q.weight": (O.Q4K, H, H), "blk.0.attn_k.weight": (O.Q8_0, 128, H), "output.weight": (O.Q4_0, 1024, H)}
+    mats = {"blk.0.attn_q.weight": (O.Q4K, H, H), "blk.0.attn_k.weight": (O.Q8_0, 128, H), "blk.0.attn_v.weight": (O.Q6K, 128, H),
+            "output.weight": (O.Q4_0, 1024, H)}
     blocks = {name: O.fill_normal_quantized(i + 3, dt, n, k, 0.02) for i, (name, (dt, n, k)) in enumerate(mats.items())}
     norm = O.fill_normal(9, H, 1.0, 0.1)
     ts = [(name, dt, (n, k), blocks[name].tobytes()) for name, (dt, n, k) in mats.items()]
@@ -104,6 +105,6 @@ def test_projection_from_gguf(tmp_path):
         with pytest.raises(candle_amd.MoeError, match="two dimensions"):
             candle_amd.QMatMul.from_gguf(g, "blk.0.attn_norm.weight")
         with pytest.raises(candle_amd.MoeError):
-            candle_amd.QMatMul.from_gguf(g, "blk.0.attn_v.weight")
+            candle_amd.QMatMul.from_gguf(g, "blk.0.attn_output.weight")
     lin = candle_amd.QMatMul.from_gguf(str(path), "output.weight")   # by path: the file is closed again
     check(O.Q4_0, lin.forward(x[:3]), O.matmul(O.Q4_0, x[:3], blocks["output.weight"], 1024))
