@@ -271,11 +271,18 @@ struct Q32Raw {
     u32x2g q;
     unsigned short d;
 };
-template <int DT>
+// ONCE: the weights are read by one pass only (non-temporal: they should not displace the activations
+// in the caches); otherwise further workgroups stream the same tiles again and should find them in L2
+template <int DT, bool ONCE>
 __device__ __forceinline__ Q32Raw load_q32_raw(const uint8_t* tile, uint32_t q_off, uint32_t d_off) {
     Q32Raw t;
-    t.q = ldg_stream<u32x2g>(tile, q_off);
-    t.d = ldg_stream<unsigned short>(tile, d_off);
+    if (ONCE) {
+        t.q = ldg_stream<u32x2g>(tile, q_off);
+        t.d = ldg_stream<unsigned short>(tile, d_off);
+    } else {
+        t.q = ldg<u32x2g>(tile, q_off);
+        t.d = ldg<unsigned short>(tile, d_off);
+    }
     return t;
 }
 template <int DT>
@@ -334,7 +341,7 @@ __device__ __forceinline__ void q32_mac_trip(const Q32Tile<DT>& w, const Q8_0Tri
 }
 
 // One wave: NT weight tile streams (tp[j], advancing TB bytes per block) against TT slot tiles, all of K.
-template <int DT, int TT, int NT, int STEP>
+template <int DT, int TT, int NT, int STEP, bool ONCE>
 __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const ActBuf& ab, int K, const int rowA[TT], const int rowD[TT][4],
                                            int lane, float acc[NT][TT][4]) {
     constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
@@ -346,7 +353,13 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT>(tp[t] + (size_t)j * TB, q_off, d_off);
+        for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off);
+    // With several slot tiles the activation operand is requested one step ahead too: the one of slot
+    // tile tt+1, or of the next trip's first slot tile, is on its way while this one is multiplied.
+    // (With one slot tile the extra registers cost a wave per SIMD, which costs more than the wait.)
+    constexpr bool AHEAD = TT > 1;
+    Q8_0Trip<STEP> An;
+    if (AHEAD) An = load_q8_0_trip<DT, STEP>(ab, K, nkb, 0, rowA[0], rowD[0], g);
     for (int kb0 = 0; kb0 < nkb; kb0 += STEP) {
         Q32Raw cur[NT][STEP];
 #pragma unroll
@@ -358,11 +371,19 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off);
+            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) {
-            const Q8_0Trip<STEP> A = load_q8_0_trip<DT, STEP>(ab, K, nkb, kb0, rowA[tt], rowD[tt], g);
+            Q8_0Trip<STEP> A;
+            if (AHEAD) {
+                A = An;
+                An = tt + 1 < TT ? load_q8_0_trip<DT, STEP>(ab, K, nkb, kb0, rowA[tt + 1 < TT ? tt + 1 : 0], rowD[tt + 1 < TT ? tt + 1 : 0], g)
+                                 : load_q8_0_trip<DT, STEP>(ab, K, nkb, kbn, rowA[0], rowD[0], g);
+                __builtin_amdgcn_sched_barrier(0);
+            } else {
+                A = load_q8_0_trip<DT, STEP>(ab, K, nkb, kb0, rowA[tt], rowD[tt], g);
+            }
 #pragma unroll
             for (int j = 0; j < STEP; j++)
 #pragma unroll
@@ -374,7 +395,7 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
 
 constexpr int Q32_STEP = 4;
 
-template <int DT, int TT>
+template <int DT, int TT, bool ONCE>
 __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
@@ -411,7 +432,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q32_engine<DT, TT, 4, Q32_STEP>(tp, p.xq, H, rowA, rowD, lane, acc);
+    q32_engine<DT, TT, 4, Q32_STEP, ONCE>(tp, p.xq, H, rowA, rowD, lane, acc);
 
     // epilogue: h = silu(w1 x) * (w3 x); the wave's 32 rows are exactly one Q8_0 block per slot
     const int nfb = F / 32;
@@ -444,7 +465,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
         }
 }
 
-template <int DT, int TT>
+template <int DT, int TT, bool ONCE>
 __global__ __launch_bounds__(Q32_THREADS) void q32_down_stream_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
@@ -477,7 +498,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_stream_kernel(ExpertPara
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[0][tt][i] = 0.f;
 
-    q32_engine<DT, TT, 1, 2 * Q32_STEP>(tp, p.hq, F, rowA, rowD, lane, acc);
+    q32_engine<DT, TT, 1, 2 * Q32_STEP, ONCE>(tp, p.hq, F, rowA, rowD, lane, acc);
 
 #pragma unroll
     for (int tt = 0; tt < TT; tt++)
@@ -500,10 +521,11 @@ static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
     const bool stream = !plain && (p.H / 32) % Q32_STEP == 0;
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 1, true>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 2, true>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
@@ -516,10 +538,11 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
     const bool stream = !plain && (p.F / 32) % (2 * Q32_STEP) == 0;
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 1, true>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, true>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
