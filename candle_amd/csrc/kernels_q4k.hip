@@ -1,4 +1,4 @@
-// Grouped expert products over Q4K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
+// Grouped expert products over Q4K, Q5K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
 //
 // Arithmetic restated from BlockQ4K::vec_dot, candle-core/src/quantized/k_quants.rs:1205-1285:
 // per 256-element super-block
@@ -90,10 +90,13 @@ __device__ inline Q8KOperand load_q8k_operand(const ActBuf& ab, int K, int nsb, 
 __device__ inline long pack64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
 
 // acc[i] += contribution of one (16 rows x 256 k) weight tile against one 16-slot operand.
-// yd[i] is the activation scale of output slot 4g+i.
-__device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
-    const uint32_t M4 = 0x0f0f0f0fu;
-    const uint32_t hdr = w.sc.x, u0 = w.sc.y, u1 = w.sc.z, u2 = w.sc.w;
+// yd[i] is the activation scale of output slot 4g+i.  FIFTH: the tile is Q5K, h0 / h1 hold the lane's
+// fifth bits (pairs 0,1 / 2,3; four bits per byte and pair), else Q4K.
+template <bool FIFTH>
+__device__ inline void q45k_mac(const uint4& q0, const uint4& q1, const uint4& sc, uint32_t h0, uint32_t h1, const Q8KOperand& A,
+                                const float yd[4], int g, float acc[4]) {
+    const uint32_t M4 = 0x0f0f0f0fu, M1 = 0x01010101u;
+    const uint32_t hdr = sc.x, u0 = sc.y, u1 = sc.z, u2 = sc.w;
     const float d = __half2float(__ushort_as_half((unsigned short)(hdr & 0xffffu)));
     const float dmin = __half2float(__ushort_as_half((unsigned short)(hdr >> 16)));
     // get_scale_min_k4 (utils.rs:50-60) for all eight sub-blocks at once
@@ -103,12 +106,20 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
     const uint32_t m47 = ((u2 >> 4) & M4) | (((u1 >> 6) & 0x03030303u) << 4);
     const v4i zero = {0, 0, 0, 0};
     v4i isum = {0, 0, 0, 0};
-    const uint32_t qw[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+    const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
 #pragma unroll
     for (int P = 0; P < 4; P++) {
         const uint32_t wx = qw[2 * P], wy = qw[2 * P + 1];
-        const long b_lo = pack64(wx & M4, wy & M4);
-        const long b_hi = pack64((wx >> 4) & M4, (wy >> 4) & M4);
+        uint32_t lx = wx & M4, ly = wy & M4, hx = (wx >> 4) & M4, hy = (wy >> 4) & M4;
+        if (FIFTH) {   // codes 0..31: nibble | fifth bit << 4
+            const uint32_t h = (P < 2 ? h0 : h1) >> (4 * (P & 1));
+            lx |= (h & M1) << 4;
+            ly |= ((h >> 1) & M1) << 4;
+            hx |= ((h >> 2) & M1) << 4;
+            hy |= ((h >> 3) & M1) << 4;
+        }
+        const long b_lo = pack64(lx, ly);
+        const long b_hi = pack64(hx, hy);
         const long a_lo = pack64(A.a[P].x, A.a[P].y);
         const long a_hi = pack64(A.a[P].z, A.a[P].w);
         v4i D0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, b_lo, zero, 0, 0, 0);
@@ -134,6 +145,29 @@ __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const floa
         acc[i] += dd * (float)isum[i];
         acc[i] -= dm * Dm[i];
     }
+}
+
+__device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+    q45k_mac<false>(w.q0, w.q1, w.sc, 0u, 0u, A, yd, g, acc);
+}
+
+// Q5K (BlockQ5K::vec_dot, k_quants.rs:1394-1485): the Q4K arithmetic on 5-bit codes
+struct Q5KTile {
+    uint4 q0, q1, sc;
+    uint2 qh;
+};
+__device__ inline Q5KTile load_q5k_tile(const uint8_t* tile, int lane) {
+    Q5KTile t;
+    t.q0 = gload_stream(tile, (uint32_t)lane * 16u);
+    t.q1 = gload_stream(tile, 1024u + (uint32_t)lane * 16u);
+    t.sc = gload_stream(tile, 2048u + (uint32_t)(lane & 15) * 16u);
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 h = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x2*>((gbytes)tile + 2304u + (uint32_t)lane * 8u));
+    t.qh = make_uint2(h.x, h.y);
+    return t;
+}
+__device__ inline void q5k_mac(const Q5KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+    q45k_mac<true>(w.q0, w.q1, w.sc, w.qh.x, w.qh.y, A, yd, g, acc);
 }
 
 struct Q6KTile {
@@ -197,6 +231,12 @@ struct FmtQ4K {
     static constexpr int TILE_BYTES = Q4K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q4k_tile(tile, lane); }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q4k_mac(w, A, yd, g, acc); }
+};
+struct FmtQ5K {
+    typedef Q5KTile Tile;
+    static constexpr int TILE_BYTES = Q5K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q5k_tile(tile, lane); }
+    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q5k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ6K {
     typedef Q6KTile Tile;
@@ -468,6 +508,13 @@ DEF_DOWN(q4k_down_t1_v1, FmtQ4K, 1, 4, 2, 3)
 DEF_DOWN_NARROW(q4k_down_t1_narrow, FmtQ4K, 8, 2, 4)
 DEF_DOWN(q4k_down_t2, FmtQ4K, 2, 4, 2, 2)
 DEF_DOWN(q4k_down_t4, FmtQ4K, 4, 8, 2, 2)
+// Q5K: the Q4K variants with two more registers per tile; one and two slot tiles per pass
+DEF_UP(q5k_up_t1, FmtQ5K, 1, 4, 2, 3)
+DEF_UP_NARROW(q5k_up_t1_narrow, FmtQ5K, 4, 2, 3)
+DEF_UP(q5k_up_t2, FmtQ5K, 2, 4, 2, 2)
+DEF_DOWN(q5k_down_t1, FmtQ5K, 1, 4, 2, 3)
+DEF_DOWN_NARROW(q5k_down_t1_narrow, FmtQ5K, 8, 2, 3)
+DEF_DOWN(q5k_down_t2, FmtQ5K, 2, 4, 2, 2)
 // Q6K: the same bodies; its tiles take five loads and seventeen registers, so every variant gets the
 // registers of a two-waves-per-SIMD launch, and four slot tiles per pass would spill: two at most
 DEF_UP(q6k_up_t1, FmtQ6K, 1, 4, 2, 2)
@@ -486,11 +533,12 @@ static int variant(const char* name, int dflt) {
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_UP_VARIANT", 1);
-    const bool q6k = p.dt == MOE_GGML_Q6K;
-    const int tt = p.slot_tiles >= 4 && !q6k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const bool q6k = p.dt == MOE_GGML_Q6K, q5k = p.dt == MOE_GGML_Q5K;
+    const int tt = p.slot_tiles >= 4 && !q6k && !q5k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (64 rows), f32 h to p.hbuf
         dim3 ngrid((unsigned)(p.F / 64), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
         if (q6k) hipLaunchKernelGGL(q6k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
+        else if (q5k) hipLaunchKernelGGL(q5k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(q4k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
@@ -498,6 +546,11 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (q6k) {
         if (tt == 2) hipLaunchKernelGGL(q6k_up_t2, grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(q6k_up_t1, grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
+    if (q5k) {
+        if (tt == 2) hipLaunchKernelGGL(q5k_up_t2, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q5k_up_t1, grid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
     if (tt == 4) hipLaunchKernelGGL(q4k_up_t4, grid, dim3(512), 0, s, p);
@@ -510,11 +563,13 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     static const int v = variant("MOE_DOWN_VARIANT", 1);
-    const bool q6k = (p.dt_down ? p.dt_down : p.dt) == MOE_GGML_Q6K;
-    const int tt = p.slot_tiles >= 4 && !q6k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const int dtd = p.dt_down ? p.dt_down : p.dt;
+    const bool q6k = dtd == MOE_GGML_Q6K, q5k = dtd == MOE_GGML_Q5K;
+    const int tt = p.slot_tiles >= 4 && !q6k && !q5k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (32 rows), eight waves split K
         dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
         if (q6k) hipLaunchKernelGGL(q6k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
+        else if (q5k) hipLaunchKernelGGL(q5k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
         else hipLaunchKernelGGL(q4k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
         return hipGetLastError();
     }
@@ -522,6 +577,11 @@ hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (q6k) {
         if (tt == 2) hipLaunchKernelGGL(q6k_down_t2, grid, dim3(256), 0, s, p);
         else hipLaunchKernelGGL(q6k_down_t1, grid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
+    if (q5k) {
+        if (tt == 2) hipLaunchKernelGGL(q5k_down_t2, grid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(q5k_down_t1, grid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
     if (tt == 4) hipLaunchKernelGGL(q4k_down_t4, grid, dim3(512), 0, s, p);

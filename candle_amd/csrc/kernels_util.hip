@@ -2,7 +2,7 @@
 // from either layout, and the stand-alone activation quantiser used by the parity hooks.
 //
 // to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0),
-// 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
+// 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1563-1595 (Q5K), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
 #include <algorithm>
 #include "act_quant.hpp"
@@ -34,6 +34,19 @@ __device__ inline float q4k_value(const uint8_t* hdr, int i, uint8_t qbyte) {
     return d1 * (float)q - m1;
 }
 
+// value of element `i` of a Q5K block: header as Q4K, nibble byte, fifth bit (k_quants.rs:1582-1591:
+// `d1 * (nibble as f32 + to_add) - m1`)
+__device__ inline float q5k_value(const uint8_t* hdr, int i, uint8_t qbyte, int hbit) {
+    float d = f16_bits_to_f32((uint16_t)(hdr[0] | (hdr[1] << 8)));
+    float mn = f16_bits_to_f32((uint16_t)(hdr[2] | (hdr[3] << 8)));
+    int sc, m;
+    scale_min_k4(i / 32, hdr + 4, &sc, &m);
+    float d1 = d * (float)sc;
+    float m1 = mn * (float)m;
+    int q = ((i / 32) & 1) ? (qbyte >> 4) : (qbyte & 0xF);
+    return d1 * ((float)q + (hbit ? 16.f : 0.f)) - m1;
+}
+
 // code (0..63) of element e (0..255) of a raw BlockQ6K: the bit fields of k_quants.rs:1772-1778
 __device__ inline int q6k_code(const uint8_t* blk, int e) {
     const int half = e / 128, q = (e % 128) / 32, l = e % 32;
@@ -53,6 +66,10 @@ __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, in
         const uint8_t* b = blocks + (i / 256) * 144;
         int e = (int)(i % 256);
         out[i] = q4k_value(b, e, b[16 + (e / 64) * 32 + (e % 32)]);
+    } else if (dt == MOE_GGML_Q5K) {
+        const uint8_t* b = blocks + (i / 256) * 176;
+        int e = (int)(i % 256);
+        out[i] = q5k_value(b, e, b[48 + (e / 64) * 32 + (e % 32)], (b[16 + e % 32] >> (e / 32)) & 1);
     } else if (dt == MOE_GGML_Q6K) {
         const uint8_t* b = blocks + (i / 256) * 210;
         int e = (int)(i % 256);
@@ -98,6 +115,35 @@ __global__ void relayout_q4k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t 
         const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
         for (int i = 0; i < 16; i++) dst[i] = blk[i];
     }
+}
+
+__global__ void relayout_q5k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
+    // one thread per (tile, lane): 32 nibble bytes and 8 bytes of fifth bits; lanes < 16 also move the header
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nsb * 64) return;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int64_t rt = tile / nsb;
+    int sb = (int)(tile % nsb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 176;
+    const uint8_t* qh = blk + 16;
+    const uint8_t* qs = blk + 48;
+    uint8_t* dst = tiled + (sb * n_rt + rt) * Q5K_TILE_BYTES;  // tiles ordered [sb][rt]
+    for (int P = 0; P < 4; P++)
+        for (int i = 0; i < 8; i++) dst[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + i] = qs[32 * P + 8 * g + i];
+    auto hb = [&](int j, int t) { return (qh[t] >> j) & 1; };   // fifth bit of element t of sub-block j
+    for (int w = 0; w < 2; w++)
+        for (int i = 0; i < 4; i++) {
+            int byte = 0;
+            for (int q = 0; q < 2; q++) {
+                const int P = 2 * w + q;
+                const int bits = hb(2 * P, 8 * g + i) | (hb(2 * P, 8 * g + 4 + i) << 1) | (hb(2 * P + 1, 8 * g + i) << 2) | (hb(2 * P + 1, 8 * g + 4 + i) << 3);
+                byte |= bits << (4 * q);
+            }
+            dst[2304 + l * 8 + w * 4 + i] = (uint8_t)byte;
+        }
+    if (g == 0)
+        for (int j = 0; j < 16; j++) dst[2048 + r * 16 + j] = blk[j];
 }
 
 __global__ void relayout_q6k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
@@ -175,6 +221,14 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         int l = g * 16 + r;
         uint8_t q = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
         out[i] = q4k_value(tile + 2048 + r * 16, e, q);
+    } else if (dt == MOE_GGML_Q5K) {
+        int sb = col / 256, e = col % 256;
+        const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q5K_TILE_BYTES;
+        int P = e / 64, sub = (e % 64) / 32, g = (e % 32) / 8, pos = e % 8;
+        int l = g * 16 + r;
+        uint8_t q = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
+        uint8_t hbyte = tile[2304 + l * 8 + (P / 2) * 4 + pos % 4];
+        out[i] = q5k_value(tile + 2048 + r * 16, e, q, (hbyte >> ((P % 2) * 4 + sub * 2 + pos / 4)) & 1);
     } else if (dt == MOE_GGML_Q6K) {
         int sb = col / 256, e = col % 256;
         const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q6K_TILE_BYTES;
@@ -260,6 +314,8 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
     if (n_rt == 0 || nkb == 0) return hipSuccess;
     if (dt == MOE_GGML_Q4K)
         hipLaunchKernelGGL(relayout_q4k_kernel, dim3(nblk(n_rt * nkb * 144, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (dt == MOE_GGML_Q5K)
+        hipLaunchKernelGGL(relayout_q5k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q6K)
         hipLaunchKernelGGL(relayout_q6k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q8_0)

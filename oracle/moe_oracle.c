@@ -97,7 +97,7 @@ static inline float rmin(float a, float b) { return fminf(a, b); }
 int64_t orc_block_elems(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return 32;
-        case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return 256;
+        case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
         default: return -1;
     }
 }
@@ -106,6 +106,7 @@ int64_t orc_block_bytes(int dtype) {
         case ORC_Q4_0: return 18;
         case ORC_Q8_0: return 34;
         case ORC_Q4K: return 144;
+        case ORC_Q5K: return 176;
         case ORC_Q6K: return 210;
         case ORC_Q8K: return 292;
         default: return -1;
@@ -114,7 +115,7 @@ int64_t orc_block_bytes(int dtype) {
 int orc_vecdot_dtype(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
-        case ORC_Q4K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
+        case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
         default: return -1;
     }
 }
@@ -342,6 +343,139 @@ static float vec_dot_q4k_q8k(int64_t n, const orc_block_q4k* xs, const orc_block
             for (int l = 0; l < 32; l++) a[l] = (int8_t)(q4[l] >> 4);
             a += 32;
             q4 += 32;
+        }
+        uint8_t scales[8], mins[8];
+        for (int j = 0; j < 8; j++) get_scale_min_k4(j, x->scales, &scales[j], &mins[j]);
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) sumi += (int32_t)y->bsums[j] * (int32_t)mins[j / 2];
+        a = aux8;
+        const int8_t* q8 = y->qs;
+        for (int s = 0; s < 8; s++) {
+            int32_t scale = scales[s];
+            for (int r = 0; r < 4; r++) {
+                for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+                for (int l = 0; l < 8; l++) aux32[l] += scale * (int32_t)aux16[l];
+                q8 += 8;
+                a += 8;
+            }
+        }
+        float d = orc_f16_to_f32(x->d) * y->d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+        float dmin = orc_f16_to_f32(x->dmin) * y->d;
+        sumf -= dmin * (float)sumi;
+    }
+    float tail = 0.f;
+    for (int l = 0; l < 8; l++) tail += sums[l];
+    return sumf + tail;
+}
+
+/* ------------------------------------------------------------------ Q5K */
+/* k_quants.rs:1487-1561 */
+static void quantize_q5k(const float* xs, int64_t k, orc_block_q5k* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float* x = xs + b * 256;
+        orc_block_q5k* block = &ys[b];
+        float mins[8], scales[8];
+        for (int j = 0; j < 8; j++) make_qkx1_quants(31, 5, x + 32 * j, 32, &scales[j], &mins[j]);
+        float max_scale = 0.f, max_min = 0.f;
+        for (int j = 0; j < 8; j++) { max_scale = rmax(scales[j], max_scale); max_min = rmax(mins[j], max_min); }
+        float inv_scale = max_scale > 0.f ? 63.0f / max_scale : 0.f;
+        float inv_min = max_min > 0.f ? 63.0f / max_min : 0.f;
+        for (int j = 0; j < 8; j++) {
+            int32_t lsi = nearest_int(inv_scale * scales[j]); if (lsi > 63) lsi = 63;
+            int32_t lmi = nearest_int(inv_min * mins[j]);     if (lmi > 63) lmi = 63;
+            uint8_t ls = (uint8_t)lsi, lm = (uint8_t)lmi;
+            if (j < 4) {
+                block->scales[j] = ls;
+                block->scales[j + 4] = lm;
+            } else {
+                block->scales[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+                block->scales[j - 4] |= (uint8_t)((ls >> 4) << 6);
+                block->scales[j] |= (uint8_t)((lm >> 4) << 6);
+            }
+        }
+        block->d = orc_f32_to_f16(max_scale / 63.0f);
+        block->dmin = orc_f32_to_f16(max_min / 63.0f);
+        uint8_t l[256];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 8; j++) {
+            uint8_t sc, m;
+            get_scale_min_k4(j, block->scales, &sc, &m);
+            float d = orc_f16_to_f32(block->d) * (float)sc;
+            if (d == 0.f) continue;
+            float dm = orc_f16_to_f32(block->dmin) * (float)m;
+            for (int ii = 0; ii < 32; ii++) {
+                int32_t lv = nearest_int((x[32 * j + ii] + dm) / d);
+                l[32 * j + ii] = (uint8_t)(lv < 0 ? 0 : lv > 31 ? 31 : lv);
+            }
+        }
+        memset(block->qh, 0, sizeof block->qh);
+        uint8_t m1 = 1, m2 = 2;
+        for (int n = 0; n < 256; n += 64) {
+            int offset = (n / 64) * 32;
+            for (int j = 0; j < 32; j++) {
+                uint8_t l1 = l[n + j], l2 = l[n + j + 32];
+                if (l1 > 15) { l1 -= 16; block->qh[j] |= m1; }
+                if (l2 > 15) { l2 -= 16; block->qh[j] |= m2; }
+                block->qs[offset + j] = (uint8_t)(l1 | (l2 << 4));
+            }
+            m1 <<= 2;
+            m2 <<= 2;
+        }
+    }
+}
+/* k_quants.rs:1563-1595 */
+static void dequantize_q5k(const orc_block_q5k* xs, int64_t k, float* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const orc_block_q5k* block = &xs[b];
+        float* y = ys + b * 256;
+        float d = orc_f16_to_f32(block->d);
+        float min = orc_f16_to_f32(block->dmin);
+        int is = 0, yi = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 256; j += 64) {
+            const uint8_t* ql = block->qs + j / 2;
+            uint8_t sc, m;
+            get_scale_min_k4(is, block->scales, &sc, &m);
+            float d1 = d * (float)sc, m1 = min * (float)m;
+            get_scale_min_k4(is + 1, block->scales, &sc, &m);
+            float d2 = d * (float)sc, m2 = min * (float)m;
+            for (int t = 0; t < 32; t++) {
+                float to_add = (block->qh[t] & u1) ? 16.f : 0.f;
+                y[yi++] = d1 * ((float)(ql[t] & 0xF) + to_add) - m1;
+            }
+            for (int t = 0; t < 32; t++) {
+                float to_add = (block->qh[t] & u2) ? 16.f : 0.f;
+                y[yi++] = d2 * ((float)(ql[t] >> 4) + to_add) - m2;
+            }
+            is += 2;
+            u1 <<= 2;
+            u2 <<= 2;
+        }
+    }
+}
+/* k_quants.rs:1394-1485 (vec_dot_unopt) */
+static float vec_dot_q5k_q8k(int64_t n, const orc_block_q5k* xs, const orc_block_q8k* ys) {
+    int8_t aux8[256];
+    int16_t aux16[8];
+    float sums[8] = {0};
+    int32_t aux32[8];
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q5k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        memset(aux32, 0, sizeof aux32);
+        int8_t* a = aux8;
+        const uint8_t* q5 = x->qs;
+        uint8_t m = 1;
+        for (int j = 0; j < 4; j++) {
+            for (int l = 0; l < 32; l++) a[l] = (int8_t)((q5[l] & 0xF) + ((x->qh[l] & m) ? 16 : 0));
+            a += 32;
+            m <<= 1;
+            for (int l = 0; l < 32; l++) a[l] = (int8_t)((q5[l] >> 4) + ((x->qh[l] & m) ? 16 : 0));
+            a += 32;
+            m <<= 1;
+            q5 += 32;
         }
         uint8_t scales[8], mins[8];
         for (int j = 0; j < 8; j++) get_scale_min_k4(j, x->scales, &scales[j], &mins[j]);
@@ -643,6 +777,7 @@ int orc_quantize(int dtype, const float* x, int64_t n, void* blocks) {
         case ORC_Q4_0: quantize_q4_0(x, n, (orc_block_q4_0*)blocks); return 0;
         case ORC_Q8_0: quantize_q8_0(x, n, (orc_block_q8_0*)blocks); return 0;
         case ORC_Q4K: memset(blocks, 0, (size_t)(n / 256) * 144); quantize_q4k(x, n, (orc_block_q4k*)blocks); return 0;
+        case ORC_Q5K: memset(blocks, 0, (size_t)(n / 256) * 176); quantize_q5k(x, n, (orc_block_q5k*)blocks); return 0;
         case ORC_Q6K: memset(blocks, 0, (size_t)(n / 256) * 210); quantize_q6k(x, n, (orc_block_q6k*)blocks); return 0;
         case ORC_Q8K: quantize_q8k(x, n, (orc_block_q8k*)blocks); return 0;
     }
@@ -655,6 +790,7 @@ int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y) {
         case ORC_Q4_0: dequantize_q4_0((const orc_block_q4_0*)blocks, n, y); return 0;
         case ORC_Q8_0: dequantize_q8_0((const orc_block_q8_0*)blocks, n, y); return 0;
         case ORC_Q4K: dequantize_q4k((const orc_block_q4k*)blocks, n, y); return 0;
+        case ORC_Q5K: dequantize_q5k((const orc_block_q5k*)blocks, n, y); return 0;
         case ORC_Q6K: dequantize_q6k((const orc_block_q6k*)blocks, n, y); return 0;
         case ORC_Q8K: dequantize_q8k((const orc_block_q8k*)blocks, n, y); return 0;
     }
@@ -665,6 +801,7 @@ float orc_vec_dot(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q4_0: return vec_dot_q4_0_q8_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return vec_dot_q8_0_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return vec_dot_q4k_q8k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q5K: return vec_dot_q5k_q8k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return vec_dot_q6k_q8k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         case ORC_Q8K: return vec_dot_q8k_q8k(n, (const orc_block_q8k*)w, (const orc_block_q8k*)a);
     }

@@ -6,6 +6,7 @@
  *   vec_dot_q4_0_q8_0  candle-core/src/quantized/avx.rs:50-68
  *   vec_dot_q8_0_q8_0  candle-core/src/quantized/avx.rs:71-87
  *   vec_dot_q4k_q8k    candle-core/src/quantized/avx.rs:443-525
+ *   vec_dot_q5k_q8k    candle-core/src/quantized/avx.rs:527-638
  *   vec_dot_q6k_q8k    candle-core/src/quantized/avx.rs:131-216
  * The integer parts are exact; the f32 accumulation order differs from the scalar
  * vec_dot_unopt, which the reference's own tests allow up to 1e-6 * k
@@ -110,6 +111,58 @@ static float dot_q4k(int64_t n, const orc_block_q4k* xs, const orc_block_q8k* ys
     return hsum_float_8(acc) + _mm_cvtss_f32(acc_m);
 }
 
+static float dot_q5k(int64_t n, const orc_block_q5k* xs, const orc_block_q8k* ys) {
+    const uint32_t KMASK1 = 0x3f3f3f3f, KMASK2 = 0x0f0f0f0f, KMASK3 = 0x03030303;
+    const __m256i m4 = _mm256_set1_epi8(0xF);
+    __m256 acc = _mm256_setzero_ps();
+    float summs = 0.f;
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q5k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        float d = y->d * orc_f16_to_f32(x->d);
+        float dmin = -y->d * orc_f16_to_f32(x->dmin);
+        uint32_t utmp[4];
+        memcpy(utmp, x->scales, 12);
+        utmp[3] = ((utmp[2] >> 4) & KMASK2) | (((utmp[1] >> 6) & KMASK3) << 4);
+        uint32_t uaux = utmp[1] & KMASK1;
+        utmp[1] = (utmp[2] & KMASK2) | (((utmp[0] >> 6) & KMASK3) << 4);
+        utmp[2] = uaux;
+        utmp[0] &= KMASK1;
+        const uint8_t* q5 = x->qs;
+        const int8_t* q8 = y->qs;
+        __m256i mins_and_scales = _mm256_cvtepu8_epi16(
+            _mm_set_epi32((int)utmp[3], (int)utmp[2], (int)utmp[1], (int)utmp[0]));
+        __m256i q8sums = _mm256_loadu_si256((const __m256i*)y->bsums);
+        __m128i q8s = _mm_hadd_epi16(_mm256_extracti128_si256(q8sums, 0), _mm256_extracti128_si256(q8sums, 1));
+        __m128i prod = _mm_madd_epi16(_mm256_extracti128_si256(mins_and_scales, 1), q8s);
+        __m128i hsum = _mm_hadd_epi32(_mm_hadd_epi32(prod, _mm_setzero_si128()), _mm_setzero_si128());
+        summs += dmin * (float)_mm_extract_epi32(hsum, 0);
+        __m128i sc128 = _mm256_extracti128_si256(mins_and_scales, 0);
+        __m256i scales = _mm256_set_m128i(sc128, sc128);
+        __m256i hbits = _mm256_loadu_si256((const __m256i*)x->qh);
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < 4; j++) {
+            __m256i scale_0 = _mm256_shuffle_epi8(scales, _mm256_set1_epi16((short)(((4 * j + 1) << 8) | (4 * j))));
+            __m256i scale_1 = _mm256_shuffle_epi8(scales, _mm256_set1_epi16((short)(((4 * j + 3) << 8) | (4 * j + 2))));
+            __m256i q5bits = _mm256_loadu_si256((const __m256i*)q5);
+            q5 += 32;
+            /* high bit 2j of every byte -> bit 4 (the reference hard-codes the same shifts per j) */
+            __m256i h0 = _mm256_and_si256(_mm256_srl_epi16(hbits, _mm_cvtsi32_si128(2 * j)), _mm256_set1_epi8(1));
+            __m256i h1 = _mm256_and_si256(_mm256_srl_epi16(hbits, _mm_cvtsi32_si128(2 * j + 1)), _mm256_set1_epi8(1));
+            __m256i q5_0 = _mm256_add_epi8(_mm256_and_si256(q5bits, m4), _mm256_slli_epi16(h0, 4));
+            __m256i q5_1 = _mm256_add_epi8(_mm256_and_si256(_mm256_srli_epi16(q5bits, 4), m4), _mm256_slli_epi16(h1, 4));
+            __m256i q8_0 = _mm256_loadu_si256((const __m256i*)q8);
+            q8 += 32;
+            __m256i q8_1 = _mm256_loadu_si256((const __m256i*)q8);
+            q8 += 32;
+            __m256i p16_0 = _mm256_madd_epi16(scale_0, _mm256_maddubs_epi16(q5_0, q8_0));
+            __m256i p16_1 = _mm256_madd_epi16(scale_1, _mm256_maddubs_epi16(q5_1, q8_1));
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(p16_0, p16_1));
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum_float_8(acc) + summs;
+}
 static float dot_q6k(int64_t n, const orc_block_q6k* xs, const orc_block_q8k* ys) {
     const __m256i m4 = _mm256_set1_epi8(0xF), m2 = _mm256_set1_epi8(3), m32s = _mm256_set1_epi8(32);
     __m256 acc = _mm256_setzero_ps();
@@ -164,6 +217,7 @@ float orc_vec_dot_avx2(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q4_0: return dot_q4_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return dot_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return dot_q4k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q5K: return dot_q5k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return dot_q6k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         default: return orc_vec_dot(dtype, n, w, a);
     }

@@ -64,7 +64,7 @@ def test_q4_0_matmul_known_answers(O, golden, simd):
     assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_neg_3_64_4"]["expected_rounded"]
 
 
-@pytest.mark.parametrize("name,dt", [("q4k_ramp", 12), ("q6k_ramp", 14), ("q8k_ramp", 15)])
+@pytest.mark.parametrize("name,dt", [("q4k_ramp", 12), ("q5k_ramp", 13), ("q6k_ramp", 14), ("q8k_ramp", 15)])
 def test_kquant_ramp_spot_values(O, golden, name, dt):
     g = golden[name]
     idx = golden["ramp_spot_indices"]
@@ -80,7 +80,7 @@ def test_kquant_ramp_spot_values(O, golden, name, dt):
         assert np.abs(dbig - big).max() < g["max_abs_err_bound_128"]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 12, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 12, 13, 14, 15])
 def test_ggml_quantization_rmse(O, golden, dt):
     src = ggml_like(0.0)
     dst = O.dequantize(dt, O.quantize(dt, src), src.size)
@@ -88,7 +88,7 @@ def test_ggml_quantization_rmse(O, golden, dt):
     assert rmse <= golden["ggml_quantization_rmse_bound"]["bound"]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 12, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 12, 13, 14, 15])
 def test_ggml_dot_error(O, golden, dt):
     # ggml_matmul_error_test, quantized_tests.rs:846-911
     g = golden["ggml_dot_error"]
@@ -114,7 +114,7 @@ def test_vec_dot_matches_dequantised_float64(O):
     # brute force: the integer block dot must equal the float dot of the dequantised operands
     rng = np.random.default_rng(3)
     n = 2048
-    for dt in (O.Q4_0, O.Q8_0, O.Q4K, O.Q6K):
+    for dt in (O.Q4_0, O.Q8_0, O.Q4K, O.Q5K, O.Q6K):
         w = rng.normal(0, 0.02, n).astype(np.float32)
         x = rng.normal(0, 1.0, n).astype(np.float32)
         wq, xq = O.quantize(dt, w), O.quantize(O.VECDOT[dt], x)
@@ -137,7 +137,7 @@ def test_seeded_matmul_spot_values(O, golden, simd):
     r3 = lambda a: [float(np.round(np.float32(1000.0) * np.float32(x)) / np.float32(1000.0)) for x in a]
     dense = (lhs.astype(np.float64) @ rhs.astype(np.float64).T).reshape(-1)
     assert r3(dense[pick]) == r3(g["dense"])  # validates the StdRng restatement itself
-    for key, dt in (("q4k", O.Q4K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
+    for key, dt in (("q4k", O.Q4K), ("q5k", O.Q5K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
         mm = O.matmul(dt, lhs, O.quantize(dt, rhs), n, simd=simd).reshape(-1)
         assert r3(mm[pick]) == r3(g[key])
 
@@ -271,3 +271,36 @@ def test_q6k_quantizer_closed_forms(O):
     z = O.quantize(O.Q6K, np.zeros(256, np.float32))
     assert z[208:210].view(np.uint16)[0] == 0x8000 and not z[:208].any()
     assert not O.dequantize(O.Q6K, z, 256).any()
+
+
+def test_q5k_layout_against_independent_decoder(O):
+    # independent numpy decoder of the published Q5_K layout, addressed by element: d, dmin, the 12 packed
+    # scale / min bytes of Q4_K, 32 bytes of high bits, 128 nibble bytes.  Element e lies in pair e//64,
+    # half (e%64)//32, column l = e%32: nibble byte qs[32*pair + l] (high nibble for the second half), fifth
+    # bit = bit 2*pair + half of qh[l].
+    rng = np.random.default_rng(12)
+    x = rng.normal(0, 0.02, 1024).astype(np.float32)
+    blocks = O.quantize(O.Q5K, x).reshape(4, 176)
+    out = np.empty((4, 256), dtype=np.float32)
+    codes = np.empty((4, 256), dtype=np.int32)
+    for b in range(4):
+        raw = blocks[b]
+        d = np.float32(raw[0:2].view(np.float16)[0])
+        dmin = np.float32(raw[2:4].view(np.float16)[0])
+        s = raw[4:16].astype(np.int32)
+        qh, qs = raw[16:48].astype(np.int32), raw[48:176].astype(np.int32)
+        for e in range(256):
+            pair, half, l = e // 64, (e % 64) // 32, e % 32
+            j = 2 * pair + half
+            if j < 4:
+                sc, mn = s[j] & 63, s[j + 4] & 63
+            else:
+                sc, mn = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4), (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+            byte = qs[32 * pair + l]
+            code = ((byte >> 4) if half else (byte & 15)) + 16 * ((qh[l] >> j) & 1)
+            codes[b, e] = code
+            out[b, e] = (d * np.float32(sc)) * np.float32(code) - dmin * np.float32(mn)
+    got = O.dequantize(O.Q5K, blocks.reshape(-1), 1024)
+    assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
+    assert codes.min() == 0 and codes.max() == 31
+    assert np.abs(got - x).max() < 0.02 * 8 / 31
