@@ -293,6 +293,16 @@ extern "C" void moe_layer_destroy(moe_layer* L) {
 // Stage marks for moe_layer_forward_timed: events recorded between the launches.
 enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_REQUANT, ST_DOWN, ST_SHARED, ST_COMBINE, ST_COUNT };
 
+// The expert kernels address quantised activation rows with 32-bit byte offsets (rows * K): a call carries
+// at most this many tokens; longer inputs are cut into chunks (tokens are independent of each other).
+static int64_t max_tokens_per_pass(const moe_layer* L) {
+    const int64_t widest = std::max(std::max(L->H, L->F), L->Fs);
+    int64_t limit = std::max<int64_t>(1, (((int64_t)1 << 31) - 1) / (L->k * widest));
+    if (const char* e = getenv("MOE_MAX_TOKENS_PER_PASS"))   // testing aid: force several passes on small inputs
+        if (atoll(e) > 0) limit = std::min<int64_t>(limit, atoll(e));
+    return limit;
+}
+
 static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
 #define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
     int rc = reserve_workspace(L, T);
@@ -317,7 +327,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
     // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
     const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k > 24 * L->E && T * L->k * std::max(L->H, L->F) < (int64_t)1 << 32;
+                       T * L->k > 24 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     const bool direct = !tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     fp.rb.direct = direct ? 1 : 0;
@@ -403,13 +413,21 @@ extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T
     if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
     std::lock_guard<std::mutex> lk(L->mu);
     if (T == 0) { L->last_T = 0; return MOE_OK; }
-    return enqueue_forward(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream));
+    const int64_t step = max_tokens_per_pass(L);
+    for (int64_t t0 = 0; t0 < T; t0 += step) {
+        const int rc = enqueue_forward(L, static_cast<const float*>(d_x) + t0 * L->H, std::min(step, T - t0),
+                                       static_cast<float*>(d_y) + t0 * L->H, static_cast<hipStream_t>(hip_stream));
+        if (rc) return rc;
+    }
+    if (T > step) L->last_T = -1;   // the routing hooks describe one pass only
+    return MOE_OK;
 }
 
 extern "C" int moe_layer_forward_timed(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream, float* stage_ms) {
     if (!L || T <= 0 || !d_x || !d_y || !stage_ms || d_x == d_y) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_timed");
     if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
     std::lock_guard<std::mutex> lk(L->mu);
+    if (T > max_tokens_per_pass(L)) return fail(MOE_E_INVALID, "moe_layer_forward_timed: more tokens than one pass carries (" + std::to_string(max_tokens_per_pass(L)) + ")");
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     hipEvent_t marks[ST_COUNT] = {};
     int rc = MOE_OK;
@@ -434,7 +452,10 @@ extern "C" int moe_layer_forward(moe_layer* L, const float* x, int64_t T, float*
     if ((rc = L->x_dev.reserve(bytes))) return rc;
     if ((rc = L->y_dev.reserve(bytes))) return rc;
     MOE_HIP_CHECK(hipMemcpyAsync(L->x_dev.p, x, bytes, hipMemcpyHostToDevice, L->stream));
-    if ((rc = enqueue_forward(L, L->x_dev.as<float>(), T, L->y_dev.as<float>(), L->stream))) return rc;
+    const int64_t step = max_tokens_per_pass(L);
+    for (int64_t t0 = 0; t0 < T; t0 += step)
+        if ((rc = enqueue_forward(L, L->x_dev.as<float>() + t0 * L->H, std::min(step, T - t0), L->y_dev.as<float>() + t0 * L->H, L->stream))) return rc;
+    if (T > step) L->last_T = -1;   // the routing hooks describe one pass only
     MOE_HIP_CHECK(hipMemcpyAsync(y, L->y_dev.p, bytes, hipMemcpyDeviceToHost, L->stream));
     MOE_HIP_CHECK(hipStreamSynchronize(L->stream));
     return MOE_OK;
@@ -620,7 +641,7 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     const int64_t row_blocks = Q->n / 128;
     const int tile_slots = row_blocks * ((m + 127) / 128) >= 512 ? 128 : 64;
     const bool tiled = !no_gemm && Q->dt == MOE_GGML_Q4K && Q->n % 128 == 0 && m >= 96 &&
-                       row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192 && m * Q->k < (int64_t)1 << 32;
+                       row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192;
     RouteBufs rb = Q->route.view();
     rb.T = (int)m; rb.k = 1;
     rb.tile_slots = tile_slots;
@@ -637,6 +658,9 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     return MOE_OK;
 }
 
+// 32-bit byte offsets into the quantised rows (rows * k): longer inputs go through in several passes
+static int64_t qlinear_rows_per_pass(const moe_qlinear* Q) { return std::max<int64_t>(1, (((int64_t)1 << 31) - 1) / Q->k); }
+
 static int check_qlinear_call(moe_qlinear* Q, const void* x, int64_t m, const void* y, const char* who) {
     if (!Q || m < 0 || (m > 0 && (!x || !y))) return fail(MOE_E_INVALID, std::string("bad argument to ") + who);
     if (m > (1 << 20)) return fail(MOE_E_INVALID, std::string(who) + ": more than 2^20 rows is not supported");
@@ -648,7 +672,12 @@ extern "C" int moe_qlinear_forward_device(moe_qlinear* Q, const void* d_x, int64
     if (rc || m == 0) return rc;
     if (d_x == d_y) return fail(MOE_E_INVALID, "d_x and d_y must not alias");
     std::lock_guard<std::mutex> lk(Q->mu);
-    return enqueue_qlinear(Q, static_cast<const float*>(d_x), m, static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream));
+    const int64_t step = qlinear_rows_per_pass(Q);
+    for (int64_t r0 = 0; r0 < m; r0 += step)
+        if ((rc = enqueue_qlinear(Q, static_cast<const float*>(d_x) + r0 * Q->k, std::min(step, m - r0), static_cast<float*>(d_y) + r0 * Q->n,
+                                  static_cast<hipStream_t>(hip_stream))))
+            return rc;
+    return MOE_OK;
 }
 
 extern "C" int moe_qlinear_forward(moe_qlinear* Q, const float* x, int64_t m, float* y) {
@@ -659,7 +688,9 @@ extern "C" int moe_qlinear_forward(moe_qlinear* Q, const float* x, int64_t m, fl
     if ((rc = Q->x_dev.reserve(xb))) return rc;
     if ((rc = Q->y_dev.reserve(yb))) return rc;
     MOE_HIP_CHECK(hipMemcpyAsync(Q->x_dev.p, x, xb, hipMemcpyHostToDevice, Q->stream));
-    if ((rc = enqueue_qlinear(Q, Q->x_dev.as<float>(), m, Q->y_dev.as<float>(), Q->stream))) return rc;
+    const int64_t step = qlinear_rows_per_pass(Q);
+    for (int64_t r0 = 0; r0 < m; r0 += step)
+        if ((rc = enqueue_qlinear(Q, Q->x_dev.as<float>() + r0 * Q->k, std::min(step, m - r0), Q->y_dev.as<float>() + r0 * Q->n, Q->stream))) return rc;
     MOE_HIP_CHECK(hipMemcpyAsync(y, Q->y_dev.p, yb, hipMemcpyDeviceToHost, Q->stream));
     MOE_HIP_CHECK(hipStreamSynchronize(Q->stream));
     return MOE_OK;

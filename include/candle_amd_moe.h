@@ -90,6 +90,9 @@ void moe_layer_destroy(moe_layer* layer);
  * x and y are HOST f32 [n_tokens, hidden]; synchronous. */
 int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float* y);
 
+/* (Both entries cut inputs of more than (2^31 - 1) / (top_k * max(hidden, ffn)) tokens into several passes;
+ * after such a call the moe_layer_last_* hooks fail, since they describe one pass.) */
+
 /* Same computation on DEVICE pointers, enqueued on `hip_stream` (a hipStream_t, NULL = default
  * stream) without synchronising.  d_x and d_y must not alias.  This is the entry a caller that
  * already keeps activations on the GPU uses (no PCIe in the path). */

@@ -289,6 +289,30 @@ def test_block_rms_residual_chain():
     gpu.close()
 
 
+def test_long_inputs_go_through_in_several_passes(monkeypatch):
+    # the kernels address quantised rows with 32-bit offsets, so a call carries a bounded number of tokens
+    # and longer inputs are cut into passes; forced here at 48 tokens per pass on a 130-token input
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
+    xs = activations(130, 512, 21)
+    whole = gpu.forward(xs)
+    monkeypatch.setenv("MOE_MAX_TOKENS_PER_PASS", "48")
+    pieces = gpu.forward(xs)
+    with pytest.raises(candle_amd.MoeError):
+        gpu.last_logits(130)          # the hooks describe one pass only
+    import torch
+    dev = gpu.forward(torch.from_numpy(xs).cuda())
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOE_MAX_TOKENS_PER_PASS")
+    assert np.array_equal(bits(pieces), bits(dev.cpu().numpy()))
+    # a token's result does not depend on which other tokens share its pass, up to the kernel chosen for the
+    # pass size (130 tokens: tiled; 48: streamed), hence the tolerance rather than bit equality
+    assert np.abs(pieces - whole).max() <= block_tol(O.Q4K, 1024) * rms(whole)
+    gpu.forward(xs[:48])
+    want = ref.forward(xs[:48], logits=gpu.last_logits(48))
+    assert np.abs(pieces[:48] - want).max() <= block_tol(O.Q4K, 1024) * rms(want)
+    gpu.close()
+
+
 def test_empty_and_shape_errors():
     ref, gpu = make_pair(256, 256, 4, 2, O.Q4_0, seed=6)
     assert gpu.forward(np.zeros((0, 256), np.float32)).shape == (0, 256)
