@@ -17,7 +17,10 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <cerrno>
 #include <cstring>
+#include <new>
+#include <stdexcept>
 #include <map>
 #include <memory>
 #include <string>
@@ -112,7 +115,7 @@ bool read_value(Reader& r, uint32_t type, Value& v, int depth, std::string& err)
             const uint32_t et = r.get<uint32_t>();
             if (et > 12) { err = "unrecognized value-type " + std::to_string(et); return false; }
             const uint64_t n = r.count();
-            if (!r.ok || n > r.len) { err = "array length past the end of the file"; return false; }
+            if (!r.ok || n > r.len - r.pos) { err = "array length past the end of the file"; return false; }   // every element takes a byte or more
             v.arr.resize((size_t)n);
             for (auto& e : v.arr)
                 if (!read_value(r, et, e, depth + 1, err)) return false;
@@ -144,9 +147,21 @@ struct moe_gguf {
     }
 };
 
+static int gguf_open_impl(const char* path, moe_gguf** out);
+
 extern "C" int moe_gguf_open(const char* path, moe_gguf** out) {
     if (!path || !out) return fail(MOE_E_INVALID, "moe_gguf_open: NULL argument");
     *out = nullptr;
+    try {
+        return gguf_open_impl(path, out);
+    } catch (const std::bad_alloc&) {   // a table that claims more entries than memory holds
+        return fail(MOE_E_NOMEM, std::string(path) + ": out of memory while reading the GGUF tables");
+    } catch (const std::exception& e) {
+        return fail(MOE_E_INVALID, std::string(path) + ": " + e.what());
+    }
+}
+
+static int gguf_open_impl(const char* path, moe_gguf** out) {
     auto g = std::make_unique<moe_gguf>();
     g->fd = open(path, O_RDONLY);
     if (g->fd < 0) return fail(MOE_E_INVALID, std::string("cannot open ") + path + ": " + strerror(errno));
@@ -202,7 +217,7 @@ extern "C" int moe_gguf_open(const char* path, moe_gguf** out) {
         if (v.type == 0 || v.type == 2 || v.type == 4) alignment = v.u;
         else if ((v.type == 1 || v.type == 3 || v.type == 5) && v.i >= 0) alignment = (uint64_t)v.i;
     }
-    if (alignment == 0) return fail(MOE_E_INVALID, "gguf: general.alignment is 0");
+    if (alignment == 0 || alignment > (1u << 30)) return fail(MOE_E_INVALID, "gguf: general.alignment is " + std::to_string(alignment));
     g->tensor_data_offset = (r.pos + alignment - 1) / alignment * alignment;
     *out = g.release();
     return MOE_OK;
@@ -280,14 +295,19 @@ extern "C" int moe_gguf_tensor(const moe_gguf* g, const char* name, int* ggml_dt
     if (it == g->tensors.end()) return fail(MOE_E_INVALID, std::string("cannot find tensor info for ") + name);
     const TensorInfo& ti = it->second;
     uint64_t elems = 1;
-    for (int64_t d : ti.dims) elems *= (uint64_t)d;
+    for (int64_t d : ti.dims) {   // a hostile table must not wrap the element count around
+        if (d < 0 || (d > 0 && elems > UINT64_MAX / (uint64_t)d))
+            return fail(MOE_E_INVALID, std::string(name) + ": tensor dimensions overflow");
+        elems *= (uint64_t)d;
+    }
     uint64_t be = 1, bb = 1;
     dtype_geometry(ti.ggml_dtype, &be, &bb);
     if (elems % be)
         return fail(MOE_E_INVALID, "the number of elements " + std::to_string(elems) + " is not divisible by the block size " + std::to_string(be));
+    if (elems / be > UINT64_MAX / bb) return fail(MOE_E_INVALID, std::string(name) + ": tensor dimensions overflow");
     const uint64_t size = elems / be * bb;
     const uint64_t start = g->tensor_data_offset + ti.offset;
-    if (start > g->len || size > g->len - start)
+    if (ti.offset > g->len || start > g->len || size > g->len - start)
         return fail(MOE_E_INVALID, "tensor data extends beyond file boundary: offset=" + std::to_string(start) + ", size=" + std::to_string(size) +
                                        ", file_len=" + std::to_string(g->len));
     if (ggml_dtype) *ggml_dtype = ti.ggml_dtype;

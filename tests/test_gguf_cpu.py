@@ -119,3 +119,44 @@ def test_tensor_size_and_bounds_checks(tmp_path):
     with candle_amd.GgufFile(str(p2)) as g:
         with pytest.raises(candle_amd.MoeError, match="tensor data extends beyond file boundary"):
             g.tensor("t")
+
+
+def test_hostile_tables_are_refused_not_followed(tmp_path):
+    # dimensions whose product wraps around 2^64 must not pass the size check as a small tensor
+    p = tmp_path / "wrap.gguf"
+    W.write_gguf(p, [], [("t", 0, (1 << 33, 1 << 33), rnd(64)), ("u", 12, (1 << 62, 1024), rnd(144))])
+    with candle_amd.GgufFile(str(p)) as g:
+        for name in ("t", "u"):
+            with pytest.raises(candle_amd.MoeError, match="overflow"):
+                g.tensor(name)
+    # a data offset near 2^64 must not wrap the start address back into the file
+    p2 = tmp_path / "offset.gguf"
+    W.write_gguf(p2, [], [("t", 0, (16,), rnd(64))])
+    blob = bytearray(open(p2, "rb").read())
+    i = blob.index(b"t", 24) + 1 + 4 + 8 + 4           # name, n_dims, one u64 dimension, dtype
+    assert struct.unpack_from("<Q", blob, i)[0] == 0
+    struct.pack_into("<Q", blob, i, (1 << 64) - 32)
+    open(p2, "wb").write(bytes(blob))
+    with candle_amd.GgufFile(str(p2)) as g:
+        with pytest.raises(candle_amd.MoeError, match="beyond file boundary"):
+            g.tensor("t")
+    # an array that claims more elements than the file has bytes left
+    p3 = tmp_path / "array.gguf"
+    W.write_gguf(p3, [("a", W.ARRAY, (W.U8, [1, 2, 3]))], [])
+    blob = bytearray(open(p3, "rb").read())
+    i = blob.index(b"a", 24) + 1 + 4 + 4               # key, value type (array), element type
+    assert struct.unpack_from("<Q", blob, i)[0] == 3
+    struct.pack_into("<Q", blob, i, 1 << 40)
+    open(p3, "wb").write(bytes(blob))
+    with pytest.raises(candle_amd.MoeError, match="array length past the end of the file"):
+        candle_amd.GgufFile(str(p3))
+    # an absurd alignment
+    p4 = tmp_path / "align.gguf"
+    W.write_gguf(p4, [("general.alignment", W.U32, 32)], [("t", 0, (8,), rnd(32))])
+    blob = bytearray(open(p4, "rb").read())
+    i = blob.index(b"general.alignment") + len("general.alignment") + 4
+    assert struct.unpack_from("<I", blob, i)[0] == 32
+    struct.pack_into("<I", blob, i, 0xFFFFFFFF)
+    open(p4, "wb").write(bytes(blob))
+    with pytest.raises(candle_amd.MoeError, match="general.alignment is 4294967295"):
+        candle_amd.GgufFile(str(p4))
