@@ -305,10 +305,17 @@ static int64_t max_tokens_per_pass(const moe_layer* L) {
 
 static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
 #define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
+    // Under stream capture (the caller records this forward into a HIP graph) nothing may be allocated, and
+    // the event that orders eager calls on different streams stays out of the graph.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    const char* const capture_msg = "forward under stream capture needs its workspace: run one forward of the same number of tokens before capturing";
+    if (capturing && T > L->cap_T) return fail(MOE_E_INVALID, capture_msg);
     int rc = reserve_workspace(L, T);
     if (rc) return rc;
     // a previous call may still be running on another stream and shares the workspace
-    MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
+    if (!capturing) MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
     const bool shared = L->Fs > 0;
     FrontParams fp;
     fp.x = d_x; fp.T = T; fp.H = (int)L->H; fp.E = (int)L->E; fp.k = (int)L->k; fp.norm_topk = L->norm_topk;
@@ -355,6 +362,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     const bool narrow = direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
                         (force_narrow >= 0 ? force_narrow > 0 : T * L->k <= L->E);
     if (tiled) {
+        if (capturing && L->hbuf.cap < (size_t)T * L->k * L->F * 4) return fail(MOE_E_INVALID, capture_msg);
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();
         ep.n_slots = T * L->k;
@@ -373,6 +381,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     } else if (narrow) {
         // very small Q4K batches: at most half of the experts can be active, so the weights are cut
         // into four times as many workgroups; those write f32 h and a small pass quantises it
+        if (capturing && L->hbuf.cap < (size_t)T * L->k * L->F * 4) return fail(MOE_E_INVALID, capture_msg);
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();
         MOE_HIP_CHECK(launch_expert_up(ep, s));
@@ -402,7 +411,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     MOE_MARK(ST_COMBINE);
 #undef MOE_MARK
     L->last_direct = direct;
-    MOE_HIP_CHECK(hipEventRecord(L->done, s));
+    if (!capturing) MOE_HIP_CHECK(hipEventRecord(L->done, s));
     L->last_T = T;
     return MOE_OK;
 }

@@ -90,6 +90,8 @@ void moe_layer_destroy(moe_layer* layer);
  * x and y are HOST f32 [n_tokens, hidden]; synchronous. */
 int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float* y);
 
+/* moe_layer_forward_device may be recorded into a HIP graph (stream capture): it then allocates nothing
+ * and fails with a message if its workspace was not reserved by an earlier forward of the same size. */
 /* (Both entries cut inputs of more than (2^31 - 1) / (top_k * max(hidden, ffn)) tokens into several passes;
  * after such a call the moe_layer_last_* hooks fail, since they describe one pass.) */
 

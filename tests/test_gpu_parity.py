@@ -313,6 +313,41 @@ def test_long_inputs_go_through_in_several_passes(monkeypatch):
     gpu.close()
 
 
+@pytest.mark.parametrize("T", [4, 32, 200])
+def test_forward_recorded_into_a_hip_graph(T):
+    # a decode loop records the layer into a graph and replays it: narrow (4), direct (32) and tiled (200)
+    # paths; every replay, with eager work and synchronisations in between, must equal the eager result
+    torch = pytest.importorskip("torch")
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
+    xs = [torch.from_numpy(activations(T, 512, 30 + i)).cuda() for i in range(3)]
+    eager = [gpu.forward(x).clone() for x in xs]
+    x_in, y_out = xs[0].clone(), torch.empty_like(xs[0])
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        gpu.forward(x_in, out=y_out)            # workspace reserved before the capture
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        gpu.forward(x_in, out=y_out)
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            x_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_out, want)
+            assert torch.equal(gpu.forward(x), want)      # eager calls between replays keep working
+    # a capture that would have to allocate is refused with a message, not recorded
+    big = torch.from_numpy(activations(T + 300, 512, 5)).cuda()
+    out = torch.empty_like(big)
+    g2 = torch.cuda.CUDAGraph()
+    with pytest.raises(candle_amd.MoeError, match="before capturing"):
+        with torch.cuda.graph(g2, stream=side):
+            gpu.forward(big, out=out)
+    torch.cuda.synchronize()
+    assert torch.equal(gpu.forward(xs[0]), eager[0])
+    gpu.close()
+
+
 def test_empty_and_shape_errors():
     ref, gpu = make_pair(256, 256, 4, 2, O.Q4_0, seed=6)
     assert gpu.forward(np.zeros((0, 256), np.float32)).shape == (0, 256)
