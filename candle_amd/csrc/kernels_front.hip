@@ -624,7 +624,11 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
         case 2: hipLaunchKernelGGL((front_fast_kernel<VDT, 2>), grid, block, 0, s, p); return true;
         case 4: hipLaunchKernelGGL((front_fast_kernel<VDT, 4>), grid, block, 0, s, p); return true;
         case 8: hipLaunchKernelGGL((front_fast_kernel<VDT, 8>), grid, block, 0, s, p); return true;
+        case 12: hipLaunchKernelGGL((front_fast_kernel<VDT, 12>), grid, block, 0, s, p); return true;
         case 16: hipLaunchKernelGGL((front_fast_kernel<VDT, 16>), grid, block, 0, s, p); return true;
+        case 20: hipLaunchKernelGGL((front_fast_kernel<VDT, 20>), grid, block, 0, s, p); return true;
+        case 24: hipLaunchKernelGGL((front_fast_kernel<VDT, 24>), grid, block, 0, s, p); return true;
+        case 28: hipLaunchKernelGGL((front_fast_kernel<VDT, 28>), grid, block, 0, s, p); return true;
         case 32: hipLaunchKernelGGL((front_fast_kernel<VDT, 32>), grid, block, 0, s, p); return true;
     }
     return false;

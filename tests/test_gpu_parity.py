@@ -219,6 +219,16 @@ def test_block_q4k_small(T):
     gpu.close()
 
 
+@pytest.mark.parametrize("H", [768, 3072, 5120, 6144, 7168])
+def test_block_other_hidden_sizes(H):
+    # hidden sizes with their own instantiation of the low-latency front kernel (3072 .. 7168) and one
+    # that takes the generic front kernel (768)
+    ref, gpu = make_pair(H, 1024, 4, 2, O.Q4K, seed=H)
+    for T in (3, 40):
+        check_block(ref, gpu, T, tol=block_tol(O.Q4K, 1024))
+    gpu.close()
+
+
 def test_block_q8_0_shared_expert_top4():
     ref, gpu = make_pair(256, 352, 12, 4, O.Q8_0, seed=3, Fs=704)
     check_block(ref, gpu, 40)
