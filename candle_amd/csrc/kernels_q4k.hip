@@ -1,4 +1,4 @@
-// Grouped expert products over Q4K, Q5K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
+// Grouped expert products over Q2K, Q4K, Q5K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
 //
 // Arithmetic restated from BlockQ4K::vec_dot, candle-core/src/quantized/k_quants.rs:1205-1285:
 // per 256-element super-block
@@ -170,6 +170,57 @@ __device__ inline void q5k_mac(const Q5KTile& w, const Q8KOperand& A, const floa
     q45k_mac<true>(w.q0, w.q1, w.sc, w.qh.x, w.qh.y, A, yd, g, acc);
 }
 
+// Q2K (BlockQ2K::vec_dot, k_quants.rs:755-805): d * y.d * sum_j sc_j * (code_j . q8_j) - dmin * y.d *
+// sum_j min_j * bsum_j over the sixteen 16-element sub-blocks, sc and min four bits each.  sc * code <= 45
+// fits a byte, so the scale goes into the weight operand (a lane's eight elements of a 32-element stretch
+// lie in one sub-block) and the eight MFMAs of a super-block accumulate into one exact integer.
+struct Q2KTile {
+    uint4 q, sc;
+    uint32_t dd;   // d | dmin << 16 of the lane's row
+};
+__device__ inline Q2KTile load_q2k_tile(const uint8_t* tile, int lane) {
+    Q2KTile t;
+    t.q = gload_stream(tile, (uint32_t)lane * 16u);
+    t.sc = gload_stream(tile, 1024u + (uint32_t)(lane & 15) * 16u);
+    t.dd = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) uint32_t*>((gbytes)tile + 1280u + (uint32_t)(lane & 15) * 4u));
+    return t;
+}
+// four bytes (each <= 3) times a scale (<= 15) with the packed 16-bit multiply: no byte overflows
+typedef unsigned short u16x2s __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t scale_codes(uint32_t q, uint32_t s) {
+    const u16x2s a = __builtin_bit_cast(u16x2s, q);
+    const u16x2s b = {(unsigned short)s, (unsigned short)s};
+    return __builtin_bit_cast(uint32_t, (u16x2s)(a * b));
+}
+__device__ inline void q2k_mac(const Q2KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+    const uint32_t M3 = 0x03030303u;
+    const float d = __half2float(__ushort_as_half((unsigned short)(w.dd & 0xffffu)));
+    const float dmin = __half2float(__ushort_as_half((unsigned short)(w.dd >> 16)));
+    const uint32_t qw[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
+    const uint32_t sw[4] = {w.sc.x, w.sc.y, w.sc.z, w.sc.w};
+    const int sel = 8 * (g >> 1);   // groups 0,1 hold the first 16 elements of a 32-element stretch, 2,3 the second
+    v4i isum = {0, 0, 0, 0};
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t q = qw[P];
+        const uint32_t s_lo = (sw[P] >> sel) & 0xFu, s_hi = (sw[P] >> (16 + sel)) & 0xFu;
+        const long b_lo = pack64(scale_codes(q & M3, s_lo), scale_codes((q >> 2) & M3, s_lo));
+        const long b_hi = pack64(scale_codes((q >> 4) & M3, s_hi), scale_codes((q >> 6) & M3, s_hi));
+        isum = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(A.a[P].x, A.a[P].y), b_lo, isum, 0, 0, 0);
+        isum = __builtin_amdgcn_mfma_i32_16x16x32_i8(pack64(A.a[P].z, A.a[P].w), b_hi, isum, 0, 0, 0);
+    }
+    // mins term: sum_j min_j * bsum_j as an exact f16 MFMA; this lane supplies sub-blocks 4g..4g+3
+    const uint32_t mg = (sw[g] >> 4) & 0x0f0f0f0fu;
+    const v4h mB = {(_Float16)(int)(mg & 0xffu), (_Float16)(int)((mg >> 8) & 0xffu), (_Float16)(int)((mg >> 16) & 0xffu), (_Float16)(int)(mg >> 24)};
+    const v4f zf = {0.f, 0.f, 0.f, 0.f};
+    v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, mB, zf, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        acc[i] += (d * yd[i]) * (float)isum[i];
+        acc[i] -= (dmin * yd[i]) * Dm[i];
+    }
+}
+
 struct Q6KTile {
     uint4 q0, q1, qh, sc;
     uint32_t d;   // f16 bits of the lane's row
@@ -231,6 +282,12 @@ struct FmtQ4K {
     static constexpr int TILE_BYTES = Q4K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q4k_tile(tile, lane); }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q4k_mac(w, A, yd, g, acc); }
+};
+struct FmtQ2K {
+    typedef Q2KTile Tile;
+    static constexpr int TILE_BYTES = Q2K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q2k_tile(tile, lane); }
+    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q2k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ5K {
     typedef Q5KTile Tile;
@@ -508,6 +565,13 @@ DEF_DOWN(q4k_down_t1_v1, FmtQ4K, 1, 4, 2, 3)
 DEF_DOWN_NARROW(q4k_down_t1_narrow, FmtQ4K, 8, 2, 4)
 DEF_DOWN(q4k_down_t2, FmtQ4K, 2, 4, 2, 2)
 DEF_DOWN(q4k_down_t4, FmtQ4K, 4, 8, 2, 2)
+// Q2K: nine registers per tile; one and two slot tiles per pass
+DEF_UP(q2k_up_t1, FmtQ2K, 1, 4, 2, 3)
+DEF_UP_NARROW(q2k_up_t1_narrow, FmtQ2K, 4, 2, 3)
+DEF_UP(q2k_up_t2, FmtQ2K, 2, 4, 2, 2)
+DEF_DOWN(q2k_down_t1, FmtQ2K, 1, 4, 2, 3)
+DEF_DOWN_NARROW(q2k_down_t1_narrow, FmtQ2K, 8, 2, 4)
+DEF_DOWN(q2k_down_t2, FmtQ2K, 2, 4, 2, 2)
 // Q5K: the Q4K variants with two more registers per tile; one and two slot tiles per pass
 DEF_UP(q5k_up_t1, FmtQ5K, 1, 4, 2, 3)
 DEF_UP_NARROW(q5k_up_t1_narrow, FmtQ5K, 4, 2, 3)
@@ -530,64 +594,62 @@ static int variant(const char* name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
+// The kernels of one weight format.  t4 (four slot tiles per pass) exists for Q4K only.
+typedef void (*ExpertKernel)(ExpertParams);
+struct KernelFamily {
+    ExpertKernel up_t1, up_narrow, up_t2, up_t4;
+    ExpertKernel down_t1, down_narrow, down_t2, down_t4;
+};
+static const KernelFamily* kernel_family(int dt) {
+    static const int uv = variant("MOE_UP_VARIANT", 1), dv = variant("MOE_DOWN_VARIANT", 1);
+    static const KernelFamily q4k = {uv == 0 ? q4k_up_t1_v0 : q4k_up_t1_v1, q4k_up_t1_narrow, q4k_up_t2, q4k_up_t4,
+                                     dv == 0 ? q4k_down_t1_v0 : q4k_down_t1_v1, q4k_down_t1_narrow, q4k_down_t2, q4k_down_t4};
+    static const KernelFamily q2k = {q2k_up_t1, q2k_up_t1_narrow, q2k_up_t2, nullptr, q2k_down_t1, q2k_down_t1_narrow, q2k_down_t2, nullptr};
+    static const KernelFamily q5k = {q5k_up_t1, q5k_up_t1_narrow, q5k_up_t2, nullptr, q5k_down_t1, q5k_down_t1_narrow, q5k_down_t2, nullptr};
+    static const KernelFamily q6k = {q6k_up_t1, q6k_up_t1_narrow, q6k_up_t2, nullptr, q6k_down_t1, q6k_down_t1_narrow, q6k_down_t2, nullptr};
+    switch (dt) {
+        case MOE_GGML_Q2K: return &q2k;
+        case MOE_GGML_Q4K: return &q4k;
+        case MOE_GGML_Q5K: return &q5k;
+        case MOE_GGML_Q6K: return &q6k;
+    }
+    return nullptr;
+}
+
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    static const int v = variant("MOE_UP_VARIANT", 1);
-    const bool q6k = p.dt == MOE_GGML_Q6K, q5k = p.dt == MOE_GGML_Q5K;
-    const int tt = p.slot_tiles >= 4 && !q6k && !q5k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const KernelFamily* f = kernel_family(p.dt);
+    if (!f) return hipErrorInvalidValue;
+    static const int uv = variant("MOE_UP_VARIANT", 1);
+    const int tt = p.slot_tiles >= 4 && f->up_t4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (64 rows), f32 h to p.hbuf
         dim3 ngrid((unsigned)(p.F / 64), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
-        if (q6k) hipLaunchKernelGGL(q6k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
-        else if (q5k) hipLaunchKernelGGL(q5k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q4k_up_t1_narrow, ngrid, dim3(256), 0, s, p);
+        hipLaunchKernelGGL(f->up_narrow, ngrid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
     dim3 grid((unsigned)(p.F / 256), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (q6k) {
-        if (tt == 2) hipLaunchKernelGGL(q6k_up_t2, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q6k_up_t1, grid, dim3(256), 0, s, p);
-        return hipGetLastError();
-    }
-    if (q5k) {
-        if (tt == 2) hipLaunchKernelGGL(q5k_up_t2, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q5k_up_t1, grid, dim3(256), 0, s, p);
-        return hipGetLastError();
-    }
-    if (tt == 4) hipLaunchKernelGGL(q4k_up_t4, grid, dim3(512), 0, s, p);
-    else if (tt == 2) hipLaunchKernelGGL(q4k_up_t2, grid, dim3(256), 0, s, p);
-    else if (v == 0) hipLaunchKernelGGL(q4k_up_t1_v0, grid, dim3(512), 0, s, p);
-    else hipLaunchKernelGGL(q4k_up_t1_v1, grid, dim3(256), 0, s, p);
+    if (tt == 4) hipLaunchKernelGGL(f->up_t4, grid, dim3(512), 0, s, p);
+    else if (tt == 2) hipLaunchKernelGGL(f->up_t2, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(f->up_t1, grid, dim3(p.dt == MOE_GGML_Q4K && uv == 0 ? 512 : 256), 0, s, p);
     return hipGetLastError();
 }
 
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    static const int v = variant("MOE_DOWN_VARIANT", 1);
     const int dtd = p.dt_down ? p.dt_down : p.dt;
-    const bool q6k = dtd == MOE_GGML_Q6K, q5k = dtd == MOE_GGML_Q5K;
-    const int tt = p.slot_tiles >= 4 && !q6k && !q5k ? 4 : p.slot_tiles >= 2 ? 2 : 1;
+    const KernelFamily* f = kernel_family(dtd);
+    if (!f) return hipErrorInvalidValue;
+    static const int dv = variant("MOE_DOWN_VARIANT", 1);
+    const int tt = p.slot_tiles >= 4 && f->down_t4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (32 rows), eight waves split K
         dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
-        if (q6k) hipLaunchKernelGGL(q6k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
-        else if (q5k) hipLaunchKernelGGL(q5k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(q4k_down_t1_narrow, ngrid, dim3(512), 0, s, p);
+        hipLaunchKernelGGL(f->down_narrow, ngrid, dim3(512), 0, s, p);
         return hipGetLastError();
     }
     dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    if (q6k) {
-        if (tt == 2) hipLaunchKernelGGL(q6k_down_t2, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q6k_down_t1, grid, dim3(256), 0, s, p);
-        return hipGetLastError();
-    }
-    if (q5k) {
-        if (tt == 2) hipLaunchKernelGGL(q5k_down_t2, grid, dim3(256), 0, s, p);
-        else hipLaunchKernelGGL(q5k_down_t1, grid, dim3(256), 0, s, p);
-        return hipGetLastError();
-    }
-    if (tt == 4) hipLaunchKernelGGL(q4k_down_t4, grid, dim3(512), 0, s, p);
-    else if (tt == 2) hipLaunchKernelGGL(q4k_down_t2, grid, dim3(256), 0, s, p);
-    else if (v == 0) hipLaunchKernelGGL(q4k_down_t1_v0, grid, dim3(512), 0, s, p);
-    else hipLaunchKernelGGL(q4k_down_t1_v1, grid, dim3(256), 0, s, p);
+    if (tt == 4) hipLaunchKernelGGL(f->down_t4, grid, dim3(512), 0, s, p);
+    else if (tt == 2) hipLaunchKernelGGL(f->down_t2, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(f->down_t1, grid, dim3(dtd == MOE_GGML_Q4K && dv == 0 ? 512 : 256), 0, s, p);
     return hipGetLastError();
 }
 

@@ -1,7 +1,7 @@
 // Layout and format kernels: re-laying GGML blocks into the tiled device layout, `to_float`
 // from either layout, and the stand-alone activation quantiser used by the parity hooks.
 //
-// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0),
+// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0), 872-908 (Q2K),
 // 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1563-1595 (Q5K), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
 #include <algorithm>
@@ -32,6 +32,12 @@ __device__ inline float q4k_value(const uint8_t* hdr, int i, uint8_t qbyte) {
     float m1 = mn * (float)m;
     int q = ((i / 32) & 1) ? (qbyte >> 4) : (qbyte & 0xF);
     return d1 * (float)q - m1;
+}
+
+// to_float of one Q2K element, k_quants.rs:885-903: `dl * code - ml` with dl = d * (sc & 0xF), ml = min * (sc >> 4)
+__device__ inline float q2k_value(float d, float mn, uint8_t sc, int code) {
+    const float dl = d * (float)(sc & 0xF), ml = mn * (float)(sc >> 4);
+    return dl * (float)code - ml;
 }
 
 // value of element `i` of a Q5K block: header as Q4K, nibble byte, fifth bit (k_quants.rs:1582-1591:
@@ -66,6 +72,11 @@ __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, in
         const uint8_t* b = blocks + (i / 256) * 144;
         int e = (int)(i % 256);
         out[i] = q4k_value(b, e, b[16 + (e / 64) * 32 + (e % 32)]);
+    } else if (dt == MOE_GGML_Q2K) {
+        const uint8_t* b = blocks + (i / 256) * 84;
+        int e = (int)(i % 256);
+        int code = (b[16 + 32 * (e / 128) + e % 32] >> (2 * ((e % 128) / 32))) & 3;
+        out[i] = q2k_value(f16_bits_to_f32((uint16_t)(b[80] | (b[81] << 8))), f16_bits_to_f32((uint16_t)(b[82] | (b[83] << 8))), b[e / 16], code);
     } else if (dt == MOE_GGML_Q5K) {
         const uint8_t* b = blocks + (i / 256) * 176;
         int e = (int)(i % 256);
@@ -114,6 +125,28 @@ __global__ void relayout_q4k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t 
         int r = ch - 128;
         const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
         for (int i = 0; i < 16; i++) dst[i] = blk[i];
+    }
+}
+
+__global__ void relayout_q2k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
+    // one thread per (tile, lane): its 64 two-bit codes; lanes < 16 also move the row's scales, d and dmin
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nsb * 64) return;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int64_t rt = tile / nsb;
+    int sb = (int)(tile % nsb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 84;
+    uint8_t* dst = tiled + (sb * n_rt + rt) * Q2K_TILE_BYTES;  // tiles ordered [sb][rt]
+    auto code = [&](int e) { return (blk[16 + 32 * (e / 128) + e % 32] >> (2 * ((e % 128) / 32))) & 3; };
+    for (int P = 0; P < 4; P++)
+        for (int i = 0; i < 4; i++) {
+            const int e = 64 * P + 8 * g + i;
+            dst[l * 16 + P * 4 + i] = (uint8_t)(code(e) | (code(e + 4) << 2) | (code(e + 32) << 4) | (code(e + 36) << 6));
+        }
+    if (g == 0) {
+        for (int j = 0; j < 16; j++) dst[1024 + r * 16 + j] = blk[j];
+        for (int j = 0; j < 4; j++) dst[1280 + r * 4 + j] = blk[80 + j];
     }
 }
 
@@ -221,6 +254,15 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         int l = g * 16 + r;
         uint8_t q = tile[(P / 2) * 1024 + l * 16 + (P % 2) * 8 + pos];
         out[i] = q4k_value(tile + 2048 + r * 16, e, q);
+    } else if (dt == MOE_GGML_Q2K) {
+        int sb = col / 256, e = col % 256;
+        const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q2K_TILE_BYTES;
+        int P = e / 64, sub = (e % 64) / 32, g = (e % 32) / 8, pos = e % 8;
+        int l = g * 16 + r;
+        int code = (tile[l * 16 + P * 4 + pos % 4] >> (2 * (2 * sub + pos / 4))) & 3;
+        const uint8_t* dd = tile + 1280 + r * 4;
+        out[i] = q2k_value(f16_bits_to_f32((uint16_t)(dd[0] | (dd[1] << 8))), f16_bits_to_f32((uint16_t)(dd[2] | (dd[3] << 8))),
+                           tile[1024 + r * 16 + e / 16], code);
     } else if (dt == MOE_GGML_Q5K) {
         int sb = col / 256, e = col % 256;
         const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q5K_TILE_BYTES;
@@ -314,6 +356,8 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
     if (n_rt == 0 || nkb == 0) return hipSuccess;
     if (dt == MOE_GGML_Q4K)
         hipLaunchKernelGGL(relayout_q4k_kernel, dim3(nblk(n_rt * nkb * 144, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (dt == MOE_GGML_Q2K)
+        hipLaunchKernelGGL(relayout_q2k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q5K)
         hipLaunchKernelGGL(relayout_q5k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q6K)

@@ -97,7 +97,7 @@ static inline float rmin(float a, float b) { return fminf(a, b); }
 int64_t orc_block_elems(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return 32;
-        case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
+        case ORC_Q2K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
         default: return -1;
     }
 }
@@ -105,6 +105,7 @@ int64_t orc_block_bytes(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: return 18;
         case ORC_Q8_0: return 34;
+        case ORC_Q2K: return 84;
         case ORC_Q4K: return 144;
         case ORC_Q5K: return 176;
         case ORC_Q6K: return 210;
@@ -115,7 +116,7 @@ int64_t orc_block_bytes(int dtype) {
 int orc_vecdot_dtype(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
-        case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
+        case ORC_Q2K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
         default: return -1;
     }
 }
@@ -367,6 +368,110 @@ static float vec_dot_q4k_q8k(int64_t n, const orc_block_q4k* xs, const orc_block
     float tail = 0.f;
     for (int l = 0; l < 8; l++) tail += sums[l];
     return sumf + tail;
+}
+
+/* ------------------------------------------------------------------ Q2K */
+/* k_quants.rs:808-870 */
+static void quantize_q2k(const float* xs, int64_t k, orc_block_q2k* ys) {
+    const float Q4SCALE = 15.0f;
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float* x = xs + b * 256;
+        orc_block_q2k* block = &ys[b];
+        float mins[16], scales[16];
+        for (int j = 0; j < 16; j++) make_qkx1_quants(3, 5, x + 16 * j, 16, &scales[j], &mins[j]);
+        float max_scale = 0.f, max_min = 0.f;
+        for (int j = 0; j < 16; j++) { max_scale = rmax(scales[j], max_scale); max_min = rmax(mins[j], max_min); }
+        if (max_scale > 0.f) {
+            float iscale = Q4SCALE / max_scale;
+            for (int j = 0; j < 16; j++) block->scales[j] = (uint8_t)nearest_int(iscale * scales[j]);
+            block->d = orc_f32_to_f16(max_scale / Q4SCALE);
+        } else {
+            for (int j = 0; j < 16; j++) block->scales[j] = 0;
+            block->d = orc_f32_to_f16(0.f);
+        }
+        if (max_min > 0.f) {
+            float iscale = Q4SCALE / max_min;
+            for (int j = 0; j < 16; j++) {
+                uint8_t l = (uint8_t)nearest_int(iscale * mins[j]);
+                block->scales[j] |= (uint8_t)(l << 4);
+            }
+            block->dmin = orc_f32_to_f16(max_min / Q4SCALE);
+        } else {
+            block->dmin = orc_f32_to_f16(0.f);
+        }
+        uint8_t big_l[256];
+        memset(big_l, 0, sizeof big_l);
+        for (int j = 0; j < 16; j++) {
+            float d = orc_f16_to_f32(block->d) * (float)(block->scales[j] & 0xF);
+            if (d == 0.f) continue;
+            float dm = orc_f16_to_f32(block->dmin) * (float)(block->scales[j] >> 4);
+            for (int ii = 0; ii < 16; ii++) {
+                int32_t ll = nearest_int((x[16 * j + ii] + dm) / d);
+                big_l[16 * j + ii] = (uint8_t)(ll < 0 ? 0 : ll > 3 ? 3 : ll);
+            }
+        }
+        for (int j = 0; j < 256; j += 128)
+            for (int ll = 0; ll < 32; ll++)
+                block->qs[j / 4 + ll] = (uint8_t)(big_l[j + ll] | (big_l[j + ll + 32] << 2) | (big_l[j + ll + 64] << 4) | (big_l[j + ll + 96] << 6));
+    }
+}
+/* k_quants.rs:872-908 */
+static void dequantize_q2k(const orc_block_q2k* xs, int64_t k, float* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const orc_block_q2k* block = &xs[b];
+        float d = orc_f16_to_f32(block->d);
+        float min = orc_f16_to_f32(block->dmin);
+        int is = 0;
+        for (int n = 0; n < 256; n += 128) {
+            const uint8_t* qs = block->qs + n / 4;
+            float* y = ys + b * 256 + n;
+            int yi = 0, shift = 0;
+            for (int j = 0; j < 4; j++) {
+                uint8_t sc = block->scales[is++];
+                float dl = d * (float)(sc & 0xF), ml = min * (float)(sc >> 4);
+                for (int l = 0; l < 16; l++) y[yi++] = dl * (float)((qs[l] >> shift) & 3) - ml;
+                sc = block->scales[is++];
+                dl = d * (float)(sc & 0xF);
+                ml = min * (float)(sc >> 4);
+                for (int l = 16; l < 32; l++) y[yi++] = dl * (float)((qs[l] >> shift) & 3) - ml;
+                shift += 2;
+            }
+        }
+    }
+}
+/* k_quants.rs:755-805 (vec_dot_unopt) */
+static float vec_dot_q2k_q8k(int64_t n, const orc_block_q2k* xs, const orc_block_q8k* ys) {
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q2k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        const uint8_t* q2 = x->qs;
+        const int8_t* q8 = y->qs;
+        int32_t summs = 0;
+        for (int j = 0; j < 16; j++) summs += (int32_t)y->bsums[j] * (int32_t)(x->scales[j] >> 4);
+        float dall = y->d * orc_f16_to_f32(x->d);
+        float dmin = y->d * orc_f16_to_f32(x->dmin);
+        int32_t isum = 0;
+        int is = 0;
+        for (int h = 0; h < 2; h++) {
+            int shift = 0;
+            for (int j = 0; j < 4; j++) {
+                int32_t d = x->scales[is++] & 0xF;
+                int32_t isuml = 0;
+                for (int l = 0; l < 16; l++) isuml += (int32_t)q8[l] * (int32_t)((q2[l] >> shift) & 3);
+                isum += d * isuml;
+                d = x->scales[is++] & 0xF;
+                isuml = 0;
+                for (int l = 16; l < 32; l++) isuml += (int32_t)q8[l] * (int32_t)((q2[l] >> shift) & 3);
+                isum += d * isuml;
+                shift += 2;
+                q8 += 32;
+            }
+            q2 += 32;
+        }
+        sumf += dall * (float)isum - dmin * (float)summs;
+    }
+    return sumf;
 }
 
 /* ------------------------------------------------------------------ Q5K */
@@ -777,6 +882,7 @@ int orc_quantize(int dtype, const float* x, int64_t n, void* blocks) {
         case ORC_Q4_0: quantize_q4_0(x, n, (orc_block_q4_0*)blocks); return 0;
         case ORC_Q8_0: quantize_q8_0(x, n, (orc_block_q8_0*)blocks); return 0;
         case ORC_Q4K: memset(blocks, 0, (size_t)(n / 256) * 144); quantize_q4k(x, n, (orc_block_q4k*)blocks); return 0;
+        case ORC_Q2K: memset(blocks, 0, (size_t)(n / 256) * 84); quantize_q2k(x, n, (orc_block_q2k*)blocks); return 0;
         case ORC_Q5K: memset(blocks, 0, (size_t)(n / 256) * 176); quantize_q5k(x, n, (orc_block_q5k*)blocks); return 0;
         case ORC_Q6K: memset(blocks, 0, (size_t)(n / 256) * 210); quantize_q6k(x, n, (orc_block_q6k*)blocks); return 0;
         case ORC_Q8K: quantize_q8k(x, n, (orc_block_q8k*)blocks); return 0;
@@ -790,6 +896,7 @@ int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y) {
         case ORC_Q4_0: dequantize_q4_0((const orc_block_q4_0*)blocks, n, y); return 0;
         case ORC_Q8_0: dequantize_q8_0((const orc_block_q8_0*)blocks, n, y); return 0;
         case ORC_Q4K: dequantize_q4k((const orc_block_q4k*)blocks, n, y); return 0;
+        case ORC_Q2K: dequantize_q2k((const orc_block_q2k*)blocks, n, y); return 0;
         case ORC_Q5K: dequantize_q5k((const orc_block_q5k*)blocks, n, y); return 0;
         case ORC_Q6K: dequantize_q6k((const orc_block_q6k*)blocks, n, y); return 0;
         case ORC_Q8K: dequantize_q8k((const orc_block_q8k*)blocks, n, y); return 0;
@@ -801,6 +908,7 @@ float orc_vec_dot(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q4_0: return vec_dot_q4_0_q8_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return vec_dot_q8_0_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return vec_dot_q4k_q8k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q2K: return vec_dot_q2k_q8k(n, (const orc_block_q2k*)w, (const orc_block_q8k*)a);
         case ORC_Q5K: return vec_dot_q5k_q8k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return vec_dot_q6k_q8k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         case ORC_Q8K: return vec_dot_q8k_q8k(n, (const orc_block_q8k*)w, (const orc_block_q8k*)a);

@@ -6,6 +6,7 @@
  *   vec_dot_q4_0_q8_0  candle-core/src/quantized/avx.rs:50-68
  *   vec_dot_q8_0_q8_0  candle-core/src/quantized/avx.rs:71-87
  *   vec_dot_q4k_q8k    candle-core/src/quantized/avx.rs:443-525
+ *   vec_dot_q2k_q8k    candle-core/src/quantized/avx.rs:224-304
  *   vec_dot_q5k_q8k    candle-core/src/quantized/avx.rs:527-638
  *   vec_dot_q6k_q8k    candle-core/src/quantized/avx.rs:131-216
  * The integer parts are exact; the f32 accumulation order differs from the scalar
@@ -111,6 +112,47 @@ static float dot_q4k(int64_t n, const orc_block_q4k* xs, const orc_block_q8k* ys
     return hsum_float_8(acc) + _mm_cvtss_f32(acc_m);
 }
 
+static float dot_q2k(int64_t n, const orc_block_q2k* xs, const orc_block_q8k* ys) {
+    const __m256i m3 = _mm256_set1_epi8(3);
+    const __m128i m4 = _mm_set1_epi8(0xF);
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q2k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        float d = y->d * orc_f16_to_f32(x->d);
+        float dmin = -y->d * orc_f16_to_f32(x->dmin);
+        const uint8_t* q2 = x->qs;
+        const int8_t* q8 = y->qs;
+        __m128i mins_and_scales = _mm_loadu_si128((const __m128i*)x->scales);
+        __m128i scales8 = _mm_and_si128(mins_and_scales, m4);
+        __m128i mins8 = _mm_and_si128(_mm_srli_epi16(mins_and_scales, 4), m4);
+        __m256i mins = _mm256_cvtepi8_epi16(mins8);
+        __m256i prod = _mm256_madd_epi16(mins, _mm256_loadu_si256((const __m256i*)y->bsums));
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(dmin), _mm256_cvtepi32_ps(prod), acc);
+        __m256i all_scales = _mm256_cvtepi8_epi16(scales8);
+        __m128i l_scales = _mm256_extracti128_si256(all_scales, 0);
+        __m128i h_scales = _mm256_extracti128_si256(all_scales, 1);
+        __m256i scales[2] = {_mm256_set_m128i(l_scales, l_scales), _mm256_set_m128i(h_scales, h_scales)};
+        __m256i sumi = _mm256_setzero_si256();
+        for (int h = 0; h < 2; h++) {
+            __m256i q2bits = _mm256_loadu_si256((const __m256i*)q2);
+            q2 += 32;
+            __m256i p[4];
+            for (int t = 0; t < 4; t++) {
+                __m256i q8v = _mm256_loadu_si256((const __m256i*)q8);
+                q8 += 32;
+                __m256i q2v = _mm256_and_si256(_mm256_srl_epi16(q2bits, _mm_cvtsi32_si128(2 * t)), m3);
+                /* 16-bit scale 2t in the low 128 bits, 2t+1 in the high (get_scale_shuffle_q3k, avx.rs:118-129) */
+                __m256i shuf = _mm256_set_m128i(_mm_set1_epi16((short)(((4 * t + 3) << 8) | (4 * t + 2))),
+                                                _mm_set1_epi16((short)(((4 * t + 1) << 8) | (4 * t))));
+                p[t] = _mm256_madd_epi16(_mm256_shuffle_epi8(scales[h], shuf), _mm256_maddubs_epi16(q2v, q8v));
+            }
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(_mm256_add_epi32(p[0], p[1]), _mm256_add_epi32(p[2], p[3])));
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum_float_8(acc);
+}
 static float dot_q5k(int64_t n, const orc_block_q5k* xs, const orc_block_q8k* ys) {
     const uint32_t KMASK1 = 0x3f3f3f3f, KMASK2 = 0x0f0f0f0f, KMASK3 = 0x03030303;
     const __m256i m4 = _mm256_set1_epi8(0xF);
@@ -217,6 +259,7 @@ float orc_vec_dot_avx2(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q4_0: return dot_q4_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return dot_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return dot_q4k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
+        case ORC_Q2K: return dot_q2k(n, (const orc_block_q2k*)w, (const orc_block_q8k*)a);
         case ORC_Q5K: return dot_q5k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return dot_q6k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         default: return orc_vec_dot(dtype, n, w, a);

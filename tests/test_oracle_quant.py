@@ -64,7 +64,7 @@ def test_q4_0_matmul_known_answers(O, golden, simd):
     assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_neg_3_64_4"]["expected_rounded"]
 
 
-@pytest.mark.parametrize("name,dt", [("q4k_ramp", 12), ("q5k_ramp", 13), ("q6k_ramp", 14), ("q8k_ramp", 15)])
+@pytest.mark.parametrize("name,dt", [("q2k_ramp", 10), ("q4k_ramp", 12), ("q5k_ramp", 13), ("q6k_ramp", 14), ("q8k_ramp", 15)])
 def test_kquant_ramp_spot_values(O, golden, name, dt):
     g = golden[name]
     idx = golden["ramp_spot_indices"]
@@ -80,15 +80,15 @@ def test_kquant_ramp_spot_values(O, golden, name, dt):
         assert np.abs(dbig - big).max() < g["max_abs_err_bound_128"]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 10, 12, 13, 14, 15])
 def test_ggml_quantization_rmse(O, golden, dt):
     src = ggml_like(0.0)
     dst = O.dequantize(dt, O.quantize(dt, src), src.size)
     rmse = np.sqrt(np.sum((src - dst).astype(np.float32) ** 2, dtype=np.float32)) / src.size
-    assert rmse <= golden["ggml_quantization_rmse_bound"]["bound"]
+    assert rmse <= golden["ggml_quantization_rmse_bound"][{10: "bound_2bits", 11: "bound_3bits"}.get(dt, "bound")]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 10, 12, 13, 14, 15])
 def test_ggml_dot_error(O, golden, dt):
     # ggml_matmul_error_test, quantized_tests.rs:846-911
     g = golden["ggml_dot_error"]
@@ -114,7 +114,7 @@ def test_vec_dot_matches_dequantised_float64(O):
     # brute force: the integer block dot must equal the float dot of the dequantised operands
     rng = np.random.default_rng(3)
     n = 2048
-    for dt in (O.Q4_0, O.Q8_0, O.Q4K, O.Q5K, O.Q6K):
+    for dt in (O.Q4_0, O.Q8_0, O.Q2K, O.Q4K, O.Q5K, O.Q6K):
         w = rng.normal(0, 0.02, n).astype(np.float32)
         x = rng.normal(0, 1.0, n).astype(np.float32)
         wq, xq = O.quantize(dt, w), O.quantize(O.VECDOT[dt], x)
@@ -137,7 +137,7 @@ def test_seeded_matmul_spot_values(O, golden, simd):
     r3 = lambda a: [float(np.round(np.float32(1000.0) * np.float32(x)) / np.float32(1000.0)) for x in a]
     dense = (lhs.astype(np.float64) @ rhs.astype(np.float64).T).reshape(-1)
     assert r3(dense[pick]) == r3(g["dense"])  # validates the StdRng restatement itself
-    for key, dt in (("q4k", O.Q4K), ("q5k", O.Q5K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
+    for key, dt in (("q2k", O.Q2K), ("q4k", O.Q4K), ("q5k", O.Q5K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
         mm = O.matmul(dt, lhs, O.quantize(dt, rhs), n, simd=simd).reshape(-1)
         assert r3(mm[pick]) == r3(g[key])
 
@@ -304,3 +304,29 @@ def test_q5k_layout_against_independent_decoder(O):
     assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
     assert codes.min() == 0 and codes.max() == 31
     assert np.abs(got - x).max() < 0.02 * 8 / 31
+
+
+def test_q2k_layout_against_independent_decoder(O):
+    # independent numpy decoder of the published Q2_K layout, addressed by element: 16 bytes of
+    # (4-bit scale | 4-bit min << 4) per 16 elements, 64 bytes of 2-bit codes, f16 d and dmin.  Element e
+    # lies in half e//128, quarter q = (e%128)//32, column l = e%32: its code is bits 2q..2q+1 of
+    # qs[32*half + l], its scale byte is scales[e//16].
+    rng = np.random.default_rng(13)
+    x = rng.normal(0, 0.02, 1024).astype(np.float32)
+    blocks = O.quantize(O.Q2K, x).reshape(4, 84)
+    out = np.empty((4, 256), dtype=np.float32)
+    codes = np.empty((4, 256), dtype=np.int32)
+    for b in range(4):
+        raw = blocks[b]
+        sc, qs = raw[:16].astype(np.int32), raw[16:80].astype(np.int32)
+        d = np.float32(raw[80:82].view(np.float16)[0])
+        dmin = np.float32(raw[82:84].view(np.float16)[0])
+        for e in range(256):
+            half, q, l = e // 128, (e % 128) // 32, e % 32
+            codes[b, e] = (qs[32 * half + l] >> (2 * q)) & 3
+            s = sc[e // 16]
+            out[b, e] = (d * np.float32(s & 15)) * np.float32(codes[b, e]) - dmin * np.float32(s >> 4)
+    got = O.dequantize(O.Q2K, blocks.reshape(-1), 1024)
+    assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
+    assert codes.min() == 0 and codes.max() == 3
+    assert np.abs(got - x).max() < 0.02 * 8 / 3
