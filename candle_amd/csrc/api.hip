@@ -173,7 +173,7 @@ static int check_desc(const moe_desc* d) {
     const int dt = d->ggml_dtype, dtd = d->ggml_dtype_down ? d->ggml_dtype_down : dt;
     if (!weight_dtype_supported(dt) || !weight_dtype_supported(dtd))
         return fail(MOE_E_INVALID, "unsupported ggml_dtype " + std::to_string(weight_dtype_supported(dt) ? dtd : dt) +
-                                       " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q4K=12, Q5K=13, Q6K=14)");
+                                       " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
     // w2 consumes the intermediate in the activation format of its own dtype; the up kernels emit the one of dt
     if (vecdot_dtype(dt) != vecdot_dtype(dtd))
         return fail(MOE_E_INVALID, "ggml_dtype " + std::to_string(dt) + " and ggml_dtype_down " + std::to_string(dtd) +
@@ -615,7 +615,7 @@ extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, i
     if (rc) return rc;
     if (!out || !w_blocks) return fail(MOE_E_INVALID, "moe_qlinear_create: NULL pointer");
     if (!weight_dtype_supported(dt))
-        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q4K=12, Q5K=13, Q6K=14)");
+        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
     const int64_t be = block_elems(dt);
     if (n <= 0 || n % 16 || k <= 0 || k % be || k > (1 << 24))
         return fail(MOE_E_INVALID, "moe_qlinear_create: need n % 16 == 0 and k a multiple of the block size (" + std::to_string(be) + ")");

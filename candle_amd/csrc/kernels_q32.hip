@@ -554,7 +554,7 @@ hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s);
 hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     switch (p.dt) {
-        case MOE_GGML_Q2K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_up(p, s);
+        case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_up(p, s);
         case MOE_GGML_Q8_0: return launch_q32_up_t<MOE_GGML_Q8_0>(p, s);
         case MOE_GGML_Q4_0: return launch_q32_up_t<MOE_GGML_Q4_0>(p, s);
     }
@@ -563,7 +563,7 @@ hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s) {
 hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
     switch (p.dt_down ? p.dt_down : p.dt) {
-        case MOE_GGML_Q2K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_down(p, s);
+        case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_down(p, s);
         case MOE_GGML_Q8_0: return launch_q32_down_t<MOE_GGML_Q8_0>(p, s);
         case MOE_GGML_Q4_0: return launch_q32_down_t<MOE_GGML_Q4_0>(p, s);
     }

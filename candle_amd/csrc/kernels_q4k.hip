@@ -1,4 +1,4 @@
-// Grouped expert products over Q2K, Q4K, Q5K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
+// Grouped expert products over Q2K, Q3K, Q4K, Q5K and Q6K weights with Q8K activations (gfx950, wave64, int8 MFMA).
 //
 // Arithmetic restated from BlockQ4K::vec_dot, candle-core/src/quantized/k_quants.rs:1205-1285:
 // per 256-element super-block
@@ -276,6 +276,60 @@ __device__ inline void q6k_mac(const Q6KTile& w, const Q8KOperand& A, const floa
     }
 }
 
+// Q3K (BlockQ3K::vec_dot, k_quants.rs:927-1045): d * y.d * sum_j (sc_j - 32) * (code_j . q8_j), codes -4..3, one
+// signed 6-bit scale per 16 elements: the Q6K scheme with 3-bit unsigned codes (code + 4 = low two bits |
+// high bit << 2) and the offset -4 taken out through the activations' 16-element sums.
+struct Q3KTile {
+    uint4 q, sc;
+    uint2 qh;
+    uint32_t d;
+};
+__device__ inline Q3KTile load_q3k_tile(const uint8_t* tile, int lane) {
+    Q3KTile t;
+    t.q = gload_stream(tile, (uint32_t)lane * 16u);
+    typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 h = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) u32x2*>((gbytes)tile + 1024u + (uint32_t)lane * 8u));
+    t.qh = make_uint2(h.x, h.y);
+    t.sc = gload_stream(tile, 1536u + (uint32_t)(lane & 15) * 16u);
+    t.d = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>((gbytes)tile + 1792u + (uint32_t)(lane & 15) * 2u));
+    return t;
+}
+__device__ inline void q3k_mac(const Q3KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+    const uint32_t M3 = 0x03030303u, M1 = 0x01010101u;
+    const float d = __half2float(__ushort_as_half((unsigned short)w.d));
+    const uint32_t first = g < 2 ? 0xffffffffu : 0u, second = ~first;
+    const v4i zero = {0, 0, 0, 0};
+    v4i isum = {0, 0, 0, 0};
+    const uint32_t qw[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
+    const uint32_t sw[4] = {w.sc.x, w.sc.y, w.sc.z, w.sc.w};
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t q = qw[P], h = (P < 2 ? w.qh.x : w.qh.y) >> (4 * (P & 1));
+        const uint32_t lx = (q & M3) | ((h & M1) << 2), ly = ((q >> 2) & M3) | (((h >> 1) & M1) << 2);
+        const uint32_t hx = ((q >> 4) & M3) | (((h >> 2) & M1) << 2), hy = ((q >> 6) & M3) | (((h >> 3) & M1) << 2);
+        const long a_lo = pack64(A.a[P].x, A.a[P].y);
+        const long a_hi = pack64(A.a[P].z, A.a[P].w);
+        v4i D0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & first, ly & first), zero, 0, 0, 0);
+        v4i D1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & second, ly & second), zero, 0, 0, 0);
+        v4i D2 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & first, hy & first), zero, 0, 0, 0);
+        v4i D3 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & second, hy & second), zero, 0, 0, 0);
+        const int s0 = (int)(int8_t)(sw[P] & 0xffu), s1 = (int)(int8_t)((sw[P] >> 8) & 0xffu);
+        const int s2 = (int)(int8_t)((sw[P] >> 16) & 0xffu), s3 = (int)(int8_t)(sw[P] >> 24);
+#pragma unroll
+        for (int i = 0; i < 4; i++) isum[i] += __mul24(s0, D0[i]) + __mul24(s1, D1[i]) + __mul24(s2, D2[i]) + __mul24(s3, D3[i]);
+    }
+    const uint32_t sg = sw[g];
+    const v4h sB = {(_Float16)(int)(int8_t)(sg & 0xffu), (_Float16)(int)(int8_t)((sg >> 8) & 0xffu),
+                    (_Float16)(int)(int8_t)((sg >> 16) & 0xffu), (_Float16)(int)(int8_t)(sg >> 24)};
+    const v4f zf = {0.f, 0.f, 0.f, 0.f};
+    v4f Ds = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, sB, zf, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int tot = isum[i] - 4 * (int)Ds[i];
+        acc[i] += (d * yd[i]) * (float)tot;
+    }
+}
+
 // Weight formats of the engine below: tile type, bytes per (16 rows x 256 k) tile, load and multiply.
 struct FmtQ4K {
     typedef Q4KTile Tile;
@@ -288,6 +342,12 @@ struct FmtQ2K {
     static constexpr int TILE_BYTES = Q2K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q2k_tile(tile, lane); }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q2k_mac(w, A, yd, g, acc); }
+};
+struct FmtQ3K {
+    typedef Q3KTile Tile;
+    static constexpr int TILE_BYTES = Q3K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q3k_tile(tile, lane); }
+    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q3k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ5K {
     typedef Q5KTile Tile;
@@ -572,6 +632,13 @@ DEF_UP(q2k_up_t2, FmtQ2K, 2, 4, 2, 2)
 DEF_DOWN(q2k_down_t1, FmtQ2K, 1, 4, 2, 3)
 DEF_DOWN_NARROW(q2k_down_t1_narrow, FmtQ2K, 8, 2, 4)
 DEF_DOWN(q2k_down_t2, FmtQ2K, 2, 4, 2, 2)
+// Q3K: eleven registers per tile, sixteen MFMAs per tile and operand like Q6K
+DEF_UP(q3k_up_t1, FmtQ3K, 1, 4, 2, 3)
+DEF_UP_NARROW(q3k_up_t1_narrow, FmtQ3K, 4, 2, 3)
+DEF_UP(q3k_up_t2, FmtQ3K, 2, 4, 2, 2)
+DEF_DOWN(q3k_down_t1, FmtQ3K, 1, 4, 2, 3)
+DEF_DOWN_NARROW(q3k_down_t1_narrow, FmtQ3K, 8, 2, 3)
+DEF_DOWN(q3k_down_t2, FmtQ3K, 2, 4, 2, 2)
 // Q5K: the Q4K variants with two more registers per tile; one and two slot tiles per pass
 DEF_UP(q5k_up_t1, FmtQ5K, 1, 4, 2, 3)
 DEF_UP_NARROW(q5k_up_t1_narrow, FmtQ5K, 4, 2, 3)
@@ -605,10 +672,12 @@ static const KernelFamily* kernel_family(int dt) {
     static const KernelFamily q4k = {uv == 0 ? q4k_up_t1_v0 : q4k_up_t1_v1, q4k_up_t1_narrow, q4k_up_t2, q4k_up_t4,
                                      dv == 0 ? q4k_down_t1_v0 : q4k_down_t1_v1, q4k_down_t1_narrow, q4k_down_t2, q4k_down_t4};
     static const KernelFamily q2k = {q2k_up_t1, q2k_up_t1_narrow, q2k_up_t2, nullptr, q2k_down_t1, q2k_down_t1_narrow, q2k_down_t2, nullptr};
+    static const KernelFamily q3k = {q3k_up_t1, q3k_up_t1_narrow, q3k_up_t2, nullptr, q3k_down_t1, q3k_down_t1_narrow, q3k_down_t2, nullptr};
     static const KernelFamily q5k = {q5k_up_t1, q5k_up_t1_narrow, q5k_up_t2, nullptr, q5k_down_t1, q5k_down_t1_narrow, q5k_down_t2, nullptr};
     static const KernelFamily q6k = {q6k_up_t1, q6k_up_t1_narrow, q6k_up_t2, nullptr, q6k_down_t1, q6k_down_t1_narrow, q6k_down_t2, nullptr};
     switch (dt) {
         case MOE_GGML_Q2K: return &q2k;
+        case MOE_GGML_Q3K: return &q3k;
         case MOE_GGML_Q4K: return &q4k;
         case MOE_GGML_Q5K: return &q5k;
         case MOE_GGML_Q6K: return &q6k;

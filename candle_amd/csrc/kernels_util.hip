@@ -1,7 +1,7 @@
 // Layout and format kernels: re-laying GGML blocks into the tiled device layout, `to_float`
 // from either layout, and the stand-alone activation quantiser used by the parity hooks.
 //
-// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0), 872-908 (Q2K),
+// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0), 872-908 (Q2K), 1131-1186 (Q3K),
 // 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1563-1595 (Q5K), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
 #include <algorithm>
@@ -38,6 +38,22 @@ __device__ inline float q4k_value(const uint8_t* hdr, int i, uint8_t qbyte) {
 __device__ inline float q2k_value(float d, float mn, uint8_t sc, int code) {
     const float dl = d * (float)(sc & 0xF), ml = mn * (float)(sc >> 4);
     return dl * (float)code - ml;
+}
+
+// Q3K: the sixteen 6-bit scales of a raw block (low nibbles in scales[0..8), two per byte; high bit pairs in
+// scales[8..12): the KMASK shuffle of k_quants.rs:1137-1145), and a code (-4..3) from its bit fields
+__device__ inline int q3k_scale_raw(const uint8_t* scales, int j) {
+    const int lo = j < 8 ? (scales[j] & 0xF) : (scales[j - 8] >> 4);
+    return lo | (((scales[8 + j % 4] >> (2 * (j / 4))) & 3) << 4);
+}
+__device__ inline int q3k_code_raw(const uint8_t* blk, int e) {
+    const int G = e / 32, l = e % 32;
+    return ((blk[32 + 32 * (G / 4) + l] >> (2 * (G % 4))) & 3) - (((blk[l] >> G) & 1) ? 0 : 4);
+}
+// to_float of one Q3K element, k_quants.rs:1160-1172: `d_all * (scale as f32 - 32.0)`, then times the code
+__device__ inline float q3k_value(float d, int8_t scale_minus_32, int code) {
+    const float dl = d * (float)scale_minus_32;
+    return dl * (float)code;
 }
 
 // value of element `i` of a Q5K block: header as Q4K, nibble byte, fifth bit (k_quants.rs:1582-1591:
@@ -77,6 +93,10 @@ __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, in
         int e = (int)(i % 256);
         int code = (b[16 + 32 * (e / 128) + e % 32] >> (2 * ((e % 128) / 32))) & 3;
         out[i] = q2k_value(f16_bits_to_f32((uint16_t)(b[80] | (b[81] << 8))), f16_bits_to_f32((uint16_t)(b[82] | (b[83] << 8))), b[e / 16], code);
+    } else if (dt == MOE_GGML_Q3K) {
+        const uint8_t* b = blocks + (i / 256) * 110;
+        int e = (int)(i % 256);
+        out[i] = q3k_value(f16_bits_to_f32((uint16_t)(b[108] | (b[109] << 8))), (int8_t)(q3k_scale_raw(b + 96, e / 16) - 32), q3k_code_raw(b, e));
     } else if (dt == MOE_GGML_Q5K) {
         const uint8_t* b = blocks + (i / 256) * 176;
         int e = (int)(i % 256);
@@ -147,6 +167,38 @@ __global__ void relayout_q2k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t 
     if (g == 0) {
         for (int j = 0; j < 16; j++) dst[1024 + r * 16 + j] = blk[j];
         for (int j = 0; j < 4; j++) dst[1280 + r * 4 + j] = blk[80 + j];
+    }
+}
+
+__global__ void relayout_q3k_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nsb) {
+    // one thread per (tile, lane): 16 bytes of low bits, 8 bytes of high bits; lanes < 16 also decode the row's scales
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nsb * 64) return;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int64_t rt = tile / nsb;
+    int sb = (int)(tile % nsb);
+    const uint8_t* blk = raw + ((rt * 16 + r) * nsb + sb) * 110;
+    uint8_t* dst = tiled + (sb * n_rt + rt) * Q3K_TILE_BYTES;  // tiles ordered [sb][rt]
+    auto cu = [&](int e) { return q3k_code_raw(blk, e) + 4; };   // 0..7: low two bits | high bit << 2
+    for (int P = 0; P < 4; P++)
+        for (int i = 0; i < 4; i++) {
+            const int e = 64 * P + 8 * g + i;
+            dst[l * 16 + P * 4 + i] = (uint8_t)((cu(e) & 3) | ((cu(e + 4) & 3) << 2) | ((cu(e + 32) & 3) << 4) | ((cu(e + 36) & 3) << 6));
+        }
+    for (int w = 0; w < 2; w++)
+        for (int i = 0; i < 4; i++) {
+            int byte = 0;
+            for (int q = 0; q < 2; q++) {
+                const int e = 64 * (2 * w + q) + 8 * g + i;
+                byte |= ((cu(e) >> 2) | ((cu(e + 4) >> 2) << 1) | ((cu(e + 32) >> 2) << 2) | ((cu(e + 36) >> 2) << 3)) << (4 * q);
+            }
+            dst[1024 + l * 8 + w * 4 + i] = (uint8_t)byte;
+        }
+    if (g == 0) {
+        for (int j = 0; j < 16; j++) dst[1536 + r * 16 + j] = (uint8_t)(int8_t)(q3k_scale_raw(blk + 96, j) - 32);
+        dst[1792 + 2 * r] = blk[108];
+        dst[1792 + 2 * r + 1] = blk[109];
     }
 }
 
@@ -263,6 +315,15 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         const uint8_t* dd = tile + 1280 + r * 4;
         out[i] = q2k_value(f16_bits_to_f32((uint16_t)(dd[0] | (dd[1] << 8))), f16_bits_to_f32((uint16_t)(dd[2] | (dd[3] << 8))),
                            tile[1024 + r * 16 + e / 16], code);
+    } else if (dt == MOE_GGML_Q3K) {
+        int sb = col / 256, e = col % 256;
+        const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q3K_TILE_BYTES;
+        int P = e / 64, sub = (e % 64) / 32, g = (e % 32) / 8, pos = e % 8;
+        int l = g * 16 + r;
+        int low = (tile[l * 16 + P * 4 + pos % 4] >> (2 * (2 * sub + pos / 4))) & 3;
+        int hb = (tile[1024 + l * 8 + (P / 2) * 4 + pos % 4] >> ((P % 2) * 4 + sub * 2 + pos / 4)) & 1;
+        float d = f16_bits_to_f32((uint16_t)(tile[1792 + 2 * r] | (tile[1792 + 2 * r + 1] << 8)));
+        out[i] = q3k_value(d, (int8_t)tile[1536 + r * 16 + e / 16], low - (hb ? 0 : 4));
     } else if (dt == MOE_GGML_Q5K) {
         int sb = col / 256, e = col % 256;
         const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q5K_TILE_BYTES;
@@ -358,6 +419,8 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
         hipLaunchKernelGGL(relayout_q4k_kernel, dim3(nblk(n_rt * nkb * 144, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q2K)
         hipLaunchKernelGGL(relayout_q2k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (dt == MOE_GGML_Q3K)
+        hipLaunchKernelGGL(relayout_q3k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q5K)
         hipLaunchKernelGGL(relayout_q5k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q6K)

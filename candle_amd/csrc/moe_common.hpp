@@ -24,13 +24,13 @@ int fail(int code, const std::string& msg);
 int ensure_device();  // 0 if a gfx950 device is usable
 
 // ---------------------------------------------------------------- GGML block formats
-// Sizes per candle-core/src/quantized/k_quants.rs:45-51 (Q4_0), 81-87 (Q8_0), 98-106 (Q2K), 118-127 (Q4K),
+// Sizes per candle-core/src/quantized/k_quants.rs:45-51 (Q4_0), 81-87 (Q8_0), 98-106 (Q2K), 108-116 (Q3K), 118-127 (Q4K),
 // 129-137 (Q5K), 142-149 (Q6K), 151-158 (Q8K).
 constexpr int QK_K = 256;
 inline int64_t block_elems(int dt) {
     switch (dt) {
         case MOE_GGML_Q4_0: case MOE_GGML_Q8_0: return 32;
-        case MOE_GGML_Q2K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: case MOE_GGML_Q8K: return 256;
+        case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: case MOE_GGML_Q8K: return 256;
         default: return -1;
     }
 }
@@ -39,6 +39,7 @@ inline int64_t block_bytes(int dt) {
         case MOE_GGML_Q4_0: return 18;
         case MOE_GGML_Q8_0: return 34;
         case MOE_GGML_Q2K: return 84;
+        case MOE_GGML_Q3K: return 110;
         case MOE_GGML_Q4K: return 144;
         case MOE_GGML_Q5K: return 176;
         case MOE_GGML_Q6K: return 210;
@@ -47,10 +48,10 @@ inline int64_t block_bytes(int dt) {
     }
 }
 inline int vecdot_dtype(int dt) {  // GgmlType::VecDotType, k_quants.rs:163,584,1189,1600
-    return (dt == MOE_GGML_Q2K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K || dt == MOE_GGML_Q8K) ? MOE_GGML_Q8K : MOE_GGML_Q8_0;
+    return (dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K || dt == MOE_GGML_Q8K) ? MOE_GGML_Q8K : MOE_GGML_Q8_0;
 }
 inline bool weight_dtype_supported(int dt) {
-    return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K;
+    return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K;
 }
 
 // ---------------------------------------------------------------- device layouts
@@ -71,6 +72,11 @@ inline bool weight_dtype_supported(int dt) {
 //                     elements 64P + 8g + i / + 4, bits 5:4 / 7:6 = codes of elements 64P + 32 + 8g + i / + 4
 //         [1024,1280) row r : the 16 (scale | min << 4) bytes, one per 16 elements
 //         [1280,1344) row r : d, dmin (f16 each)
+//  Q3K  tile(rt, sb) = 1824 B, ordered [sb][rt]:
+//         [0,1024)    lane l: the low two bits of the codes, placed as in the Q2K tile
+//         [1024,1536) lane l: 8 bytes of high bits, placed as the fifth bits of the Q5K tile (set = no -4)
+//         [1536,1792) row r : the sixteen scales, decoded to i8 (stored value - 32)
+//         [1792,1824) row r : d (f16)
 //  Q5K  tile(rt, sb) = 2816 B: the Q4K tile (nibbles, then d / dmin / scales of the 16 rows) followed by
 //         [2304,2816) lane l: 8 bytes of fifth bits; byte i of word w (0..3, 0..1) holds, for pair 2w in
 //                     bits 0..3 and pair 2w+1 in bits 4..7: the bits of elements 8g+i and 8g+4+i of the
@@ -92,7 +98,7 @@ inline bool weight_dtype_supported(int dt) {
 //       MFMA k-chunk g of a Q4_0 block covers elements {0-7, 16-23, 8-15, 24-31}[g]: low / high
 //       nibbles of byte half g>>1 ... see experts_q32.hip.
 //
-// ACTIVATIONS are quantised exactly as the reference does (Q8K for Q2K, Q4K, Q5K and Q6K weights, Q8_0
+// ACTIVATIONS are quantised exactly as the reference does (Q8K for Q2K ... Q6K weights, Q8_0
 // otherwise) and stored per row as
 //  Q8K  qs[K] with element k at ((k/64)*64 + ((k%32)/8)*16 + ((k/32)%2)*8 + k%8), so that lane
 //       (row, g) fetches sub-blocks 2P and 2P+1, chunk g, with one 16-byte load;
@@ -101,6 +107,7 @@ inline bool weight_dtype_supported(int dt) {
 //       bsum[K/32] i32 = sum of the block's 32 quants (used for Q4_0's -8 offset).
 constexpr int Q4K_TILE_BYTES = 2304;
 constexpr int Q2K_TILE_BYTES = 1344;
+constexpr int Q3K_TILE_BYTES = 1824;
 constexpr int Q5K_TILE_BYTES = 2816;
 constexpr int Q6K_TILE_BYTES = 3360;
 constexpr int Q8_0_TILE_BYTES = 544;
@@ -110,6 +117,7 @@ inline int64_t tile_bytes(int dt) {
     switch (dt) {
         case MOE_GGML_Q4K: return Q4K_TILE_BYTES;
         case MOE_GGML_Q2K: return Q2K_TILE_BYTES;
+        case MOE_GGML_Q3K: return Q3K_TILE_BYTES;
         case MOE_GGML_Q5K: return Q5K_TILE_BYTES;
         case MOE_GGML_Q6K: return Q6K_TILE_BYTES;
         case MOE_GGML_Q8_0: return Q8_0_TILE_BYTES;

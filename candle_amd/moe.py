@@ -11,8 +11,8 @@ import os
 
 import numpy as np
 
-GGML_Q4_0, GGML_Q8_0, GGML_Q2K, GGML_Q4K, GGML_Q5K, GGML_Q6K, GGML_Q8K = 2, 8, 10, 12, 13, 14, 15
-_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q2K: (256, 84), GGML_Q4K: (256, 144), GGML_Q5K: (256, 176), GGML_Q6K: (256, 210),
+GGML_Q4_0, GGML_Q8_0, GGML_Q2K, GGML_Q3K, GGML_Q4K, GGML_Q5K, GGML_Q6K, GGML_Q8K = 2, 8, 10, 11, 12, 13, 14, 15
+_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q2K: (256, 84), GGML_Q3K: (256, 110), GGML_Q4K: (256, 144), GGML_Q5K: (256, 176), GGML_Q6K: (256, 210),
           GGML_Q8K: (256, 292)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))

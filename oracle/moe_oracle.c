@@ -97,7 +97,7 @@ static inline float rmin(float a, float b) { return fminf(a, b); }
 int64_t orc_block_elems(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return 32;
-        case ORC_Q2K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
+        case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
         default: return -1;
     }
 }
@@ -106,6 +106,7 @@ int64_t orc_block_bytes(int dtype) {
         case ORC_Q4_0: return 18;
         case ORC_Q8_0: return 34;
         case ORC_Q2K: return 84;
+        case ORC_Q3K: return 110;
         case ORC_Q4K: return 144;
         case ORC_Q5K: return 176;
         case ORC_Q6K: return 210;
@@ -116,7 +117,7 @@ int64_t orc_block_bytes(int dtype) {
 int orc_vecdot_dtype(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
-        case ORC_Q2K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
+        case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
         default: return -1;
     }
 }
@@ -472,6 +473,175 @@ static float vec_dot_q2k_q8k(int64_t n, const orc_block_q2k* xs, const orc_block
         sumf += dall * (float)isum - dmin * (float)summs;
     }
     return sumf;
+}
+
+/* ------------------------------------------------------------------ Q3K */
+/* make_q3_quants, utils.rs:262-328 */
+static float make_q3_quants(const float* x, int n, int nmax, int do_rmse) {
+    int8_t l[16];
+    float max = 0.f, amax = 0.f;
+    for (int i = 0; i < n; i++) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) { amax = ax; max = x[i]; }
+    }
+    if (amax == 0.f) return 0.f;
+    float iscale = -(float)nmax / max;
+    if (do_rmse) {
+        float sumlx = 0.f, suml2 = 0.f;
+        for (int i = 0; i < n; i++) {
+            int32_t li = nearest_int(iscale * x[i]);
+            li = li < -nmax ? -nmax : li > nmax - 1 ? nmax - 1 : li;
+            l[i] = (int8_t)li;
+            float w = x[i] * x[i];
+            sumlx += w * x[i] * (float)li;
+            suml2 += w * (float)(li * li);
+        }
+        for (int t = 0; t < 5; t++) {
+            int n_changed = 0;
+            for (int i = 0; i < n; i++) {
+                float w = x[i] * x[i];
+                float slx = sumlx - w * x[i] * (float)l[i];
+                if (slx > 0.f) {
+                    float sl2 = suml2 - w * (float)((int32_t)l[i] * (int32_t)l[i]);
+                    int32_t new_l = nearest_int(x[i] * sl2 / slx);
+                    new_l = new_l < -nmax ? -nmax : new_l > nmax - 1 ? nmax - 1 : new_l;
+                    if (new_l != (int32_t)l[i]) {
+                        slx += w * x[i] * (float)new_l;
+                        sl2 += w * (float)(new_l * new_l);
+                        if (sl2 > 0.f && slx * slx * suml2 > sumlx * sumlx * sl2) {
+                            l[i] = (int8_t)new_l;
+                            sumlx = slx;
+                            suml2 = sl2;
+                            n_changed++;
+                        }
+                    }
+                }
+            }
+            if (n_changed == 0) break;
+        }
+        return sumlx / suml2;
+    }
+    return 1.0f / iscale;
+}
+/* the sixteen 6-bit scales (stored + 32) of a block: low four bits in scales[0..8) (two per byte), high
+ * two bits in scales[8..12) -- the KMASK shuffle of k_quants.rs:1013-1019 / 1137-1145 */
+static inline int q3k_scale(const uint8_t* scales, int j) {
+    int lo = j < 8 ? (scales[j] & 0xF) : (scales[j - 8] >> 4);
+    int hi = (scales[8 + j % 4] >> (2 * (j / 4))) & 3;
+    return lo | (hi << 4);
+}
+/* k_quants.rs:1047-1129 */
+static void quantize_q3k(const float* xs, int64_t k, orc_block_q3k* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const float* x = xs + b * 256;
+        orc_block_q3k* block = &ys[b];
+        float scales[16];
+        for (int j = 0; j < 16; j++) scales[j] = make_q3_quants(x + 16 * j, 16, 4, 1);
+        float max_scale = 0.f;
+        for (int j = 0; j < 16; j++)
+            if (fabsf(scales[j]) > fabsf(max_scale)) max_scale = scales[j];
+        memset(block->scales, 0, sizeof block->scales);
+        if (max_scale != 0.f) {
+            float iscale = -32.0f / max_scale;
+            for (int j = 0; j < 16; j++) {
+                int32_t lv = nearest_int(iscale * scales[j]);
+                lv = (lv < -32 ? -32 : lv > 31 ? 31 : lv) + 32;
+                if (j < 8) block->scales[j] = (uint8_t)(lv & 0xF);
+                else block->scales[j - 8] |= (uint8_t)((lv & 0xF) << 4);
+                lv >>= 4;
+                block->scales[j % 4 + 8] |= (uint8_t)(lv << (2 * (j / 4)));
+            }
+            block->d = orc_f32_to_f16(1.0f / iscale);
+        } else {
+            block->d = orc_f32_to_f16(0.f);
+        }
+        int8_t l[256];
+        memset(l, 0, sizeof l);
+        for (int j = 0; j < 16; j++) {
+            int sc = q3k_scale(block->scales, j) - 32;
+            float d = orc_f16_to_f32(block->d) * (float)sc;
+            if (d != 0.f)
+                for (int ii = 0; ii < 16; ii++) {
+                    int32_t lv = nearest_int(x[16 * j + ii] / d);
+                    l[16 * j + ii] = (int8_t)((lv < -4 ? -4 : lv > 3 ? 3 : lv) + 4);
+                }
+        }
+        memset(block->hmask, 0, sizeof block->hmask);
+        int m = 0;
+        uint8_t hm = 1;
+        for (int i = 0; i < 256; i++) {
+            if (l[i] > 3) { block->hmask[m] |= hm; l[i] -= 4; }
+            if (++m == 32) { m = 0; hm <<= 1; }
+        }
+        for (int j = 0; j < 256; j += 128)
+            for (int lv = 0; lv < 32; lv++)
+                block->qs[j / 4 + lv] = (uint8_t)(l[j + lv] | (l[j + lv + 32] << 2) | (l[j + lv + 64] << 4) | (l[j + lv + 96] << 6));
+    }
+}
+/* k_quants.rs:1131-1186 */
+static void dequantize_q3k(const orc_block_q3k* xs, int64_t k, float* ys) {
+    for (int64_t b = 0; b < k / 256; b++) {
+        const orc_block_q3k* block = &xs[b];
+        float d_all = orc_f16_to_f32(block->d);
+        uint8_t m = 1;
+        int is = 0;
+        for (int n = 0; n < 256; n += 128) {
+            const uint8_t* qs = block->qs + n / 4;
+            float* y = ys + b * 256 + n;
+            int shift = 0;
+            for (int j = 0; j < 4; j++) {
+                for (int half = 0; half < 2; half++) {
+                    float dl = d_all * ((float)(int8_t)q3k_scale(block->scales, is) - 32.0f);
+                    for (int i = 0; i < 16; i++) {
+                        int8_t q = (int8_t)((int8_t)((qs[i + 16 * half] >> shift) & 3) - ((block->hmask[i + 16 * half] & m) == 0 ? 4 : 0));
+                        y[32 * j + 16 * half + i] = dl * (float)q;
+                    }
+                    is++;
+                }
+                shift += 2;
+                m <<= 1;
+            }
+        }
+    }
+}
+/* k_quants.rs:927-1045 (vec_dot_unopt) */
+static float vec_dot_q3k_q8k(int64_t n, const orc_block_q3k* xs, const orc_block_q8k* ys) {
+    int8_t aux8[256];
+    int16_t aux16[8];
+    float sums[8] = {0};
+    int32_t aux32[8];
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q3k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        memset(aux32, 0, sizeof aux32);
+        int8_t* a = aux8;
+        const uint8_t* q3 = x->qs;
+        uint8_t m = 1;
+        for (int h = 0; h < 2; h++) {
+            for (int sh = 0; sh < 8; sh += 2) {
+                for (int l = 0; l < 32; l++) a[l] = (int8_t)(((q3[l] >> sh) & 3) - ((x->hmask[l] & m) ? 0 : 4));
+                a += 32;
+                m <<= 1;
+            }
+            q3 += 32;
+        }
+        a = aux8;
+        const int8_t* q8 = y->qs;
+        for (int j = 0; j < 16; j++) {
+            int32_t scale = (int32_t)(int8_t)q3k_scale(x->scales, j) - 32;
+            for (int r = 0; r < 2; r++) {
+                for (int l = 0; l < 8; l++) aux16[l] = (int16_t)((int16_t)q8[l] * (int16_t)a[l]);
+                for (int l = 0; l < 8; l++) aux32[l] += scale * (int32_t)aux16[l];
+                q8 += 8;
+                a += 8;
+            }
+        }
+        float d = orc_f16_to_f32(x->d) * y->d;
+        for (int l = 0; l < 8; l++) sums[l] += d * (float)aux32[l];
+    }
+    float total = 0.f;
+    for (int l = 0; l < 8; l++) total += sums[l];
+    return total;
 }
 
 /* ------------------------------------------------------------------ Q5K */
@@ -883,6 +1053,7 @@ int orc_quantize(int dtype, const float* x, int64_t n, void* blocks) {
         case ORC_Q8_0: quantize_q8_0(x, n, (orc_block_q8_0*)blocks); return 0;
         case ORC_Q4K: memset(blocks, 0, (size_t)(n / 256) * 144); quantize_q4k(x, n, (orc_block_q4k*)blocks); return 0;
         case ORC_Q2K: memset(blocks, 0, (size_t)(n / 256) * 84); quantize_q2k(x, n, (orc_block_q2k*)blocks); return 0;
+        case ORC_Q3K: memset(blocks, 0, (size_t)(n / 256) * 110); quantize_q3k(x, n, (orc_block_q3k*)blocks); return 0;
         case ORC_Q5K: memset(blocks, 0, (size_t)(n / 256) * 176); quantize_q5k(x, n, (orc_block_q5k*)blocks); return 0;
         case ORC_Q6K: memset(blocks, 0, (size_t)(n / 256) * 210); quantize_q6k(x, n, (orc_block_q6k*)blocks); return 0;
         case ORC_Q8K: quantize_q8k(x, n, (orc_block_q8k*)blocks); return 0;
@@ -897,6 +1068,7 @@ int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y) {
         case ORC_Q8_0: dequantize_q8_0((const orc_block_q8_0*)blocks, n, y); return 0;
         case ORC_Q4K: dequantize_q4k((const orc_block_q4k*)blocks, n, y); return 0;
         case ORC_Q2K: dequantize_q2k((const orc_block_q2k*)blocks, n, y); return 0;
+        case ORC_Q3K: dequantize_q3k((const orc_block_q3k*)blocks, n, y); return 0;
         case ORC_Q5K: dequantize_q5k((const orc_block_q5k*)blocks, n, y); return 0;
         case ORC_Q6K: dequantize_q6k((const orc_block_q6k*)blocks, n, y); return 0;
         case ORC_Q8K: dequantize_q8k((const orc_block_q8k*)blocks, n, y); return 0;
@@ -909,6 +1081,7 @@ float orc_vec_dot(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q8_0: return vec_dot_q8_0_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return vec_dot_q4k_q8k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
         case ORC_Q2K: return vec_dot_q2k_q8k(n, (const orc_block_q2k*)w, (const orc_block_q8k*)a);
+        case ORC_Q3K: return vec_dot_q3k_q8k(n, (const orc_block_q3k*)w, (const orc_block_q8k*)a);
         case ORC_Q5K: return vec_dot_q5k_q8k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return vec_dot_q6k_q8k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         case ORC_Q8K: return vec_dot_q8k_q8k(n, (const orc_block_q8k*)w, (const orc_block_q8k*)a);

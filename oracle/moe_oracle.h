@@ -16,6 +16,8 @@
  *                          (11,512,21) mat-mul spot values of :1102-1121 through a restated rand-0.9 StdRng
  *   q2k  quantize/dequant  spot values and error bounds of quantized_tests.rs:471-517, ggml dot error :821-911,
  *                          the seeded (11,512,21) mat-mul spot values of :1048-1074, independent decoder
+ *   q3k  quantize/dequant  spot values and error bounds of quantized_tests.rs:519-563, ggml dot error :821-911,
+ *                          the seeded (11,512,21) mat-mul spot values of :1076-1100, independent decoder
  *   q5k  quantize/dequant  spot values and error bounds of quantized_tests.rs:613-658, ggml dot error :821-911,
  *                          the seeded (11,512,21) mat-mul spot values of :1129-1152, independent decoder
  *   q6k  quantize/dequant  spot values and error bound of quantized_tests.rs:660-700, ggml dot error :821-911,
@@ -40,13 +42,14 @@ extern "C" {
 #endif
 
 /* ggml dtype numbering: candle-core/src/quantized/mod.rs:153-174 */
-enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q2K = 10, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14, ORC_Q8K = 15 };
+enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14, ORC_Q8K = 15 };
 
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } orc_block_q4_0;            /* k_quants.rs:45-51  */
 typedef struct { uint16_t d; int8_t qs[32]; } orc_block_q8_0;             /* k_quants.rs:81-87  */
 typedef struct { uint16_t d, dmin; uint8_t scales[12]; uint8_t qs[128]; } orc_block_q4k; /* :118-127 */
 typedef struct { uint8_t scales[16]; uint8_t qs[64]; uint16_t d, dmin; } orc_block_q2k;   /* k_quants.rs:98-106 */
+typedef struct { uint8_t hmask[32]; uint8_t qs[64]; uint8_t scales[12]; uint16_t d; } orc_block_q3k; /* k_quants.rs:108-116 */
 typedef struct { uint16_t d, dmin; uint8_t scales[12]; uint8_t qh[32]; uint8_t qs[128]; } orc_block_q5k; /* :129-137 */
 typedef struct { uint8_t ql[128]; uint8_t qh[64]; int8_t scales[16]; uint16_t d; } orc_block_q6k; /* :142-149 */
 typedef struct { float d; int8_t qs[256]; int16_t bsums[16]; } orc_block_q8k;            /* :151-158 */
@@ -62,18 +65,18 @@ int64_t orc_block_bytes(int dtype);
 /* VecDotType of a weight dtype: k_quants.rs:163,584,1189 */
 int     orc_vecdot_dtype(int dtype);
 
-/* from_float / to_float: k_quants.rs:166-224 (Q4_0), 587-634 (Q8_0), 808-908 (Q2K), 1287-1374 (Q4K), 1487-1595 (Q5K), 1673-1790 (Q6K),
+/* from_float / to_float: k_quants.rs:166-224 (Q4_0), 587-634 (Q8_0), 808-908 (Q2K), 1047-1186 (Q3K), 1287-1374 (Q4K), 1487-1595 (Q5K), 1673-1790 (Q6K),
  * 1819-1871 (Q8K).
  * n must be a multiple of the block size.  Return 0 or -1 (bad dtype / size). */
 int orc_quantize(int dtype, const float* x, int64_t n, void* blocks);
 int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y);
 
-/* vec_dot_unopt: k_quants.rs:241-258, 650-668, 755-805 (Q2K), 1205-1285, 1394-1485 (Q5K), 1613-1671 (Q6K) */
+/* vec_dot_unopt: k_quants.rs:241-258, 650-668, 755-805 (Q2K), 927-1045 (Q3K), 1205-1285, 1394-1485 (Q5K), 1613-1671 (Q6K) */
 float orc_vec_dot(int dtype, int64_t n, const void* w_blocks, const void* act_blocks);
 
 /* k_quants::matmul, k_quants.rs:1873-1920: dst[m,n] = lhs[m,k] . rhs_t[n,k]^T, lhs quantised
  * row by row to the VecDotType.  simd=0 uses vec_dot_unopt, simd=1 the AVX2 loops that restate
- * candle-core/src/quantized/avx.rs:50-87,131-216,224-304,443-638 (falls back to 0 if the CPU lacks AVX2+FMA).
+ * candle-core/src/quantized/avx.rs:50-87,131-216,224-441,443-638 (falls back to 0 if the CPU lacks AVX2+FMA).
  * threads<=1 runs serially; otherwise output columns are split over threads as rayon does. */
 int orc_matmul(int dtype, int64_t m, int64_t k, int64_t n, const float* lhs, const void* rhs_t,
                float* dst, int simd, int threads);

@@ -7,6 +7,7 @@
  *   vec_dot_q8_0_q8_0  candle-core/src/quantized/avx.rs:71-87
  *   vec_dot_q4k_q8k    candle-core/src/quantized/avx.rs:443-525
  *   vec_dot_q2k_q8k    candle-core/src/quantized/avx.rs:224-304
+ *   vec_dot_q3k_q8k    candle-core/src/quantized/avx.rs:306-441
  *   vec_dot_q5k_q8k    candle-core/src/quantized/avx.rs:527-638
  *   vec_dot_q6k_q8k    candle-core/src/quantized/avx.rs:131-216
  * The integer parts are exact; the f32 accumulation order differs from the scalar
@@ -153,6 +154,52 @@ static float dot_q2k(int64_t n, const orc_block_q2k* xs, const orc_block_q8k* ys
     }
     return hsum_float_8(acc);
 }
+static float dot_q3k(int64_t n, const orc_block_q3k* xs, const orc_block_q8k* ys) {
+    const uint32_t KMASK1 = 0x03030303, KMASK2 = 0x0f0f0f0f;
+    const __m256i m3 = _mm256_set1_epi8(3), mone = _mm256_set1_epi8(1);
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t b = 0; b < n / 256; b++) {
+        const orc_block_q3k* x = &xs[b];
+        const orc_block_q8k* y = &ys[b];
+        float d = y->d * orc_f16_to_f32(x->d);
+        const uint8_t* q3 = x->qs;
+        const int8_t* q8 = y->qs;
+        uint32_t aux[3];
+        memcpy(aux, x->scales, 12);
+        __m128i scales128 = _mm_set_epi32((int)(((aux[1] >> 4) & KMASK2) | (((aux[2] >> 6) & KMASK1) << 4)),
+                                          (int)(((aux[0] >> 4) & KMASK2) | (((aux[2] >> 4) & KMASK1) << 4)),
+                                          (int)((aux[1] & KMASK2) | (((aux[2] >> 2) & KMASK1) << 4)),
+                                          (int)((aux[0] & KMASK2) | ((aux[2] & KMASK1) << 4)));
+        scales128 = _mm_sub_epi8(scales128, _mm_set1_epi8(32));
+        __m256i all_scales = _mm256_cvtepi8_epi16(scales128);
+        __m128i l_scales = _mm256_extracti128_si256(all_scales, 0);
+        __m128i h_scales = _mm256_extracti128_si256(all_scales, 1);
+        __m256i scales[2] = {_mm256_set_m128i(l_scales, l_scales), _mm256_set_m128i(h_scales, h_scales)};
+        __m256i hbits = _mm256_loadu_si256((const __m256i*)x->hmask);
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < 2; j++) {
+            __m256i q3bits = _mm256_loadu_si256((const __m256i*)q3);
+            q3 += 32;
+            __m256i p[4];
+            for (int t = 0; t < 4; t++) {
+                const int bit = 4 * j + t;
+                __m256i q3l = _mm256_and_si256(_mm256_srl_epi16(q3bits, _mm_cvtsi32_si128(2 * t)), m3);
+                /* 4 where the high bit is NOT set, else 0 */
+                __m256i q3h = _mm256_slli_epi16(
+                    _mm256_srl_epi16(_mm256_andnot_si256(hbits, _mm256_sll_epi16(mone, _mm_cvtsi32_si128(bit))), _mm_cvtsi32_si128(bit)), 2);
+                __m256i q8v = _mm256_loadu_si256((const __m256i*)q8);
+                q8 += 32;
+                __m256i p16 = _mm256_sub_epi16(_mm256_maddubs_epi16(q3l, q8v), _mm256_maddubs_epi16(q3h, q8v));
+                __m256i shuf = _mm256_set_m128i(_mm_set1_epi16((short)(((4 * t + 3) << 8) | (4 * t + 2))),
+                                                _mm_set1_epi16((short)(((4 * t + 1) << 8) | (4 * t))));
+                p[t] = _mm256_madd_epi16(_mm256_shuffle_epi8(scales[j], shuf), p16);
+            }
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(_mm256_add_epi32(p[0], p[1]), _mm256_add_epi32(p[2], p[3])));
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum_float_8(acc);
+}
 static float dot_q5k(int64_t n, const orc_block_q5k* xs, const orc_block_q8k* ys) {
     const uint32_t KMASK1 = 0x3f3f3f3f, KMASK2 = 0x0f0f0f0f, KMASK3 = 0x03030303;
     const __m256i m4 = _mm256_set1_epi8(0xF);
@@ -260,6 +307,7 @@ float orc_vec_dot_avx2(int dtype, int64_t n, const void* w, const void* a) {
         case ORC_Q8_0: return dot_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q4K: return dot_q4k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
         case ORC_Q2K: return dot_q2k(n, (const orc_block_q2k*)w, (const orc_block_q8k*)a);
+        case ORC_Q3K: return dot_q3k(n, (const orc_block_q3k*)w, (const orc_block_q8k*)a);
         case ORC_Q5K: return dot_q5k(n, (const orc_block_q5k*)w, (const orc_block_q8k*)a);
         case ORC_Q6K: return dot_q6k(n, (const orc_block_q6k*)w, (const orc_block_q8k*)a);
         default: return orc_vec_dot(dtype, n, w, a);

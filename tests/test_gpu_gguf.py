@@ -78,11 +78,11 @@ def test_loader_errors(tmp_path):
     W.moe_layer_file(pm, 0, gate, w1, w3, w2_q8, O.Q4K, k, down_dtype=O.Q8_0)
     with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):
         candle_amd.SparseMoeBlock.from_gguf(str(pm), 0)
-    # an unsupported dtype among the experts (Q3K = 11)
-    pu = tmp_path / "q3k.gguf"
-    w2_q3 = [np.zeros(H * F // 256 * 110, np.uint8) for _ in range(E)]
-    W.moe_layer_file(pu, 0, gate, w1, w3, w2_q3, O.Q4K, k, down_dtype=11)
-    with pytest.raises(candle_amd.MoeError, match="unsupported ggml_dtype 11"):
+    # an unsupported dtype among the experts (Q5_0 = 6)
+    pu = tmp_path / "q5_0.gguf"
+    w2_q5 = [np.zeros(H * F // 32 * 22, np.uint8) for _ in range(E)]
+    W.moe_layer_file(pu, 0, gate, w1, w3, w2_q5, O.Q4K, k, down_dtype=6)
+    with pytest.raises(candle_amd.MoeError, match="unsupported ggml_dtype 6"):
         candle_amd.SparseMoeBlock.from_gguf(str(pu), 0)
 
 

@@ -39,7 +39,7 @@ def test_device_is_gfx950():
     assert candle_amd.device_arch().startswith("gfx950")
 
 
-@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q2K, O.Q4K, O.Q5K, O.Q6K, O.Q8K])
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K, O.Q8K])
 def test_to_float_bit_exact(dt):
     n = 256 * 96
     x = O.fill_normal(dt, n, 0.0, 0.02)
@@ -51,7 +51,7 @@ def test_to_float_bit_exact(dt):
     # arbitrary bit patterns in the quant payload (scale fields kept finite)
     rng = np.random.default_rng(dt)
     raw = blocks.copy().reshape(-1, O.BLOCK_BYTES[dt])
-    lo, hi = {O.Q4_0: (2, 18), O.Q8_0: (2, 34), O.Q2K: (0, 80), O.Q4K: (4, 144), O.Q5K: (4, 176), O.Q6K: (0, 208), O.Q8K: (4, 292)}[dt]
+    lo, hi = {O.Q4_0: (2, 18), O.Q8_0: (2, 34), O.Q2K: (0, 80), O.Q3K: (0, 108), O.Q4K: (4, 144), O.Q5K: (4, 176), O.Q6K: (0, 208), O.Q8K: (4, 292)}[dt]
     raw[:, lo:hi] = rng.integers(0, 256, raw[:, lo:hi].shape, dtype=np.uint8)
     raw = raw.reshape(-1)
     assert np.array_equal(bits(candle_amd.dequantize(dt, raw, n)), bits(O.dequantize(dt, raw, n)))
@@ -126,6 +126,7 @@ def test_route_zipf_bias_lists():
 
 @pytest.mark.parametrize("dt,n,k,m", [(O.Q4K, 64, 512, 5), (O.Q4K, 4096, 1024, 33), (O.Q8_0, 48, 96, 3),
                                        (O.Q2K, 64, 512, 5), (O.Q2K, 1040, 1024, 33), (O.Q2K, 256, 2304, 150),
+                                       (O.Q3K, 64, 512, 5), (O.Q3K, 1040, 1024, 33), (O.Q3K, 256, 2304, 150),
                                        (O.Q5K, 64, 512, 5), (O.Q5K, 1040, 1024, 33), (O.Q5K, 256, 2304, 150),
                                        (O.Q6K, 64, 512, 5), (O.Q6K, 1040, 1024, 33), (O.Q6K, 256, 2304, 150),
                                        (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70)])
@@ -254,7 +255,7 @@ def test_block_q4k_tile_sizes_and_paths():
 
 
 @pytest.mark.parametrize("dt,dt_down", [(O.Q6K, None), (O.Q4K, O.Q6K), (O.Q6K, O.Q4K), (O.Q5K, None), (O.Q5K, O.Q6K),
-                                        (O.Q2K, None), (O.Q2K, O.Q4K)])
+                                        (O.Q2K, None), (O.Q2K, O.Q4K), (O.Q3K, None), (O.Q3K, O.Q5K)])
 def test_block_q6k_and_mixed_down_dtype(dt, dt_down):
     # all-Q6K and all-Q5K experts, the Q4_K_M arrangement (Q4K gate / up with Q6K down), its reverse, and
     # the Q5_K_M arrangement (Q5K with Q6K down).

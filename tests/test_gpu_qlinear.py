@@ -26,7 +26,7 @@ def check(dt, got, want):
         assert np.abs(got - want).max() <= Q4K_TOL * rms(want)
 
 
-@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q6K, 528, 768), (O.Q5K, 528, 768), (O.Q2K, 528, 768), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024)])
+@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q6K, 528, 768), (O.Q5K, 528, 768), (O.Q2K, 528, 768), (O.Q3K, 528, 768), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024)])
 def test_resident_projection_over_batch_sizes(dt, n, k):
     # one object, many calls: decode rows, mid batches, and (Q4K, n % 128 == 0) the tiled kernel
     # at 64- and 128-row tiles with ragged last tiles; shrinking and growing batches reuse the workspace
@@ -79,7 +79,7 @@ def test_argument_checks():
     with pytest.raises(candle_amd.MoeError, match="n % 16"):
         candle_amd.QMatMul(O.Q8_0, w[: 34 * 48], 24, 64)
     with pytest.raises(candle_amd.MoeError):
-        candle_amd.QMatMul(11, w, 32, 64)      # Q3K
+        candle_amd.QMatMul(7, w, 32, 64)       # Q5_1
     lin = candle_amd.QMatMul(O.Q8_0, w, 32, 64)
     with pytest.raises(candle_amd.MoeError, match="expected"):
         lin.forward(np.zeros((3, 32), dtype=np.float32))

@@ -64,7 +64,7 @@ def test_q4_0_matmul_known_answers(O, golden, simd):
     assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_neg_3_64_4"]["expected_rounded"]
 
 
-@pytest.mark.parametrize("name,dt", [("q2k_ramp", 10), ("q4k_ramp", 12), ("q5k_ramp", 13), ("q6k_ramp", 14), ("q8k_ramp", 15)])
+@pytest.mark.parametrize("name,dt", [("q2k_ramp", 10), ("q3k_ramp", 11), ("q4k_ramp", 12), ("q5k_ramp", 13), ("q6k_ramp", 14), ("q8k_ramp", 15)])
 def test_kquant_ramp_spot_values(O, golden, name, dt):
     g = golden[name]
     idx = golden["ramp_spot_indices"]
@@ -80,7 +80,7 @@ def test_kquant_ramp_spot_values(O, golden, name, dt):
         assert np.abs(dbig - big).max() < g["max_abs_err_bound_128"]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 10, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 10, 11, 12, 13, 14, 15])
 def test_ggml_quantization_rmse(O, golden, dt):
     src = ggml_like(0.0)
     dst = O.dequantize(dt, O.quantize(dt, src), src.size)
@@ -88,7 +88,7 @@ def test_ggml_quantization_rmse(O, golden, dt):
     assert rmse <= golden["ggml_quantization_rmse_bound"][{10: "bound_2bits", 11: "bound_3bits"}.get(dt, "bound")]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 10, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 8, 10, 11, 12, 13, 14, 15])
 def test_ggml_dot_error(O, golden, dt):
     # ggml_matmul_error_test, quantized_tests.rs:846-911
     g = golden["ggml_dot_error"]
@@ -114,7 +114,7 @@ def test_vec_dot_matches_dequantised_float64(O):
     # brute force: the integer block dot must equal the float dot of the dequantised operands
     rng = np.random.default_rng(3)
     n = 2048
-    for dt in (O.Q4_0, O.Q8_0, O.Q2K, O.Q4K, O.Q5K, O.Q6K):
+    for dt in (O.Q4_0, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K):
         w = rng.normal(0, 0.02, n).astype(np.float32)
         x = rng.normal(0, 1.0, n).astype(np.float32)
         wq, xq = O.quantize(dt, w), O.quantize(O.VECDOT[dt], x)
@@ -137,7 +137,7 @@ def test_seeded_matmul_spot_values(O, golden, simd):
     r3 = lambda a: [float(np.round(np.float32(1000.0) * np.float32(x)) / np.float32(1000.0)) for x in a]
     dense = (lhs.astype(np.float64) @ rhs.astype(np.float64).T).reshape(-1)
     assert r3(dense[pick]) == r3(g["dense"])  # validates the StdRng restatement itself
-    for key, dt in (("q2k", O.Q2K), ("q4k", O.Q4K), ("q5k", O.Q5K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
+    for key, dt in (("q2k", O.Q2K), ("q3k", O.Q3K), ("q4k", O.Q4K), ("q5k", O.Q5K), ("q6k", O.Q6K), ("q8k", O.Q8K)):
         mm = O.matmul(dt, lhs, O.quantize(dt, rhs), n, simd=simd).reshape(-1)
         assert r3(mm[pick]) == r3(g[key])
 
@@ -330,3 +330,34 @@ def test_q2k_layout_against_independent_decoder(O):
     assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
     assert codes.min() == 0 and codes.max() == 3
     assert np.abs(got - x).max() < 0.02 * 8 / 3
+
+
+def test_q3k_layout_against_independent_decoder(O):
+    # independent numpy decoder of the published Q3_K layout, addressed by element: 32 bytes of high bits,
+    # 64 bytes of 2-bit codes, 12 bytes holding sixteen 6-bit scales (stored + 32), f16 d.  Element e lies in
+    # 32-element group G = e//32 (half G//4, quarter G%4), column l = e%32: low bits 2(G%4).. of
+    # qs[32*(G//4) + l], high bit = bit G of hmask[l] (clear means -4); scale j = e//16 has its low nibble in
+    # scales[j%8] (upper nibble for j >= 8) and its two high bits at 2*(j//4) of scales[8 + j%4].
+    rng = np.random.default_rng(14)
+    x = rng.normal(0, 0.02, 1024).astype(np.float32)
+    blocks = O.quantize(O.Q3K, x).reshape(4, 110)
+    out = np.empty((4, 256), dtype=np.float32)
+    codes = np.empty((4, 256), dtype=np.int32)
+    scs = np.empty((4, 16), dtype=np.int32)
+    for b in range(4):
+        raw = blocks[b]
+        hmask, qs, sc = raw[:32].astype(np.int32), raw[32:96].astype(np.int32), raw[96:108].astype(np.int32)
+        d = np.float32(raw[108:110].view(np.float16)[0])
+        for j in range(16):
+            lo = (sc[j % 8] >> (4 if j >= 8 else 0)) & 15
+            hi = (sc[8 + j % 4] >> (2 * (j // 4))) & 3
+            scs[b, j] = (lo | (hi << 4)) - 32
+        for e in range(256):
+            G, l = e // 32, e % 32
+            low = (qs[32 * (G // 4) + l] >> (2 * (G % 4))) & 3
+            codes[b, e] = low - (0 if (hmask[l] >> G) & 1 else 4)
+            out[b, e] = (d * np.float32(scs[b, e // 16])) * np.float32(codes[b, e])
+    got = O.dequantize(O.Q3K, blocks.reshape(-1), 1024)
+    assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
+    assert codes.min() == -4 and codes.max() == 3 and scs.min() == -32 and scs.max() > 0
+    assert np.abs(got - x).max() < 0.02 * 8 / 4
