@@ -599,6 +599,10 @@ struct moe_qlinear {
     RouteStore route;
     ActStore xq;
     int64_t cap_m = -1;
+    int64_t routed_m = -1;          // row count the identity routing table currently describes (with routed_tile)
+    int routed_tile = 0;
+    bool routed_tab = false;
+    hipStream_t routed_stream = nullptr;
     DevBuf x_dev, y_dev;
     hipStream_t stream = nullptr;
 };
@@ -639,10 +643,18 @@ extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, i
 // quantise the rows, then one pass over the matrix: streamed for short batches, tiled MFMA beyond
 static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d_y, hipStream_t s) {
     int rc;
+    // under stream capture nothing may be allocated, and the graph carries its own copy of the routing table pass
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    if (capturing && m > Q->cap_m)
+        return fail(MOE_E_INVALID, "forward under stream capture needs its workspace: run one forward of the same number of rows before capturing");
+    if (capturing) Q->routed_m = -1;
     if (m > Q->cap_m) {
         if ((rc = Q->route.reserve(m, 1, 1, false))) return rc;
         if ((rc = Q->xq.reserve(Q->vdt, m, Q->k))) return rc;
         Q->cap_m = m;
+        Q->routed_m = -1;   // the table's buffers may have moved
     }
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
     // The tiled MFMA kernel runs one workgroup per (128 weight rows, tile of 64 or 128 x rows): it pays
@@ -656,7 +668,14 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     rb.tile_slots = tile_slots;
     if (!tiled) rb.tile_tab = nullptr;
     MOE_HIP_CHECK(launch_quantize_rows(Q->vdt, d_x, m, (int)Q->k, Q->xq.view(), s));
-    MOE_HIP_CHECK(launch_identity_routing(rb, m, s));
+    // the identity table depends on the row count only: a decode loop that calls with the same m finds it in place
+    // (calls on one object are serialised, and a call on another stream waits for nothing it did not enqueue itself:
+    // the table is rewritten whenever the previous call used another stream)
+    if (Q->routed_m != m || Q->routed_tile != tile_slots || Q->routed_tab != tiled || Q->routed_stream != s) {
+        MOE_HIP_CHECK(launch_identity_routing(rb, m, s));
+        Q->routed_m = m; Q->routed_tile = tile_slots; Q->routed_tab = tiled; Q->routed_stream = s;
+        if (capturing) Q->routed_m = -1;   // an eager call after the capture writes the table again
+    }
     ExpertParams ep;
     ep.dt = Q->dt; ep.H = (int)Q->n; ep.F = (int)Q->k; ep.n_groups = 1; ep.group0 = 0;
     ep.groups = Q->group.as<GroupWeights>();

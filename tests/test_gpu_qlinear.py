@@ -108,3 +108,26 @@ def test_projection_from_gguf(tmp_path):
             candle_amd.QMatMul.from_gguf(g, "blk.0.attn_output.weight")
     lin = candle_amd.QMatMul.from_gguf(str(path), "output.weight")   # by path: the file is closed again
     check(O.Q4_0, lin.forward(x[:3]), O.matmul(O.Q4_0, x[:3], blocks["output.weight"], 1024))
+
+
+def test_projection_recorded_into_a_hip_graph():
+    torch = pytest.importorskip("torch")
+    dt, n, k, m = O.Q4K, 512, 1024, 8
+    w = O.fill_normal_quantized(6, dt, n, k, 0.02)
+    lin = candle_amd.QMatMul(dt, w, n, k)
+    xs = [torch.from_numpy(activations(m, k, seed=60 + i)).cuda() for i in range(3)]
+    eager = [lin.forward(x).clone() for x in xs]
+    x_in, y_out = xs[0].clone(), torch.empty(m, n, device="cuda")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        lin.forward(x_in, out=y_out)
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            x_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_out, want)
+            # eager calls with other row counts in between rewrite the routing table; the graph carries its own pass
+            lin.forward(torch.from_numpy(activations(3, k, seed=1)).cuda())
+            torch.cuda.synchronize()
