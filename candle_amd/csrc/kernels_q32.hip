@@ -349,11 +349,15 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
     const int nkb = K / 32;
     const uint32_t q_off = DT == MOE_GGML_Q8_0 ? (uint32_t)lane * 8u : (uint32_t)(r * 16 + 8 * (g >> 1));
     const uint32_t d_off = (DT == MOE_GGML_Q8_0 ? 512u : 256u) + 2u * (uint32_t)r;
-    Q32Raw nxt[NT][STEP];
+    // ONCE (the weights come from HBM): the next trip's tiles are requested a whole trip ahead.  Otherwise they
+    // are in L2 after the first pass and are fetched where they are used: half the registers, twice the waves.
+    Q32Raw nxt[ONCE ? NT : 1][ONCE ? STEP : 1];
+    if (ONCE) {
 #pragma unroll
-    for (int t = 0; t < NT; t++)
+        for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off);
+            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off);
+    }
     // With several slot tiles the activation operand is requested one step ahead too: the one of slot
     // tile tt+1, or of the next trip's first slot tile, is on its way while this one is multiplied.
     // (With one slot tile the extra registers cost a wave per SIMD, which costs more than the wait.)
@@ -362,16 +366,23 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
     if (AHEAD) An = load_q8_0_trip<DT, STEP>(ab, K, nkb, 0, rowA[0], rowD[0], g);
     for (int kb0 = 0; kb0 < nkb; kb0 += STEP) {
         Q32Raw cur[NT][STEP];
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-#pragma unroll
-            for (int j = 0; j < STEP; j++) cur[t][j] = nxt[t][j];
         // the trip after this one; past the end the last trip is requested again (no branch around a load)
         const int kbn = kb0 + STEP < nkb ? kb0 + STEP : kb0;
+        if (ONCE) {
 #pragma unroll
-        for (int t = 0; t < NT; t++)
+            for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off);
+                for (int j = 0; j < STEP; j++) cur[t][j] = nxt[t][j];
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off);
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; t++)
+#pragma unroll
+                for (int j = 0; j < STEP; j++) cur[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kb0 + j) * TB, q_off, d_off);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) {
@@ -498,7 +509,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_stream_kernel(ExpertPara
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[0][tt][i] = 0.f;
 
-    q32_engine<DT, TT, 1, 2 * Q32_STEP, ONCE>(tp, p.hq, F, rowA, rowD, lane, acc);
+    q32_engine<DT, TT, 1, ONCE ? 2 * Q32_STEP : Q32_STEP, ONCE>(tp, p.hq, F, rowA, rowD, lane, acc);
 
 #pragma unroll
     for (int tt = 0; tt < TT; tt++)
@@ -537,12 +548,13 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
     const bool stream = !plain && (p.F / 32) % (2 * Q32_STEP) == 0;
+    const bool stream_again = !plain && (p.F / 32) % Q32_STEP == 0;   // the several-pass variant walks K in shorter trips
     if (tt == 1) {
         if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 1, true>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
         if (stream && grid.z == 1) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, true>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream_again && grid.z > 1) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
