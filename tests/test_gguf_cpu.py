@@ -160,3 +160,32 @@ def test_hostile_tables_are_refused_not_followed(tmp_path):
     open(p4, "wb").write(bytes(blob))
     with pytest.raises(candle_amd.MoeError, match="general.alignment is 4294967295"):
         candle_amd.GgufFile(str(p4))
+
+
+def test_reader_survives_mutated_files_under_sanitizers(tmp_path):
+    # gguf.cpp (host code only) built with AddressSanitizer + UBSan around stubs that read every byte the reader
+    # hands out; 2000 mutated copies of a valid MoE file (byte and bit flips, extreme 64-bit fields, truncations)
+    # go through every public call of the reader.  Any out-of-bounds read, overflow or leak aborts the harness.
+    import shutil
+    import subprocess
+    gxx = shutil.which("g++")
+    if gxx is None or not os.path.isdir("/opt/rocm/include"):
+        pytest.skip("needs g++ and the ROCm headers")
+    here = os.path.dirname(os.path.abspath(__file__))
+    exe = tmp_path / "gguf_fuzz"
+    cmd = [gxx, "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all", "-D__HIP_PLATFORM_AMD__",
+           "-I/opt/rocm/include", os.path.join(here, "gguf_fuzz_harness.cpp"),
+           os.path.join(here, "..", "candle_amd", "csrc", "gguf.cpp"), "-o", str(exe)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rng = np.random.default_rng(0)
+    H, F, E = 256, 256, 4
+    blk = lambda: rng.integers(0, 256, H * F // 256 * 144, dtype=np.uint8)
+    gate = rng.standard_normal((E, H)).astype(np.float32)
+    good = tmp_path / "good.gguf"
+    W.moe_layer_file(good, 0, gate, [blk() for _ in range(E)], [blk() for _ in range(E)], [blk() for _ in range(E)], 12, 2,
+                     extra_metadata=[("tokenizer.ggml.tokens", W.ARRAY, (W.STRING, ["a", "bb", "ccc"]))])
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0")
+    r = subprocess.run([str(exe), str(good), str(tmp_path / "mut.gguf"), "2000", "7"], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0, (r.stdout[-500:], r.stderr[-3000:])
+    assert "2000 mutants survived" in r.stdout
