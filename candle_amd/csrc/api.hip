@@ -328,13 +328,13 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.xq = L->xq.view();
     fp.rb = L->route.view();
     fp.rb.T = (int)T; fp.rb.k = (int)L->k;
-    // Q4K batches with more than ~24 rows per expert take the tiled MFMA kernels (F a multiple of 64,
+    // Q4K batches with more than ~36 rows per expert take the tiled MFMA kernels (F a multiple of 64,
     // H of 128; those kernels address activation rows with 32-bit byte offsets).  Their tiles hold 64
     // slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
     // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
     const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k > 24 * L->E;
+                       T * L->k > 36 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     const bool direct = !tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     fp.rb.direct = direct ? 1 : 0;
@@ -355,7 +355,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.max_rows = T;
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
-    ep.slot_tiles = (T * L->k > 24 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
+    // tiles per pass up to ~40 rows per expert)
+    ep.slot_tiles = (T * L->k > 40 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
     static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
     if (force_st) ep.slot_tiles = force_st;
     static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;

@@ -247,9 +247,10 @@ def test_block_q4k_shared_expert_slot_tiles(T):
 
 
 def test_block_q4k_tile_sizes_and_paths():
-    # 25 rows per expert and more go to the tiled kernels: 64-slot tiles up to ~96 rows per expert, 128 beyond
+    # two slot tiles per streamed pass with a second pass for lists beyond 32 rows (T = 104, 130); from 37 rows per
+    # expert the tiled kernels: 64-slot tiles (T = 150, 300) up to ~96 rows per expert, 128 beyond (T = 400, 600)
     ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
-    for T in (104, 130, 400, 600):
+    for T in (104, 130, 150, 300, 400, 600):
         check_block(ref, gpu, T)
     gpu.close()
 
