@@ -2,6 +2,7 @@
 // k_quants::matmul applies to every lhs row before the integer dot products:
 //   BlockQ8K::from_float   candle-core/src/quantized/k_quants.rs:1819-1856
 //   BlockQ8_0::from_float  candle-core/src/quantized/k_quants.rs:605-634
+//   BlockQ8_1::from_float  candle-core/src/quantized/k_quants.rs:700-729
 // so the int8 operands are bit-identical to the CPU path's.
 #pragma once
 #include "moe_common.hpp"
@@ -57,9 +58,19 @@ __device__ inline void quantize_q8k_block(float4 v, int lane, int8_t* qs_block, 
     if (lane == 0) *d_out = 1.0f / iscale;
 }
 
-// Half a wave (32 lanes) quantises one 32-element block; lane holds element (lane & 31).
-//   q_out: the element's quant byte; d_out: f16-rounded scale widened to f32; bsum_out: sum of quants.
-__device__ inline void quantize_q8_0_block(float x, int lane, int8_t* q_out, float* d_out, int32_t* bsum_out) {
+// The word kept beside a 32-element activation block.  Q8_0: the sum of the block's quants (the -8 / -16 code
+// offsets of Q4_0 / Q5_0 weights leave through it).  Q8_1: the block's `s` widened to f32, s = f16(sum) * d in
+// binary16 arithmetic (two 11-bit significands: the f32 product is exact, so one rounding to f16 remains).
+__device__ inline int32_t q8_block_word(int vdt, int sum, float d_f16) {
+    if (vdt != MOE_GGML_Q8_1) return sum;
+    const float fs = __half2float(__float2half_rn((float)sum));
+    return __float_as_int(__half2float(__float2half_rn(fs * d_f16)));
+}
+
+// Half a wave (32 lanes) quantises one 32-element block; lane holds element (lane & 31).  Q8_0 and Q8_1 blocks
+// hold the same scale and quants.
+//   q_out: the element's quant byte; d_out: f16-rounded scale widened to f32; word_out: see q8_block_word.
+__device__ inline void quantize_q8_0_block(int vdt, float x, int lane, int8_t* q_out, float* d_out, int32_t* word_out) {
     float amax = fabsf(x);
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
@@ -71,8 +82,9 @@ __device__ inline void quantize_q8_0_block(float x, int lane, int8_t* q_out, flo
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
     if ((lane & 31) == 0) {
-        *d_out = __half2float(__float2half_rn(d));
-        *bsum_out = sum;
+        const float dh = __half2float(__float2half_rn(d));
+        *d_out = dh;
+        *word_out = q8_block_word(vdt, sum, dh);
     }
 }
 

@@ -173,11 +173,11 @@ static int check_desc(const moe_desc* d) {
     const int dt = d->ggml_dtype, dtd = d->ggml_dtype_down ? d->ggml_dtype_down : dt;
     if (!weight_dtype_supported(dt) || !weight_dtype_supported(dtd))
         return fail(MOE_E_INVALID, "unsupported ggml_dtype " + std::to_string(weight_dtype_supported(dt) ? dtd : dt) +
-                                       " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
+                                       " (supported: Q4_0=2, Q4_1=3, Q5_0=6, Q5_1=7, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
     // w2 consumes the intermediate in the activation format of its own dtype; the up kernels emit the one of dt
     if (vecdot_dtype(dt) != vecdot_dtype(dtd))
         return fail(MOE_E_INVALID, "ggml_dtype " + std::to_string(dt) + " and ggml_dtype_down " + std::to_string(dtd) +
-                                       " quantise activations differently (Q8_0 vs Q8K); such a layer is not supported");
+                                       " quantise activations differently (Q8_0, Q8_1 or Q8K); such a layer is not supported");
     const int64_t be = block_elems(dt);
     if (d->hidden <= 0 || d->ffn <= 0) return fail(MOE_E_INVALID, "hidden and ffn must be positive");
     // the reference rejects a last dimension that is not a multiple of the block size
@@ -555,7 +555,8 @@ extern "C" int moe_dequantize(int32_t dt, const void* blocks, int64_t n, float* 
     int rc = ensure_device();
     if (rc) return rc;
     const int64_t be = block_elems(dt);
-    if (be < 0) return fail(MOE_E_INVALID, "moe_dequantize: unsupported dtype " + std::to_string(dt));
+    if (be < 0 || dt == MOE_GGML_Q8_1)   // BlockQ8_1 has no to_float (k_quants.rs:731-733)
+        return fail(MOE_E_INVALID, "moe_dequantize: unsupported dtype " + std::to_string(dt));
     if (n < 0 || n % be) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
     if (n == 0) return MOE_OK;
     if (!blocks || !out) return fail(MOE_E_INVALID, "NULL pointer");
@@ -572,7 +573,7 @@ extern "C" int moe_dequantize(int32_t dt, const void* blocks, int64_t n, float* 
 extern "C" int moe_quantize_act(int32_t vdt, const float* x, int64_t rows, int64_t k, void* out) {
     int rc = ensure_device();
     if (rc) return rc;
-    if (vdt != MOE_GGML_Q8_0 && vdt != MOE_GGML_Q8K) return fail(MOE_E_INVALID, "vecdot_dtype must be Q8_0 (8) or Q8K (15)");
+    if (vdt != MOE_GGML_Q8_0 && vdt != MOE_GGML_Q8_1 && vdt != MOE_GGML_Q8K) return fail(MOE_E_INVALID, "vecdot_dtype must be Q8_0 (8), Q8_1 (9) or Q8K (15)");
     const int64_t be = block_elems(vdt);
     if (rows < 0 || k <= 0 || k % be || k > (1 << 24)) return fail(MOE_E_INVALID, "k must be a positive multiple of the block size");
     if (rows == 0) return MOE_OK;
@@ -621,7 +622,7 @@ extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, i
     if (rc) return rc;
     if (!out || !w_blocks) return fail(MOE_E_INVALID, "moe_qlinear_create: NULL pointer");
     if (!weight_dtype_supported(dt))
-        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
+        return fail(MOE_E_INVALID, "moe_qlinear_create: unsupported ggml_dtype " + std::to_string(dt) + " (supported: Q4_0=2, Q4_1=3, Q5_0=6, Q5_1=7, Q8_0=8, Q2K=10, Q3K=11, Q4K=12, Q5K=13, Q6K=14)");
     const int64_t be = block_elems(dt);
     if (n <= 0 || n % 16 || k <= 0 || k % be || k > (1 << 24))
         return fail(MOE_E_INVALID, "moe_qlinear_create: need n % 16 == 0 and k a multiple of the block size (" + std::to_string(be) + ")");

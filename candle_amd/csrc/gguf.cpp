@@ -360,10 +360,10 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     else if (dt == 1) {
         const uint16_t* h = static_cast<const uint16_t*>(data);
         for (size_t i = 0; i < gate.size(); i++) gate[i] = half_bits_to_float(h[i]);
-    } else if (dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K) {
+    } else if (moe::weight_dtype_supported(dt)) {
         if ((rc = moe_dequantize(dt, data, E * H, gate.data()))) return rc;   // on the GPU
     } else
-        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: unsupported dtype " + std::to_string(dt) + " (supported: F32, F16, Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K)");
+        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: unsupported dtype " + std::to_string(dt) + " (supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K)");
 
     std::vector<const void*> w1((size_t)E), w2((size_t)E), w3((size_t)E);
     int up_dt = -1, down_dt = -1;   // gate / up matrices share one dtype, down matrices one
@@ -409,7 +409,7 @@ extern "C" int moe_qlinear_create_from_gguf(const moe_gguf* g, const char* tenso
     int rc = moe_gguf_tensor(g, tensor_name, &dt, &nd, dims, &data, &nbytes);
     if (rc) return rc;
     if (nd != 2) return fail(MOE_E_INVALID, std::string(tensor_name) + ": a projection matrix has two dimensions, this tensor has " + std::to_string(nd));
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q2K && dt != MOE_GGML_Q3K && dt != MOE_GGML_Q4K && dt != MOE_GGML_Q5K && dt != MOE_GGML_Q6K)
-        return fail(MOE_E_INVALID, std::string(tensor_name) + ": unsupported dtype " + std::to_string(dt) + " (supported: Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K)");
+    if (!moe::weight_dtype_supported(dt))
+        return fail(MOE_E_INVALID, std::string(tensor_name) + ": unsupported dtype " + std::to_string(dt) + " (supported: Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K)");
     return moe_qlinear_create(dt, data, dims[0], dims[1], out);
 }

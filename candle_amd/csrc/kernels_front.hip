@@ -317,7 +317,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
         const int nb = H / 32;
         for (int h = tid; h < H; h += FRONT_THREADS) {
             int b = h / 32;
-            quantize_q8_0_block(xrow[h], lane, p.xq.qs + t * H + h, p.xq.d + t * nb + b,
+            quantize_q8_0_block(p.vdt, xrow[h], lane, p.xq.qs + t * H + h, p.xq.d + t * nb + b,
                                 reinterpret_cast<int32_t*>(p.xq.bsum) + t * nb + b);
         }
     }
@@ -420,8 +420,9 @@ __device__ inline void quantize_chunk(const FrontParams& p, int64_t t, int H, in
         *reinterpret_cast<uint32_t*>(p.xq.qs + t * H + chunk * 256 + lane * 4) = packed;
         if ((lane & 7) == 0) {
             const int b = chunk * 8 + (lane >> 3);
-            p.xq.d[t * nb + b] = __half2float(__float2half_rn(d));
-            reinterpret_cast<int32_t*>(p.xq.bsum)[t * nb + b] = sum;
+            const float dh = __half2float(__float2half_rn(d));
+            p.xq.d[t * nb + b] = dh;
+            reinterpret_cast<int32_t*>(p.xq.bsum)[t * nb + b] = q8_block_word(p.vdt, sum, dh);
         }
     }
 }

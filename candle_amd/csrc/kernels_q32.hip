@@ -1,13 +1,16 @@
-// Grouped expert products over Q4_0 / Q8_0 weights with Q8_0 activations (gfx950, int8 MFMA).
+// Grouped expert products over the 32-element block formats (gfx950, int8 MFMA): Q4_0, Q5_0, Q8_0 weights
+// with Q8_0 activations, Q4_1 and Q5_1 weights with Q8_1 activations.
 //
-// Arithmetic restated from candle-core/src/quantized/k_quants.rs:241-258 (Q4_0 . Q8_0) and
-// :650-668 (Q8_0 . Q8_0): per 32-element block  sumf += (sum_i as f32) * d_w * d_x.  One
+// Arithmetic restated from candle-core/src/quantized/k_quants.rs:241-258 (Q4_0 . Q8_0), :381-402
+// (Q5_0 . Q8_0) and :650-668 (Q8_0 . Q8_0): per 32-element block  sumf += (sum_i as f32) * d_w * d_x;
+// :270-297 (Q4_1 . Q8_1) and :477-509 (Q5_1 . Q8_1): sumf += (sum_i as f32) * d_w * d_x + m_w * s_x.  One
 // v_mfma_i32_16x16x32_i8 yields the exact integer dot of a block for 16 rows x 16 slots, and every
 // lane adds its (row, slot) blocks in ascending block order with separately rounded products, so
 // the f32 result is bit-identical to the scalar reference loop.
 //
-// Q4_0 stores nibble - 8; the kernel multiplies the raw nibbles (0..15) and subtracts
-// 8 * sum(q8) of the block, which is the same integer.
+// Q4_0 stores nibble - 8 and Q5_0 code - 16; the kernel multiplies the raw codes (0..15, 0..31) and
+// subtracts 8 or 16 times sum(q8) of the block, which is the same integer.  Q4_1 and Q5_1 codes are
+// unsigned as stored.
 #include <cstdlib>
 #include "act_quant.hpp"
 #include "kernels.hpp"
@@ -17,45 +20,28 @@ namespace moe {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
+// Placement of one format's 16-row tile (see moe_common.hpp) and what its block carries.
+template <int DT>
+struct Q32Fmt {
+    static constexpr bool NIB = DT != MOE_GGML_Q8_0;                             // two codes per byte
+    static constexpr bool FIFTH = DT == MOE_GGML_Q5_0 || DT == MOE_GGML_Q5_1;    // a fifth bit per code
+    static constexpr bool HAS_M = DT == MOE_GGML_Q4_1 || DT == MOE_GGML_Q5_1;    // a block minimum (and Q8_1 activations)
+    static constexpr int OFFSET = DT == MOE_GGML_Q4_0 ? 8 : DT == MOE_GGML_Q5_0 ? 16 : 0;  // stored code - value
+    static constexpr int TB = DT == MOE_GGML_Q8_0 ? Q8_0_TILE_BYTES : DT == MOE_GGML_Q4_0 ? Q4_0_TILE_BYTES
+                            : DT == MOE_GGML_Q4_1 ? Q4_1_TILE_BYTES : DT == MOE_GGML_Q5_0 ? Q5_0_TILE_BYTES : Q5_1_TILE_BYTES;
+    static constexpr uint32_t H_OFF = 256;
+    static constexpr uint32_t D_OFF = !NIB ? 512 : FIFTH ? 320 : 256;
+    static constexpr uint32_t D_STRIDE = HAS_M ? 4 : 2;
+    __device__ static uint32_t q_off(int lane) { return NIB ? (uint32_t)((lane & 15) * 16 + 8 * (lane >> 5)) : (uint32_t)lane * 8u; }
+    __device__ static uint32_t d_off(int lane) { return D_OFF + D_STRIDE * (uint32_t)(lane & 15); }
+    __device__ static uint32_t h_off(int lane) { return H_OFF + 4u * (uint32_t)(lane & 15); }
+};
+
 template <int DT>
 struct Q32Tile {
     uint2 q;
     float d;
-};
-
-// weight tiles are read once per launch: non-temporal loads keep them from displacing the activations
-// and routing lists in the caches
-typedef uint32_t u32x2_q32 __attribute__((ext_vector_type(2)));
-__device__ inline uint2 load_stream8(const uint8_t* p) {
-    const u32x2_q32 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_q32*>(p));
-    return make_uint2(v.x, v.y);
-}
-__device__ inline float load_stream_half(const uint8_t* p) {
-    const unsigned short h = __builtin_nontemporal_load(reinterpret_cast<const unsigned short*>(p));
-    return __half2float(__ushort_as_half(h));
-}
-
-template <int DT>
-__device__ inline Q32Tile<DT> load_q32_tile(const uint8_t* tile, int lane) {
-    Q32Tile<DT> t;
-    const int r = lane & 15, g = lane >> 4;
-    if (DT == MOE_GGML_Q8_0) {
-        t.q = load_stream8(tile + lane * 8);
-        t.d = load_stream_half(tile + 512 + 2 * r);
-    } else {
-        uint2 w = load_stream8(tile + r * 16 + 8 * (g >> 1));
-        if (g & 1) { w.x >>= 4; w.y >>= 4; }
-        t.q.x = w.x & 0x0f0f0f0fu;
-        t.q.y = w.y & 0x0f0f0f0fu;
-        t.d = load_stream_half(tile + 256 + 2 * r);
-    }
-    return t;
-}
-
-struct Q8_0Operand {
-    uint2 a;
-    float yd[4];
-    int bs[4];
+    float m;   // formats with a block minimum only
 };
 
 // element offset inside a block of this lane's 8-element MFMA chunk
@@ -64,6 +50,79 @@ __device__ inline int chunk_start(int g) {
     return DT == MOE_GGML_Q8_0 ? 8 * g : (g & 1) * 16 + (g >> 1) * 8;
 }
 
+typedef const __attribute__((address_space(1))) uint8_t* gbytes32;
+typedef uint32_t u32x2g __attribute__((ext_vector_type(2)));
+typedef float f32x4g __attribute__((ext_vector_type(4)));
+typedef int i32x4g __attribute__((ext_vector_type(4)));
+template <typename T>
+__device__ __forceinline__ T ldg(const void* uniform_base, uint32_t off) {
+    return *reinterpret_cast<const __attribute__((address_space(1))) T*>((gbytes32)uniform_base + off);
+}
+template <typename T>
+__device__ __forceinline__ T ldg_stream(const void* uniform_base, uint32_t off) {
+    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) T*>((gbytes32)uniform_base + off));
+}
+
+// One lane's share of a tile as it is fetched: 8 code bytes, the row's d (and m), the row's fifth bits.
+struct Q32Raw {
+    u32x2g q;
+    uint32_t dm;
+    uint32_t h;
+};
+// ONCE: the weights are read by one pass only (non-temporal: they should not displace the activations
+// in the caches); otherwise further workgroups stream the same tiles again and should find them in L2
+template <int DT, bool ONCE>
+__device__ __forceinline__ Q32Raw load_q32_raw(const uint8_t* tile, uint32_t q_off, uint32_t d_off, uint32_t h_off) {
+    typedef Q32Fmt<DT> F;
+    Q32Raw t;
+    t.h = 0;
+    if (ONCE) {
+        t.q = ldg_stream<u32x2g>(tile, q_off);
+        t.dm = F::HAS_M ? ldg_stream<uint32_t>(tile, d_off) : (uint32_t)ldg_stream<unsigned short>(tile, d_off);
+        if (F::FIFTH) t.h = ldg_stream<uint32_t>(tile, h_off);
+    } else {
+        t.q = ldg<u32x2g>(tile, q_off);
+        t.dm = F::HAS_M ? ldg<uint32_t>(tile, d_off) : (uint32_t)ldg<unsigned short>(tile, d_off);
+        if (F::FIFTH) t.h = ldg<uint32_t>(tile, h_off);
+    }
+    return t;
+}
+// bits 0..3 of x to bit 4 of bytes 0..3 (the four shifted copies of x do not overlap, so no carries)
+__device__ __forceinline__ uint32_t fifth_bits(uint32_t x) { return ((x * 0x00204081u) & 0x01010101u) << 4; }
+template <int DT>
+__device__ __forceinline__ Q32Tile<DT> q32_unpack(const Q32Raw& raw, int g) {
+    typedef Q32Fmt<DT> F;
+    Q32Tile<DT> t;
+    if (!F::NIB) {
+        t.q = make_uint2(raw.q.x, raw.q.y);
+    } else {
+        uint32_t x = raw.q.x, y = raw.q.y;
+        if (g & 1) { x >>= 4; y >>= 4; }
+        x &= 0x0f0f0f0fu; y &= 0x0f0f0f0fu;
+        if (F::FIFTH) {   // bit e of the word belongs to element e; this lane's elements start at chunk_start
+            const uint32_t hb = raw.h >> chunk_start<DT>(g);
+            x |= fifth_bits(hb & 15u);
+            y |= fifth_bits((hb >> 4) & 15u);
+        }
+        t.q = make_uint2(x, y);
+    }
+    t.d = __half2float(__ushort_as_half((unsigned short)(raw.dm & 0xffffu)));
+    t.m = F::HAS_M ? __half2float(__ushort_as_half((unsigned short)(raw.dm >> 16))) : 0.f;
+    return t;
+}
+
+template <int DT>
+__device__ inline Q32Tile<DT> load_q32_tile(const uint8_t* tile, int lane) {
+    typedef Q32Fmt<DT> F;
+    return q32_unpack<DT>(load_q32_raw<DT, true>(tile, F::q_off(lane), F::d_off(lane), F::h_off(lane)), lane >> 4);
+}
+
+struct Q8_0Operand {
+    uint2 a;
+    float yd[4];
+    int bs[4];
+};
+
 template <int DT>
 __device__ inline Q8_0Operand load_q8_0_operand(const ActBuf& ab, int K, int nkb, int kb, int rowA, const int rowD[4], int g) {
     Q8_0Operand o;
@@ -71,7 +130,7 @@ __device__ inline Q8_0Operand load_q8_0_operand(const ActBuf& ab, int K, int nkb
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         o.yd[i] = ab.d[(int64_t)rowD[i] * nkb + kb];
-        o.bs[i] = (DT == MOE_GGML_Q4_0) ? reinterpret_cast<const int32_t*>(ab.bsum)[(int64_t)rowD[i] * nkb + kb] : 0;
+        o.bs[i] = (Q32Fmt<DT>::OFFSET || Q32Fmt<DT>::HAS_M) ? reinterpret_cast<const int32_t*>(ab.bsum)[(int64_t)rowD[i] * nkb + kb] : 0;
     }
     return o;
 }
@@ -85,9 +144,10 @@ __device__ inline void q32_mac(const Q32Tile<DT>& w, const Q8_0Operand& A, float
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         int isum = D[i];
-        if (DT == MOE_GGML_Q4_0) isum -= 8 * A.bs[i];
+        if (Q32Fmt<DT>::OFFSET) isum -= Q32Fmt<DT>::OFFSET * A.bs[i];
         float t = (float)isum * w.d;
         t = t * A.yd[i];
+        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __int_as_float(A.bs[i]);   // the word holds the activation block's s
         acc[i] += t;
     }
 }
@@ -108,7 +168,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
     const int H = p.H, F = p.F, nkb = H / 32;
     const int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
     if (rt0 >= F / 16) return;
-    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+    constexpr int TB = Q32Fmt<DT>::TB;
 
     int rowA[TT], rowD[TT][4];
 #pragma unroll
@@ -174,8 +234,9 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
                 p.hq.qs[hrow * F + rt0 * 16 + r] = (int8_t)q0;
                 p.hq.qs[hrow * F + rt0 * 16 + 16 + r] = (int8_t)q1;
                 if (r == 0) {
-                    p.hq.d[hrow * nfb + fb] = __half2float(__float2half_rn(d));
-                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + fb] = sum;
+                    const float dh = __half2float(__float2half_rn(d));
+                    p.hq.d[hrow * nfb + fb] = dh;
+                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + fb] = q8_block_word(vecdot_dtype(DT), sum, dh);
                 }
             }
         }
@@ -195,7 +256,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
     const int H = p.H, F = p.F, nkb = F / 32;
     const int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
     if (rt >= H / 16) return;
-    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+    constexpr int TB = Q32Fmt<DT>::TB;
 
     int rowA[TT], rowD[TT][4];
 #pragma unroll
@@ -254,51 +315,6 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
 // non-temporal global loads with a scalar base and 32-bit lane offsets, the activation scales and
 // block sums of a trip fetched as one 16-byte load per output slot.  They need K / 32 to be a
 // multiple of STEP; other shapes take the kernels above.
-typedef const __attribute__((address_space(1))) uint8_t* gbytes32;
-typedef uint32_t u32x2g __attribute__((ext_vector_type(2)));
-typedef float f32x4g __attribute__((ext_vector_type(4)));
-typedef int i32x4g __attribute__((ext_vector_type(4)));
-template <typename T>
-__device__ __forceinline__ T ldg(const void* uniform_base, uint32_t off) {
-    return *reinterpret_cast<const __attribute__((address_space(1))) T*>((gbytes32)uniform_base + off);
-}
-template <typename T>
-__device__ __forceinline__ T ldg_stream(const void* uniform_base, uint32_t off) {
-    return __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) T*>((gbytes32)uniform_base + off));
-}
-
-struct Q32Raw {
-    u32x2g q;
-    unsigned short d;
-};
-// ONCE: the weights are read by one pass only (non-temporal: they should not displace the activations
-// in the caches); otherwise further workgroups stream the same tiles again and should find them in L2
-template <int DT, bool ONCE>
-__device__ __forceinline__ Q32Raw load_q32_raw(const uint8_t* tile, uint32_t q_off, uint32_t d_off) {
-    Q32Raw t;
-    if (ONCE) {
-        t.q = ldg_stream<u32x2g>(tile, q_off);
-        t.d = ldg_stream<unsigned short>(tile, d_off);
-    } else {
-        t.q = ldg<u32x2g>(tile, q_off);
-        t.d = ldg<unsigned short>(tile, d_off);
-    }
-    return t;
-}
-template <int DT>
-__device__ __forceinline__ Q32Tile<DT> q32_unpack(const Q32Raw& raw, int g) {
-    Q32Tile<DT> t;
-    if (DT == MOE_GGML_Q8_0) {
-        t.q = make_uint2(raw.q.x, raw.q.y);
-    } else {
-        uint32_t x = raw.q.x, y = raw.q.y;
-        if (g & 1) { x >>= 4; y >>= 4; }
-        t.q = make_uint2(x & 0x0f0f0f0fu, y & 0x0f0f0f0fu);
-    }
-    t.d = __half2float(__ushort_as_half(raw.d));
-    return t;
-}
-
 // activation operand of one 16-slot tile for STEP consecutive blocks
 template <int STEP>
 struct Q8_0Trip {
@@ -318,7 +334,7 @@ __device__ __forceinline__ Q8_0Trip<STEP> load_q8_0_trip(const ActBuf& ab, int K
 #pragma unroll
         for (int q = 0; q < STEP / 4; q++) {
             o.yd[i][q] = ldg<f32x4g>(ab.d, doff + q * 16);
-            if (DT == MOE_GGML_Q4_0) o.bs[i][q] = ldg<i32x4g>(ab.bsum, doff + q * 16);
+            if (Q32Fmt<DT>::OFFSET || Q32Fmt<DT>::HAS_M) o.bs[i][q] = ldg<i32x4g>(ab.bsum, doff + q * 16);
         }
     }
     return o;
@@ -333,9 +349,10 @@ __device__ __forceinline__ void q32_mac_trip(const Q32Tile<DT>& w, const Q8_0Tri
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         int isum = D[i];
-        if (DT == MOE_GGML_Q4_0) isum -= 8 * A.bs[i][j / 4][j % 4];
+        if (Q32Fmt<DT>::OFFSET) isum -= Q32Fmt<DT>::OFFSET * A.bs[i][j / 4][j % 4];
         float t = (float)isum * w.d;
         t = t * A.yd[i][j / 4][j % 4];
+        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __int_as_float(A.bs[i][j / 4][j % 4]);
         acc[i] += t;
     }
 }
@@ -344,11 +361,10 @@ __device__ __forceinline__ void q32_mac_trip(const Q32Tile<DT>& w, const Q8_0Tri
 template <int DT, int TT, int NT, int STEP, bool ONCE>
 __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const ActBuf& ab, int K, const int rowA[TT], const int rowD[TT][4],
                                            int lane, float acc[NT][TT][4]) {
-    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
-    const int r = lane & 15, g = lane >> 4;
+    constexpr int TB = Q32Fmt<DT>::TB;
+    const int g = lane >> 4;
     const int nkb = K / 32;
-    const uint32_t q_off = DT == MOE_GGML_Q8_0 ? (uint32_t)lane * 8u : (uint32_t)(r * 16 + 8 * (g >> 1));
-    const uint32_t d_off = (DT == MOE_GGML_Q8_0 ? 512u : 256u) + 2u * (uint32_t)r;
+    const uint32_t q_off = Q32Fmt<DT>::q_off(lane), d_off = Q32Fmt<DT>::d_off(lane), h_off = Q32Fmt<DT>::h_off(lane);
     // ONCE (the weights come from HBM): the next trip's tiles are requested a whole trip ahead.  Otherwise they
     // are in L2 after the first pass and are fetched where they are used: half the registers, twice the waves.
     Q32Raw nxt[ONCE ? NT : 1][ONCE ? STEP : 1];
@@ -356,7 +372,7 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
 #pragma unroll
         for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off);
+            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off, h_off);
     }
     // With several slot tiles the activation operand is requested one step ahead too: the one of slot
     // tile tt+1, or of the next trip's first slot tile, is on its way while this one is multiplied.
@@ -376,12 +392,12 @@ __device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const Ac
 #pragma unroll
             for (int t = 0; t < NT; t++)
 #pragma unroll
-                for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off);
+                for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off, h_off);
         } else {
 #pragma unroll
             for (int t = 0; t < NT; t++)
 #pragma unroll
-                for (int j = 0; j < STEP; j++) cur[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kb0 + j) * TB, q_off, d_off);
+                for (int j = 0; j < STEP; j++) cur[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kb0 + j) * TB, q_off, d_off, h_off);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -419,7 +435,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
     const int H = p.H, F = p.F, nkb = H / 32;
     const int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
     if (rt0 >= F / 16) return;
-    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+    constexpr int TB = Q32Fmt<DT>::TB;
 
     int rowA[TT], rowD[TT][4];
 #pragma unroll
@@ -469,8 +485,9 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
                 p.hq.qs[hrow * F + rt0 * 16 + r] = (int8_t)q0;
                 p.hq.qs[hrow * F + rt0 * 16 + 16 + r] = (int8_t)q1;
                 if (r == 0) {
-                    p.hq.d[hrow * nfb + fb] = __half2float(__float2half_rn(d));
-                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + fb] = sum;
+                    const float dh = __half2float(__float2half_rn(d));
+                    p.hq.d[hrow * nfb + fb] = dh;
+                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + fb] = q8_block_word(vecdot_dtype(DT), sum, dh);
                 }
             }
         }
@@ -489,7 +506,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_stream_kernel(ExpertPara
     const int H = p.H, F = p.F, nkb = F / 32;
     const int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
     if (rt >= H / 16) return;
-    constexpr int TB = (DT == MOE_GGML_Q8_0) ? Q8_0_TILE_BYTES : Q4_0_TILE_BYTES;
+    constexpr int TB = Q32Fmt<DT>::TB;
 
     int rowA[TT], rowD[TT][4];
 #pragma unroll
@@ -569,6 +586,9 @@ hipError_t launch_expert_up(const ExpertParams& p, hipStream_t s) {
         case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_up(p, s);
         case MOE_GGML_Q8_0: return launch_q32_up_t<MOE_GGML_Q8_0>(p, s);
         case MOE_GGML_Q4_0: return launch_q32_up_t<MOE_GGML_Q4_0>(p, s);
+        case MOE_GGML_Q4_1: return launch_q32_up_t<MOE_GGML_Q4_1>(p, s);
+        case MOE_GGML_Q5_0: return launch_q32_up_t<MOE_GGML_Q5_0>(p, s);
+        case MOE_GGML_Q5_1: return launch_q32_up_t<MOE_GGML_Q5_1>(p, s);
     }
     return hipErrorInvalidValue;
 }
@@ -578,6 +598,9 @@ hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s) {
         case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: return launch_q4k_down(p, s);
         case MOE_GGML_Q8_0: return launch_q32_down_t<MOE_GGML_Q8_0>(p, s);
         case MOE_GGML_Q4_0: return launch_q32_down_t<MOE_GGML_Q4_0>(p, s);
+        case MOE_GGML_Q4_1: return launch_q32_down_t<MOE_GGML_Q4_1>(p, s);
+        case MOE_GGML_Q5_0: return launch_q32_down_t<MOE_GGML_Q5_0>(p, s);
+        case MOE_GGML_Q5_1: return launch_q32_down_t<MOE_GGML_Q5_1>(p, s);
     }
     return hipErrorInvalidValue;
 }

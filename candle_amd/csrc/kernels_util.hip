@@ -1,7 +1,7 @@
 // Layout and format kernels: re-laying GGML blocks into the tiled device layout, `to_float`
 // from either layout, and the stand-alone activation quantiser used by the parity hooks.
 //
-// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 587-603 (Q8_0), 872-908 (Q2K), 1131-1186 (Q3K),
+// to_float restated from candle-core/src/quantized/k_quants.rs:166-186 (Q4_0), 340-359 (Q4_1), 443-465 (Q5_0), 556-581 (Q5_1), 587-603 (Q8_0), 872-908 (Q2K), 1131-1186 (Q3K),
 // 1347-1374 (Q4K, with get_scale_min_k4 of utils.rs:50-60), 1563-1595 (Q5K), 1753-1790 (Q6K) and 1858-1870 (Q8K).  The library is
 // built with -ffp-contract=off: `d1 * q - m1` must round the product before the subtraction.
 #include <algorithm>
@@ -81,6 +81,31 @@ __device__ inline int q6k_code(const uint8_t* blk, int e) {
 __device__ inline float q6k_value(float d, int8_t sc, int code) { return d * (float)sc * (float)(int8_t)(code - 32); }
 
 // ------------------------------------------------------------------ standard layout to_float
+// 32-element block formats with two codes per byte (Q4_0, Q4_1, Q5_0, Q5_1): where the pieces of a raw block sit
+// (d first; m, the fifth-bit word and the 16 nibble bytes after it) and where the tile keeps them.
+// to_float: k_quants.rs:166-186, 340-359, 443-465, 556-581.
+struct NibFmt {
+    int bytes, m_pos, h_pos, q_pos;   // raw block; a position of 0 = the format has no such field
+    int offset;                       // stored code - value (formats without a minimum)
+    int tile_bytes, tile_d, tile_d_stride;
+};
+__host__ __device__ inline bool is_nib(int dt) { return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q5_1; }
+__host__ __device__ inline NibFmt nib_fmt(int dt) {
+    switch (dt) {
+        case MOE_GGML_Q4_1: return {20, 2, 0, 4, 0, Q4_1_TILE_BYTES, 256, 4};
+        case MOE_GGML_Q5_0: return {22, 0, 2, 6, 16, Q5_0_TILE_BYTES, 320, 2};
+        case MOE_GGML_Q5_1: return {24, 2, 4, 8, 0, Q5_1_TILE_BYTES, 320, 4};
+        default: return {18, 0, 0, 2, 8, Q4_0_TILE_BYTES, 256, 2};
+    }
+}
+// element e of a block: low nibbles are elements 0..15, high nibbles 16..31, bit e of h is the fifth bit
+__device__ inline float nib_value(const NibFmt& f, uint16_t d_bits, uint16_t m_bits, uint8_t q, uint32_t h, int e) {
+    const int code = (e < 16 ? (q & 0xF) : (q >> 4)) | (int)(((h >> e) & 1u) << 4);
+    const float d = f16_bits_to_f32(d_bits);
+    if (!f.m_pos) return (float)(code - f.offset) * d;
+    return (float)code * d + f16_bits_to_f32(m_bits);
+}
+
 __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, int64_t n) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
@@ -105,13 +130,12 @@ __global__ void dequant_std_kernel(int dt, const uint8_t* blocks, float* out, in
         const uint8_t* b = blocks + (i / 256) * 210;
         int e = (int)(i % 256);
         out[i] = q6k_value(f16_bits_to_f32((uint16_t)(b[208] | (b[209] << 8))), (int8_t)b[192 + e / 16], q6k_code(b, e));
-    } else if (dt == MOE_GGML_Q4_0) {
-        const uint8_t* b = blocks + (i / 32) * 18;
+    } else if (is_nib(dt)) {
+        const NibFmt f = nib_fmt(dt);
+        const uint8_t* b = blocks + (i / 32) * f.bytes;
         int e = (int)(i % 32);
-        float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
-        uint8_t q = b[2 + (e % 16)];
-        int v = (e < 16 ? (q & 0xF) : (q >> 4)) - 8;
-        out[i] = (float)v * d;
+        uint32_t h = f.h_pos ? (uint32_t)b[f.h_pos] | ((uint32_t)b[f.h_pos + 1] << 8) | ((uint32_t)b[f.h_pos + 2] << 16) | ((uint32_t)b[f.h_pos + 3] << 24) : 0u;
+        out[i] = nib_value(f, (uint16_t)(b[0] | (b[1] << 8)), (uint16_t)(b[2] | (b[3] << 8)), b[f.q_pos + (e % 16)], h, e);
     } else if (dt == MOE_GGML_Q8_0) {
         const uint8_t* b = blocks + (i / 32) * 34;
         float d = f16_bits_to_f32((uint16_t)(b[0] | (b[1] << 8)));
@@ -273,19 +297,21 @@ __global__ void relayout_q8_0_kernel(const uint8_t* raw, uint8_t* tiled, int64_t
     if (g == 0) { dst[512 + 2 * r] = blk[0]; dst[512 + 2 * r + 1] = blk[1]; }
 }
 
-__global__ void relayout_q4_0_kernel(const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nkb) {
+__global__ void relayout_nib_kernel(int dt, const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nkb) {
     // one thread per (tile, row)
     int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= n_rt * nkb * 16) return;
+    const NibFmt f = nib_fmt(dt);
     int64_t tile = c / 16;
     int r = (int)(c % 16);
     int64_t rt = tile / nkb;
     int kb = (int)(tile % nkb);
-    const uint8_t* blk = raw + ((rt * 16 + r) * nkb + kb) * 18;
-    uint8_t* dst = tiled + tile * Q4_0_TILE_BYTES;
-    for (int i = 0; i < 16; i++) dst[r * 16 + i] = blk[2 + i];
-    dst[256 + 2 * r] = blk[0];
-    dst[256 + 2 * r + 1] = blk[1];
+    const uint8_t* blk = raw + ((rt * 16 + r) * nkb + kb) * f.bytes;
+    uint8_t* dst = tiled + tile * f.tile_bytes;
+    for (int i = 0; i < 16; i++) dst[r * 16 + i] = blk[f.q_pos + i];
+    if (f.h_pos)
+        for (int i = 0; i < 4; i++) dst[256 + 4 * r + i] = blk[f.h_pos + i];
+    for (int i = 0; i < f.tile_d_stride; i++) dst[f.tile_d + f.tile_d_stride * r + i] = blk[i];   // d, then m, lead the block
 }
 
 // ------------------------------------------------------------------ to_float from the tiled layout
@@ -348,13 +374,15 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         float d = f16_bits_to_f32((uint16_t)(tile[512 + 2 * r] | (tile[512 + 2 * r + 1] << 8)));
         int l = (e / 8) * 16 + r;
         out[i] = (float)(int8_t)tile[l * 8 + e % 8] * d;
-    } else {  // Q4_0
+    } else {  // Q4_0, Q4_1, Q5_0, Q5_1
+        const NibFmt f = nib_fmt(dt);
         int nkb = (int)(k / 32), kb = col / 32, e = col % 32;
-        const uint8_t* tile = tiled + (rt * nkb + kb) * Q4_0_TILE_BYTES;
-        float d = f16_bits_to_f32((uint16_t)(tile[256 + 2 * r] | (tile[256 + 2 * r + 1] << 8)));
-        uint8_t q = tile[r * 16 + e % 16];
-        int v = (e < 16 ? (q & 0xF) : (q >> 4)) - 8;
-        out[i] = (float)v * d;
+        const uint8_t* tile = tiled + (rt * nkb + kb) * f.tile_bytes;
+        const uint8_t* dm = tile + f.tile_d + f.tile_d_stride * r;
+        const uint8_t* hp = tile + 256 + 4 * r;
+        uint32_t h = f.h_pos ? (uint32_t)hp[0] | ((uint32_t)hp[1] << 8) | ((uint32_t)hp[2] << 16) | ((uint32_t)hp[3] << 24) : 0u;
+        uint16_t m_bits = f.m_pos ? (uint16_t)(dm[2] | (dm[3] << 8)) : (uint16_t)0;
+        out[i] = nib_value(f, (uint16_t)(dm[0] | (dm[1] << 8)), m_bits, tile[r * 16 + e % 16], h, e);
     }
 }
 
@@ -375,13 +403,13 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int6
     } else {
         const int nb = k / 32;
         for (int h = blockIdx.y * 256 + tid; h < k; h += 256 * gridDim.y)
-            quantize_q8_0_block(xr[h], lane, out.qs + row * k + h, out.d + row * nb + h / 32,
+            quantize_q8_0_block(VDT, xr[h], lane, out.qs + row * k + h, out.d + row * nb + h / 32,
                                 reinterpret_cast<int32_t*>(out.bsum) + row * nb + h / 32);
     }
 }
 
 // ActBuf -> the reference's block structs (BlockQ8K 292 B: d f32, qs[256], bsums i16[16];
-// BlockQ8_0 34 B: d f16, qs[32])
+// BlockQ8_0 34 B: d f16, qs[32]; BlockQ8_1 36 B: d f16, s f16, qs[32])
 __global__ void actbuf_to_std_kernel(int vdt, ActBuf in, int64_t rows, int k, uint8_t* out) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= rows * k) return;
@@ -397,13 +425,18 @@ __global__ void actbuf_to_std_kernel(int vdt, ActBuf in, int64_t rows, int k, ui
             __builtin_memcpy(blk + 260 + 2 * e, &s, 2);
         }
     } else {
+        const bool q81 = vdt == MOE_GGML_Q8_1;
         int nb = k / 32, b = col / 32, e = col % 32;
-        uint8_t* blk = out + (row * nb + b) * 34;
-        blk[2 + e] = (uint8_t)in.qs[row * k + col];
+        uint8_t* blk = out + (row * nb + b) * (q81 ? 36 : 34);
+        blk[(q81 ? 4 : 2) + e] = (uint8_t)in.qs[row * k + col];
         if (e == 0) {
-            // the stored f32 is an exactly widened f16
+            // the stored f32 values are exactly widened f16
             uint16_t h = __half_as_ushort(__float2half_rn(in.d[row * nb + b]));
             __builtin_memcpy(blk, &h, 2);
+            if (q81) {
+                uint16_t sh = __half_as_ushort(__float2half_rn(reinterpret_cast<const float*>(in.bsum)[row * nb + b]));
+                __builtin_memcpy(blk + 2, &sh, 2);
+            }
         }
     }
 }
@@ -428,7 +461,7 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
     else if (dt == MOE_GGML_Q8_0)
         hipLaunchKernelGGL(relayout_q8_0_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else
-        hipLaunchKernelGGL(relayout_q4_0_kernel, dim3(nblk(n_rt * nkb * 16, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+        hipLaunchKernelGGL(relayout_nib_kernel, dim3(nblk(n_rt * nkb * 16, 256)), dim3(256), 0, s, dt, raw, tiled, n_rt, nkb);
     return hipGetLastError();
 }
 
@@ -450,6 +483,8 @@ hipError_t launch_quantize_rows(int vdt, const float* x, int64_t rows, int k, co
     const unsigned split = (unsigned)std::max<int64_t>(1, std::min<int64_t>(per_row, 2048 / rows));
     if (vdt == MOE_GGML_Q8K)
         hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8K>, dim3((unsigned)rows, split), dim3(256), 0, s, x, rows, k, out);
+    else if (vdt == MOE_GGML_Q8_1)
+        hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8_1>, dim3((unsigned)rows, split), dim3(256), 0, s, x, rows, k, out);
     else
         hipLaunchKernelGGL(quantize_rows_kernel<MOE_GGML_Q8_0>, dim3((unsigned)rows, split), dim3(256), 0, s, x, rows, k, out);
     return hipGetLastError();

@@ -24,12 +24,12 @@ int fail(int code, const std::string& msg);
 int ensure_device();  // 0 if a gfx950 device is usable
 
 // ---------------------------------------------------------------- GGML block formats
-// Sizes per candle-core/src/quantized/k_quants.rs:45-51 (Q4_0), 81-87 (Q8_0), 98-106 (Q2K), 108-116 (Q3K), 118-127 (Q4K),
+// Sizes per candle-core/src/quantized/k_quants.rs:45-51 (Q4_0), 53-60 (Q4_1), 62-69 (Q5_0), 71-79 (Q5_1), 81-87 (Q8_0), 89-96 (Q8_1), 98-106 (Q2K), 108-116 (Q3K), 118-127 (Q4K),
 // 129-137 (Q5K), 142-149 (Q6K), 151-158 (Q8K).
 constexpr int QK_K = 256;
 inline int64_t block_elems(int dt) {
     switch (dt) {
-        case MOE_GGML_Q4_0: case MOE_GGML_Q8_0: return 32;
+        case MOE_GGML_Q4_0: case MOE_GGML_Q4_1: case MOE_GGML_Q5_0: case MOE_GGML_Q5_1: case MOE_GGML_Q8_0: case MOE_GGML_Q8_1: return 32;
         case MOE_GGML_Q2K: case MOE_GGML_Q3K: case MOE_GGML_Q4K: case MOE_GGML_Q5K: case MOE_GGML_Q6K: case MOE_GGML_Q8K: return 256;
         default: return -1;
     }
@@ -37,7 +37,11 @@ inline int64_t block_elems(int dt) {
 inline int64_t block_bytes(int dt) {
     switch (dt) {
         case MOE_GGML_Q4_0: return 18;
+        case MOE_GGML_Q4_1: return 20;
+        case MOE_GGML_Q5_0: return 22;
+        case MOE_GGML_Q5_1: return 24;
         case MOE_GGML_Q8_0: return 34;
+        case MOE_GGML_Q8_1: return 36;
         case MOE_GGML_Q2K: return 84;
         case MOE_GGML_Q3K: return 110;
         case MOE_GGML_Q4K: return 144;
@@ -47,11 +51,12 @@ inline int64_t block_bytes(int dt) {
         default: return -1;
     }
 }
-inline int vecdot_dtype(int dt) {  // GgmlType::VecDotType, k_quants.rs:163,584,1189,1600
-    return (dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K || dt == MOE_GGML_Q8K) ? MOE_GGML_Q8K : MOE_GGML_Q8_0;
+__host__ __device__ constexpr int vecdot_dtype(int dt) {  // GgmlType::VecDotType, k_quants.rs:163,264,365,471,584,1189,1600
+    return (dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K || dt == MOE_GGML_Q8K) ? MOE_GGML_Q8K
+         : (dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_1 || dt == MOE_GGML_Q8_1) ? MOE_GGML_Q8_1 : MOE_GGML_Q8_0;
 }
 inline bool weight_dtype_supported(int dt) {
-    return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K;
+    return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q5_1 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K;
 }
 
 // ---------------------------------------------------------------- device layouts
@@ -96,15 +101,20 @@ inline bool weight_dtype_supported(int dt) {
 //         [0,256)   (row r, half h): qs[row r][8h .. 8h+8)   (16 rows x 2 x 8 B)
 //         [256,288) row r : d (f16)
 //       MFMA k-chunk g of a Q4_0 block covers elements {0-7, 16-23, 8-15, 24-31}[g]: low / high
-//       nibbles of byte half g>>1 ... see experts_q32.hip.
+//       nibbles of byte half g>>1.
+//  Q4_1 / Q5_0 / Q5_1 tiles (320 / 352 / 384 B): the 256 nibble bytes as in the Q4_0 tile, then, for the
+//       five-bit formats, row r's 32 fifth bits as one little-endian word (bit e = element e), then row
+//       r's d (f16) and, for the formats with a block minimum, m (f16) as one 4-byte pair.
 //
-// ACTIVATIONS are quantised exactly as the reference does (Q8K for Q2K ... Q6K weights, Q8_0
-// otherwise) and stored per row as
+// ACTIVATIONS are quantised exactly as the reference does (Q8K for Q2K ... Q6K weights, Q8_1 for Q4_1 and
+// Q5_1, Q8_0 otherwise) and stored per row as
 //  Q8K  qs[K] with element k at ((k/64)*64 + ((k%32)/8)*16 + ((k/32)%2)*8 + k%8), so that lane
 //       (row, g) fetches sub-blocks 2P and 2P+1, chunk g, with one 16-byte load;
 //       d[K/256] f32;  bsums[K/256][16] as f16 (|sum of 16 quants| <= 2048 is exact in f16).
 //  Q8_0 qs[K] in natural order; d[K/32] f32 (the f16-rounded scale widened);
-//       bsum[K/32] i32 = sum of the block's 32 quants (used for Q4_0's -8 offset).
+//       bsum[K/32] i32 = sum of the block's 32 quants (used for the -8 / -16 offsets of Q4_0 / Q5_0).
+//  Q8_1 as Q8_0, except that the word beside every block holds the block's `s` widened to f32:
+//       s = f16(sum of quants) * d in binary16 arithmetic (k_quants.rs:727).
 constexpr int Q4K_TILE_BYTES = 2304;
 constexpr int Q2K_TILE_BYTES = 1344;
 constexpr int Q3K_TILE_BYTES = 1824;
@@ -112,6 +122,9 @@ constexpr int Q5K_TILE_BYTES = 2816;
 constexpr int Q6K_TILE_BYTES = 3360;
 constexpr int Q8_0_TILE_BYTES = 544;
 constexpr int Q4_0_TILE_BYTES = 288;
+constexpr int Q4_1_TILE_BYTES = 320;
+constexpr int Q5_0_TILE_BYTES = 352;
+constexpr int Q5_1_TILE_BYTES = 384;
 
 inline int64_t tile_bytes(int dt) {
     switch (dt) {
@@ -122,6 +135,9 @@ inline int64_t tile_bytes(int dt) {
         case MOE_GGML_Q6K: return Q6K_TILE_BYTES;
         case MOE_GGML_Q8_0: return Q8_0_TILE_BYTES;
         case MOE_GGML_Q4_0: return Q4_0_TILE_BYTES;
+        case MOE_GGML_Q4_1: return Q4_1_TILE_BYTES;
+        case MOE_GGML_Q5_0: return Q5_0_TILE_BYTES;
+        case MOE_GGML_Q5_1: return Q5_1_TILE_BYTES;
         default: return -1;
     }
 }
@@ -134,7 +150,7 @@ inline int64_t relaid_bytes(int dt, int64_t rows, int64_t k) {
 struct ActBuf {
     int8_t* qs = nullptr;    // [rows][K]
     float* d = nullptr;      // [rows][K/block]
-    void* bsum = nullptr;    // Q8K: __half [rows][K/256][16]; Q8_0: int32 [rows][K/32]
+    void* bsum = nullptr;    // Q8K: __half [rows][K/256][16]; Q8_0: int32 [rows][K/32]; Q8_1: float s [rows][K/32]
 };
 
 // ---------------------------------------------------------------- exp with the CPU's rounding

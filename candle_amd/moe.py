@@ -11,8 +11,10 @@ import os
 
 import numpy as np
 
-GGML_Q4_0, GGML_Q8_0, GGML_Q2K, GGML_Q3K, GGML_Q4K, GGML_Q5K, GGML_Q6K, GGML_Q8K = 2, 8, 10, 11, 12, 13, 14, 15
-_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q8_0: (32, 34), GGML_Q2K: (256, 84), GGML_Q3K: (256, 110), GGML_Q4K: (256, 144), GGML_Q5K: (256, 176), GGML_Q6K: (256, 210),
+GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1, GGML_Q8_0, GGML_Q8_1 = 2, 3, 6, 7, 8, 9
+GGML_Q2K, GGML_Q3K, GGML_Q4K, GGML_Q5K, GGML_Q6K, GGML_Q8K = 10, 11, 12, 13, 14, 15
+_BLOCK = {GGML_Q4_0: (32, 18), GGML_Q4_1: (32, 20), GGML_Q5_0: (32, 22), GGML_Q5_1: (32, 24), GGML_Q8_0: (32, 34), GGML_Q8_1: (32, 36),
+          GGML_Q2K: (256, 84), GGML_Q3K: (256, 110), GGML_Q4K: (256, 144), GGML_Q5K: (256, 176), GGML_Q6K: (256, 210),
           GGML_Q8K: (256, 292)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -287,7 +289,7 @@ class SparseMoeBlock:
         L = load_library()
         dtype_down = ggml_dtype if ggml_dtype_down is None else ggml_dtype_down
         for dt in (ggml_dtype, dtype_down):
-            if dt not in _BLOCK or dt == GGML_Q8K:
+            if dt not in _BLOCK or dt in (GGML_Q8K, GGML_Q8_1):
                 raise MoeError("unsupported ggml_dtype %r" % (dt,))
         self.dtype_down = dtype_down
         if len(w1) != n_experts or len(w2) != n_experts or len(w3) != n_experts:
@@ -428,7 +430,7 @@ class QMatMul:
     of quantized_llama.rs:590-593, 608)."""
 
     def __init__(self, ggml_dtype, w_blocks, n, k):
-        if ggml_dtype not in _BLOCK or ggml_dtype == GGML_Q8K:
+        if ggml_dtype not in _BLOCK or ggml_dtype in (GGML_Q8K, GGML_Q8_1):
             raise MoeError("unsupported ggml_dtype %r" % (ggml_dtype,))
         w_blocks = _blocks(w_blocks, ggml_dtype, n * k, "QMatMul")
         h = C.c_void_p()

@@ -33,7 +33,11 @@ extern "C" {
 
 /* GgmlDType numbering, candle-core/src/quantized/mod.rs:153-174 (also the GGUF on-disk ids). */
 #define MOE_GGML_Q4_0 2
+#define MOE_GGML_Q4_1 3
+#define MOE_GGML_Q5_0 6
+#define MOE_GGML_Q5_1 7
 #define MOE_GGML_Q8_0 8
+#define MOE_GGML_Q8_1 9   /* activations only (VecDotType of Q4_1 and Q5_1) */
 #define MOE_GGML_Q2K 10
 #define MOE_GGML_Q3K 11
 #define MOE_GGML_Q4K 12
@@ -59,7 +63,7 @@ typedef struct {
     int64_t ffn;                 /* F: per-expert intermediate size */
     int64_t n_experts;           /* E (1..256) */
     int64_t top_k;               /* n_expert_used (1..min(E,16)) */
-    int32_t ggml_dtype;          /* MOE_GGML_Q4_0 | Q8_0 | Q2K | Q3K | Q4K | Q5K | Q6K: dtype of every w1 and w3 (and of w2
+    int32_t ggml_dtype;          /* MOE_GGML_Q4_0 | Q4_1 | Q5_0 | Q5_1 | Q8_0 | Q2K | Q3K | Q4K | Q5K | Q6K: dtype of every w1 and w3 (and of w2
                                     unless ggml_dtype_down says otherwise) */
     int32_t norm_topk;           /* 1: weights renormalised over the selected experts (Mixtral,
                                     quantized_llama.rs:175-178); 0: raw softmax probability
@@ -80,7 +84,8 @@ typedef struct {
     float rms_eps;
     /* dtype of every w2 (and shared_w2) when it differs from ggml_dtype, 0 = the same.  GGUF files of
      * the Q4_K_M flavour store ffn_down of some layers as Q6K beside Q4K gate / up matrices; the two
-     * dtypes must quantise activations the same way (Q2K ... Q6K use Q8K; Q4_0 and Q8_0 use Q8_0). */
+     * dtypes must quantise activations the same way (Q2K ... Q6K use Q8K; Q4_0, Q5_0 and Q8_0 use Q8_0;
+     * Q4_1 and Q5_1 use Q8_1). */
     int32_t ggml_dtype_down;
 } moe_desc;
 
@@ -132,13 +137,13 @@ int moe_layer_dequantize_weight(moe_layer* layer, int64_t expert, int which, flo
 int moe_route(const float* logits, int64_t n_tokens, int64_t n_experts, int64_t top_k, int32_t norm_topk,
               int32_t* topk_idx, float* topk_w, int32_t* expert_offsets, int32_t* perm_token, float* perm_w);
 
-/* Parity hook: GgmlType::to_float on raw blocks (host pointers), k_quants.rs:166-186 (Q4_0),
- * 587-603 (Q8_0), 872-908 (Q2K), 1131-1186 (Q3K), 1347-1374 (Q4K), 1563-1595 (Q5K), 1753-1790 (Q6K), 1858-1870 (Q8K). */
+/* Parity hook: GgmlType::to_float on raw blocks (host pointers), k_quants.rs:166-186 (Q4_0), 340-359 (Q4_1),
+ * 443-465 (Q5_0), 556-581 (Q5_1), 587-603 (Q8_0), 872-908 (Q2K), 1131-1186 (Q3K), 1347-1374 (Q4K), 1563-1595 (Q5K), 1753-1790 (Q6K), 1858-1870 (Q8K). */
 int moe_dequantize(int32_t ggml_dtype, const void* blocks, int64_t n_elems, float* out);
 
 /* Parity hook: the activation quantiser k_quants::matmul applies to every lhs row
- * (k_quants.rs:1893-1903): vecdot_dtype MOE_GGML_Q8_0 (k_quants.rs:605-634) or MOE_GGML_Q8K
- * (k_quants.rs:1819-1856).  x is host f32 [rows, k]; out receives rows*k/block standard blocks. */
+ * (k_quants.rs:1893-1903): vecdot_dtype MOE_GGML_Q8_0 (k_quants.rs:605-634), MOE_GGML_Q8_1
+ * (k_quants.rs:700-729) or MOE_GGML_Q8K (k_quants.rs:1819-1856).  x is host f32 [rows, k]; out receives rows*k/block standard blocks. */
 int moe_quantize_act(int32_t vecdot_dtype, const float* x, int64_t rows, int64_t k, void* out);
 
 /* Parity hook: QMatMul::forward on one quantized matrix (quantized/mod.rs:533-537 ->
@@ -151,7 +156,7 @@ int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, 
  * 533-537 (forward): the attention projections and the output head around the MoE block
  * (quantized_llama.rs:590-593 attention_wq/wk/wv/wo, :608 output; applied at :275-277, :345, :897).
  * create uploads the [n, k] matrix of raw GGML blocks once (n % 16 == 0, k a multiple of the block
- * size; Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K) and keeps it resident in the kernels' layout; forward quantises the m rows
+ * size; Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K) and keeps it resident in the kernels' layout; forward quantises the m rows
  * of x as k_quants::matmul does (k_quants.rs:1893-1903) and writes y[m, n] = x . W^T.
  * forward takes host pointers and returns when y is filled; forward_device takes device pointers and
  * enqueues on hip_stream.  Calls on one object serialise; dequantize is QMatMul::dequantize

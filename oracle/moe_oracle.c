@@ -96,7 +96,7 @@ static inline float rmin(float a, float b) { return fminf(a, b); }
 
 int64_t orc_block_elems(int dtype) {
     switch (dtype) {
-        case ORC_Q4_0: case ORC_Q8_0: return 32;
+        case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_Q8_0: case ORC_Q8_1: return 32;
         case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return 256;
         default: return -1;
     }
@@ -104,7 +104,11 @@ int64_t orc_block_elems(int dtype) {
 int64_t orc_block_bytes(int dtype) {
     switch (dtype) {
         case ORC_Q4_0: return 18;
+        case ORC_Q4_1: return 20;
+        case ORC_Q5_0: return 22;
+        case ORC_Q5_1: return 24;
         case ORC_Q8_0: return 34;
+        case ORC_Q8_1: return 36;
         case ORC_Q2K: return 84;
         case ORC_Q3K: return 110;
         case ORC_Q4K: return 144;
@@ -116,7 +120,8 @@ int64_t orc_block_bytes(int dtype) {
 }
 int orc_vecdot_dtype(int dtype) {
     switch (dtype) {
-        case ORC_Q4_0: case ORC_Q8_0: return ORC_Q8_0;
+        case ORC_Q4_0: case ORC_Q5_0: case ORC_Q8_0: return ORC_Q8_0;
+        case ORC_Q4_1: case ORC_Q5_1: case ORC_Q8_1: return ORC_Q8_1;
         case ORC_Q2K: case ORC_Q3K: case ORC_Q4K: case ORC_Q5K: case ORC_Q6K: case ORC_Q8K: return ORC_Q8K;
         default: return -1;
     }
@@ -167,6 +172,205 @@ static float vec_dot_q4_0_q8_0(int64_t n, const orc_block_q4_0* xs, const orc_bl
             int v1 = (int)(xs[b].qs[j] >> 4) - 8;
             sum_i += v0 * (int)ys[b].qs[j] + v1 * (int)ys[b].qs[j + 16];
         }
+        sumf += (float)sum_i * orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d);
+    }
+    return sumf;
+}
+
+/* ------------------------------------------------------------------ Q4_1 */
+/* k_quants.rs:299-337 */
+static void quantize_q4_1(const float* xs, int64_t k, orc_block_q4_1* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        const float* x = xs + i * qk;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < qk; j++) { min = rmin(x[j], min); max = rmax(x[j], max); }
+        float d = (max - min) / 15.0f;
+        float id = (d != 0.f) ? 1.f / d : 0.f;
+        ys[i].d = orc_f32_to_f16(d);
+        ys[i].m = orc_f32_to_f16(min);
+        for (int j = 0; j < qk / 2; j++) {
+            float x0 = (x[j] - min) * id;
+            float x1 = (x[qk / 2 + j] - min) * id;
+            uint8_t xi0 = sat_u8(x0 + 0.5f); if (xi0 > 15) xi0 = 15;
+            uint8_t xi1 = sat_u8(x1 + 0.5f); if (xi1 > 15) xi1 = 15;
+            ys[i].qs[j] = (uint8_t)(xi0 | (xi1 << 4));
+        }
+    }
+}
+/* k_quants.rs:340-359 */
+static void dequantize_q4_1(const orc_block_q4_1* xs, int64_t k, float* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        float d = orc_f16_to_f32(xs[i].d), m = orc_f16_to_f32(xs[i].m);
+        for (int j = 0; j < qk / 2; j++) {
+            int x0 = xs[i].qs[j] & 0x0F, x1 = xs[i].qs[j] >> 4;
+            ys[i * qk + j] = (float)x0 * d + m;
+            ys[i * qk + j + qk / 2] = (float)x1 * d + m;
+        }
+    }
+}
+/* k_quants.rs:270-297 */
+static float vec_dot_q4_1_q8_1(int64_t n, const orc_block_q4_1* xs, const orc_block_q8_1* ys) {
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 32; b++) {
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int v0 = xs[b].qs[j] & 0x0F, v1 = xs[b].qs[j] >> 4;
+            sumi += v0 * (int)ys[b].qs[j] + v1 * (int)ys[b].qs[j + 16];
+        }
+        sumf += (float)sumi * orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d)
+              + orc_f16_to_f32(xs[b].m) * orc_f16_to_f32(ys[b].s);
+    }
+    return sumf;
+}
+
+/* ------------------------------------------------------------------ Q5_0 */
+static inline uint32_t rd_u32le(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24); }
+static inline void wr_u32le(uint8_t* p, uint32_t v) { p[0] = (uint8_t)v; p[1] = (uint8_t)(v >> 8); p[2] = (uint8_t)(v >> 16); p[3] = (uint8_t)(v >> 24); }
+/* k_quants.rs:404-440 */
+static void quantize_q5_0(const float* xs, int64_t k, orc_block_q5_0* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        const float* x = xs + i * qk;
+        float amax = 0.f, max = 0.f;
+        for (int j = 0; j < qk; j++) {
+            if (amax < fabsf(x[j])) { amax = fabsf(x[j]); max = x[j]; }
+        }
+        float d = max / -16.0f;
+        float id = (d != 0.f) ? 1.f / d : 0.f;
+        ys[i].d = orc_f32_to_f16(d);
+        uint32_t qh = 0;
+        for (int j = 0; j < qk / 2; j++) {
+            float x0 = x[j] * id, x1 = x[j + qk / 2] * id;
+            int8_t s0 = sat_i8(x0 + 16.5f); if (s0 > 31) s0 = 31;     /* `as i8` then .min(31) then `as u8` */
+            int8_t s1 = sat_i8(x1 + 16.5f); if (s1 > 31) s1 = 31;
+            uint8_t xi0 = (uint8_t)s0, xi1 = (uint8_t)s1;
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + qk / 2);
+        }
+        wr_u32le(ys[i].qh, qh);
+    }
+}
+/* k_quants.rs:443-465 */
+static void dequantize_q5_0(const orc_block_q5_0* xs, int64_t k, float* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        float d = orc_f16_to_f32(xs[i].d);
+        uint32_t qh = rd_u32le(xs[i].qh);
+        for (int j = 0; j < qk / 2; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh >> j) << 4) & 0x10);
+            uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            int x0 = (int)((xs[i].qs[j] & 0x0F) | xh_0) - 16;
+            int x1 = (int)((xs[i].qs[j] >> 4) | xh_1) - 16;
+            ys[i * qk + j] = (float)x0 * d;
+            ys[i * qk + j + qk / 2] = (float)x1 * d;
+        }
+    }
+}
+/* k_quants.rs:381-402 (vec_dot is vec_dot_unopt on every target, :367-379) */
+static float vec_dot_q5_0_q8_0(int64_t n, const orc_block_q5_0* xs, const orc_block_q8_0* ys) {
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 32; b++) {
+        uint32_t qh = rd_u32le(xs[b].qh);
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh & (1u << j)) >> j) << 4);
+            uint8_t xh_1 = (uint8_t)((qh & (1u << (j + 16))) >> (j + 12));
+            int x0 = ((int)(xs[b].qs[j] & 0x0F) | (int)xh_0) - 16;
+            int x1 = ((int)(xs[b].qs[j] >> 4) | (int)xh_1) - 16;
+            sumi += x0 * (int)ys[b].qs[j] + x1 * (int)ys[b].qs[j + 16];
+        }
+        sumf += (float)sumi * orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d);
+    }
+    return sumf;
+}
+
+/* ------------------------------------------------------------------ Q5_1 */
+/* k_quants.rs:511-553 */
+static void quantize_q5_1(const float* xs, int64_t k, orc_block_q5_1* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        const float* x = xs + i * qk;
+        float min = INFINITY, max = -INFINITY;
+        for (int j = 0; j < qk; j++) { min = rmin(x[j], min); max = rmax(x[j], max); }
+        float d = (max - min) / 31.0f;
+        float id = (d != 0.f) ? 1.f / d : 0.f;
+        ys[i].d = orc_f32_to_f16(d);
+        ys[i].m = orc_f32_to_f16(min);
+        uint32_t qh = 0;
+        for (int j = 0; j < qk / 2; j++) {
+            float x0 = (x[j] - min) * id, x1 = (x[qk / 2 + j] - min) * id;
+            uint8_t xi0 = sat_u8(x0 + 0.5f), xi1 = sat_u8(x1 + 0.5f);
+            ys[i].qs[j] = (uint8_t)((xi0 & 0x0F) | ((xi1 & 0x0F) << 4));
+            qh |= (((uint32_t)xi0 & 0x10u) >> 4) << j;
+            qh |= (((uint32_t)xi1 & 0x10u) >> 4) << (j + qk / 2);
+        }
+        wr_u32le(ys[i].qh, qh);
+    }
+}
+/* k_quants.rs:556-581 */
+static void dequantize_q5_1(const orc_block_q5_1* xs, int64_t k, float* ys) {
+    const int qk = 32;
+    for (int64_t i = 0; i < k / qk; i++) {
+        float d = orc_f16_to_f32(xs[i].d), m = orc_f16_to_f32(xs[i].m);
+        uint32_t qh = rd_u32le(xs[i].qh);
+        for (int j = 0; j < qk / 2; j++) {
+            uint8_t xh_0 = (uint8_t)(((qh >> j) << 4) & 0x10);
+            uint8_t xh_1 = (uint8_t)((qh >> (j + 12)) & 0x10);
+            int x0 = (xs[i].qs[j] & 0x0F) | xh_0;
+            int x1 = (xs[i].qs[j] >> 4) | xh_1;
+            ys[i * qk + j] = (float)x0 * d + m;
+            ys[i * qk + j + qk / 2] = (float)x1 * d + m;
+        }
+    }
+}
+/* k_quants.rs:477-509 */
+static float vec_dot_q5_1_q8_1(int64_t n, const orc_block_q5_1* xs, const orc_block_q8_1* ys) {
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 32; b++) {
+        uint32_t qh = rd_u32le(xs[b].qh);
+        int32_t sumi = 0;
+        for (int j = 0; j < 16; j++) {
+            int xh_0 = (int)(((qh >> j) << 4) & 0x10);
+            int xh_1 = (int)((qh >> (j + 12)) & 0x10);
+            int x0 = (xs[b].qs[j] & 0xF) | xh_0;
+            int x1 = (xs[b].qs[j] >> 4) | xh_1;
+            sumi += x0 * (int)ys[b].qs[j] + x1 * (int)ys[b].qs[j + 16];
+        }
+        sumf += (float)sumi * orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d)
+              + orc_f16_to_f32(xs[b].m) * orc_f16_to_f32(ys[b].s);
+    }
+    return sumf;
+}
+
+/* ------------------------------------------------------------------ Q8_1 */
+/* k_quants.rs:700-729.  `s` is computed in f16 arithmetic: f16(sum) * d, i.e. the two f16 values widened,
+ * multiplied in f32 and rounded once (half 2.5.0, binary16 arithmetic through f32). */
+static void quantize_q8_1(const float* xs, int64_t k, orc_block_q8_1* ys) {
+    for (int64_t i = 0; i < k / 32; i++) {
+        const float* x = xs + i * 32;
+        float amax = 0.f;
+        for (int j = 0; j < 32; j++) amax = rmax(amax, fabsf(x[j]));
+        float d = amax / 127.0f;
+        float id = (d != 0.f) ? 1.f / d : 0.f;
+        ys[i].d = orc_f32_to_f16(d);
+        int32_t sum = 0;
+        for (int j = 0; j < 16; j++) {
+            ys[i].qs[j] = sat_i8(roundf(x[j] * id));
+            ys[i].qs[j + 16] = sat_i8(roundf(x[j + 16] * id));
+            sum += (int32_t)ys[i].qs[j] + (int32_t)ys[i].qs[j + 16];
+        }
+        ys[i].s = orc_f32_to_f16(orc_f16_to_f32(orc_f32_to_f16((float)sum)) * orc_f16_to_f32(ys[i].d));
+    }
+}
+/* k_quants.rs:680-698 */
+static float vec_dot_q8_1_q8_1(int64_t n, const orc_block_q8_1* xs, const orc_block_q8_1* ys) {
+    float sumf = 0.f;
+    for (int64_t b = 0; b < n / 32; b++) {
+        int32_t sum_i = 0;
+        for (int j = 0; j < 32; j++) sum_i += (int)xs[b].qs[j] * (int)ys[b].qs[j];
         sumf += (float)sum_i * orc_f16_to_f32(xs[b].d) * orc_f16_to_f32(ys[b].d);
     }
     return sumf;
@@ -1051,6 +1255,10 @@ int orc_quantize(int dtype, const float* x, int64_t n, void* blocks) {
     switch (dtype) {
         case ORC_Q4_0: quantize_q4_0(x, n, (orc_block_q4_0*)blocks); return 0;
         case ORC_Q8_0: quantize_q8_0(x, n, (orc_block_q8_0*)blocks); return 0;
+        case ORC_Q4_1: quantize_q4_1(x, n, (orc_block_q4_1*)blocks); return 0;
+        case ORC_Q5_0: quantize_q5_0(x, n, (orc_block_q5_0*)blocks); return 0;
+        case ORC_Q5_1: quantize_q5_1(x, n, (orc_block_q5_1*)blocks); return 0;
+        case ORC_Q8_1: quantize_q8_1(x, n, (orc_block_q8_1*)blocks); return 0;
         case ORC_Q4K: memset(blocks, 0, (size_t)(n / 256) * 144); quantize_q4k(x, n, (orc_block_q4k*)blocks); return 0;
         case ORC_Q2K: memset(blocks, 0, (size_t)(n / 256) * 84); quantize_q2k(x, n, (orc_block_q2k*)blocks); return 0;
         case ORC_Q3K: memset(blocks, 0, (size_t)(n / 256) * 110); quantize_q3k(x, n, (orc_block_q3k*)blocks); return 0;
@@ -1066,6 +1274,9 @@ int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y) {
     switch (dtype) {
         case ORC_Q4_0: dequantize_q4_0((const orc_block_q4_0*)blocks, n, y); return 0;
         case ORC_Q8_0: dequantize_q8_0((const orc_block_q8_0*)blocks, n, y); return 0;
+        case ORC_Q4_1: dequantize_q4_1((const orc_block_q4_1*)blocks, n, y); return 0;
+        case ORC_Q5_0: dequantize_q5_0((const orc_block_q5_0*)blocks, n, y); return 0;
+        case ORC_Q5_1: dequantize_q5_1((const orc_block_q5_1*)blocks, n, y); return 0;
         case ORC_Q4K: dequantize_q4k((const orc_block_q4k*)blocks, n, y); return 0;
         case ORC_Q2K: dequantize_q2k((const orc_block_q2k*)blocks, n, y); return 0;
         case ORC_Q3K: dequantize_q3k((const orc_block_q3k*)blocks, n, y); return 0;
@@ -1079,6 +1290,10 @@ float orc_vec_dot(int dtype, int64_t n, const void* w, const void* a) {
     switch (dtype) {
         case ORC_Q4_0: return vec_dot_q4_0_q8_0(n, (const orc_block_q4_0*)w, (const orc_block_q8_0*)a);
         case ORC_Q8_0: return vec_dot_q8_0_q8_0(n, (const orc_block_q8_0*)w, (const orc_block_q8_0*)a);
+        case ORC_Q4_1: return vec_dot_q4_1_q8_1(n, (const orc_block_q4_1*)w, (const orc_block_q8_1*)a);
+        case ORC_Q5_0: return vec_dot_q5_0_q8_0(n, (const orc_block_q5_0*)w, (const orc_block_q8_0*)a);
+        case ORC_Q5_1: return vec_dot_q5_1_q8_1(n, (const orc_block_q5_1*)w, (const orc_block_q8_1*)a);
+        case ORC_Q8_1: return vec_dot_q8_1_q8_1(n, (const orc_block_q8_1*)w, (const orc_block_q8_1*)a);
         case ORC_Q4K: return vec_dot_q4k_q8k(n, (const orc_block_q4k*)w, (const orc_block_q8k*)a);
         case ORC_Q2K: return vec_dot_q2k_q8k(n, (const orc_block_q2k*)w, (const orc_block_q8k*)a);
         case ORC_Q3K: return vec_dot_q3k_q8k(n, (const orc_block_q3k*)w, (const orc_block_q8k*)a);

@@ -42,11 +42,15 @@ extern "C" {
 #endif
 
 /* ggml dtype numbering: candle-core/src/quantized/mod.rs:153-174 */
-enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14, ORC_Q8K = 15 };
+enum { ORC_Q4_0 = 2, ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q8_0 = 8, ORC_Q8_1 = 9, ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14, ORC_Q8K = 15 };
 
 #pragma pack(push, 1)
 typedef struct { uint16_t d; uint8_t qs[16]; } orc_block_q4_0;            /* k_quants.rs:45-51  */
 typedef struct { uint16_t d; int8_t qs[32]; } orc_block_q8_0;             /* k_quants.rs:81-87  */
+typedef struct { uint16_t d, m; uint8_t qs[16]; } orc_block_q4_1;         /* k_quants.rs:53-60  */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } orc_block_q5_0;     /* k_quants.rs:62-69  */
+typedef struct { uint16_t d, m; uint8_t qh[4]; uint8_t qs[16]; } orc_block_q5_1;  /* k_quants.rs:71-79  */
+typedef struct { uint16_t d, s; int8_t qs[32]; } orc_block_q8_1;          /* k_quants.rs:89-96  */
 typedef struct { uint16_t d, dmin; uint8_t scales[12]; uint8_t qs[128]; } orc_block_q4k; /* :118-127 */
 typedef struct { uint8_t scales[16]; uint8_t qs[64]; uint16_t d, dmin; } orc_block_q2k;   /* k_quants.rs:98-106 */
 typedef struct { uint8_t hmask[32]; uint8_t qs[64]; uint8_t scales[12]; uint16_t d; } orc_block_q3k; /* k_quants.rs:108-116 */

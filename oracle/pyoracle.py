@@ -12,10 +12,13 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libmoe_oracle.so")
 
-Q4_0, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 8, 10, 11, 12, 13, 14, 15
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q2K: 256, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
-BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q2K: 84, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
-VECDOT = {Q4_0: Q8_0, Q8_0: Q8_0, Q2K: Q8K, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q8_1, Q2K, Q3K, Q4K, Q5K, Q6K, Q8K = 2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15
+BLOCK_ELEMS = {Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: 32, Q8_1: 32,
+               Q2K: 256, Q3K: 256, Q4K: 256, Q5K: 256, Q6K: 256, Q8K: 256}
+BLOCK_BYTES = {Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34, Q8_1: 36,
+               Q2K: 84, Q3K: 110, Q4K: 144, Q5K: 176, Q6K: 210, Q8K: 292}
+VECDOT = {Q4_0: Q8_0, Q5_0: Q8_0, Q8_0: Q8_0, Q4_1: Q8_1, Q5_1: Q8_1, Q8_1: Q8_1,
+          Q2K: Q8K, Q3K: Q8K, Q4K: Q8K, Q5K: Q8K, Q6K: Q8K, Q8K: Q8K}
 
 
 def build(force=False):

@@ -21,7 +21,7 @@ def build(dt, H=512, F=1024, E=8, seed=11):
     return gate, w1, w3, w2
 
 
-@pytest.mark.parametrize("dt", [O.Q4K, O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("dt", [O.Q4K, O.Q8_0, O.Q4_0, O.Q5_0, O.Q5_1])
 @pytest.mark.parametrize("version", [2, 3])
 def test_layer_from_gguf_equals_layer_from_arrays(tmp_path, dt, version):
     H, F, E, k = 512, 1024, 8, 2
@@ -78,11 +78,11 @@ def test_loader_errors(tmp_path):
     W.moe_layer_file(pm, 0, gate, w1, w3, w2_q8, O.Q4K, k, down_dtype=O.Q8_0)
     with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):
         candle_amd.SparseMoeBlock.from_gguf(str(pm), 0)
-    # an unsupported dtype among the experts (Q5_0 = 6)
-    pu = tmp_path / "q5_0.gguf"
-    w2_q5 = [np.zeros(H * F // 32 * 22, np.uint8) for _ in range(E)]
-    W.moe_layer_file(pu, 0, gate, w1, w3, w2_q5, O.Q4K, k, down_dtype=6)
-    with pytest.raises(candle_amd.MoeError, match="unsupported ggml_dtype 6"):
+    # an unsupported dtype among the experts (Q8_1 = 9, an activation format)
+    pu = tmp_path / "q8_1.gguf"
+    w2_q81 = [np.zeros(H * F // 32 * 36, np.uint8) for _ in range(E)]
+    W.moe_layer_file(pu, 0, gate, w1, w3, w2_q81, O.Q4K, k, down_dtype=9)
+    with pytest.raises(candle_amd.MoeError, match="unsupported ggml_dtype 9"):
         candle_amd.SparseMoeBlock.from_gguf(str(pu), 0)
 
 

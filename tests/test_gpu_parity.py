@@ -39,7 +39,7 @@ def test_device_is_gfx950():
     assert candle_amd.device_arch().startswith("gfx950")
 
 
-@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K, O.Q8K])
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K, O.Q8K])
 def test_to_float_bit_exact(dt):
     n = 256 * 96
     x = O.fill_normal(dt, n, 0.0, 0.02)
@@ -51,7 +51,7 @@ def test_to_float_bit_exact(dt):
     # arbitrary bit patterns in the quant payload (scale fields kept finite)
     rng = np.random.default_rng(dt)
     raw = blocks.copy().reshape(-1, O.BLOCK_BYTES[dt])
-    lo, hi = {O.Q4_0: (2, 18), O.Q8_0: (2, 34), O.Q2K: (0, 80), O.Q3K: (0, 108), O.Q4K: (4, 144), O.Q5K: (4, 176), O.Q6K: (0, 208), O.Q8K: (4, 292)}[dt]
+    lo, hi = {O.Q4_0: (2, 18), O.Q4_1: (4, 20), O.Q5_0: (2, 22), O.Q5_1: (4, 24), O.Q8_0: (2, 34), O.Q2K: (0, 80), O.Q3K: (0, 108), O.Q4K: (4, 144), O.Q5K: (4, 176), O.Q6K: (0, 208), O.Q8K: (4, 292)}[dt]
     raw[:, lo:hi] = rng.integers(0, 256, raw[:, lo:hi].shape, dtype=np.uint8)
     raw = raw.reshape(-1)
     assert np.array_equal(bits(candle_amd.dequantize(dt, raw, n)), bits(O.dequantize(dt, raw, n)))
@@ -79,7 +79,7 @@ def test_weight_quantiser_bit_exact(dt, golden):
     assert np.array_equal(out.cpu().numpy(), O.quantize(dt, x))
 
 
-@pytest.mark.parametrize("vdt", [O.Q8_0, O.Q8K])
+@pytest.mark.parametrize("vdt", [O.Q8_0, O.Q8_1, O.Q8K])
 def test_activation_quantiser_bit_exact(vdt):
     rows, k = 37, 2048
     x = O.fill_normal(5 + vdt, rows * k).reshape(rows, k)
@@ -91,6 +91,8 @@ def test_activation_quantiser_bit_exact(vdt):
     x[5] *= 1e-20
     x[6] *= 1e20
     x[7, ::2] = 0.5                 # exact .5 ties after scaling
+    x[8, :32] = 3.0                 # block sum 32 * 127 = 4064 is not representable in f16 (Q8_1's s rounds it)
+    x[9] *= 1e-7                    # Q8_1: s = f16(sum) * d falls among the f16 subnormals
     got = candle_amd.quantize_act(vdt, x)
     want = O.quantize(vdt, x)
     assert np.array_equal(got, want)
@@ -129,13 +131,16 @@ def test_route_zipf_bias_lists():
                                        (O.Q3K, 64, 512, 5), (O.Q3K, 1040, 1024, 33), (O.Q3K, 256, 2304, 150),
                                        (O.Q5K, 64, 512, 5), (O.Q5K, 1040, 1024, 33), (O.Q5K, 256, 2304, 150),
                                        (O.Q6K, 64, 512, 5), (O.Q6K, 1040, 1024, 33), (O.Q6K, 256, 2304, 150),
-                                       (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70)])
+                                       (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70),
+                                       (O.Q5_0, 48, 96, 3), (O.Q5_0, 256, 1408, 40), (O.Q5_0, 128, 1024, 70),
+                                       (O.Q4_1, 48, 96, 3), (O.Q4_1, 256, 1408, 40), (O.Q4_1, 128, 1024, 70),
+                                       (O.Q5_1, 48, 96, 3), (O.Q5_1, 256, 1408, 40), (O.Q5_1, 128, 1024, 70)])
 def test_qmatmul_against_oracle(dt, n, k, m):
     w = O.fill_normal_quantized(n + k, dt, n, k, 0.02)
     x = activations(m, k, seed=n)
     got = candle_amd.qmatmul(dt, w, n, k, x)
     want = O.matmul(dt, x, w, n)
-    if dt in (O.Q4_0, O.Q8_0):
+    if O.BLOCK_ELEMS[dt] == 32:
         # same per-block values added in the same order as the scalar reference loop
         assert np.array_equal(bits(got), bits(want))
     else:
@@ -278,7 +283,31 @@ def test_block_q6k_shared_expert():
     gpu.close()
 
 
+@pytest.mark.parametrize("dt,dt_down", [(O.Q5_0, None), (O.Q4_1, None), (O.Q5_1, None), (O.Q4_0, O.Q5_0), (O.Q5_0, O.Q8_0),
+                                        (O.Q5_1, O.Q4_1)])
+def test_block_legacy_five_bit_and_min_formats(dt, dt_down):
+    # Q5_0 (Q8_0 activations, code - 16), Q4_1 and Q5_1 (Q8_1 activations, block minimum times the activation
+    # block's s), alone and mixed with another format of the same activation type; with the always-on expert.
+    # T = 1, 8: one slot tile; 33: two; 70: a second pass; 300: dispatched lists
+    ref, gpu = make_pair(256, 512, 8, 2, dt, seed=31, Fs=256, dt_down=dt_down)
+    for T in (1, 8, 33, 70, 300):
+        check_block(ref, gpu, T, tol=TOL)
+    for e, which, wdt in ((0, 1, dt), (7, 3, dt), (5, 2, dt_down or dt)):
+        want = O.dequantize(wdt, getattr(ref, "w%d" % which)[e], 256 * 512)
+        assert np.array_equal(bits(gpu.dequantize_weight(e, which)).reshape(-1), bits(want))
+    gpu.close()
+    # an odd number of 32-element blocks per row and a row count that is not a multiple of 64: the plain kernels
+    ref, gpu = make_pair(96, 160, 3, 2, dt, seed=32, dt_down=dt_down)
+    for T in (2, 40):
+        check_block(ref, gpu, T, tol=TOL)
+    gpu.close()
+
+
 def test_mixed_dtypes_need_one_activation_format():
+    ref41, _ = make_pair(256, 256, 4, 2, O.Q4_1, seed=6, want_gpu=False)
+    with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):   # Q8_1 against Q8_0
+        candle_amd.SparseMoeBlock(256, 256, 4, 2, O.Q4_1, ref41.gate, ref41.w1, ref41.w3,
+                                  [O.fill_normal_quantized(i, O.Q4_0, 256, 256, 0.02) for i in range(4)], ggml_dtype_down=O.Q4_0)
     ref, _ = make_pair(256, 256, 4, 2, O.Q4_0, seed=6, want_gpu=False)
     with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):
         candle_amd.SparseMoeBlock(256, 256, 4, 2, O.Q4_0, ref.gate, ref.w1, ref.w3,

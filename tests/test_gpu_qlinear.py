@@ -20,13 +20,14 @@ def bits(a):
 
 
 def check(dt, got, want):
-    if dt in (O.Q4_0, O.Q8_0):
+    if O.BLOCK_ELEMS[dt] == 32:
         assert np.array_equal(bits(got), bits(want))
     else:
         assert np.abs(got - want).max() <= Q4K_TOL * rms(want)
 
 
-@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q6K, 528, 768), (O.Q5K, 528, 768), (O.Q2K, 528, 768), (O.Q3K, 528, 768), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024)])
+@pytest.mark.parametrize("dt,n,k", [(O.Q4K, 512, 1024), (O.Q4K, 4096, 512), (O.Q4K, 272, 512), (O.Q6K, 528, 768), (O.Q5K, 528, 768), (O.Q2K, 528, 768), (O.Q3K, 528, 768), (O.Q8_0, 256, 1408), (O.Q4_0, 128, 1024),
+                                   (O.Q4_1, 128, 1024), (O.Q5_0, 256, 1408), (O.Q5_1, 128, 1024)])
 def test_resident_projection_over_batch_sizes(dt, n, k):
     # one object, many calls: decode rows, mid batches, and (Q4K, n % 128 == 0) the tiled kernel
     # at 64- and 128-row tiles with ragged last tiles; shrinking and growing batches reuse the workspace

@@ -51,6 +51,21 @@ def test_q4_0_roundtrip_known_answer(O, golden):
     assert np.array_equal(dst.view(np.uint32), want.view(np.uint32))  # includes the two -0.0
 
 
+def round3_half_away(v):
+    # round_vector, quantized_tests.rs:407-412: f32::round(1000 x) / 1000 (ties away from zero)
+    t = np.float32(1000.0) * np.asarray(v, dtype=np.float32)
+    return (np.sign(t) * np.floor(np.abs(t) + np.float32(0.5))).astype(np.float32) / np.float32(1000.0)
+
+
+@pytest.mark.parametrize("name,dt", [("q4_1", 3), ("q5_0", 6), ("q5_1", 7)])
+def test_legacy_roundtrip_known_answers(O, golden, name, dt):
+    # quantize_q4_1 / quantize_q5_0 / quantize_q5_1: 0..128 through from_float and to_float, to three decimals
+    src = np.arange(128, dtype=np.float32)
+    dst = O.dequantize(dt, O.quantize(dt, src), 128)
+    want = np.array(golden[name + "_roundtrip_0_127"]["expected_rounded_3"], dtype=np.float32)
+    assert round3_half_away(dst).tolist() == want.tolist()
+
+
 @pytest.mark.parametrize("simd", [False, True])
 def test_q4_0_matmul_known_answers(O, golden, simd):
     m, k, n = 3, 64, 4
@@ -80,7 +95,7 @@ def test_kquant_ramp_spot_values(O, golden, name, dt):
         assert np.abs(dbig - big).max() < g["max_abs_err_bound_128"]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 10, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 3, 6, 7, 8, 10, 11, 12, 13, 14, 15])
 def test_ggml_quantization_rmse(O, golden, dt):
     src = ggml_like(0.0)
     dst = O.dequantize(dt, O.quantize(dt, src), src.size)
@@ -88,7 +103,7 @@ def test_ggml_quantization_rmse(O, golden, dt):
     assert rmse <= golden["ggml_quantization_rmse_bound"][{10: "bound_2bits", 11: "bound_3bits"}.get(dt, "bound")]
 
 
-@pytest.mark.parametrize("dt", [2, 8, 10, 11, 12, 13, 14, 15])
+@pytest.mark.parametrize("dt", [2, 3, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15])
 def test_ggml_dot_error(O, golden, dt):
     # ggml_matmul_error_test, quantized_tests.rs:846-911
     g = golden["ggml_dot_error"]
@@ -114,12 +129,18 @@ def test_vec_dot_matches_dequantised_float64(O):
     # brute force: the integer block dot must equal the float dot of the dequantised operands
     rng = np.random.default_rng(3)
     n = 2048
-    for dt in (O.Q4_0, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K):
+    for dt in (O.Q4_0, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K):
         w = rng.normal(0, 0.02, n).astype(np.float32)
+        if dt in (O.Q4_1, O.Q5_1):
+            w += np.float32(0.05)  # a block minimum that matters
         x = rng.normal(0, 1.0, n).astype(np.float32)
         wq, xq = O.quantize(dt, w), O.quantize(O.VECDOT[dt], x)
         wd = O.dequantize(dt, wq, n).astype(np.float64)
-        xd = O.dequantize(O.VECDOT[dt], xq, n).astype(np.float64)
+        if O.VECDOT[dt] == O.Q8_1:  # the reference has no to_float for Q8_1: d * qs, decoded here
+            blk = xq.reshape(-1, 36)
+            xd = (blk[:, :2].copy().view(np.float16).astype(np.float64) * blk[:, 4:].view(np.int8)).reshape(-1)
+        else:
+            xd = O.dequantize(O.VECDOT[dt], xq, n).astype(np.float64)
         want = float(wd @ xd)
         for simd in (False, True):
             got = O.vec_dot(dt, n, wq, xq, simd=simd)
@@ -185,6 +206,51 @@ def test_q8_quantizer_closed_forms(O):
     assert not O.quantize(O.Q8_0, np.zeros(32, np.float32)).any()
     z4 = O.quantize(O.Q4_0, np.zeros(32, np.float32))  # d = 0/-8 = -0.0, every nibble 8
     assert z4[:2].view(np.uint16)[0] == 0x8000 and (z4[2:] == 0x88).all()
+
+
+def test_q8_1_closed_forms(O):
+    # Q8_1 = the Q8_0 block plus s = f16(sum of quants) * d in binary16 arithmetic (k_quants.rs:716-727)
+    rng = np.random.default_rng(6)
+    x = rng.normal(0, 1, 32 * 64).astype(np.float32)
+    x[:32] = 3.0   # sum = 32 * 127 = 4064: not a multiple of 4, so f16(sum) rounds
+    x[32:64] = 0.0
+    b1 = O.quantize(O.Q8_1, x).reshape(-1, 36)
+    b0 = O.quantize(O.Q8_0, x).reshape(-1, 34)
+    assert np.array_equal(b1[:, :2], b0[:, :2]) and np.array_equal(b1[:, 4:], b0[:, 2:])
+    d = b1[:, :2].copy().view(np.float16).reshape(-1)
+    sums = b1[:, 4:].view(np.int8).astype(np.int32).sum(1)
+    assert sums[0] == 4064
+    want = (sums.astype(np.float16).astype(np.float32) * d.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(b1[:, 2:4].copy().view(np.float16).reshape(-1).view(np.uint16), want.view(np.uint16))
+    assert not b1[1].any()
+
+
+def test_legacy_layouts_against_independent_decoders(O):
+    # numpy decoders of the published block layouts: Q4_1 (d, m, 16 nibble bytes), Q5_0 (d, 32 fifth bits, nibbles),
+    # Q5_1 (d, m, fifth bits, nibbles); element j < 16 is the low nibble of byte j, element j + 16 the high one,
+    # and the fifth bit of element e is bit e of the 32-bit little-endian word
+    rng = np.random.default_rng(12)
+    x = (rng.normal(0, 1, 32 * 40) + 0.3).astype(np.float32)
+    for dt, nb, has_m, has_h in ((O.Q4_1, 20, True, False), (O.Q5_0, 22, False, True), (O.Q5_1, 24, True, True)):
+        blk = O.quantize(dt, x).reshape(-1, nb)
+        pos = 2
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32)
+        m = np.zeros_like(d)
+        if has_m:
+            m = blk[:, 2:4].copy().view(np.float16).astype(np.float32); pos = 4
+        hi = np.zeros((blk.shape[0], 32), dtype=np.int32)
+        if has_h:
+            word = blk[:, pos:pos + 4].copy().view("<u4").reshape(-1, 1)
+            hi = ((word >> np.arange(32, dtype=np.uint32)) & 1).astype(np.int32) << 4
+            pos += 4
+        qs = blk[:, pos:pos + 16].astype(np.int32)
+        code = np.concatenate([qs & 15, qs >> 4], axis=1) | hi
+        if dt == O.Q5_0:
+            code = code - 16
+        want = code.astype(np.float32) * d + m if has_m else code.astype(np.float32) * d
+        got = O.dequantize(dt, blk.reshape(-1), x.size).reshape(-1, 32)
+        assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
+        assert np.abs(got.reshape(-1) - x).max() <= (np.abs(d).max() * (0.51 if dt != O.Q5_0 else 1.01))
 
 
 def test_q4k_layout_against_independent_decoder(O):
