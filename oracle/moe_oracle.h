@@ -11,6 +11,10 @@
  *   f16 conversions        exhaustive against numpy float16
  *   q4_0 quantize/dequant  exact 128-value vector of candle-core/tests/quantized_tests.rs:262-291
  *   q4_0 x q8_0 matmul     exact integers of quantized_tests.rs:89-104 and :149-169
+ *   q4_1, q5_0, q5_1       exact 128-value round trips of quantized_tests.rs:296-392 (to three decimals, as the reference
+ *                          states them), ggml RMSE / dot-error bounds :821-911, independent numpy block decoders,
+ *                          float64 dot of the dequantised operands
+ *   q8_1 quantize, dots    closed form (the Q8_0 block plus s = f16(sum) * d), ggml dot-error bound :836
  *   q8_0 quantize/dequant  closed form + ggml RMSE / dot-error bounds (quantized_tests.rs:428-469,821-911)
  *   q4k  quantize/dequant  spot values and error bounds of quantized_tests.rs:566-611, and the seeded
  *                          (11,512,21) mat-mul spot values of :1102-1121 through a restated rand-0.9 StdRng
@@ -69,13 +73,13 @@ int64_t orc_block_bytes(int dtype);
 /* VecDotType of a weight dtype: k_quants.rs:163,584,1189 */
 int     orc_vecdot_dtype(int dtype);
 
-/* from_float / to_float: k_quants.rs:166-224 (Q4_0), 587-634 (Q8_0), 808-908 (Q2K), 1047-1186 (Q3K), 1287-1374 (Q4K), 1487-1595 (Q5K), 1673-1790 (Q6K),
+/* from_float / to_float: k_quants.rs:166-224 (Q4_0), 299-359 (Q4_1), 404-465 (Q5_0), 511-581 (Q5_1), 587-634 (Q8_0), 700-729 (Q8_1, from_float only), 808-908 (Q2K), 1047-1186 (Q3K), 1287-1374 (Q4K), 1487-1595 (Q5K), 1673-1790 (Q6K),
  * 1819-1871 (Q8K).
  * n must be a multiple of the block size.  Return 0 or -1 (bad dtype / size). */
 int orc_quantize(int dtype, const float* x, int64_t n, void* blocks);
 int orc_dequantize(int dtype, const void* blocks, int64_t n, float* y);
 
-/* vec_dot_unopt: k_quants.rs:241-258, 650-668, 755-805 (Q2K), 927-1045 (Q3K), 1205-1285, 1394-1485 (Q5K), 1613-1671 (Q6K) */
+/* vec_dot_unopt: k_quants.rs:241-258, 270-297 (Q4_1), 381-402 (Q5_0), 477-509 (Q5_1), 650-668, 680-698 (Q8_1), 755-805 (Q2K), 927-1045 (Q3K), 1205-1285, 1394-1485 (Q5K), 1613-1671 (Q6K) */
 float orc_vec_dot(int dtype, int64_t n, const void* w_blocks, const void* act_blocks);
 
 /* k_quants::matmul, k_quants.rs:1873-1920: dst[m,n] = lhs[m,k] . rhs_t[n,k]^T, lhs quantised
