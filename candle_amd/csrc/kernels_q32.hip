@@ -310,147 +310,217 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Streaming versions of the two kernels above (same arithmetic, same order of additions): STEP blocks
-// per trip, the next trip's weight tiles requested before this trip's arithmetic (double buffer),
-// non-temporal global loads with a scalar base and 32-bit lane offsets, the activation scales and
-// block sums of a trip fetched as one 16-byte load per output slot.  They need K / 32 to be a
-// multiple of STEP; other shapes take the kernels above.
-// activation operand of one 16-slot tile for STEP consecutive blocks
-template <int STEP>
-struct Q8_0Trip {
-    u32x2g a[STEP];
-    f32x4g yd[4][STEP / 4];
-    i32x4g bs[4][STEP / 4];
+// Streaming versions of the two kernels above (same arithmetic, same order of additions) for matrices
+// whose K is a multiple of 128: those are kept in "super-tiles" of 16 rows x four blocks (moe_common.hpp),
+// so a lane fetches the codes of four blocks with one or two 16-byte loads and their scales with one.
+//
+// The four waves of a workgroup work on different rows against the SAME slots, so the activation operand
+// is staged once per workgroup: every K step (four blocks) the 256 threads copy the 16 x 128 quants of each
+// slot tile and their 64 (scale, word) pairs from global memory into LDS in MFMA operand order (double
+// buffered, one barrier per step); the waves read them back with conflict-free 8-byte reads and broadcast
+// 16-byte reads.  The weights go global -> registers, one step ahead.
+typedef uint32_t u32x4g __attribute__((ext_vector_type(4)));
+
+template <int DT>
+struct Q32SFmt {
+    typedef Q32Fmt<DT> F;
+    static constexpr uint32_t QB = F::NIB ? 1024 : 2048;     // codes: lane l at 16 l (Q8_0: blocks 0,1 then, 1 KiB on, 2,3)
+    static constexpr uint32_t HB = F::FIFTH ? 256 : 0;       // fifth-bit words: row r at 16 r, one word per block
+    static constexpr uint32_t DB = F::HAS_M ? 256 : 128;     // d (and m) per block: row r at 8 r (16 r)
+    static constexpr uint32_t STB = QB + HB + DB;            // = 4 tiles of the one-block layout
 };
-template <int DT, int STEP>
-__device__ __forceinline__ Q8_0Trip<STEP> load_q8_0_trip(const ActBuf& ab, int K, int nkb, int kb0, int rowA, const int rowD[4], int g) {
-    Q8_0Trip<STEP> o;
-    const uint32_t abase = (uint32_t)rowA * (uint32_t)K + (uint32_t)(kb0 * 32 + chunk_start<DT>(g));
-#pragma unroll
-    for (int j = 0; j < STEP; j++) o.a[j] = ldg<u32x2g>(ab.qs, abase + j * 32);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t doff = ((uint32_t)rowD[i] * (uint32_t)nkb + (uint32_t)kb0) * 4;
-#pragma unroll
-        for (int q = 0; q < STEP / 4; q++) {
-            o.yd[i][q] = ldg<f32x4g>(ab.d, doff + q * 16);
-            if (Q32Fmt<DT>::OFFSET || Q32Fmt<DT>::HAS_M) o.bs[i][q] = ldg<i32x4g>(ab.bsum, doff + q * 16);
-        }
+
+template <int DT>
+struct Q32SRaw {
+    u32x4g q0, q1;   // q1: Q8_0 only
+    u32x4g h;        // five-bit formats only
+    u32x4g dm;       // formats with a minimum: (d, m) of the four blocks; else .x / .y = the four d
+};
+template <int DT, bool ONCE>
+__device__ __forceinline__ Q32SRaw<DT> load_q32s(const uint8_t* tile, int lane) {
+    typedef Q32Fmt<DT> F;
+    typedef Q32SFmt<DT> S;
+    Q32SRaw<DT> t;
+    const uint32_t r = (uint32_t)(lane & 15);
+    t.q0 = ONCE ? ldg_stream<u32x4g>(tile, (uint32_t)lane * 16u) : ldg<u32x4g>(tile, (uint32_t)lane * 16u);
+    if (!F::NIB) t.q1 = ONCE ? ldg_stream<u32x4g>(tile, 1024u + (uint32_t)lane * 16u) : ldg<u32x4g>(tile, 1024u + (uint32_t)lane * 16u);
+    if (F::FIFTH) t.h = ONCE ? ldg_stream<u32x4g>(tile, S::QB + 16u * r) : ldg<u32x4g>(tile, S::QB + 16u * r);
+    if (F::HAS_M) {
+        t.dm = ONCE ? ldg_stream<u32x4g>(tile, S::QB + S::HB + 16u * r) : ldg<u32x4g>(tile, S::QB + S::HB + 16u * r);
+    } else {
+        const u32x2g d = ONCE ? ldg_stream<u32x2g>(tile, S::QB + S::HB + 8u * r) : ldg<u32x2g>(tile, S::QB + S::HB + 8u * r);
+        t.dm.x = d.x; t.dm.y = d.y;
     }
-    return o;
+    return t;
+}
+// Block b (compile-time) of a super-tile as an MFMA operand.  Lane (row, g) holds the codes of elements
+// 4g .. 4g+3 (low word) and 16+4g .. 16+4g+3 (high word) of the block.
+template <int DT, int B>
+__device__ __forceinline__ Q32Tile<DT> q32s_block(const Q32SRaw<DT>& raw, int g) {
+    typedef Q32Fmt<DT> F;
+    Q32Tile<DT> t;
+    if (!F::NIB) {
+        const u32x4g& q = B < 2 ? raw.q0 : raw.q1;
+        t.q = (B & 1) ? make_uint2(q.z, q.w) : make_uint2(q.x, q.y);
+    } else {
+        const uint32_t w = raw.q0[B];
+        uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;
+        if (F::FIFTH) {   // bit e of the word belongs to element e
+            const uint32_t hb = raw.h[B] >> (4 * g);
+            lo |= fifth_bits(hb & 15u);
+            hi |= fifth_bits((hb >> 16) & 15u);
+        }
+        t.q = make_uint2(lo, hi);
+    }
+    if (F::HAS_M) {
+        t.d = __half2float(__ushort_as_half((unsigned short)(raw.dm[B] & 0xffffu)));
+        t.m = __half2float(__ushort_as_half((unsigned short)(raw.dm[B] >> 16)));
+    } else {
+        const uint32_t w = B < 2 ? raw.dm.x : raw.dm.y;
+        t.d = __half2float(__ushort_as_half((unsigned short)((B & 1) ? (w >> 16) : (w & 0xffffu))));
+        t.m = 0.f;
+    }
+    return t;
 }
 
-template <int DT, int STEP>
-__device__ __forceinline__ void q32_mac_trip(const Q32Tile<DT>& w, const Q8_0Trip<STEP>& A, int j, float acc[4]) {
+constexpr int Q32S_ACT_Q = 2048;                  // LDS bytes of one slot tile's quants for one K step
+constexpr int Q32S_ACT_BYTES = Q32S_ACT_Q + 512;  // ... and of its 4 x 16 (scale, word) pairs
+
+// Which rows of the activation buffer this thread copies: quants of slot tid / 16 (8 bytes at element 8 (tid % 16) of
+// the step), and the (scale, word) pair of slot (tid / 4) % 16, block tid % 4 (the four waves copy the same 64 pairs:
+// no divergent branch in the K loop, whose body has to stay one basic block for the scheduler fences to hold).
+template <int TT>
+struct Q32SStage {
+    uint32_t q_row[TT], s_row[TT];
+    u32x2g q[TT];
+    float d[TT];
+    int w[TT];
+};
+template <int TT>
+__device__ __forceinline__ void q32s_issue(Q32SStage<TT>& st, const ActBuf& ab, int K, int nkb, int ks, int tid) {
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        st.q[tt] = ldg<u32x2g>(ab.qs, st.q_row[tt] * (uint32_t)K + (uint32_t)(ks * 128 + 8 * (tid & 15)));
+        const uint32_t off = (st.s_row[tt] * (uint32_t)nkb + (uint32_t)(ks * 4 + (tid & 3))) * 4u;
+        st.d[tt] = ldg<float>(ab.d, off);
+        st.w[tt] = ldg<int>(ab.bsum, off);
+    }
+}
+// OFFSET: the block sums are stored times the format's code offset (the products need isum - OFFSET * sum)
+template <int TT, int OFFSET>
+__device__ __forceinline__ void q32s_commit(const Q32SStage<TT>& st, uint8_t* buf, int tid) {
+    const int slot = tid >> 4, c = tid & 15, b = c >> 2, cc = c & 3;
+    // elements 8cc .. 8cc+3 of the block belong to chunk g0 = 2 (cc % 2), the next four to chunk g0 + 1; both are the
+    // low (cc < 2) or the high half of their lane's operand
+    const int at = ((b * 64 + 2 * (cc & 1) * 16 + slot) * 8) + (cc >> 1) * 4;
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+        uint8_t* base = buf + tt * Q32S_ACT_BYTES;
+        *reinterpret_cast<uint32_t*>(base + at) = st.q[tt].x;
+        *reinterpret_cast<uint32_t*>(base + at + 128) = st.q[tt].y;
+        *reinterpret_cast<uint2*>(base + Q32S_ACT_Q + ((tid & 3) * 16 + ((tid >> 2) & 15)) * 8) = make_uint2(__float_as_uint(st.d[tt]), (uint32_t)(OFFSET ? st.w[tt] * OFFSET : st.w[tt]));
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ void q32s_mac(const Q32Tile<DT>& w, uint2 a, const uint4& s01, const uint4& s23, float acc[4]) {
     const v4i zero = {0, 0, 0, 0};
-    const long a = (long)(((uint64_t)A.a[j].y << 32) | A.a[j].x);
-    const long b = (long)(((uint64_t)w.q.y << 32) | w.q.x);
-    v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, zero, 0, 0, 0);
+    const long av = (long)(((uint64_t)a.y << 32) | a.x);
+    const long bv = (long)(((uint64_t)w.q.y << 32) | w.q.x);
+    v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, zero, 0, 0, 0);
+    const uint32_t yd[4] = {s01.x, s01.z, s23.x, s23.z}, wd[4] = {s01.y, s01.w, s23.y, s23.w};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         int isum = D[i];
-        if (Q32Fmt<DT>::OFFSET) isum -= Q32Fmt<DT>::OFFSET * A.bs[i][j / 4][j % 4];
+        if (Q32Fmt<DT>::OFFSET) isum -= (int)wd[i];   // staged as OFFSET * sum of the block's quants
         float t = (float)isum * w.d;
-        t = t * A.yd[i][j / 4][j % 4];
-        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __int_as_float(A.bs[i][j / 4][j % 4]);
+        t = t * __uint_as_float(yd[i]);
+        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __uint_as_float(wd[i]);   // the word holds the activation block's s
         acc[i] += t;
     }
 }
 
-// One wave: NT weight tile streams (tp[j], advancing TB bytes per block) against TT slot tiles, all of K.
-template <int DT, int TT, int NT, int STEP, bool ONCE>
-__device__ __forceinline__ void q32_engine(const uint8_t* const tp[NT], const ActBuf& ab, int K, const int rowA[TT], const int rowD[TT][4],
-                                           int lane, float acc[NT][TT][4]) {
-    constexpr int TB = Q32Fmt<DT>::TB;
+// Block B of the step: every slot tile's operand and scales from LDS against the NT weight tiles.
+template <int DT, int TT, int NT, int B>
+__device__ __forceinline__ void q32s_step(const Q32SRaw<DT> (&cur)[NT], const uint8_t* buf, int lane, float acc[NT][TT][4]) {
     const int g = lane >> 4;
-    const int nkb = K / 32;
-    const uint32_t q_off = Q32Fmt<DT>::q_off(lane), d_off = Q32Fmt<DT>::d_off(lane), h_off = Q32Fmt<DT>::h_off(lane);
-    // ONCE (the weights come from HBM): the next trip's tiles are requested a whole trip ahead.  Otherwise they
-    // are in L2 after the first pass and are fetched where they are used: half the registers, twice the waves.
-    Q32Raw nxt[ONCE ? NT : 1][ONCE ? STEP : 1];
-    if (ONCE) {
+    Q32Tile<DT> w[NT];
 #pragma unroll
-        for (int t = 0; t < NT; t++)
+    for (int t = 0; t < NT; t++) w[t] = q32s_block<DT, B>(cur[t], g);
 #pragma unroll
-            for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)j * TB, q_off, d_off, h_off);
+    for (int tt = 0; tt < TT; tt++) {
+        const uint8_t* base = buf + tt * Q32S_ACT_BYTES;
+        const uint2 a = *reinterpret_cast<const uint2*>(base + (B * 64 + lane) * 8);
+        const uint4 s01 = *reinterpret_cast<const uint4*>(base + Q32S_ACT_Q + (B * 16 + 4 * g) * 8);
+        const uint4 s23 = *reinterpret_cast<const uint4*>(base + Q32S_ACT_Q + (B * 16 + 4 * g + 2) * 8);
+#pragma unroll
+        for (int t = 0; t < NT; t++) q32s_mac<DT>(w[t], a, s01, s23, acc[t][tt]);
     }
-    // With several slot tiles the activation operand is requested one step ahead too: the one of slot
-    // tile tt+1, or of the next trip's first slot tile, is on its way while this one is multiplied.
-    // (With one slot tile the extra registers cost a wave per SIMD, which costs more than the wait.)
-    constexpr bool AHEAD = TT > 1;
-    Q8_0Trip<STEP> An;
-    if (AHEAD) An = load_q8_0_trip<DT, STEP>(ab, K, nkb, 0, rowA[0], rowD[0], g);
-    for (int kb0 = 0; kb0 < nkb; kb0 += STEP) {
-        Q32Raw cur[NT][STEP];
-        // the trip after this one; past the end the last trip is requested again (no branch around a load)
-        const int kbn = kb0 + STEP < nkb ? kb0 + STEP : kb0;
-        if (ONCE) {
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One wave: NT super-tile streams (tp[t], advancing `stride` bytes per K step) against the workgroup's TT slot tiles,
+// all of K.  Every thread of the workgroup must call it (barriers).
+template <int DT, int TT, int NT, bool ONCE>
+__device__ __forceinline__ void q32s_engine(const uint8_t* const tp[NT], size_t stride, const ActBuf& ab, int K, Q32SStage<TT>& st,
+                                            uint8_t* act_lds, int tid, float acc[NT][TT][4]) {
+    const int lane = tid & 63, g = lane >> 4;
+    const int nkb = K / 32, nks = K / 128;
+    q32s_issue<TT>(st, ab, K, nkb, 0, tid);
+    Q32SRaw<DT> nxt[NT];
 #pragma unroll
-            for (int t = 0; t < NT; t++)
+    for (int t = 0; t < NT; t++) nxt[t] = load_q32s<DT, ONCE>(tp[t], lane);
+    q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st, act_lds, tid);
+    q32s_issue<TT>(st, ab, K, nkb, nks > 1 ? 1 : 0, tid);
+    __syncthreads();
+    for (int ks = 0; ks < nks; ks++) {
+        Q32SRaw<DT> cur[NT];
+        // past the end the last step is requested again (no branch around a load)
+        const int ksn = ks + 1 < nks ? ks + 1 : ks;
 #pragma unroll
-                for (int j = 0; j < STEP; j++) cur[t][j] = nxt[t][j];
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-#pragma unroll
-                for (int j = 0; j < STEP; j++) nxt[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kbn + j) * TB, q_off, d_off, h_off);
-        } else {
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-#pragma unroll
-                for (int j = 0; j < STEP; j++) cur[t][j] = load_q32_raw<DT, ONCE>(tp[t] + (size_t)(kb0 + j) * TB, q_off, d_off, h_off);
-        }
+        for (int t = 0; t < NT; t++) { cur[t] = nxt[t]; nxt[t] = load_q32s<DT, ONCE>(tp[t] + (size_t)ksn * stride, lane); }
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int tt = 0; tt < TT; tt++) {
-            Q8_0Trip<STEP> A;
-            if (AHEAD) {
-                A = An;
-                An = tt + 1 < TT ? load_q8_0_trip<DT, STEP>(ab, K, nkb, kb0, rowA[tt + 1 < TT ? tt + 1 : 0], rowD[tt + 1 < TT ? tt + 1 : 0], g)
-                                 : load_q8_0_trip<DT, STEP>(ab, K, nkb, kbn, rowA[0], rowD[0], g);
-                __builtin_amdgcn_sched_barrier(0);
-            } else {
-                A = load_q8_0_trip<DT, STEP>(ab, K, nkb, kb0, rowA[tt], rowD[tt], g);
-            }
-#pragma unroll
-            for (int j = 0; j < STEP; j++)
-#pragma unroll
-                for (int t = 0; t < NT; t++) q32_mac_trip<DT, STEP>(q32_unpack<DT>(cur[t][j], g), A, j, acc[t][tt]);
-        }
+        const uint8_t* buf = act_lds + (ks & 1) * (TT * Q32S_ACT_BYTES);
+        q32s_step<DT, TT, NT, 0>(cur, buf, lane, acc);
+        q32s_step<DT, TT, NT, 1>(cur, buf, lane, acc);
+        q32s_step<DT, TT, NT, 2>(cur, buf, lane, acc);
+        q32s_step<DT, TT, NT, 3>(cur, buf, lane, acc);
         __builtin_amdgcn_sched_barrier(0);
+        // (after the last step this stages the last step once more, into the buffer nobody reads again)
+        q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st, act_lds + ((ks + 1) & 1) * (TT * Q32S_ACT_BYTES), tid);
+        q32s_issue<TT>(st, ab, K, nkb, ks + 2 < nks ? ks + 2 : nks - 1, tid);
+        __syncthreads();
     }
 }
 
-constexpr int Q32_STEP = 4;
-
-template <int DT, int TT, bool ONCE>
-__global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams p) {
+// (a fixed number of waves per SIMD also makes the compiler keep the MFMA results in ordinary registers)
+template <int DT, int TT, bool ONCE, int WPE>
+__global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void q32s_up_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
+    __shared__ __align__(16) uint8_t act_lds[2 * TT * Q32S_ACT_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = blockIdx.y;
     const GroupSlots gs = group_slots<Q32_THREADS>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
     if (tg0 >= gs.n) return;
-    const int H = p.H, F = p.F, nkb = H / 32;
-    const int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
-    if (rt0 >= F / 16) return;
-    constexpr int TB = Q32Fmt<DT>::TB;
+    const int H = p.H, F = p.F, n_rt = F / 16;
+    int rt0 = (blockIdx.x * (Q32_THREADS / 64) + wave) * 2;
+    const bool live = rt0 < n_rt;      // a wave past the last rows still stages activations and meets the barriers
+    if (!live) rt0 = 0;
+    constexpr size_t STB = Q32SFmt<DT>::STB;
 
-    int rowA[TT], rowD[TT][4];
+    Q32SStage<TT> st;
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        int ia = tg0 + tt * 16 + r;
-        rowA[tt] = slot_token(p, gs.slot(ia < gs.n ? ia : gs.n - 1));
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int id = tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = slot_token(p, gs.slot(id < gs.n ? id : gs.n - 1));
-        }
+        const int iq = tg0 + tt * 16 + (tid >> 4), is = tg0 + tt * 16 + ((tid >> 2) & 15);
+        st.q_row[tt] = (uint32_t)slot_token(p, gs.slot(iq < gs.n ? iq : gs.n - 1));
+        st.s_row[tt] = (uint32_t)slot_token(p, gs.slot(is < gs.n ? is : gs.n - 1));
     }
     const GroupWeights gw = p.groups[grp];
-    const uint8_t* tp[4] = {gw.w1 + (size_t)rt0 * nkb * TB, gw.w1 + (size_t)(rt0 + 1) * nkb * TB,
-                            gw.w3 + (size_t)rt0 * nkb * TB, gw.w3 + (size_t)(rt0 + 1) * nkb * TB};
+    const uint8_t* tp[4] = {gw.w1 + (size_t)rt0 * STB, gw.w1 + (size_t)(rt0 + 1) * STB,
+                            gw.w3 + (size_t)rt0 * STB, gw.w3 + (size_t)(rt0 + 1) * STB};
     float acc[4][TT][4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -459,7 +529,8 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q32_engine<DT, TT, 4, Q32_STEP, ONCE>(tp, p.xq, H, rowA, rowD, lane, acc);
+    q32s_engine<DT, TT, 4, ONCE>(tp, (size_t)n_rt * STB, p.xq, H, st, act_lds, tid, acc);
+    if (!live) return;
 
     // epilogue: h = silu(w1 x) * (w3 x); the wave's 32 rows are exactly one Q8_0 block per slot
     const int nfb = F / 32;
@@ -493,40 +564,39 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_stream_kernel(ExpertParams
         }
 }
 
-template <int DT, int TT, bool ONCE>
-__global__ __launch_bounds__(Q32_THREADS) void q32_down_stream_kernel(ExpertParams p) {
+template <int DT, int TT, bool ONCE, int WPE>
+__global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void q32s_down_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
+    __shared__ __align__(16) uint8_t act_lds[2 * TT * Q32S_ACT_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = blockIdx.y;
     const GroupSlots gs = group_slots<Q32_THREADS>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
     if (tg0 >= gs.n) return;
-    const int H = p.H, F = p.F, nkb = F / 32;
-    const int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
-    if (rt >= H / 16) return;
-    constexpr int TB = Q32Fmt<DT>::TB;
+    const int H = p.H, F = p.F, n_rt = H / 16;
+    int rt = blockIdx.x * (Q32_THREADS / 64) + wave;
+    const bool live = rt < n_rt;
+    if (!live) rt = 0;
+    constexpr size_t STB = Q32SFmt<DT>::STB;
 
-    int rowA[TT], rowD[TT][4];
+    Q32SStage<TT> st;
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        int ia = tg0 + tt * 16 + r;
-        rowA[tt] = gs.slot(ia < gs.n ? ia : gs.n - 1) - p.slot_origin;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int id = tg0 + tt * 16 + 4 * g + i;
-            rowD[tt][i] = gs.slot(id < gs.n ? id : gs.n - 1) - p.slot_origin;
-        }
+        const int iq = tg0 + tt * 16 + (tid >> 4), is = tg0 + tt * 16 + ((tid >> 2) & 15);
+        st.q_row[tt] = (uint32_t)(gs.slot(iq < gs.n ? iq : gs.n - 1) - p.slot_origin);
+        st.s_row[tt] = (uint32_t)(gs.slot(is < gs.n ? is : gs.n - 1) - p.slot_origin);
     }
-    const uint8_t* tp[1] = {p.groups[grp].w2 + (size_t)rt * nkb * TB};
+    const uint8_t* tp[1] = {p.groups[grp].w2 + (size_t)rt * STB};
     float acc[1][TT][4];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[0][tt][i] = 0.f;
 
-    q32_engine<DT, TT, 1, ONCE ? 2 * Q32_STEP : Q32_STEP, ONCE>(tp, p.hq, F, rowA, rowD, lane, acc);
+    q32s_engine<DT, TT, 1, ONCE>(tp, (size_t)n_rt * STB, p.hq, F, st, act_lds, tid, acc);
+    if (!live) return;
 
 #pragma unroll
     for (int tt = 0; tt < TT; tt++)
@@ -547,13 +617,15 @@ static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
     const int n_pairs = p.F / 32;
     dim3 grid((unsigned)((n_pairs + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
-    const bool stream = !plain && (p.H / 32) % Q32_STEP == 0;
+    const bool stream = !plain && q32_super_layout(p.H);
+    // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
+    constexpr int UP1 = Q32Fmt<DT>::FIFTH ? 3 : 4, UP2 = (Q32Fmt<DT>::FIFTH && Q32Fmt<DT>::HAS_M) ? 2 : 3;
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 1, true>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 1, true, UP1>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 2, true>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32_up_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, true, UP2>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, false, UP2>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
@@ -564,14 +636,13 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     const int wpb = Q32_THREADS / 64;
     dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
-    const bool stream = !plain && (p.F / 32) % (2 * Q32_STEP) == 0;
-    const bool stream_again = !plain && (p.F / 32) % Q32_STEP == 0;   // the several-pass variant walks K in shorter trips
+    const bool stream = !plain && q32_super_layout(p.F);
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 1, true>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, 8>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, true>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream_again && grid.z > 1) hipLaunchKernelGGL((q32_down_stream_kernel<DT, 2, false>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, true, 6>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, false, 6>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();

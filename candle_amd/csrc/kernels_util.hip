@@ -314,6 +314,47 @@ __global__ void relayout_nib_kernel(int dt, const uint8_t* raw, uint8_t* tiled, 
     for (int i = 0; i < f.tile_d_stride; i++) dst[f.tile_d + f.tile_d_stride * r + i] = blk[i];   // d, then m, lead the block
 }
 
+// Super-tiles of the 32-element formats (K % 128 == 0): 16 rows x four blocks, ordered [step][row-tile].
+// One thread per (super-tile, lane l = (row r, chunk g)): the lane's 4 (nibble formats) or 8 (Q8_0) code bytes of each
+// of the four blocks; the lanes of chunk 0 also move the row's fifth-bit words and scales.
+struct SuperFmt {
+    uint32_t qb, hb, db;   // section sizes: codes, fifth-bit words, scales
+};
+__host__ __device__ inline SuperFmt super_fmt(int dt) {
+    const uint32_t qb = dt == MOE_GGML_Q8_0 ? 2048u : 1024u;
+    const uint32_t hb = (dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q5_1) ? 256u : 0u;
+    const uint32_t db = (dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_1) ? 256u : 128u;
+    return {qb, hb, db};
+}
+__global__ void relayout_q32_super_kernel(int dt, const uint8_t* raw, uint8_t* tiled, int64_t n_rt, int nks) {
+    int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_rt * nks * 64) return;
+    const SuperFmt sf = super_fmt(dt);
+    const bool nib = is_nib(dt);
+    const NibFmt f = nib_fmt(dt);
+    const int bytes = nib ? f.bytes : 34, q_pos = nib ? f.q_pos : 2, m_pos = nib ? f.m_pos : 0, h_pos = nib ? f.h_pos : 0;
+    int64_t tile = c / 64;
+    int l = (int)(c % 64), r = l % 16, g = l / 16;
+    int ks = (int)(tile / n_rt);
+    int64_t rt = tile % n_rt;
+    uint8_t* dst = tiled + tile * (sf.qb + sf.hb + sf.db);
+    for (int b = 0; b < 4; b++) {
+        const uint8_t* blk = raw + ((rt * 16 + r) * (int64_t)(nks * 4) + ks * 4 + b) * bytes;
+        if (nib) {
+            for (int i = 0; i < 4; i++) dst[l * 16 + 4 * b + i] = blk[q_pos + 4 * g + i];
+        } else {
+            uint8_t* q = dst + (b / 2) * 1024 + l * 16 + (b & 1) * 8;
+            for (int i = 0; i < 4; i++) { q[i] = blk[q_pos + 4 * g + i]; q[4 + i] = blk[q_pos + 16 + 4 * g + i]; }
+        }
+        if (g == 0) {
+            if (h_pos)
+                for (int i = 0; i < 4; i++) dst[sf.qb + 16 * r + 4 * b + i] = blk[h_pos + i];
+            const int nd = m_pos ? 4 : 2;   // d, then m, lead the block
+            for (int i = 0; i < nd; i++) dst[sf.qb + sf.hb + nd * 4 * r + nd * b + i] = blk[i];
+        }
+    }
+}
+
 // ------------------------------------------------------------------ to_float from the tiled layout
 __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, int64_t rows, int64_t k) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -368,6 +409,24 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
         int code = (sub ? (nb >> 4) : (nb & 0xF)) | (((hb >> (2 * (2 * sub + pos / 4))) & 3) << 4);
         float d = f16_bits_to_f32((uint16_t)(tile[3328 + 2 * r] | (tile[3328 + 2 * r + 1] << 8)));
         out[i] = q6k_value(d, (int8_t)tile[3072 + r * 16 + e / 16], code);
+    } else if (q32_super_layout(k)) {  // the 32-element formats in super-tiles
+        const SuperFmt sf = super_fmt(dt);
+        const int ks = col / 128, b = (col % 128) / 32, e = col % 32;
+        const uint8_t* tile = tiled + ((int64_t)ks * (rows / 16) + rt) * (sf.qb + sf.hb + sf.db);
+        const int g = (e % 16) / 4, bi = e % 4, l = g * 16 + r;
+        if (dt == MOE_GGML_Q8_0) {
+            const uint8_t* dp = tile + sf.qb + 8 * r + 2 * b;
+            float d = f16_bits_to_f32((uint16_t)(dp[0] | (dp[1] << 8)));
+            out[i] = (float)(int8_t)tile[(b / 2) * 1024 + l * 16 + (b & 1) * 8 + (e / 16) * 4 + bi] * d;
+        } else {
+            const NibFmt f = nib_fmt(dt);
+            const int nd = f.m_pos ? 4 : 2;
+            const uint8_t* dm = tile + sf.qb + sf.hb + nd * 4 * r + nd * b;
+            const uint8_t* hp = tile + sf.qb + 16 * r + 4 * b;
+            uint32_t h = f.h_pos ? (uint32_t)hp[0] | ((uint32_t)hp[1] << 8) | ((uint32_t)hp[2] << 16) | ((uint32_t)hp[3] << 24) : 0u;
+            uint16_t m_bits = f.m_pos ? (uint16_t)(dm[2] | (dm[3] << 8)) : (uint16_t)0;
+            out[i] = nib_value(f, (uint16_t)(dm[0] | (dm[1] << 8)), m_bits, tile[l * 16 + 4 * b + bi], h, e);
+        }
     } else if (dt == MOE_GGML_Q8_0) {
         int nkb = (int)(k / 32), kb = col / 32, e = col % 32;
         const uint8_t* tile = tiled + (rt * nkb + kb) * Q8_0_TILE_BYTES;
@@ -458,6 +517,8 @@ hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t r
         hipLaunchKernelGGL(relayout_q5k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else if (dt == MOE_GGML_Q6K)
         hipLaunchKernelGGL(relayout_q6k_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
+    else if (q32_super_layout(k))
+        hipLaunchKernelGGL(relayout_q32_super_kernel, dim3(nblk(n_rt * (nkb / 4) * 64, 256)), dim3(256), 0, s, dt, raw, tiled, n_rt, nkb / 4);
     else if (dt == MOE_GGML_Q8_0)
         hipLaunchKernelGGL(relayout_q8_0_kernel, dim3(nblk(n_rt * nkb * 64, 256)), dim3(256), 0, s, raw, tiled, n_rt, nkb);
     else

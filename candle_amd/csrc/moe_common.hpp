@@ -105,6 +105,14 @@ inline bool weight_dtype_supported(int dt) {
 //  Q4_1 / Q5_0 / Q5_1 tiles (320 / 352 / 384 B): the 256 nibble bytes as in the Q4_0 tile, then, for the
 //       five-bit formats, row r's 32 fifth bits as one little-endian word (bit e = element e), then row
 //       r's d (f16) and, for the formats with a block minimum, m (f16) as one 4-byte pair.
+//  Super-tiles of these five formats (matrices with K % 128 == 0; 16 rows x blocks 4s .. 4s+3, ordered
+//       [step s][row-tile], four times the bytes of the one-block tile).  MFMA k-chunk g of a block covers
+//       elements 4g .. 4g+3 and 16+4g .. 16+4g+3:
+//         codes   lane l = (row l%16, g = l/16) at 16 l.  Nibble formats: word b = bytes 4g .. 4g+3 of block b's qs
+//                 (low nibbles = elements 4g .., high nibbles = elements 16+4g ..).  Q8_0: 2 KiB, blocks 0,1 then 2,3;
+//                 per block 8 bytes: elements 4g .. 4g+3, then 16+4g .. 16+4g+3.
+//         fifth bits (Q5_0, Q5_1)  row r at 16 r: the four blocks' words
+//         scales  row r at 8 r: the four d (f16); with a minimum, at 16 r: (d, m) per block
 //
 // ACTIVATIONS are quantised exactly as the reference does (Q8K for Q2K ... Q6K weights, Q8_1 for Q4_1 and
 // Q5_1, Q8_0 otherwise) and stored per row as
@@ -141,6 +149,9 @@ inline int64_t tile_bytes(int dt) {
         default: return -1;
     }
 }
+// The 32-element formats keep a matrix whose K is a multiple of 128 in super-tiles of 16 rows x four blocks
+// (same bytes in total), other matrices in the one-block tiles.
+__host__ __device__ inline bool q32_super_layout(int64_t k) { return k % 128 == 0; }
 // bytes of a re-laid [rows, k] matrix (rows % 16 == 0)
 inline int64_t relaid_bytes(int dt, int64_t rows, int64_t k) {
     return (rows / 16) * (k / block_elems(dt)) * tile_bytes(dt);
