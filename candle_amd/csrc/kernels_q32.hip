@@ -390,25 +390,39 @@ constexpr int Q32S_ACT_BYTES = Q32S_ACT_Q + 512;  // ... and of its 4 x 16 (scal
 // the step), and the (scale, word) pair of slot (tid / 4) % 16, block tid % 4 (the four waves copy the same 64 pairs:
 // no divergent branch in the K loop, whose body has to stay one basic block for the scheduler fences to hold).
 template <int TT>
-struct Q32SStage {
+struct Q32SRows {
     uint32_t q_row[TT], s_row[TT];
+};
+template <int TT>
+struct Q32SStage {
     u32x2g q[TT];
     float d[TT];
     int w[TT];
 };
+// Requests step ks of the activations.  A step past the end of K (the K loop runs in whole rounds of its prefetch
+// ring) re-reads the last one; q32s_commit zeroes its scale and word, so that its products add +-0.  (Nothing here
+// may touch the loaded values: that would wait for the loads where they are issued.)
 template <int TT>
-__device__ __forceinline__ void q32s_issue(Q32SStage<TT>& st, const ActBuf& ab, int K, int nkb, int ks, int tid) {
+__device__ __forceinline__ void q32s_issue(Q32SStage<TT>& st, const Q32SRows<TT>& rows, const ActBuf& ab, int K, int nkb, int ks, int tid) {
+    const int nks = K / 128;
+    const int kc = ks >= nks ? nks - 1 : ks;
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
-        st.q[tt] = ldg<u32x2g>(ab.qs, st.q_row[tt] * (uint32_t)K + (uint32_t)(ks * 128 + 8 * (tid & 15)));
-        const uint32_t off = (st.s_row[tt] * (uint32_t)nkb + (uint32_t)(ks * 4 + (tid & 3))) * 4u;
+        st.q[tt] = ldg<u32x2g>(ab.qs, rows.q_row[tt] * (uint32_t)K + (uint32_t)(kc * 128 + 8 * (tid & 15)));
+        const uint32_t off = (rows.s_row[tt] * (uint32_t)nkb + (uint32_t)(kc * 4 + (tid & 3))) * 4u;
         st.d[tt] = ldg<float>(ab.d, off);
         st.w[tt] = ldg<int>(ab.bsum, off);
     }
 }
-// OFFSET: the block sums are stored times the format's code offset (the products need isum - OFFSET * sum)
+// The integer products reach the vector ALU as floats without a conversion: the MFMA's addend is the bit pattern of
+// 1.5 * 2^23, so its result, read as a float, is exactly 1.5 * 2^23 + isum (|isum| < 2^22), and
+// fma(that, d, -(1.5 * 2^23) * d) = isum * d with one rounding, as (isum as f32) * d has (the subtrahend is exact:
+// d has an 11-bit significand).  OFFSET: the format's code offset leaves through the same addend, staged per
+// block and slot as magic - OFFSET * (sum of the block's quants).
+constexpr int Q32S_MAGIC_BITS = 0x4B400000;
+constexpr float Q32S_MAGIC = 12582912.0f;
 template <int TT, int OFFSET>
-__device__ __forceinline__ void q32s_commit(const Q32SStage<TT>& st, uint8_t* buf, int tid) {
+__device__ __forceinline__ void q32s_commit(const Q32SStage<TT>& st, uint8_t* buf, int tid, bool past) {
     const int slot = tid >> 4, c = tid & 15, b = c >> 2, cc = c & 3;
     // elements 8cc .. 8cc+3 of the block belong to chunk g0 = 2 (cc % 2), the next four to chunk g0 + 1; both are the
     // low (cc < 2) or the high half of their lane's operand
@@ -418,24 +432,24 @@ __device__ __forceinline__ void q32s_commit(const Q32SStage<TT>& st, uint8_t* bu
         uint8_t* base = buf + tt * Q32S_ACT_BYTES;
         *reinterpret_cast<uint32_t*>(base + at) = st.q[tt].x;
         *reinterpret_cast<uint32_t*>(base + at + 128) = st.q[tt].y;
-        *reinterpret_cast<uint2*>(base + Q32S_ACT_Q + ((tid & 3) * 16 + ((tid >> 2) & 15)) * 8) = make_uint2(__float_as_uint(st.d[tt]), (uint32_t)(OFFSET ? st.w[tt] * OFFSET : st.w[tt]));
+        const int at_s = Q32S_ACT_Q + ((tid & 3) * 16 + ((tid >> 2) & 15)) * 4;   // [block][slot] scales, then words
+        *reinterpret_cast<float*>(base + at_s) = past ? 0.f : st.d[tt];
+        *reinterpret_cast<int*>(base + at_s + 256) = OFFSET ? Q32S_MAGIC_BITS - st.w[tt] * OFFSET : (past ? 0 : st.w[tt]);
     }
 }
 
 template <int DT>
-__device__ __forceinline__ void q32s_mac(const Q32Tile<DT>& w, uint2 a, const uint4& s01, const uint4& s23, float acc[4]) {
-    const v4i zero = {0, 0, 0, 0};
+__device__ __forceinline__ void q32s_mac(const Q32Tile<DT>& w, uint2 a, const f32x4g& yd, const v4i& wd, float acc[4]) {
+    const v4i magic = {Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS};
     const long av = (long)(((uint64_t)a.y << 32) | a.x);
     const long bv = (long)(((uint64_t)w.q.y << 32) | w.q.x);
-    v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, zero, 0, 0, 0);
-    const uint32_t yd[4] = {s01.x, s01.z, s23.x, s23.z}, wd[4] = {s01.y, s01.w, s23.y, s23.w};
+    v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, Q32Fmt<DT>::OFFSET ? wd : magic, 0, 0, 0);
+    const float c = -(Q32S_MAGIC * w.d);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        int isum = D[i];
-        if (Q32Fmt<DT>::OFFSET) isum -= (int)wd[i];   // staged as OFFSET * sum of the block's quants
-        float t = (float)isum * w.d;
-        t = t * __uint_as_float(yd[i]);
-        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __uint_as_float(wd[i]);   // the word holds the activation block's s
+        float t = __builtin_fmaf(__int_as_float(D[i]), w.d, c);
+        t = t * yd[i];
+        if (Q32Fmt<DT>::HAS_M) t = t + w.m * __int_as_float(wd[i]);   // the word holds the activation block's s
         acc[i] += t;
     }
 }
@@ -451,45 +465,57 @@ __device__ __forceinline__ void q32s_step(const Q32SRaw<DT> (&cur)[NT], const ui
     for (int tt = 0; tt < TT; tt++) {
         const uint8_t* base = buf + tt * Q32S_ACT_BYTES;
         const uint2 a = *reinterpret_cast<const uint2*>(base + (B * 64 + lane) * 8);
-        const uint4 s01 = *reinterpret_cast<const uint4*>(base + Q32S_ACT_Q + (B * 16 + 4 * g) * 8);
-        const uint4 s23 = *reinterpret_cast<const uint4*>(base + Q32S_ACT_Q + (B * 16 + 4 * g + 2) * 8);
+        const f32x4g yd = *reinterpret_cast<const f32x4g*>(base + Q32S_ACT_Q + (B * 16 + 4 * g) * 4);
+        v4i wd = {0, 0, 0, 0};
+        if (Q32Fmt<DT>::OFFSET || Q32Fmt<DT>::HAS_M) wd = *reinterpret_cast<const v4i*>(base + Q32S_ACT_Q + 256 + (B * 16 + 4 * g) * 4);
 #pragma unroll
-        for (int t = 0; t < NT; t++) q32s_mac<DT>(w[t], a, s01, s23, acc[t][tt]);
+        for (int t = 0; t < NT; t++) q32s_mac<DT>(w[t], a, yd, wd, acc[t][tt]);
     }
     __builtin_amdgcn_sched_barrier(0);
 }
 
 // One wave: NT super-tile streams (tp[t], advancing `stride` bytes per K step) against the workgroup's TT slot tiles,
-// all of K.  Every thread of the workgroup must call it (barriers).
-template <int DT, int TT, int NT, bool ONCE>
-__device__ __forceinline__ void q32s_engine(const uint8_t* const tp[NT], size_t stride, const ActBuf& ab, int K, Q32SStage<TT>& st,
+// all of K.  Every thread of the workgroup must call it (barriers).  D = steps the weights and the activations are
+// requested ahead (register rings; the K loop is unrolled D times so that ring positions are compile-time).  A wave
+// with one weight stream does little arithmetic per step, so only a deep ring keeps enough bytes in flight.
+template <int DT, int TT, int NT, bool ONCE, int D>
+__device__ __forceinline__ void q32s_engine(const uint8_t* const tp[NT], size_t stride, const ActBuf& ab, int K, const Q32SRows<TT>& rows,
                                             uint8_t* act_lds, int tid, float acc[NT][TT][4]) {
-    const int lane = tid & 63, g = lane >> 4;
+    const int lane = tid & 63;
     const int nkb = K / 32, nks = K / 128;
-    q32s_issue<TT>(st, ab, K, nkb, 0, tid);
-    Q32SRaw<DT> nxt[NT];
+    Q32SStage<TT> st[D];
+    Q32SRaw<DT> ring[D][NT];
 #pragma unroll
-    for (int t = 0; t < NT; t++) nxt[t] = load_q32s<DT, ONCE>(tp[t], lane);
-    q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st, act_lds, tid);
-    q32s_issue<TT>(st, ab, K, nkb, nks > 1 ? 1 : 0, tid);
-    __syncthreads();
-    for (int ks = 0; ks < nks; ks++) {
-        Q32SRaw<DT> cur[NT];
+    for (int j = 0; j < D; j++) {
+        q32s_issue<TT>(st[j], rows, ab, K, nkb, j, tid);
         // past the end the last step is requested again (no branch around a load)
-        const int ksn = ks + 1 < nks ? ks + 1 : ks;
 #pragma unroll
-        for (int t = 0; t < NT; t++) { cur[t] = nxt[t]; nxt[t] = load_q32s<DT, ONCE>(tp[t] + (size_t)ksn * stride, lane); }
-        __builtin_amdgcn_sched_barrier(0);
-        const uint8_t* buf = act_lds + (ks & 1) * (TT * Q32S_ACT_BYTES);
-        q32s_step<DT, TT, NT, 0>(cur, buf, lane, acc);
-        q32s_step<DT, TT, NT, 1>(cur, buf, lane, acc);
-        q32s_step<DT, TT, NT, 2>(cur, buf, lane, acc);
-        q32s_step<DT, TT, NT, 3>(cur, buf, lane, acc);
-        __builtin_amdgcn_sched_barrier(0);
-        // (after the last step this stages the last step once more, into the buffer nobody reads again)
-        q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st, act_lds + ((ks + 1) & 1) * (TT * Q32S_ACT_BYTES), tid);
-        q32s_issue<TT>(st, ab, K, nkb, ks + 2 < nks ? ks + 2 : nks - 1, tid);
-        __syncthreads();
+        for (int t = 0; t < NT; t++) ring[j][t] = load_q32s<DT, ONCE>(tp[t] + (size_t)(j < nks ? j : nks - 1) * stride, lane);
+    }
+    q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st[0], act_lds, tid, false);
+    q32s_issue<TT>(st[0], rows, ab, K, nkb, D, tid);
+    __syncthreads();
+    for (int ks0 = 0; ks0 < nks; ks0 += D) {
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            const int ks = ks0 + j;
+            Q32SRaw<DT> cur[NT];
+            const int ksn = ks + D < nks ? ks + D : nks - 1;
+#pragma unroll
+            for (int t = 0; t < NT; t++) { cur[t] = ring[j][t]; ring[j][t] = load_q32s<DT, ONCE>(tp[t] + (size_t)ksn * stride, lane); }
+            __builtin_amdgcn_sched_barrier(0);
+            const uint8_t* buf = act_lds + (ks & 1) * (TT * Q32S_ACT_BYTES);
+            q32s_step<DT, TT, NT, 0>(cur, buf, lane, acc);
+            q32s_step<DT, TT, NT, 1>(cur, buf, lane, acc);
+            q32s_step<DT, TT, NT, 2>(cur, buf, lane, acc);
+            q32s_step<DT, TT, NT, 3>(cur, buf, lane, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            // step ks + 1 goes into the other buffer (nobody reads it before the barrier below), its ring position
+            // takes the request for step ks + 1 + D
+            q32s_commit<TT, Q32Fmt<DT>::OFFSET>(st[(j + 1) % D], act_lds + ((ks + 1) & 1) * (TT * Q32S_ACT_BYTES), tid, ks + 1 >= nks);
+            q32s_issue<TT>(st[(j + 1) % D], rows, ab, K, nkb, ks + 1 + D, tid);
+            __syncthreads();
+        }
     }
 }
 
@@ -511,7 +537,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
     if (!live) rt0 = 0;
     constexpr size_t STB = Q32SFmt<DT>::STB;
 
-    Q32SStage<TT> st;
+    Q32SRows<TT> st;
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
         const int iq = tg0 + tt * 16 + (tid >> 4), is = tg0 + tt * 16 + ((tid >> 2) & 15);
@@ -529,7 +555,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q32s_engine<DT, TT, 4, ONCE>(tp, (size_t)n_rt * STB, p.xq, H, st, act_lds, tid, acc);
+    q32s_engine<DT, TT, 4, ONCE, 1>(tp, (size_t)n_rt * STB, p.xq, H, st, act_lds, tid, acc);
     if (!live) return;
 
     // epilogue: h = silu(w1 x) * (w3 x); the wave's 32 rows are exactly one Q8_0 block per slot
@@ -564,7 +590,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
         }
 }
 
-template <int DT, int TT, bool ONCE, int WPE>
+template <int DT, int TT, bool ONCE, int WPE, int DEPTH>
 __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void q32s_down_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
@@ -581,7 +607,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
     if (!live) rt = 0;
     constexpr size_t STB = Q32SFmt<DT>::STB;
 
-    Q32SStage<TT> st;
+    Q32SRows<TT> st;
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
         const int iq = tg0 + tt * 16 + (tid >> 4), is = tg0 + tt * 16 + ((tid >> 2) & 15);
@@ -595,7 +621,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[0][tt][i] = 0.f;
 
-    q32s_engine<DT, TT, 1, ONCE>(tp, (size_t)n_rt * STB, p.hq, F, st, act_lds, tid, acc);
+    q32s_engine<DT, TT, 1, ONCE, DEPTH>(tp, (size_t)n_rt * STB, p.hq, F, st, act_lds, tid, acc);
     if (!live) return;
 
 #pragma unroll
@@ -619,7 +645,7 @@ static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
     const bool stream = !plain && q32_super_layout(p.H);
     // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
-    constexpr int UP1 = Q32Fmt<DT>::FIFTH ? 3 : 4, UP2 = (Q32Fmt<DT>::FIFTH && Q32Fmt<DT>::HAS_M) ? 2 : 3;
+    constexpr int UP1 = (Q32Fmt<DT>::FIFTH || Q32Fmt<DT>::HAS_M || !Q32Fmt<DT>::NIB) ? 3 : 4, UP2 = Q32Fmt<DT>::FIFTH ? 2 : 3;
     if (tt == 1) {
         if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 1, true, UP1>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
@@ -637,12 +663,15 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
     static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
     const bool stream = !plain && q32_super_layout(p.F);
+    constexpr int DN1 = Q32Fmt<DT>::FIFTH ? 3 : 4, DN2 = 4;
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, 8>), grid, dim3(Q32_THREADS), 0, s, p);
+        // one weight stream per wave: a deep request ring when K is long enough to pay for its prologue
+        if (stream && p.F >= 24 * 128) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, DN1, 6>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, DN1 + 1, 2>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, true, 6>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, false, 6>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, true, DN2, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, false, DN2, 2>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
