@@ -520,7 +520,7 @@ __device__ __forceinline__ void q32s_engine(const uint8_t* const tp[NT], size_t 
 }
 
 // (a fixed number of waves per SIMD also makes the compiler keep the MFMA results in ordinary registers)
-template <int DT, int TT, bool ONCE, int WPE>
+template <int DT, int TT, bool ONCE, int WPE, int DEPTH>
 __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void q32s_up_kernel(ExpertParams p) {
     __shared__ int list_lds[DIRECT_MAX_SLOTS];
     __shared__ int wtot_lds[Q32_THREADS / 64];
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q32s_engine<DT, TT, 4, ONCE, 1>(tp, (size_t)n_rt * STB, p.xq, H, st, act_lds, tid, acc);
+    q32s_engine<DT, TT, 4, ONCE, DEPTH>(tp, (size_t)n_rt * STB, p.xq, H, st, act_lds, tid, acc);
     if (!live) return;
 
     // epilogue: h = silu(w1 x) * (w3 x); the wave's 32 rows are exactly one Q8_0 block per slot
@@ -647,11 +647,11 @@ static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
     // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
     constexpr int UP1 = (Q32Fmt<DT>::FIFTH || Q32Fmt<DT>::HAS_M || !Q32Fmt<DT>::NIB) ? 3 : 4, UP2 = Q32Fmt<DT>::FIFTH ? 2 : 3;
     if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 1, true, UP1>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 1, true, UP1, 1>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, true, UP2>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, false, UP2>), grid, dim3(Q32_THREADS), 0, s, p);
+        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, true, UP2, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+        else if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, false, UP2, 1>), grid, dim3(Q32_THREADS), 0, s, p);
         else hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
