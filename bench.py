@@ -10,6 +10,9 @@ activations already resident in HBM.  Prints ONE JSON line.
 
 `--workload prefill` measures BASELINE config 3 instead (same layer, 4096 tokens, router bias that makes
 the expert load follow Zipf(1)); its roofline object is the int8-MFMA one of the tiled up kernel.
+`--workload config4` measures BASELINE config 4 (hidden 2048, 60 experts of FFN 1408, top-4, one always-on
+shared expert of FFN 5632 behind a sigmoid gate, Q8_0 weights, 512 tokens); its line carries the time of the
+dispatch (histogram, scan, permutation) beside the other stages.
 """
 import argparse
 import re
@@ -23,7 +26,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 H, F, E, TOPK = 4096, 14336, 8, 2
-Q4K = 12
+Q4K, Q8_0 = 12, 8
+CFG4 = dict(H=2048, F=1408, E=60, k=4, Fs=5632)   # BASELINE config 4
 EXPERT_BYTES = 3 * H * F * 144 // 256          # 99,090,432 B of Q4_K blocks per expert
 HBM_PEAK_GBS = 8000.0                          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0                        # MI355X dense int8 MFMA, published
@@ -31,20 +35,31 @@ INT8_PEAK_TOPS = 5000.0                        # MI355X dense int8 MFMA, publish
 ZIPF_BIAS = [0.0, -1.158, -1.581, -1.845, -2.033, -2.186, -2.299, -2.398]
 
 
-def build_layer(torch, candle_amd, seed=0, gate_bias=None):
+def build_layer(torch, candle_amd, seed=0, gate_bias=None, cfg4=False):
     """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel
     (bit-identical to candle's CPU quantiser), kept as host bytes for the CPU baseline too."""
+    h, f, e_n, k, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, TOPK, Q4K, 0)
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
+
+    def draw(shape):
+        x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
+        return candle_amd.quantize_weights(dt, x).cpu().numpy()
+
     w = {"w1": [], "w3": [], "w2": []}
-    for e in range(E):
-        for name, shape in (("w1", (F, H)), ("w3", (F, H)), ("w2", (H, F))):
-            x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
-            w[name].append(candle_amd.quantize_weights(Q4K, x).cpu().numpy())
-            del x
+    for e in range(e_n):
+        for name, shape in (("w1", (f, h)), ("w3", (f, h)), ("w2", (h, f))):
+            w[name].append(draw(shape))
+    kw = {}
+    if fs:
+        w["shared"] = (draw((fs, h)), draw((fs, h)), draw((h, fs)))
     g.manual_seed(seed + 1)
-    gate = (torch.randn((E, H), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
-    layer = candle_amd.SparseMoeBlock(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+    gate = (torch.randn((e_n, h), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
+    if fs:
+        w["shared_gate"] = (torch.randn((h,), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
+        kw = dict(shared_ffn=fs, shared_w1=w["shared"][0], shared_w3=w["shared"][1], shared_w2=w["shared"][2],
+                  shared_gate=w["shared_gate"])
+    layer = candle_amd.SparseMoeBlock(h, f, e_n, k, dt, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias, **kw)
     return layer, gate, w
 
 
@@ -58,7 +73,7 @@ def hip_events():
     return hip
 
 
-def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None):
+def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=False):
     """candle's CPU path restated (the oracle: serial rows, columns threaded, AVX2 inner loops of
     candle's x86 build) on all host cores: the same batch, same weight bytes, same routing,
     repeated until `min_seconds` of wall time have passed."""
@@ -67,7 +82,11 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None):
 
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
-    layer = O.Layer(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+    if cfg4:
+        layer = O.Layer(CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, gate, w["w1"], w["w3"], w["w2"], Fs=CFG4["Fs"],
+                        sw1=w["shared"][0], sw3=w["shared"][1], sw2=w["shared"][2], shared_gate=w["shared_gate"])
+    else:
+        layer = O.Layer(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
     layer.forward(xs_host[:1], logits=logits_host[:1], simd=True, threads=cores)  # warm the pages
     reps, t0 = 0, time.perf_counter()
     while True:
@@ -100,8 +119,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill)")
-    ap.add_argument("--workload", choices=("decode", "prefill"), default="decode")
+    ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill, 512 for config4)")
+    ap.add_argument("--workload", choices=("decode", "prefill", "config4"), default="decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
@@ -127,13 +146,15 @@ def main():
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
     prefill = args.workload == "prefill"
-    B = args.batch or (4096 if prefill else 32)
+    cfg4 = args.workload == "config4"
+    B = args.batch or (4096 if prefill else 512 if cfg4 else 32)
     bias = np.array(ZIPF_BIAS, dtype=np.float32) if prefill else None
-    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias)
+    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias, cfg4=cfg4)
+    n_exp, hid = (CFG4["E"], CFG4["H"]) if cfg4 else (E, H)
     g = torch.Generator(device="cuda")
     g.manual_seed(2)
     # several distinct activation batches, rotated, so that no step repeats the previous one's input
-    xs = [torch.randn((B, H), generator=g, device="cuda", dtype=torch.float32) for _ in range(4)]
+    xs = [torch.randn((B, hid), generator=g, device="cuda", dtype=torch.float32) for _ in range(4)]
     ys = [torch.empty_like(x) for x in xs]
 
     stream = torch.cuda.Stream()
@@ -142,7 +163,7 @@ def main():
         for i in range(args.warmup):
             layer.forward(xs[i % 4], out=ys[i % 4])
         stream.synchronize()
-        loads = np.diff(layer.last_routing(B)[2])[:E]
+        loads = np.diff(layer.last_routing(B)[2])[:n_exp]
         n_active = int((loads > 0).sum())
         ev = [C.c_void_p() for _ in range(2)]
         for e in ev:
@@ -170,7 +191,26 @@ def main():
     stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
 
     step_bytes = n_active * EXPERT_BYTES + E * H * 4 + 2 * B * H * 4
-    if prefill:
+    metric = "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, %s)" % args.workload
+    if cfg4:
+        # Weights are Q8_0 (34 bytes per 32 elements); every routed expert with a token and the shared expert are
+        # read at least once per step.  The up kernel (w1, w3 of the routed experts) is the longest launch.
+        c = CFG4
+        expert_bytes = 3 * c["H"] * c["F"] * 34 // 32
+        shared_bytes = 3 * c["H"] * c["Fs"] * 34 // 32
+        step_bytes = n_active * expert_bytes + shared_bytes + c["E"] * c["H"] * 4 + 2 * B * c["H"] * 4
+        up_bytes = n_active * (2 * c["H"] * c["F"] * 34 // 32)
+        achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+        step_ops = 2.0 * B * 3 * c["H"] * (c["k"] * c["F"] + c["Fs"])
+        roofline = {"bound": "hbm", "kernel": "q32s_up (routed w1, w3, SiLU, Q8_0 re-quantisation; lists beyond 32 rows re-read the weights from L2)",
+                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": None, "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+        workload = ("BASELINE config 4: hidden 2048, 60 experts of ffn 1408, top-4 renormalised, shared expert of ffn 5632 "
+                    "with sigmoid gate, Q8_0 weights, %d tokens" % B)
+        extra = {"step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                 "step_int8_ops": step_ops, "dispatch_us": stage_us["dispatch"], "max_expert_load": int(loads.max())}
+        metric = "MoE layer tokens/s (Qwen-MoE shape, Q8_0, 512-token batch)"
+    elif prefill:
         # Roofline of the dominant kernel, the tiled up projection: 2 * slots * 2 * H * F integer
         # multiply-adds (w1 and w3) per launch against the dense int8 MFMA peak.
         up_ops = 2.0 * B * TOPK * 2 * H * F
@@ -201,7 +241,7 @@ def main():
         extra = {"step_algorithmic_bytes": step_bytes,
                  "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
     out = {
-        "metric": "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, %s)" % args.workload, "value": tokens_per_s, "unit": "tokens/s",
+        "metric": metric, "value": tokens_per_s, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8",
         "data": "synthetic",
@@ -215,7 +255,7 @@ def main():
         # a bounded sample: the CPU path does ~1 k tokens/s, so a prefill batch is cut to its first 64 tokens
         n_cpu = min(B, 64)
         out["cpu_baseline"] = cpu_baseline(gate, w, xs[0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu],
-                                           args.cpu_seconds, gate_bias=bias)
+                                           args.cpu_seconds, gate_bias=bias, cfg4=cfg4)
     print(json.dumps(out))
 
 

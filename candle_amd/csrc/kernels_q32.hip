@@ -11,7 +11,6 @@
 // Q4_0 stores nibble - 8 and Q5_0 code - 16; the kernel multiplies the raw codes (0..15, 0..31) and
 // subtracts 8 or 16 times sum(q8) of the block, which is the same integer.  Q4_1 and Q5_1 codes are
 // unsigned as stored.
-#include <cstdlib>
 #include "act_quant.hpp"
 #include "kernels.hpp"
 #include "slots.hpp"
@@ -642,8 +641,7 @@ static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
     const int wpb = Q32_THREADS / 64;
     const int n_pairs = p.F / 32;
     dim3 grid((unsigned)((n_pairs + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
-    const bool stream = !plain && q32_super_layout(p.H);
+    const bool stream = q32_super_layout(p.H);   // the layout of w1 / w3 decides
     // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
     constexpr int UP1 = (Q32Fmt<DT>::FIFTH || Q32Fmt<DT>::HAS_M || !Q32Fmt<DT>::NIB) ? 3 : 4, UP2 = Q32Fmt<DT>::FIFTH ? 2 : 3;
     if (tt == 1) {
@@ -661,8 +659,7 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     const int tt = p.slot_tiles >= 2 ? 2 : 1;
     const int wpb = Q32_THREADS / 64;
     dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    static const bool plain = getenv("MOE_Q32_PLAIN") != nullptr;
-    const bool stream = !plain && q32_super_layout(p.F);
+    const bool stream = q32_super_layout(p.F);   // the layout of w2 decides
     constexpr int DN1 = Q32Fmt<DT>::FIFTH ? 3 : 4, DN2 = 4;
     if (tt == 1) {
         // one weight stream per wave: a deep request ring when K is long enough to pay for its prologue
