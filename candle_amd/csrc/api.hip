@@ -358,6 +358,8 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
     // tiles per pass up to ~40 rows per expert)
     ep.slot_tiles = (T * L->k > 40 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    // (the 32-element kernels carry at most two tiles: three or four per pass measured slower at the Mixtral shape and
+    // 8 % faster at best where sixty small experts' weights exceed the caches)
     static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
     if (force_st) ep.slot_tiles = force_st;
     static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;

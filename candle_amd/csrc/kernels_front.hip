@@ -105,12 +105,25 @@ struct DispatchShared {
 // tok_slots is written and re-read inside one workgroup: bypass the vector cache on the re-read
 __device__ inline int ld_i32(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 
+// Mask of the valid lanes whose expert index equals this lane's: one ballot per bit of the index, whatever the number
+// of distinct experts among the 64 lanes (a loop over the distinct values takes ~40 rounds with 60 experts and top-4).
+__device__ inline unsigned long long same_expert_lanes(int e, bool valid, int ebits) {
+    unsigned long long m = __ballot(valid);
+    for (int b = 0; b < ebits; b++) {
+        const unsigned long long set = __ballot((e >> b) & 1);
+        m &= ((e >> b) & 1) ? set : ~set;
+    }
+    return m;
+}
+
 __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, bool shared, DispatchShared& sh) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int NW = DISPATCH_THREADS / 64;
     const int64_t A = T * k;
     const int64_t chunk = ((A + NW - 1) / NW + 63) / 64 * 64;
     const int64_t lo = wave * chunk, hi = (lo + chunk < A) ? lo + chunk : A;
+    const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));   // the lanes below this one
+    const int ebits = 32 - __clz(E > 1 ? E - 1 : 1);                              // bits of an expert index
     for (int i = tid; i < NW * MAX_E; i += DISPATCH_THREADS) (&sh.cnt[0][0])[i] = 0;
     __syncthreads();
     // phase 1: per-wave histogram from ballots (topk_idx comes from the previous kernel: plain loads,
@@ -121,14 +134,9 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
             const int e = e_next;
             const bool valid = base + lane < hi;
             e_next = (base + 64 + lane < hi) ? rb.topk_idx[base + 64 + lane] : -1;
-            unsigned long long rem = __ballot(valid);
-            while (rem) {
-                int leader = __ffsll((long long)rem) - 1;
-                int e0 = __shfl(e, leader, 64);
-                unsigned long long m = __ballot(valid && e == e0);
-                if (lane == leader) sh.cnt[wave][e0] += __popcll(m);
-                rem &= ~m;
-            }
+            // lanes of this wave with the same expert; the lowest of them adds the group's size
+            const unsigned long long m = same_expert_lanes(e, valid, ebits);
+            if (valid && (m & lt) == 0) sh.cnt[wave][e] += __popcll(m);
         }
     }
     __syncthreads();
@@ -189,7 +197,6 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
     {
         int e_next = (lo + lane < hi) ? rb.topk_idx[lo + lane] : -1;
         float w_next = (lo + lane < hi) ? rb.topk_w[lo + lane] : 0.f;
-        const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
         for (int64_t base = lo; base < hi; base += 64) {
             const int64_t a = base + lane;
             const bool valid = a < hi;
@@ -197,17 +204,13 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
             const float w = w_next;
             e_next = (a + 64 < hi) ? rb.topk_idx[a + 64] : -1;
             w_next = (a + 64 < hi) ? rb.topk_w[a + 64] : 0.f;
-            unsigned long long rem = __ballot(valid);
+            const unsigned long long m = same_expert_lanes(e, valid, ebits);
             int slot = -1;
-            while (rem) {
-                int leader = __ffsll((long long)rem) - 1;
-                int e0 = __shfl(e, leader, 64);
-                unsigned long long m = __ballot(valid && e == e0);
-                int cur = sh.cnt[wave][e0];
-                if (valid && e == e0) slot = cur + __popcll(m & lt);
-                // all lanes have read `cur` before the leader updates it (same wave, program order)
-                if (lane == leader) sh.cnt[wave][e0] = cur + __popcll(m);
-                rem &= ~m;
+            if (valid) {
+                const int cur = sh.cnt[wave][e];
+                slot = cur + __popcll(m & lt);
+                // every lane of the group has read `cur` before its lowest lane updates it (one wave, program order)
+                if ((m & lt) == 0) sh.cnt[wave][e] = cur + __popcll(m);
             }
             if (valid) {
                 int t = (int)(a / k);

@@ -635,41 +635,58 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
         }
 }
 
+template <int DT, int TT>
+static void launch_q32s_up(const ExpertParams& p, dim3 grid, hipStream_t s) {
+    // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
+    constexpr bool fat = Q32Fmt<DT>::FIFTH || Q32Fmt<DT>::HAS_M || !Q32Fmt<DT>::NIB;
+    constexpr int WPE = TT == 1 ? (fat ? 3 : 4) : (Q32Fmt<DT>::FIFTH ? 2 : 3);
+    // one-tile launches are chosen for short lists: a second pass is the exception there, and the stream stays non-temporal
+    if (TT == 1 || grid.z == 1) hipLaunchKernelGGL((q32s_up_kernel<DT, TT, true, WPE, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q32s_up_kernel<DT, TT, false, WPE, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+}
 template <int DT>
 static hipError_t launch_q32_up_t(const ExpertParams& p, hipStream_t s) {
+    const bool stream = q32_super_layout(p.H);   // the layout of w1 / w3 decides
     const int tt = p.slot_tiles >= 2 ? 2 : 1;
     const int wpb = Q32_THREADS / 64;
     const int n_pairs = p.F / 32;
     dim3 grid((unsigned)((n_pairs + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    const bool stream = q32_super_layout(p.H);   // the layout of w1 / w3 decides
-    // waves per SIMD the register count of each variant allows (the five-bit formats carry their fifth-bit words)
-    constexpr int UP1 = (Q32Fmt<DT>::FIFTH || Q32Fmt<DT>::HAS_M || !Q32Fmt<DT>::NIB) ? 3 : 4, UP2 = Q32Fmt<DT>::FIFTH ? 2 : 3;
-    if (tt == 1) {
-        if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 1, true, UP1, 1>), grid, dim3(Q32_THREADS), 0, s, p);
-        else hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+    if (stream) {
+        if (tt == 1) launch_q32s_up<DT, 1>(p, grid, s);
+        else launch_q32s_up<DT, 2>(p, grid, s);
+    } else if (tt == 1) {
+        hipLaunchKernelGGL((q32_up_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, true, UP2, 1>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32s_up_kernel<DT, 2, false, UP2, 1>), grid, dim3(Q32_THREADS), 0, s, p);
-        else hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+        hipLaunchKernelGGL((q32_up_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
 }
+template <int DT, int TT>
+static void launch_q32s_down(const ExpertParams& p, dim3 grid, hipStream_t s) {
+    constexpr int WPE = TT == 1 ? (Q32Fmt<DT>::FIFTH ? 3 : 4) : 4;
+    if constexpr (TT == 1) {
+        // one weight stream per wave: a deep request ring when K is long enough to pay for its prologue
+        if (p.F >= 24 * 128) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, WPE, 6>), grid, dim3(Q32_THREADS), 0, s, p);
+        else hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, WPE + 1, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+    } else if (grid.z == 1) {
+        hipLaunchKernelGGL((q32s_down_kernel<DT, TT, true, WPE, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+    } else {
+        hipLaunchKernelGGL((q32s_down_kernel<DT, TT, false, WPE, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+    }
+}
 template <int DT>
 static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
+    const bool stream = q32_super_layout(p.F);   // the layout of w2 decides
     const int tt = p.slot_tiles >= 2 ? 2 : 1;
     const int wpb = Q32_THREADS / 64;
     dim3 grid((unsigned)((p.H / 16 + wpb - 1) / wpb), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
-    const bool stream = q32_super_layout(p.F);   // the layout of w2 decides
-    constexpr int DN1 = Q32Fmt<DT>::FIFTH ? 3 : 4, DN2 = 4;
-    if (tt == 1) {
-        // one weight stream per wave: a deep request ring when K is long enough to pay for its prologue
-        if (stream && p.F >= 24 * 128) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, DN1, 6>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 1, true, DN1 + 1, 2>), grid, dim3(Q32_THREADS), 0, s, p);
-        else hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
+    if (stream) {
+        if (tt == 1) launch_q32s_down<DT, 1>(p, grid, s);
+        else launch_q32s_down<DT, 2>(p, grid, s);
+    } else if (tt == 1) {
+        hipLaunchKernelGGL((q32_down_kernel<DT, 1>), grid, dim3(Q32_THREADS), 0, s, p);
     } else {
-        if (stream && grid.z == 1) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, true, DN2, 2>), grid, dim3(Q32_THREADS), 0, s, p);
-        else if (stream) hipLaunchKernelGGL((q32s_down_kernel<DT, 2, false, DN2, 2>), grid, dim3(Q32_THREADS), 0, s, p);
-        else hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
+        hipLaunchKernelGGL((q32_down_kernel<DT, 2>), grid, dim3(Q32_THREADS), 0, s, p);
     }
     return hipGetLastError();
 }
