@@ -303,6 +303,24 @@ def test_block_legacy_five_bit_and_min_formats(dt, dt_down):
     gpu.close()
 
 
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_0])
+def test_block_32_element_formats_ragged_row_tiles(dt):
+    # The super-tile kernels (K % 128 == 0) run four waves per workgroup behind common barriers; these shapes leave
+    # waves without rows: 3 and 5 pairs of row tiles in the up projection (F = 96, 160), 6 row tiles in the down
+    # projection (H = 96), and mix super-tile matrices with one-block ones (the other projection's K is not a
+    # multiple of 128).
+    for H, F in ((128, 96), (128, 160), (96, 256), (384, 640)):
+        ref, gpu = make_pair(H, F, 3, 2, dt, seed=40 + H + F, Fs=F)
+        for T in (1, 20, 45):
+            check_block(ref, gpu, T, tol=TOL)
+        gpu.close()
+    # dense products with 3 and 5 row tiles, one and three K steps
+    for n, k, m in ((48, 128, 3), (80, 384, 40)):
+        w = O.fill_normal_quantized(n + k, dt, n, k, 0.02)
+        x = activations(m, k, seed=n)
+        assert np.array_equal(bits(candle_amd.qmatmul(dt, w, n, k, x)), bits(O.matmul(dt, x, w, n)))
+
+
 def test_mixed_dtypes_need_one_activation_format():
     ref41, _ = make_pair(256, 256, 4, 2, O.Q4_1, seed=6, want_gpu=False)
     with pytest.raises(candle_amd.MoeError, match="quantise activations differently"):   # Q8_1 against Q8_0
