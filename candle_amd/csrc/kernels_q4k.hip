@@ -140,6 +140,10 @@ __device__ inline void q45k_mac(const uint4& q0, const uint4& q1, const uint4& s
     v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, mB, zf, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+        // The reference rounds d_w * d_x first and then each product; (d_w isum - dmin_w mins) d_x with fused
+        // multiply-adds would save two instructions per result, but every rounding that differs from the reference's
+        // moves more intermediate values across a re-quantisation boundary (measured: the 64-token case of the
+        // Mixtral-shape test went from inside to outside the 2e-3 bar).
         const float dd = d * yd[i];
         const float dm = dmin * yd[i];
         acc[i] += dd * (float)isum[i];
@@ -149,6 +153,72 @@ __device__ inline void q45k_mac(const uint4& q0, const uint4& q1, const uint4& s
 
 __device__ inline void q4k_mac(const Q4KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
     q45k_mac<false>(w.q0, w.q1, w.sc, 0u, 0u, A, yd, g, acc);
+}
+
+// The same Q4K contribution with the 6-bit scale inside the weight operand, for workgroups that carry two or four
+// slot tiles: sc = 8 hi + lo (3-bit digits), the byte planes hi * q4 and lo * q4 (<= 105, packed 16-bit multiplies,
+// no carry between bytes) are each multiplied by the activations with v_mfma_i32_16x16x64_i8 (a pair of sub-blocks
+// per instruction, its two scales already applied) and accumulated over the super-block; 8 acc_hi + acc_lo is the
+// integer of vec_dot.  The planes are built once per weight tile and serve every slot tile, whereas q45k_mac spends
+// an integer multiply-add per result and sub-block: 80 + 32 TT vector instructions per tile against 39 + 72 TT.
+typedef unsigned short u16x2p __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t digit_times_codes(uint32_t q, uint32_t digit) {
+    const u16x2p a = __builtin_bit_cast(u16x2p, q);
+    const u16x2p b = {(unsigned short)digit, (unsigned short)digit};
+    return __builtin_bit_cast(uint32_t, (u16x2p)(a * b));
+}
+struct Q4KPlanes {
+    v4i hi[4], lo[4];   // pair P: operand of one 16x16x64 MFMA (sub-block 2P chunk, sub-block 2P+1 chunk)
+    float d, dmin;
+    v4h mB;
+};
+__device__ inline Q4KPlanes q4k_planes(const Q4KTile& w, int g) {
+    const uint32_t M4 = 0x0f0f0f0fu;
+    Q4KPlanes pl;
+    const uint32_t hdr = w.sc.x, u0 = w.sc.y, u1 = w.sc.z, u2 = w.sc.w;
+    pl.d = __half2float(__ushort_as_half((unsigned short)(hdr & 0xffffu)));
+    pl.dmin = __half2float(__ushort_as_half((unsigned short)(hdr >> 16)));
+    const uint32_t sc03 = u0 & 0x3f3f3f3fu;
+    const uint32_t sc47 = (u2 & M4) | (((u0 >> 6) & 0x03030303u) << 4);
+    const uint32_t m03 = u1 & 0x3f3f3f3fu;
+    const uint32_t m47 = ((u2 >> 4) & M4) | (((u1 >> 6) & 0x03030303u) << 4);
+    const uint32_t qw[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t wx = qw[2 * P], wy = qw[2 * P + 1];
+        const uint32_t lx = wx & M4, ly = wy & M4, hx = (wx >> 4) & M4, hy = (wy >> 4) & M4;
+        // the digits of four scales at a time, then one bit-field extract per digit
+        const uint32_t scw = (P < 2) ? sc03 : sc47;
+        const uint32_t hiw = (scw >> 3) & 0x07070707u, low = scw & 0x07070707u;
+        const uint32_t s0h = (hiw >> (16 * (P & 1))) & 0xffu, s1h = (hiw >> (16 * (P & 1) + 8)) & 0xffu;
+        const uint32_t s0l = (low >> (16 * (P & 1))) & 0xffu, s1l = (low >> (16 * (P & 1) + 8)) & 0xffu;
+        pl.hi[P] = v4i{(int)digit_times_codes(lx, s0h), (int)digit_times_codes(ly, s0h), (int)digit_times_codes(hx, s1h), (int)digit_times_codes(hy, s1h)};
+        pl.lo[P] = v4i{(int)digit_times_codes(lx, s0l), (int)digit_times_codes(ly, s0l), (int)digit_times_codes(hx, s1l), (int)digit_times_codes(hy, s1l)};
+    }
+    const uint32_t mw = (g < 2) ? m03 : m47;
+    const _Float16 ma = (_Float16)(int)((mw >> (16 * (g & 1))) & 0xffu);
+    const _Float16 mb = (_Float16)(int)((mw >> (16 * (g & 1) + 8)) & 0xffu);
+    pl.mB = v4h{ma, ma, mb, mb};
+    return pl;
+}
+__device__ inline void q4k_mac_planes(const Q4KPlanes& pl, const Q8KOperand& A, const float yd[4], float acc[4]) {
+    const v4i zero = {0, 0, 0, 0};
+    v4i acc_hi = zero, acc_lo = zero;
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const v4i a = {(int)A.a[P].x, (int)A.a[P].y, (int)A.a[P].z, (int)A.a[P].w};
+        acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.hi[P], acc_hi, 0, 0, 0);
+        acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.lo[P], acc_lo, 0, 0, 0);
+    }
+    const v4f zf = {0.f, 0.f, 0.f, 0.f};
+    v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, pl.mB, zf, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float dd = pl.d * yd[i];
+        const float dm = pl.dmin * yd[i];
+        acc[i] += dd * (float)(8 * acc_hi[i] + acc_lo[i]);
+        acc[i] -= dm * Dm[i];
+    }
 }
 
 // Q5K (BlockQ5K::vec_dot, k_quants.rs:1394-1485): the Q4K arithmetic on 5-bit codes
@@ -335,30 +405,43 @@ struct FmtQ4K {
     typedef Q4KTile Tile;
     static constexpr int TILE_BYTES = Q4K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q4k_tile(tile, lane); }
+    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q4k_mac(w, A, yd, g, acc); }
+};
+// Q4K with the scales inside the weight operand (see q4k_planes): for two and four slot tiles per pass
+struct FmtQ4KP {
+    typedef Q4KTile Tile;
+    static constexpr int TILE_BYTES = Q4K_TILE_BYTES;
+    static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q4k_tile(tile, lane); }
+    static __device__ inline Q4KPlanes prepare(const Tile& w, int g) { return q4k_planes(w, g); }
+    static __device__ inline void mac(const Q4KPlanes& pl, const Q8KOperand& A, const float yd[4], int, float acc[4]) { q4k_mac_planes(pl, A, yd, acc); }
 };
 struct FmtQ2K {
     typedef Q2KTile Tile;
     static constexpr int TILE_BYTES = Q2K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q2k_tile(tile, lane); }
+    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q2k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ3K {
     typedef Q3KTile Tile;
     static constexpr int TILE_BYTES = Q3K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q3k_tile(tile, lane); }
+    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q3k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ5K {
     typedef Q5KTile Tile;
     static constexpr int TILE_BYTES = Q5K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q5k_tile(tile, lane); }
+    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q5k_mac(w, A, yd, g, acc); }
 };
 struct FmtQ6K {
     typedef Q6KTile Tile;
     static constexpr int TILE_BYTES = Q6K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q6k_tile(tile, lane); }
+    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
     static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q6k_mac(w, A, yd, g, acc); }
 };
 
@@ -420,8 +503,9 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride,
                 sbn = sbn < sb_hi ? sbn : sb_hi - 1;
                 t[idx % RING] = FMT::load(tp[jn] + (size_t)sbn * sb_stride, lane);
                 __builtin_amdgcn_sched_barrier(0);
+                const auto prep = FMT::prepare(w, g);   // what of the tile's unpacking serves every slot tile
 #pragma unroll
-                for (int tt = 0; tt < TT; tt++) FMT::mac(w, A[tt], yd[tt], g, acc[j][tt]);
+                for (int tt = 0; tt < TT; tt++) FMT::mac(prep, A[tt], yd[tt], g, acc[j][tt]);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
@@ -618,13 +702,13 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
 DEF_UP(q4k_up_t1_v0, FmtQ4K, 1, 8, 2, 4)
 DEF_UP(q4k_up_t1_v1, FmtQ4K, 1, 4, 2, 3)
 DEF_UP_NARROW(q4k_up_t1_narrow, FmtQ4K, 4, 2, 3)
-DEF_UP(q4k_up_t2, FmtQ4K, 2, 4, 2, 2)
-DEF_UP(q4k_up_t4, FmtQ4K, 4, 8, 2, 2)
+DEF_UP(q4k_up_t2, FmtQ4KP, 2, 4, 2, 2)
+DEF_UP(q4k_up_t4, FmtQ4KP, 4, 8, 2, 2)
 DEF_DOWN(q4k_down_t1_v0, FmtQ4K, 1, 8, 2, 4)
 DEF_DOWN(q4k_down_t1_v1, FmtQ4K, 1, 4, 2, 3)
 DEF_DOWN_NARROW(q4k_down_t1_narrow, FmtQ4K, 8, 2, 4)
-DEF_DOWN(q4k_down_t2, FmtQ4K, 2, 4, 2, 2)
-DEF_DOWN(q4k_down_t4, FmtQ4K, 4, 8, 2, 2)
+DEF_DOWN(q4k_down_t2, FmtQ4KP, 2, 4, 2, 2)
+DEF_DOWN(q4k_down_t4, FmtQ4KP, 4, 8, 2, 2)
 // Q2K: nine registers per tile; one and two slot tiles per pass
 DEF_UP(q2k_up_t1, FmtQ2K, 1, 4, 2, 3)
 DEF_UP_NARROW(q2k_up_t1_narrow, FmtQ2K, 4, 2, 3)

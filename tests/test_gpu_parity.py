@@ -195,7 +195,9 @@ def check_block(ref, gpu, T, seed=2, tol=None):
     moe = want - xs if ref.rms_alpha is not None else want
     err = np.abs(ys - want).max()
     assert err <= tol * rms(moe), (err, rms(moe))
-    assert rms(ys - want) <= 2e-4 * rms(moe)  # a wrong term or index moves the whole result, not one element
+    # a wrong term or index moves the whole result, not one element; the flipped quants of a narrow intermediate
+    # weigh more (the same sqrt(14336 / F) by which block_tol widens the max-abs bar)
+    assert rms(ys - want) <= 2e-4 * (tol / TOL) * rms(moe)
     return ys, want
 
 
