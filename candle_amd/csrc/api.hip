@@ -388,12 +388,14 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         if (capturing && L->hbuf.cap < (size_t)T * L->k * L->F * 4) return fail(MOE_E_INVALID, capture_msg);
         if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
         ep.hbuf = L->hbuf.as<float>();
+        ep.by_assignment = T * L->k <= L->E ? 1 : 0;   // one row of workgroups per assignment: none for idle experts
         MOE_HIP_CHECK(launch_expert_up(ep, s));
         MOE_MARK(ST_UP);
         MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_REQUANT);
         MOE_HIP_CHECK(launch_expert_down(ep, s));
         MOE_MARK(ST_DOWN);
+        ep.by_assignment = 0;
     } else {
         MOE_HIP_CHECK(launch_expert_up(ep, s));   // re-quantises the intermediate in its epilogue
         MOE_MARK(ST_UP);

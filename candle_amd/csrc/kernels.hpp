@@ -73,6 +73,10 @@ struct ExpertParams {
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
     int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1, 2 or, Q4K only, 4)
     int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)
+    // Narrow launches of tiny batches (direct slot numbering, T*k <= E): the grid's y dimension counts assignments
+    // instead of experts, workgroup row y serves the expert of assignment y unless an earlier assignment names the
+    // same expert.  No workgroups (and no weight prefetches) for experts without tokens.
+    int by_assignment = 0;
     float* hbuf = nullptr;          // tiled path only: f32 intermediate [slots, F] before re-quantisation
     int64_t n_slots = 0;            // tiled path only: total slots (bounds the tile grid)
 };

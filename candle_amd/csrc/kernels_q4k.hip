@@ -534,7 +534,8 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
     constexpr int NT = 2 * RTW;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
-    const int grp = blockIdx.y;
+    const int grp = __builtin_amdgcn_readfirstlane(group_of_row(p, blockIdx.y));
+    if (grp < 0) return;
     const int H = p.H, F = p.F, nsb = H / 256;
     const int rb = blockIdx.x;
     const GroupWeights gw = p.groups[grp];
@@ -611,7 +612,8 @@ template <class FMT, int TT, int NW, int RING, int NTD = 4>
 __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * TT * 4][64], int* list_lds, int* wtot_lds) {
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: tile addresses stay in scalar registers
-    const int grp = blockIdx.y;
+    const int grp = __builtin_amdgcn_readfirstlane(group_of_row(p, blockIdx.y));
+    if (grp < 0) return;
     const int H = p.H, F = p.F, nsb = F / 256;
     const int n_rt = H / 16;
     const int rt0 = blockIdx.x * NTD;
@@ -776,7 +778,7 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     static const int uv = variant("MOE_UP_VARIANT", 1);
     const int tt = p.slot_tiles >= 4 && f->up_t4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (64 rows), f32 h to p.hbuf
-        dim3 ngrid((unsigned)(p.F / 64), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
+        dim3 ngrid((unsigned)(p.F / 64), (unsigned)(p.by_assignment ? p.rb.T * p.rb.k : p.n_groups), (unsigned)((p.max_rows + 15) / 16));
         hipLaunchKernelGGL(f->up_narrow, ngrid, dim3(256), 0, s, p);
         return hipGetLastError();
     }
@@ -795,7 +797,7 @@ hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
     static const int dv = variant("MOE_DOWN_VARIANT", 1);
     const int tt = p.slot_tiles >= 4 && f->down_t4 ? 4 : p.slot_tiles >= 2 ? 2 : 1;
     if (p.hbuf && tt == 1) {   // narrow workgroups (32 rows), eight waves split K
-        dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)p.n_groups, (unsigned)((p.max_rows + 15) / 16));
+        dim3 ngrid((unsigned)((p.H / 16 + 1) / 2), (unsigned)(p.by_assignment ? p.rb.T * p.rb.k : p.n_groups), (unsigned)((p.max_rows + 15) / 16));
         hipLaunchKernelGGL(f->down_narrow, ngrid, dim3(512), 0, s, p);
         return hipGetLastError();
     }

@@ -57,6 +57,17 @@ __device__ inline GroupSlots group_slots(const ExpertParams& p, int grp, int* li
     return gs;
 }
 
+// Group of a workgroup row.  Regular launches: the row index.  Launches by assignment: the expert of assignment
+// `row`, or -1 when an earlier assignment has the same expert (its workgroups do the work).  Uniform per workgroup.
+__device__ inline int group_of_row(const ExpertParams& p, int row) {
+    if (!p.by_assignment) return row;
+    const int lane = threadIdx.x & 63;
+    const int e = p.rb.topk_idx[row];
+    bool dup = false;
+    for (int a = lane; a < row; a += 64) dup |= p.rb.topk_idx[a] == e;
+    return __any(dup) ? -1 : e - p.group0;
+}
+
 // token row / routing weight of a slot
 __device__ inline int slot_token(const ExpertParams& p, int slot) {
     if (!p.rb.direct) return p.rb.perm_token[slot];
