@@ -328,13 +328,16 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.xq = L->xq.view();
     fp.rb = L->route.view();
     fp.rb.T = (int)T; fp.rb.k = (int)L->k;
-    // Q4K batches with more than ~36 rows per expert take the tiled MFMA kernels (F a multiple of 64,
-    // H of 128; those kernels address activation rows with 32-bit byte offsets).  Their tiles hold 64
-    // slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
+    // Q4K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
+    // multiple of 64, H of 128; those kernels address activation rows with 32-bit byte offsets), from ~64 rows per
+    // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
+    // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
+    // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
     static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
     // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
     const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k > 36 * L->E;
+                       T * L->k > 38 * L->E;
+    const bool tiled_down = tiled && L->dt_down == MOE_GGML_Q4K && T * L->k > 64 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     const bool direct = !tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     fp.rb.direct = direct ? 1 : 0;
@@ -356,8 +359,8 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
     // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
-    // tiles per pass up to ~40 rows per expert)
-    ep.slot_tiles = (T * L->k > 40 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    // tiles per pass up to ~34 rows per expert)
+    ep.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
     // (the 32-element kernels carry at most two tiles: three or four per pass measured slower at the Mixtral shape and
     // 8 % faster at best where sixty small experts' weights exceed the caches)
     static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
@@ -374,7 +377,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         MOE_MARK(ST_UP);
         MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_REQUANT);
-        if (L->dt_down == MOE_GGML_Q4K) {
+        if (tiled_down) {
             MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
         } else {
             ExpertParams dp = ep;
