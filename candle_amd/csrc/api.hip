@@ -149,10 +149,28 @@ struct moe_layer {
     ActStore xq, hq, hq_shared;
     DevBuf yw, x_dev, y_dev, hbuf;
     hipStream_t stream = nullptr;   // used by the host-pointer entry
-    hipEvent_t done = nullptr;      // end of the last enqueued forward
+    // Calls share the workspace, so a call must not start before the previous one has finished.  On one stream the
+    // stream's own order sees to that; the event is recorded (on the previous call's stream) only when a call arrives on
+    // another stream or the host wants the results: an event record between every two forwards costs a 5.6 us bubble.
+    hipEvent_t done = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool pending = false;           // work enqueued on last_stream that `done` does not cover yet
     int64_t last_T = 0;
     bool last_direct = false;       // the last forward skipped the dispatch pass
 };
+
+// Marks the end of everything enqueued for the layer so far in L->done.  If the stream of the last call has gone
+// (the caller destroyed it; its work completes all the same) the device is synchronised instead.
+static int close_pending(moe_layer* L) {
+    if (!L->pending) return MOE_OK;
+    if (hipEventRecord(L->done, L->last_stream) != hipSuccess) {
+        (void)hipGetLastError();
+        MOE_HIP_CHECK(hipDeviceSynchronize());
+        MOE_HIP_CHECK(hipEventRecord(L->done, nullptr));
+    }
+    L->pending = false;
+    return MOE_OK;
+}
 
 static int reserve_workspace(moe_layer* L, int64_t T) {
     if (T <= L->cap_T) return MOE_OK;
@@ -315,7 +333,10 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     int rc = reserve_workspace(L, T);
     if (rc) return rc;
     // a previous call may still be running on another stream and shares the workspace
-    if (!capturing) MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
+    if (!capturing && (!L->pending || L->last_stream != s)) {
+        if ((rc = close_pending(L))) return rc;
+        MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
+    }
     const bool shared = L->Fs > 0;
     FrontParams fp;
     fp.x = d_x; fp.T = T; fp.H = (int)L->H; fp.E = (int)L->E; fp.k = (int)L->k; fp.norm_topk = L->norm_topk;
@@ -420,7 +441,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     MOE_MARK(ST_COMBINE);
 #undef MOE_MARK
     L->last_direct = direct;
-    if (!capturing) MOE_HIP_CHECK(hipEventRecord(L->done, s));
+    if (!capturing) { L->last_stream = s; L->pending = true; }
     L->last_T = T;
     return MOE_OK;
 }
@@ -489,6 +510,7 @@ extern "C" int moe_layer_last_logits(moe_layer* L, float* logits, int64_t T) {
     if (!L || !logits) return fail(MOE_E_INVALID, "bad argument to moe_layer_last_logits");
     std::lock_guard<std::mutex> lk(L->mu);
     if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
+    if (int rc = close_pending(L)) return rc;
     MOE_HIP_CHECK(hipEventSynchronize(L->done));
     return d2h(logits, L->route.logits.p, (size_t)T * L->E * 4);
 }
@@ -498,8 +520,9 @@ extern "C" int moe_layer_last_routing(moe_layer* L, int64_t T, int32_t* topk_idx
     if (!L) return fail(MOE_E_INVALID, "layer is NULL");
     std::lock_guard<std::mutex> lk(L->mu);
     if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
-    MOE_HIP_CHECK(hipEventSynchronize(L->done));
     int rc;
+    if ((rc = close_pending(L))) return rc;
+    MOE_HIP_CHECK(hipEventSynchronize(L->done));
     const size_t A = (size_t)T * L->k;
     if (L->last_direct && T > 0) {  // the forward needed no lists; build them now for the caller
         RouteBufs rb = L->route.view();

@@ -440,6 +440,33 @@ def test_device_entry_point_matches_host_entry_point():
     gpu.close()
 
 
+def test_forward_alternating_between_streams():
+    # Calls on one layer share its workspace.  On one stream the stream's order serialises them; a call on another
+    # stream has to wait for the previous call's kernels (the library records its ordering event only then).
+    import torch
+    ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=17)
+    xs = [torch.from_numpy(activations(T, 512, 60 + i)).cuda() for i, T in enumerate((40, 3, 40, 17, 64, 5))]
+    want = [gpu.forward(x).cpu().numpy() for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.current_stream()]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        outs = []
+        for i, x in enumerate(xs):
+            st = streams[(i + rep) % 3]
+            st.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(st):
+                outs.append((st, gpu.forward(x)))
+        for (st, y), w in zip(outs, want):
+            st.synchronize()
+            assert np.array_equal(bits(y.cpu().numpy()), bits(w))
+    # the parity hooks wait for the last call wherever it ran
+    with torch.cuda.stream(streams[0]):
+        y = gpu.forward(xs[0])
+    assert gpu.last_logits(40).shape == (40, 8)
+    assert np.array_equal(bits(y.cpu().numpy()), bits(want[0]))
+    gpu.close()
+
+
 def test_concurrent_forward_from_several_threads():
     # QuantizedType is Send + Sync (candle-core/src/quantized/mod.rs:256): candle calls a layer from any thread.
     # Four threads share two layers (calls on one layer are serialised inside the library) and use their own inputs.
