@@ -100,14 +100,15 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg
                       "(AVX2 vec_dot, %d threads over output columns)" % (reps, xs_host.shape[0], dt, cores)}
 
 
-def measured_traffic(batch):
+def measured_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
     """HBM bytes per launch of the up kernel from the committed rocprofv3 counter summary (FETCH_SIZE +
     WRITE_SIZE, scaled by the copy kernel), or None when the summary does not cover this batch size."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "q4k_up_decode_hbm_traffic.md")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", name)
+    key = key or "batch=%d" % batch
     try:
         for line in open(path):
-            m = re.match(r"traffic_bytes_per_launch\[batch=(\d+)\]:\s*(\d+)", line.strip())
-            if m and int(m.group(1)) == batch:
+            m = re.match(r"traffic_bytes_per_launch\[([^\]]+)\]:\s*(\d+)", line.strip())
+            if m and m.group(1) == key:
                 return int(m.group(2))
     except OSError:
         pass
@@ -204,7 +205,8 @@ def main():
         step_ops = 2.0 * B * 3 * c["H"] * (c["k"] * c["F"] + c["Fs"])
         roofline = {"bound": "hbm", "kernel": "q32s_up (routed w1, w3, SiLU, Q8_0 re-quantisation; lists beyond 32 rows re-read the weights from L2)",
                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                    "traffic": None, "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+                    "traffic": measured_traffic(B, "q32s_config4_kernel_trace.md", "config4") if B == 512 else None,
+                    "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
         workload = ("BASELINE config 4: hidden 2048, 60 experts of ffn 1408, top-4 renormalised, shared expert of ffn 5632 "
                     "with sigmoid gate, Q8_0 weights, %d tokens" % B)
         extra = {"step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
