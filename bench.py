@@ -10,6 +10,8 @@ activations already resident in HBM.  Prints ONE JSON line.
 
 `--workload prefill` measures BASELINE config 3 instead (same layer, 4096 tokens, router bias that makes
 the expert load follow Zipf(1)); its roofline object is the int8-MFMA one of the tiled up kernel.
+`--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with
+another GGML format (random block payloads with small finite scales: timing does not depend on the values).
 `--workload config4` measures BASELINE config 4 (hidden 2048, 60 experts of FFN 1408, top-4, one always-on
 shared expert of FFN 5632 behind a sigmoid gate, Q8_0 weights, 512 tokens); its line carries the time of the
 dispatch (histogram, scan, permutation) beside the other stages.
@@ -27,6 +29,10 @@ sys.path.insert(0, ROOT)
 
 H, F, E, TOPK = 4096, 14336, 8, 2
 Q4K, Q8_0 = 12, 8
+# other weight formats for the decode workload: name -> (GGML dtype, block elements, block bytes, offsets of the f16 scale fields)
+FORMATS = {"q4_k": (12, 256, 144, (0, 2)), "q4_0": (2, 32, 18, (0,)), "q4_1": (3, 32, 20, (0, 2)), "q5_0": (6, 32, 22, (0,)),
+           "q5_1": (7, 32, 24, (0, 2)), "q8_0": (8, 32, 34, (0,)), "q2_k": (10, 256, 84, (80, 82)), "q3_k": (11, 256, 110, (108,)),
+           "q5_k": (13, 256, 176, (0, 2)), "q6_k": (14, 256, 210, (208,))}
 CFG4 = dict(H=2048, F=1408, E=60, k=4, Fs=5632)   # BASELINE config 4
 EXPERT_BYTES = 3 * H * F * 144 // 256          # 99,090,432 B of Q4_K blocks per expert
 HBM_PEAK_GBS = 8000.0                          # MI355X HBM3E, published
@@ -35,14 +41,32 @@ INT8_PEAK_TOPS = 5000.0                        # MI355X dense int8 MFMA, publish
 ZIPF_BIAS = [0.0, -1.158, -1.581, -1.845, -2.033, -2.186, -2.299, -2.398]
 
 
-def build_layer(torch, candle_amd, seed=0, gate_bias=None, cfg4=False):
+def random_blocks(np, rng, fmt, n_elems):
+    """Raw GGML blocks with random payloads; the f16 scale fields are set to 0.001 so that every value is finite."""
+    _, be, bb, scale_at = FORMATS[fmt]
+    raw = rng.integers(0, 256, (n_elems // be, bb), dtype=np.uint8)
+    d = int(np.float16(0.001).view(np.uint16))
+    for o in scale_at:
+        raw[:, o] = d & 255
+        raw[:, o + 1] = d >> 8
+    return raw.reshape(-1)
+
+
+def build_layer(torch, candle_amd, seed=0, gate_bias=None, cfg4=False, fmt="q4_k"):
     """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel
     (bit-identical to candle's CPU quantiser), kept as host bytes for the CPU baseline too."""
     h, f, e_n, k, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, TOPK, Q4K, 0)
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
 
+    if fmt != "q4_k" and not cfg4:
+        import numpy as np
+        dt = FORMATS[fmt][0]
+        rng = np.random.default_rng(seed)
+
     def draw(shape):
+        if fmt != "q4_k" and not cfg4:
+            return random_blocks(np, rng, fmt, shape[0] * shape[1])
         x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
         return candle_amd.quantize_weights(dt, x).cpu().numpy()
 
@@ -73,7 +97,7 @@ def hip_events():
     return hip
 
 
-def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=False):
+def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=False, dt=Q4K):
     """candle's CPU path restated (the oracle: serial rows, columns threaded, AVX2 inner loops of
     candle's x86 build) on all host cores: the same batch, same weight bytes, same routing,
     repeated until `min_seconds` of wall time have passed."""
@@ -86,7 +110,7 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg
         layer = O.Layer(CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, gate, w["w1"], w["w3"], w["w2"], Fs=CFG4["Fs"],
                         sw1=w["shared"][0], sw3=w["shared"][1], sw2=w["shared"][2], shared_gate=w["shared_gate"])
     else:
-        layer = O.Layer(H, F, E, TOPK, Q4K, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+        layer = O.Layer(H, F, E, TOPK, dt, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
     layer.forward(xs_host[:1], logits=logits_host[:1], simd=True, threads=cores)  # warm the pages
     reps, t0 = 0, time.perf_counter()
     while True:
@@ -122,6 +146,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill, 512 for config4)")
     ap.add_argument("--workload", choices=("decode", "prefill", "config4"), default="decode")
+    ap.add_argument("--weights", choices=sorted(FORMATS), default="q4_k", help="GGML format of the expert matrices (decode workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
@@ -150,7 +175,10 @@ def main():
     cfg4 = args.workload == "config4"
     B = args.batch or (4096 if prefill else 512 if cfg4 else 32)
     bias = np.array(ZIPF_BIAS, dtype=np.float32) if prefill else None
-    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias, cfg4=cfg4)
+    if args.weights != "q4_k" and args.workload != "decode":
+        sys.exit("bench.py: --weights applies to the decode workload only")
+    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias, cfg4=cfg4, fmt=args.weights)
+    fmt_dt, fmt_be, fmt_bb, _ = FORMATS[args.weights]
     n_exp, hid = (CFG4["E"], CFG4["H"]) if cfg4 else (E, H)
     g = torch.Generator(device="cuda")
     g.manual_seed(2)
@@ -191,7 +219,8 @@ def main():
                 stage[k] += v / args.stage_iters
     stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
 
-    step_bytes = n_active * EXPERT_BYTES + E * H * 4 + 2 * B * H * 4
+    expert_bytes = 3 * H * F * fmt_bb // fmt_be
+    step_bytes = n_active * expert_bytes + E * H * 4 + 2 * B * H * 4
     metric = "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, %s)" % args.workload
     if cfg4:
         # Weights are Q8_0 (34 bytes per 32 elements); every routed expert with a token and the shared expert are
@@ -233,13 +262,18 @@ def main():
         # Roofline of the dominant kernel, the up projection (w1, w3 + SiLU): it streams w1 and w3 of
         # every active expert exactly once per launch; algorithmic bytes = Q4_K bytes of those matrices
         # plus the quantised activations it reads and the quantised intermediate it writes.
-        up_bytes = n_active * (2 * H * F * 144 // 256) + B * (H + H // 256 * 36) + B * TOPK * (F + F // 256 * 36)
+        act = 36 / 256 if fmt_be == 256 else 8 / 32    # bytes of scales and sums per quantised activation element
+        up_bytes = n_active * (2 * H * F * fmt_bb // fmt_be) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
         achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)", "achieved": achieved,
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                    "traffic": measured_traffic(B),
+        q4k = args.weights == "q4_k"
+        roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)" if q4k else "up projection (w1, w3, SiLU, re-quantisation), %s" % args.weights,
+                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": measured_traffic(B) if q4k else None,
                     "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
         workload = "BASELINE config 2: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, decode batch %d" % B
+        if not q4k:
+            workload = "BASELINE config 2's layer with %s weights (random block payloads), decode batch %d" % (args.weights, B)
+            metric = "MoE layer tokens/s (Mixtral-8x7B shape, %s, decode)" % args.weights
         extra = {"step_algorithmic_bytes": step_bytes,
                  "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
     out = {
@@ -257,7 +291,7 @@ def main():
         # a bounded sample: the CPU path does ~1 k tokens/s, so a prefill batch is cut to its first 64 tokens
         n_cpu = min(B, 64)
         out["cpu_baseline"] = cpu_baseline(gate, w, xs[0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu],
-                                           args.cpu_seconds, gate_bias=bias, cfg4=cfg4)
+                                           args.cpu_seconds, gate_bias=bias, cfg4=cfg4, dt=fmt_dt)
     print(json.dumps(out))
 
 
