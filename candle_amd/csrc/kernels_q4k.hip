@@ -364,39 +364,60 @@ __device__ inline Q3KTile load_q3k_tile(const uint8_t* tile, int lane) {
     t.d = __builtin_nontemporal_load(reinterpret_cast<const __attribute__((address_space(1))) uint16_t*>((gbytes)tile + 1792u + (uint32_t)(lane & 15) * 2u));
     return t;
 }
-__device__ inline void q3k_mac(const Q3KTile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) {
+// The scale of a 16-element group goes into the weight operand, as for Q4K with several slot tiles: a lane's eight
+// codes of a 32-element stretch lie in one group, so the lane knows its scale.  sc * (code - 4) can reach +128, one too
+// many for a byte; instead sc + 32 = 8 hi + lo (3-bit digits) multiplies the unsigned code (<= 49 per plane) and the
+// plain codes form a third plane:
+//     sum sc (code - 4) a = 8 P_hi + P_lo - 32 P_code - 4 sum_j sc_j bsum_j
+// (the last term the exact f16 MFMA over the 16-element sums as before).  Twelve v_mfma_i32_16x16x64_i8 per tile and
+// slot tile instead of sixteen half-masked 16x16x32 ones, and no integer multiply-add per result and group.
+struct Q3KPlanes {
+    v4i hi[4], lo[4], code[4];
+    float d;
+    v4h sB;
+};
+__device__ inline Q3KPlanes q3k_planes(const Q3KTile& w, int g) {
     const uint32_t M3 = 0x03030303u, M1 = 0x01010101u;
-    const float d = __half2float(__ushort_as_half((unsigned short)w.d));
-    const uint32_t first = g < 2 ? 0xffffffffu : 0u, second = ~first;
-    const v4i zero = {0, 0, 0, 0};
-    v4i isum = {0, 0, 0, 0};
+    Q3KPlanes pl;
+    pl.d = __half2float(__ushort_as_half((unsigned short)w.d));
     const uint32_t qw[4] = {w.q.x, w.q.y, w.q.z, w.q.w};
     const uint32_t sw[4] = {w.sc.x, w.sc.y, w.sc.z, w.sc.w};
+    const int half = g < 2 ? 0 : 8;   // which group of its stretch this lane's codes belong to
 #pragma unroll
     for (int P = 0; P < 4; P++) {
         const uint32_t q = qw[P], h = (P < 2 ? w.qh.x : w.qh.y) >> (4 * (P & 1));
         const uint32_t lx = (q & M3) | ((h & M1) << 2), ly = ((q >> 2) & M3) | (((h >> 1) & M1) << 2);
         const uint32_t hx = ((q >> 4) & M3) | (((h >> 2) & M1) << 2), hy = ((q >> 6) & M3) | (((h >> 3) & M1) << 2);
-        const long a_lo = pack64(A.a[P].x, A.a[P].y);
-        const long a_hi = pack64(A.a[P].z, A.a[P].w);
-        v4i D0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & first, ly & first), zero, 0, 0, 0);
-        v4i D1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_lo, pack64(lx & second, ly & second), zero, 0, 0, 0);
-        v4i D2 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & first, hy & first), zero, 0, 0, 0);
-        v4i D3 = __builtin_amdgcn_mfma_i32_16x16x32_i8(a_hi, pack64(hx & second, hy & second), zero, 0, 0, 0);
-        const int s0 = (int)(int8_t)(sw[P] & 0xffu), s1 = (int)(int8_t)((sw[P] >> 8) & 0xffu);
-        const int s2 = (int)(int8_t)((sw[P] >> 16) & 0xffu), s3 = (int)(int8_t)(sw[P] >> 24);
-#pragma unroll
-        for (int i = 0; i < 4; i++) isum[i] += __mul24(s0, D0[i]) + __mul24(s1, D1[i]) + __mul24(s2, D2[i]) + __mul24(s3, D3[i]);
+        // stored scale - 32 was decoded at re-lay time; + 32 gives back the unsigned 6-bit value
+        const uint32_t s_lo = (uint32_t)((int)(int8_t)((sw[P] >> half) & 0xffu) + 32);
+        const uint32_t s_hi = (uint32_t)((int)(int8_t)((sw[P] >> (16 + half)) & 0xffu) + 32);
+        pl.hi[P] = v4i{(int)digit_times_codes(lx, s_lo >> 3), (int)digit_times_codes(ly, s_lo >> 3),
+                       (int)digit_times_codes(hx, s_hi >> 3), (int)digit_times_codes(hy, s_hi >> 3)};
+        pl.lo[P] = v4i{(int)digit_times_codes(lx, s_lo & 7u), (int)digit_times_codes(ly, s_lo & 7u),
+                       (int)digit_times_codes(hx, s_hi & 7u), (int)digit_times_codes(hy, s_hi & 7u)};
+        pl.code[P] = v4i{(int)lx, (int)ly, (int)hx, (int)hy};
     }
     const uint32_t sg = sw[g];
-    const v4h sB = {(_Float16)(int)(int8_t)(sg & 0xffu), (_Float16)(int)(int8_t)((sg >> 8) & 0xffu),
-                    (_Float16)(int)(int8_t)((sg >> 16) & 0xffu), (_Float16)(int)(int8_t)(sg >> 24)};
+    pl.sB = v4h{(_Float16)(int)(int8_t)(sg & 0xffu), (_Float16)(int)(int8_t)((sg >> 8) & 0xffu),
+                (_Float16)(int)(int8_t)((sg >> 16) & 0xffu), (_Float16)(int)(int8_t)(sg >> 24)};
+    return pl;
+}
+__device__ inline void q3k_mac(const Q3KPlanes& pl, const Q8KOperand& A, const float yd[4], float acc[4]) {
+    const v4i zero = {0, 0, 0, 0};
+    v4i p_hi = zero, p_lo = zero, p_c = zero;
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const v4i a = {(int)A.a[P].x, (int)A.a[P].y, (int)A.a[P].z, (int)A.a[P].w};
+        p_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.hi[P], p_hi, 0, 0, 0);
+        p_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.lo[P], p_lo, 0, 0, 0);
+        p_c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.code[P], p_c, 0, 0, 0);
+    }
     const v4f zf = {0.f, 0.f, 0.f, 0.f};
-    v4f Ds = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, sB, zf, 0, 0, 0);
+    v4f Ds = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, pl.sB, zf, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int tot = isum[i] - 4 * (int)Ds[i];
-        acc[i] += (d * yd[i]) * (float)tot;
+        const int tot = 8 * p_hi[i] + p_lo[i] - 32 * p_c[i] - 4 * (int)Ds[i];   // exact: |tot| < 2^28
+        acc[i] += (pl.d * yd[i]) * (float)tot;
     }
 }
 
@@ -427,8 +448,8 @@ struct FmtQ3K {
     typedef Q3KTile Tile;
     static constexpr int TILE_BYTES = Q3K_TILE_BYTES;
     static __device__ inline Tile load(const uint8_t* tile, int lane) { return load_q3k_tile(tile, lane); }
-    static __device__ inline const Tile& prepare(const Tile& w, int) { return w; }
-    static __device__ inline void mac(const Tile& w, const Q8KOperand& A, const float yd[4], int g, float acc[4]) { q3k_mac(w, A, yd, g, acc); }
+    static __device__ inline Q3KPlanes prepare(const Tile& w, int g) { return q3k_planes(w, g); }
+    static __device__ inline void mac(const Q3KPlanes& pl, const Q8KOperand& A, const float yd[4], int, float acc[4]) { q3k_mac(pl, A, yd, acc); }
 };
 struct FmtQ5K {
     typedef Q5KTile Tile;
