@@ -429,6 +429,9 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     }
     if (shared) {
         ExpertParams sp = ep;
+        // the always-on expert takes the regular kernels (which quantise its intermediate in their epilogue) also when
+        // the routed experts of a tiny batch took the narrow ones with their separate quantisation pass
+        sp.hbuf = nullptr; sp.by_assignment = 0;
         sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
         sp.groups = L->groups.as<GroupWeights>() + L->E;
         sp.hq = L->hq_shared.view(); sp.slot_origin = (int)(T * L->k);

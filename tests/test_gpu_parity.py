@@ -280,6 +280,20 @@ def test_block_q6k_and_mixed_down_dtype(dt, dt_down):
     gpu.close()
 
 
+@pytest.mark.parametrize("dt", [O.Q4K, O.Q6K, O.Q2K])
+def test_block_kquant_shared_expert_tiny_batches(dt):
+    # at most E assignments: the routed experts take the narrow kernels (f32 intermediate, separate quantisation pass),
+    # the always-on expert the regular ones
+    ref, gpu = make_pair(512, 512, 8, 2, dt, seed=14, Fs=1024)
+    for T in (1, 2, 4):
+        check_block(ref, gpu, T, tol=block_tol(O.Q4K, 512))
+    gpu.close()
+    ref, gpu = make_pair(768, 768, 8, 1, dt, seed=15, Fs=1536)
+    for T in (1, 8):
+        check_block(ref, gpu, T, tol=block_tol(O.Q4K, 768))
+    gpu.close()
+
+
 def test_block_q6k_shared_expert():
     ref, gpu = make_pair(512, 512, 8, 2, O.Q4K, seed=13, Fs=1024, dt_down=O.Q6K)
     for T in (5, 40, 70):
