@@ -1,0 +1,65 @@
+"""Randomised parity sweep (fixed seeds): layer shapes, expert counts, formats, mixed up / down formats, shared expert,
+rms-norm and batch sizes drawn at random, each compared with the oracle like the hand-picked cases.  It exists because
+such a sweep found what those cases had missed (a K-quant layer with a shared expert at a batch of one or two tokens)."""
+import random
+
+import numpy as np
+import pytest
+
+import candle_amd
+import pyoracle as O
+from helpers import activations, make_pair, rms
+from test_gpu_parity import TOL, bits, check_block
+
+pytestmark = pytest.mark.gpu
+
+KQ = [O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K]
+Q80 = [O.Q4_0, O.Q5_0, O.Q8_0]   # formats with Q8_0 activations
+Q81 = [O.Q4_1, O.Q5_1]           # ... with Q8_1 activations
+
+
+@pytest.mark.parametrize("seed", [2, 3])
+def test_random_layers(seed):
+    rnd = random.Random(seed)
+    for case in range(30):
+        fam = rnd.choice(["k", "k", "80", "81"])
+        if fam == "k":
+            dt, dtd, mult = rnd.choice(KQ), rnd.choice(KQ + [None, None]), 256
+            H, F = 256 * rnd.choice([1, 2, 3, 4]), 256 * rnd.choice([1, 2, 3, 5])
+        else:
+            pool = Q80 if fam == "80" else Q81
+            dt, dtd, mult = rnd.choice(pool), rnd.choice(pool + [None]), 32
+            H, F = 32 * rnd.choice([1, 3, 4, 5, 8, 12, 16]), 32 * rnd.choice([1, 2, 4, 5, 8, 11, 16, 20])
+        E = rnd.choice([1, 2, 3, 4, 8, 13, 32, 60])
+        k = rnd.choice([kk for kk in (1, 2, 4, 6) if kk <= E])
+        Fs = rnd.choice([0, 0, F, 2 * F])
+        rmsn, norm = rnd.random() < 0.2, rnd.random() < 0.8
+        Ts = sorted(set(rnd.choice([1, 2, 3, 5, 8, 16, 17, 31, 33, 40, 64, 70, 100, 129, 200, 300, 520, 1100]) for _ in range(3)))
+        ref, gpu = make_pair(H, F, E, k, dt, seed=1000 + case, Fs=Fs, rms=rmsn, norm_topk=norm, dt_down=dtd)
+        # one flipped re-quantised value weighs more the narrower the intermediate (see block_tol in test_gpu_parity)
+        tol = TOL * max(1.0, float(np.sqrt((14336.0 if mult == 256 else 4096.0) / F)))
+        for T in Ts:
+            try:
+                check_block(ref, gpu, T, seed=case, tol=tol)
+            except AssertionError as e:
+                raise AssertionError("case %r: %s" % (dict(dt=dt, dtd=dtd, H=H, F=F, E=E, k=k, Fs=Fs, rms=rmsn, norm=norm, T=T), e))
+        gpu.close()
+
+
+def test_random_dense_projections():
+    rnd = random.Random(1)
+    for case in range(50):
+        dt = rnd.choice(Q80 + Q81 + KQ)
+        be = O.BLOCK_ELEMS[dt]
+        n = 16 * rnd.choice([1, 2, 3, 5, 8, 17, 32, 64, 100, 256])
+        k = be * rnd.choice([1, 2, 3, 4, 5, 8, 11, 16] if be == 32 else [1, 2, 3, 4, 6])
+        w = O.fill_normal_quantized(case + 7, dt, n, k, 0.02)
+        lin = candle_amd.QMatMul(dt, w, n, k)
+        for m in sorted(set(rnd.choice([1, 2, 7, 16, 17, 32, 33, 48, 64, 65, 96, 130, 300, 700]) for _ in range(4))):
+            x = activations(m, k, seed=case * 31 + m)
+            got, want = lin.forward(x), O.matmul(dt, x, w, n)
+            if be == 32:   # same block values added in the reference's order
+                assert np.array_equal(bits(got), bits(want)), (dt, n, k, m)
+            else:
+                assert np.abs(got - want).max() <= 1e-4 * rms(want), (dt, n, k, m)
+        lin.close()
