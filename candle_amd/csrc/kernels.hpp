@@ -77,6 +77,7 @@ struct ExpertParams {
     // instead of experts, workgroup row y serves the expert of assignment y unless an earlier assignment names the
     // same expert.  No workgroups (and no weight prefetches) for experts without tokens.
     int by_assignment = 0;
+    int down_interleaved = 0;   // down projection: wave w of a workgroup takes super-blocks w, w + NW, ... instead of a contiguous range
     float* hbuf = nullptr;          // tiled path only: f32 intermediate [slots, F] before re-quantisation
     int64_t n_slots = 0;            // tiled path only: total slots (bounds the tile grid)
 };

@@ -490,13 +490,13 @@ __device__ inline void q4k_engine_prefetch(const uint8_t* const tp[NT], size_t s
 // past the end multiplies its surplus super-blocks by a zero activation scale.
 template <class FMT, int TT, int NT, int RING>
 __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride, typename FMT::Tile t[RING], const ActBuf& ab, int K, int nsb,
-                                  int sb_lo, int sb_hi, const int rowA[TT], int lane, int g, float acc[NT][TT][4]) {
+                                  int sb_lo, int sb_hi, const int rowA[TT], int lane, int g, float acc[NT][TT][4], int a_step = 1, int a_off = 0) {
     static_assert(NT % RING == 0 || RING % NT == 0, "ring must divide, or be a multiple of, the tiles per super-block");
     constexpr int U = RING > NT ? RING / NT : 1;   // super-blocks per trip
     if (sb_lo >= sb_hi) return;
     Q8KOperand A[TT];
 #pragma unroll
-    for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_lo, rowA[tt], g);
+    for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_lo * a_step + a_off, rowA[tt], g);
     // The loop body is one basic block: prefetches past the end are redirected to the last
     // super-block (a harmless repeated load) instead of being branched around, so that the
     // scheduling fences below really bound the live ranges.
@@ -530,7 +530,7 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride,
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next, rowA[tt], g);
+            for (int tt = 0; tt < TT; tt++) A[tt] = load_q8k_operand(ab, K, nsb, sb_next * a_step + a_off, rowA[tt], g);
         }
     }
 }
@@ -645,10 +645,21 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
         int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;  // tiles past the last row are computed and dropped
         tp[j] = w2 + (size_t)rt * FMT::TILE_BYTES;
     }
-    const size_t sb_stride = (size_t)n_rt * FMT::TILE_BYTES;
-    const int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
+    size_t sb_stride = (size_t)n_rt * FMT::TILE_BYTES;
+    int sb_lo = (int)((int64_t)nsb * wave / NW), sb_hi = (int)((int64_t)nsb * (wave + 1) / NW);
+    int a_step = 1, a_off = 0;
+    const bool ILV = p.down_interleaved != 0;
+    if (ILV) {   // wave w takes super-blocks w, w + NW, ...: the waves of a workgroup read neighbouring slabs of the matrix
+        const int mine = wave < nsb ? (nsb - wave + NW - 1) / NW : 0;
+        a_step = NW; a_off = mine ? wave : 0;
+#pragma unroll
+        for (int j = 0; j < NTD; j++) tp[j] += (size_t)a_off * sb_stride;
+        sb_stride *= NW;
+        sb_lo = 0; sb_hi = mine;
+    }
     typename FMT::Tile ring[RING];
-    q4k_engine_prefetch<FMT, NTD, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, sb_hi > sb_lo ? sb_hi - 1 : (sb_lo < nsb ? sb_lo : nsb - 1), lane, ring);
+    if (ILV) q4k_engine_prefetch<FMT, NTD, RING>(tp, sb_stride, 0, sb_hi > 0 ? sb_hi - 1 : 0, lane, ring);
+    else q4k_engine_prefetch<FMT, NTD, RING>(tp, sb_stride, sb_lo < nsb ? sb_lo : nsb - 1, sb_hi > sb_lo ? sb_hi - 1 : (sb_lo < nsb ? sb_lo : nsb - 1), lane, ring);
 
     const GroupSlots gs = group_slots<NW * 64>(p, grp, list_lds, wtot_lds);
     const int tg0 = blockIdx.z * (TT * 16);
@@ -668,7 +679,7 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<FMT, TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc);
+    q4k_engine<FMT, TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc, a_step, a_off);
 
 #pragma unroll
     for (int j = 0; j < NTD; j++)
@@ -810,8 +821,11 @@ hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s) {
-    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
+hipError_t launch_q4k_down(const ExpertParams& p_in, hipStream_t s) {
+    if (p_in.max_rows == 0 || p_in.n_groups == 0) return hipSuccess;
+    static const int ilv = variant("MOE_DOWN_ILV", 1);
+    ExpertParams p = p_in;
+    p.down_interleaved = ilv;
     const int dtd = p.dt_down ? p.dt_down : p.dt;
     const KernelFamily* f = kernel_family(dtd);
     if (!f) return hipErrorInvalidValue;
