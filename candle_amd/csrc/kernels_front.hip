@@ -256,15 +256,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     const float* x = p.x + t * H;
 
     // ---- load the row (and normalise it if the layer carries the pre-norm)
-    float sum2 = 0.f;
-    for (int h = tid * 4; h < H; h += FRONT_THREADS * 4) {
-        float4 v = *reinterpret_cast<const float4*>(x + h);
-        *reinterpret_cast<float4*>(xrow + h) = v;
-        sum2 += v.x * v.x;
-        sum2 += v.y * v.y;
-        sum2 += v.z * v.z;
-        sum2 += v.w * v.w;
-    }
+    for (int h = tid * 4; h < H; h += FRONT_THREADS * 4) *reinterpret_cast<float4*>(xrow + h) = *reinterpret_cast<const float4*>(x + h);
     if (p.rms_alpha) {
         // sum of squares left to right, as the reference does (see front_fast_kernel)
         __syncthreads();

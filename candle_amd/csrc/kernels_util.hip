@@ -364,7 +364,7 @@ __global__ void dequant_tiled_kernel(int dt, const uint8_t* tiled, float* out, i
     int64_t rt = row / 16;
     int r = (int)(row % 16);
     if (dt == MOE_GGML_Q4K) {
-        int nsb = (int)(k / 256), sb = col / 256, e = col % 256;
+        int sb = col / 256, e = col % 256;
         const uint8_t* tile = tiled + ((int64_t)sb * (rows / 16) + rt) * Q4K_TILE_BYTES;
         // original qs byte index of element e: (e/64)*32 + e%32 ; that byte sits in pair P = byte/32,
         // chunk g = (byte%32)/8, position byte%8
