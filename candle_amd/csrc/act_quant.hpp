@@ -58,6 +58,55 @@ __device__ inline void quantize_q8k_block(float4 v, int lane, int8_t* qs_block, 
     if (lane == 0) *d_out = 1.0f / iscale;
 }
 
+// N blocks at once, lane l holding elements 4l..4l+3 of each: the arithmetic of quantize_q8k_block without its
+// branch, so that the N chains of wave reductions and the divisions overlap instead of running one after the other
+// (the epilogue of the up projection, where nothing else hides their latency).  Blocks with valid[n] == false are
+// computed and not stored.
+template <int N>
+__device__ inline void quantize_q8k_blocks(const float4 (&v)[N], const bool (&valid)[N], int lane, int8_t* const (&qs_block)[N],
+                                           float* const (&d_out)[N], __half* const (&bs_out)[N]) {
+    float amax[N], mx[N], wmax[N], iscale[N];
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+        const float e[4] = {v[n].x, v[n].y, v[n].z, v[n].w};
+        amax[n] = 0.f; mx[n] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float a = fabsf(e[i]);
+            if (amax[n] < a) { amax[n] = a; mx[n] = e[i]; }
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < N; n++) wmax[n] = wave_max(amax[n]);
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+        const unsigned long long winners = __ballot(amax[n] == wmax[n]);
+        const int first = __ffsll((long long)winners) - 1;
+        const float max = __shfl(mx[n], first, 64);
+        iscale[n] = wmax[n] == 0.f ? 0.f : -128.0f / max;   // an all-zero block quantises to zeros with d = 0
+    }
+#pragma unroll
+    for (int n = 0; n < N; n++) {
+        const float e[4] = {v[n].x, v[n].y, v[n].z, v[n].w};
+        int sum = 0;
+        uint32_t packed = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float r = roundf(iscale[n] * e[i]);
+            const int q = sat_i8(fminf(r, 127.f));
+            sum += q;
+            packed |= (uint32_t)(uint8_t)q << (8 * i);
+        }
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        if (valid[n]) {
+            *reinterpret_cast<uint32_t*>(qs_block[n] + q8k_act_offset(4 * lane)) = packed;
+            if ((lane & 3) == 0) bs_out[n][lane >> 2] = __int2half_rn(sum);
+            if (lane == 0) *d_out[n] = wmax[n] == 0.f ? 0.f : 1.0f / iscale[n];
+        }
+    }
+}
+
 // The word kept beside a 32-element activation block.  Q8_0: the sum of the block's quants (the -8 / -16 code
 // offsets of Q4_0 / Q5_0 weights leave through it).  Q8_1: the block's `s` widened to f32, s = f16(sum) * d in
 // binary16 arithmetic (two 11-bit significands: the f32 product is exact, so one rounding to f16 remains).

@@ -128,7 +128,14 @@ __device__ inline void q45k_mac(const uint4& q0, const uint4& q1, const uint4& s
         const int s0 = (int)((scw >> (16 * (P & 1))) & 0xffu);
         const int s1 = (int)((scw >> (16 * (P & 1) + 8)) & 0xffu);
 #pragma unroll
-        for (int i = 0; i < 4; i++) isum[i] += __mul24(s0, D0[i]) + __mul24(s1, D1[i]);
+        for (int i = 0; i < 4; i++) {
+            // one v_mad_i32_i24 per product: the empty asm keeps the compiler from regrouping the two into two
+            // multiplies and a three-way add (1.5 instructions per product)
+            isum[i] += __mul24(s0, D0[i]);
+            asm("" : "+v"(isum[i]));
+            isum[i] += __mul24(s1, D1[i]);
+            asm("" : "+v"(isum[i]));
+        }
     }
     // mins term: sum_k bsum16[slot][k] * m[row][k/2], k = 0..15, as an exact f16 MFMA; this lane
     // supplies k = 4g..4g+3, i.e. sub-blocks 2g and 2g+1
@@ -616,13 +623,24 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
                 hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
     __syncthreads();
     const int nfb = F / 256;
-    for (int tok = wave; tok < TT * 16; tok += NW) {
-        if (tg0 + tok >= gs.n) break;
-        float4 v = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
-        int64_t hrow = gs.slot(tg0 + tok) - p.slot_origin;
-        quantize_q8k_block(v, lane, p.hq.qs + hrow * F + rb * 256, p.hq.d + hrow * nfb + rb,
-                           reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16);
+    // every wave quantises its TT*16/NW tokens side by side
+    constexpr int NQ = TT * 16 / NW;
+    float4 v[NQ];
+    bool valid[NQ];
+    int8_t* qs_out[NQ];
+    float* d_out[NQ];
+    __half* bs_out[NQ];
+#pragma unroll
+    for (int n = 0; n < NQ; n++) {
+        const int tok = wave + n * NW;
+        valid[n] = tg0 + tok < gs.n;
+        v[n] = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
+        const int64_t hrow = gs.slot(valid[n] ? tg0 + tok : gs.n - 1) - p.slot_origin;
+        qs_out[n] = p.hq.qs + hrow * F + rb * 256;
+        d_out[n] = p.hq.d + hrow * nfb + rb;
+        bs_out[n] = reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16;
     }
+    quantize_q8k_blocks<NQ>(v, valid, lane, qs_out, d_out, bs_out);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -688,8 +706,13 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
 #pragma unroll
             for (int i = 0; i < 4; i++) part[wave][(j * TT + tt) * 4 + i][lane] = acc[j][tt][i];
     __syncthreads();
-    // NTD*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ...
-    for (int v = wave; v < NTD * TT * 4; v += NW) {
+    // NTD*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ... (a fixed trip count, so that the routing
+    // weights of all its planes are fetched together rather than one per trip)
+    constexpr int NPL = NTD * TT * 4;
+#pragma unroll
+    for (int n = 0; n < (NPL + NW - 1) / NW; n++) {
+        const int v = wave + n * NW;
+        if (NPL % NW != 0 && v >= NPL) break;
         float sum = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; w++) sum += part[w][v][lane];
