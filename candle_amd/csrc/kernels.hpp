@@ -40,6 +40,7 @@ struct FrontParams {
     const float* shared_gate = nullptr; // [H] or null
     const float* rms_alpha = nullptr;   // [H] or null
     float rms_eps = 0.f;
+    int rms_serial = 0;                 // 1: the fast kernel adds the squares of a row term by term (checks the chunked evaluation)
     int vdt = MOE_GGML_Q8K;             // activation format
     ActBuf xq;                          // token-indexed quantised activations (output)
     RouteBufs rb;

@@ -422,6 +422,114 @@ __device__ inline void quantize_chunk(const FrontParams& p, int64_t t, int H, in
     }
 }
 
+// Sum of the squares of a row in the reference's order: ((x0^2 + x1^2) + x2^2) + ..., every product and every
+// partial sum rounded to f32 (candle-nn/src/ops.rs:504-515 folds the row with `sum::<f32>()`).  Taken literally that is
+// a chain of H dependent adds, ten cycles each for a lone wave (20 us at H = 4096).  The chain is cut into 64 chunks:
+// while a running sum S = k * u (k its 24-bit significand, u its ulp) stays inside one binade, adding a term v moves
+// k by round-to-nearest-even(v / u), i.e. by floor(v / u), plus one if the fraction exceeds 1/2, plus the parity of the
+// result if the fraction is exactly 1/2.  Such steps compose: a run of them maps k to k + (k even ? a0 : a1), and two
+// runs compose into a pair of the same kind.  Every chunk is summarised this way in parallel for the binade that an
+// approximate prefix sum predicts for it; one wave then walks the chunks with the exact running sum and takes the
+// summary when the sum enters the chunk in the predicted binade and leaves it in the same one (the partial sums only
+// grow, so the end decides), and adds the chunk term by term otherwise (chunk 0, binade crossings, NaN / overflow: a
+// handful of chunks per row).  Either way the bits equal those of the term-by-term sum.  Call with all FAST_THREADS
+// threads; every wave holds the row (xr[4 i + j] = x[256 i + 4 lane + j]); `serial_only` adds every chunk term by term.
+template <int NCH>
+__device__ inline float ordered_sum_of_squares(const float* xr, int tid, bool serial_only) {
+    constexpr int L = NCH * 4, LP = L + 1;     // chunk length; chunks are padded by one word so that lanes reading
+    __shared__ float sqp[64 * LP];             // the same position of 64 chunks hit 64 different banks
+    __shared__ int part[8][64][2];
+    __shared__ float result;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr bool kSummaries = NCH >= 4 && NCH % 2 == 0;
+    const bool summaries = kSummaries && !serial_only;
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+        if ((i & 7) == wave) {
+            const int idx = i * 256 + lane * 4;
+            float* d = sqp + idx + idx / L;
+            d[0] = xr[4 * i] * xr[4 * i]; d[1] = xr[4 * i + 1] * xr[4 * i + 1];
+            d[2] = xr[4 * i + 2] * xr[4 * i + 2]; d[3] = xr[4 * i + 3] * xr[4 * i + 3];
+        }
+    __syncthreads();
+    const float* mine = sqp + lane * LP;
+    int e = 0;   // biased exponent predicted for the running sum at the start of chunk `lane`; 0 = no summary
+    if (summaries) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+        for (int j = 0; j < L; j += 4) { s0 += mine[j]; s1 += mine[j + 1]; s2 += mine[j + 2]; s3 += mine[j + 3]; }
+        float incl = (s0 + s1) + (s2 + s3);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const float o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        const float excl = __shfl_up(incl, 1, 64);
+        const int eb = (int)(__float_as_uint(excl) >> 23);
+        // 1 / u = 2^(150 - eb) has to be a normal float
+        if (lane > 0 && eb >= 23 && eb <= 254) e = eb;
+        int a0 = 0, a1 = 0;
+        if (e) {
+            const float inv_u = __uint_as_float((uint32_t)(277 - e) << 23);
+#pragma unroll
+            for (int jj = 0; jj < L / 8; jj++) {
+                float sc = mine[wave * (L / 8) + jj] * inv_u;   // a power of two: exact
+                if (!(sc < 16777216.f)) sc = 16777216.f;         // too large for this binade (or NaN): the end test fails
+                const float q = floorf(sc), f = sc - q;
+                const int n = (int)q + (f > 0.5f ? 1 : 0);
+                const bool tie = f == 0.5f;
+                a0 += n + (tie ? ((a0 + n) & 1) : 0);
+                a1 += n + (tie ? ((1 + a1 + n) & 1) : 0);
+            }
+        }
+        part[wave][lane][0] = a0;
+        part[wave][lane][1] = a1;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int a0 = 0, a1 = 0;
+        if (summaries) {
+            a0 = part[0][lane][0]; a1 = part[0][lane][1];
+#pragma unroll
+            for (int w = 1; w < 8; w++) {
+                const int b0 = part[w][lane][0], b1 = part[w][lane][1];
+                a0 += (a0 & 1) ? b1 : b0;
+                a1 += ((1 + a1) & 1) ? b1 : b0;
+                a0 = a0 < (1 << 25) ? a0 : (1 << 25);   // anything from 2^24 on fails the end test; keeps the sums in range
+                a1 = a1 < (1 << 25) ? a1 : (1 << 25);
+            }
+        }
+        // bits of the first float of the predicted binade; all ones where the chunk has no summary
+        const uint32_t lo_v = e ? (uint32_t)e << 23 : 0xffffffffu;
+        uint32_t b = 0;   // bits of the running sum, the same in every lane
+        for (int c = 0; c < 64; c++) {
+            const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)lo_v, c);
+            const uint32_t s0 = (uint32_t)__builtin_amdgcn_readlane(a0, c), s1 = (uint32_t)__builtin_amdgcn_readlane(a1, c);
+            const uint32_t nb = b + ((b & 1u) ? s1 : s0);   // inside a binade the significand's increment adds to the bits
+            // taken when the sum enters the chunk in the predicted binade and leaves it there: both share lo's top nine bits
+            if ((((b ^ lo) | (nb ^ lo)) >> 23) == 0u) {
+                b = nb;
+            } else {
+                float S = __uint_as_float(b);
+                const float* ch = sqp + c * LP;
+#pragma unroll
+                for (int j0 = 0; j0 < L; j0 += 16) {
+                    float v[16];
+#pragma unroll
+                    for (int j = 0; j < 16 && j0 + j < L; j++) v[j] = ch[j0 + j];
+#pragma unroll
+                    for (int j = 0; j < 16 && j0 + j < L; j++) S += v[j];
+                }
+                b = __builtin_amdgcn_readfirstlane(__float_as_uint(S));
+            }
+        }
+        if (lane == 0) result = __uint_as_float(b);
+    }
+    __syncthreads();
+    return result;
+}
+
 template <int VDT, int NCH>
 __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p) {
     __shared__ float logit_lds[64];
@@ -440,37 +548,9 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
     if (p.rms_alpha) {
         // rms_norm (candle-nn/src/ops.rs:504-515) sums the squares left to right in f32.  A different
         // order changes the divisor in the last ulp, which flips quantised activations now and then
-        // and moves a whole output row by 1e-3 of its rms, so the sum is taken serially by one lane
-        // (H dependent adds, a few microseconds) to keep the normalised row bit-identical.
-        __shared__ float sq[H];
-        __shared__ float m_lds;
-        if (wave == 0) {
-#pragma unroll
-            for (int i = 0; i < NCH; i++)
-                *reinterpret_cast<float4*>(&sq[i * 256 + lane * 4]) =
-                    make_float4(xr[4 * i] * xr[4 * i], xr[4 * i + 1] * xr[4 * i + 1], xr[4 * i + 2] * xr[4 * i + 2], xr[4 * i + 3] * xr[4 * i + 3]);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            // the chain of H dependent adds is the cost; the operands are fetched 32 at a time ahead of it
-            float sum2 = 0.f;
-            float4 nxt[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) nxt[j] = *reinterpret_cast<const float4*>(&sq[4 * j]);
-            for (int h = 0; h < H; h += 32) {
-                float4 cur[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) cur[j] = nxt[j];
-                const int hn = h + 32 < H ? h + 32 : h;
-#pragma unroll
-                for (int j = 0; j < 8; j++) nxt[j] = *reinterpret_cast<const float4*>(&sq[hn + 4 * j]);
-#pragma unroll
-                for (int j = 0; j < 8; j++) { sum2 += cur[j].x; sum2 += cur[j].y; sum2 += cur[j].z; sum2 += cur[j].w; }
-            }
-            m_lds = sqrtf(sum2 / (float)H + p.rms_eps);
-        }
-        __syncthreads();
-        const float m = m_lds;
+        // and moves a whole output row by 1e-3 of its rms, so the sum keeps the reference's order.
+        const float sum2 = ordered_sum_of_squares<NCH>(xr, tid, p.rms_serial != 0);
+        const float m = sqrtf(sum2 / (float)H + p.rms_eps);
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const float4 a = *reinterpret_cast<const float4*>(p.rms_alpha + i * 256 + lane * 4);
@@ -632,7 +712,8 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
 
 hipError_t launch_front(const FrontParams& p_in, hipStream_t s) {
     if (p_in.T == 0) return hipSuccess;
-    const FrontParams& p = p_in;
+    FrontParams p = p_in;
+    p.rms_serial = getenv("MOE_RMS_SERIAL") != nullptr;   // read per call: the tests compare the two evaluations in one process
     static const bool no_fast = getenv("MOE_FRONT_GENERIC") != nullptr;
     const bool q8k = p.vdt == MOE_GGML_Q8K;
     if (!no_fast && (q8k ? launch_front_fast<MOE_GGML_Q8K>(p, s) : launch_front_fast<MOE_GGML_Q8_0>(p, s))) return hipGetLastError();

@@ -368,6 +368,45 @@ def test_block_rms_residual_chain():
     gpu.close()
 
 
+@pytest.mark.parametrize("H", [1024, 3072, 4096])
+def test_rms_norm_sum_keeps_the_reference_order(H, monkeypatch):
+    """rms_norm folds the squares of a row left to right in f32 (candle-nn/src/ops.rs:504-515).  The fast front kernel
+    evaluates that fold in chunks (per-chunk significand increments, exact while the running sum stays in one binade);
+    MOE_RMS_SERIAL makes it add term by term instead.  Logits and outputs of the two must agree bit for bit on rows
+    chosen to stress the chunked form: many exact rounding ties (few mantissa bits), outliers that jump binades, tiny
+    terms under a large sum, an all-zero row, a row that overflows to infinity.  The term-by-term form itself is held
+    to the oracle by the tolerance tests of the rms-norm layers."""
+    ref, gpu = make_pair(H, 256, 4, 2, O.Q4K, seed=6, rms=True)
+    rng = np.random.default_rng(H)
+    rows = [rng.standard_normal(H),
+            rng.integers(-8, 9, H) / 4.0,
+            rng.standard_normal(H) * np.exp(3.0 * rng.standard_normal(H)),
+            rng.integers(0, 3, H) * 2.0 ** -10,
+            np.round(rng.standard_normal(H) * 16) / 16,
+            np.zeros(H),
+            rng.standard_normal(H) * 1e-20,
+            np.full(H, 0.5),
+            rng.integers(1, 4, H) * 2.0 ** 60]
+    rows[3][rng.integers(0, H, 3)] = 37.5
+    rows[8][H // 2] = 1.5e19   # its square is near the top of the f32 range; the sum ends up infinite
+    xs = np.ascontiguousarray(np.stack(rows), dtype=np.float32)
+    T = xs.shape[0]
+    with np.errstate(all="ignore"):
+        fast = gpu.forward(xs)
+        fast_logits = gpu.last_logits(T)
+        monkeypatch.setenv("MOE_RMS_SERIAL", "1")
+        serial = gpu.forward(xs)
+        serial_logits = gpu.last_logits(T)
+        monkeypatch.delenv("MOE_RMS_SERIAL")
+    assert np.array_equal(bits(fast_logits), bits(serial_logits))
+    assert np.array_equal(bits(fast), bits(serial))
+    finite = np.isfinite(serial).all(axis=1)
+    assert finite[:5].all()
+    want = ref.forward(xs[:5], logits=serial_logits[:5])
+    assert np.abs(serial[:5] - want).max() <= block_tol(O.Q4K, 256) * rms(want - xs[:5])
+    gpu.close()
+
+
 def test_long_inputs_go_through_in_several_passes(monkeypatch):
     # the kernels address quantised rows with 32-bit offsets, so a call carries a bounded number of tokens
     # and longer inputs are cut into passes; forced here at 48 tokens per pass on a 130-token input
