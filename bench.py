@@ -15,6 +15,9 @@ another GGML format (random block payloads with small finite scales: timing does
 `--workload config4` measures BASELINE config 4 (hidden 2048, 60 experts of FFN 1408, top-4, one always-on
 shared expert of FFN 5632 behind a sigmoid gate, Q8_0 weights, 512 tokens); its line carries the time of the
 dispatch (histogram, scan, permutation) beside the other stages.
+`--workload stack` measures BASELINE config 5: 32 such layers chained on one GPU (26 GB of Q4_K blocks resident),
+each y = x + moe(rms_norm(x)), a 32-token batch run for `--steps` (default 128) consecutive steps, each step
+feeding the previous output plus N(0, 0.1) noise; a "step" is one pass through all 32 layers.
 """
 import argparse
 import re
@@ -139,13 +142,98 @@ def measured_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
     return None
 
 
+def run_stack(args, np, torch, candle_amd):
+    """BASELINE config 5: `--layers` Mixtral-shape MoE layers chained, each with its own resident copy of its
+    weights and its own gate; layer l's experts are the drawn eight rotated by l places (timing does not depend on
+    the values, and drawing 26 GB of distinct blocks would only lengthen the set-up)."""
+    B = args.batch or 32
+    _, gate0, w = build_layer(torch, candle_amd)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    layers = []
+    for l in range(args.layers):
+        r = l % E
+        gate = (torch.randn((E, H), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
+        alpha = (1.0 + 0.1 * torch.randn((H,), generator=g, device="cuda", dtype=torch.float32)).cpu().numpy()
+        layers.append(candle_amd.SparseMoeBlock(H, F, E, TOPK, Q4K, gate, w["w1"][r:] + w["w1"][:r], w["w3"][r:] + w["w3"][:r],
+                                                w["w2"][r:] + w["w2"][:r], rms_alpha=alpha, rms_eps=1e-5))
+    x0 = torch.randn((B, H), generator=g, device="cuda", dtype=torch.float32)
+    bufs = [torch.empty_like(x0) for _ in range(2)]
+    noise, x_next = torch.empty_like(x0), torch.empty_like(x0)
+
+    def step(h):
+        for i, layer in enumerate(layers):
+            layer.forward(h, out=bufs[i & 1])
+            h = bufs[i & 1]
+        noise.normal_(0.0, 0.1, generator=g)
+        return torch.add(h, noise, out=x_next)   # the next step's input
+
+    stream = torch.cuda.Stream()
+    hip = hip_events()
+    with torch.cuda.stream(stream):
+        h = x0
+        for _ in range(args.warmup):
+            h = step(h)
+        stream.synchronize()
+        ev = [C.c_void_p() for _ in range(2)]
+        for e in ev:
+            hip.hipEventCreate(C.byref(e))
+        sh = C.c_void_p(stream.cuda_stream)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        hip.hipEventRecord(ev[0], sh)
+        for _ in range(args.steps):
+            h = step(h)
+        hip.hipEventRecord(ev[1], sh)
+        hip.hipEventSynchronize(ev[1])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms = C.c_float()
+        hip.hipEventElapsedTime(C.byref(ms), ev[0], ev[1])
+        ms_per_step = ms.value / args.steps
+        finite = bool(torch.isfinite(h).all())
+        # stage times of a mid-stack layer, measured right after its predecessors ran (its weights and gate are cold)
+        mid = len(layers) // 2
+        stage = {k: 0.0 for k in layers[mid].STAGES}
+        for _ in range(5):
+            hh = x0
+            for i, layer in enumerate(layers[:mid]):
+                layer.forward(hh, out=bufs[i & 1])
+                hh = bufs[i & 1]
+            for k, v in layers[mid].forward_timed(hh, bufs[mid & 1]).items():
+                stage[k] += v / 5
+    stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
+    n_active = E   # a 32-token batch reaches every expert (64 assignments over 8 experts)
+    act = 36 / 256
+    up_bytes = n_active * (2 * H * F * 144 // 256) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
+    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+    step_bytes = len(layers) * (n_active * EXPERT_BYTES + E * H * 4 + 3 * B * H * 4)
+    out = {
+        "metric": "MoE stack tokens/s end to end (%d Mixtral-8x7B MoE layers, Q4_K, decode)" % len(layers),
+        "value": B / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8", "data": "synthetic",
+        "config": {"workload": "BASELINE config 5: %d chained MoE layers (hidden 4096, ffn 14336, 8 experts, top-2, Q4_K, %.1f GB "
+                               "resident), y = x + moe(rms_norm(x)) per layer, %d-token batch, each step fed the previous output "
+                               "plus N(0, 0.1) noise" % (len(layers), len(layers) * E * EXPERT_BYTES / 1e9, B),
+                   "layers": len(layers), "us_per_layer": ms_per_step * 1e3 / len(layers), "wall_ms_per_step": wall * 1e3 / args.steps,
+                   "mid_stack_stage_us": stage_us, "output_finite": finite,
+                   "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "roofline": {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation), layer %d of the stack" % mid,
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 200; 128 for the stack workload)")
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill, 512 for config4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "config4"), default="decode")
+    ap.add_argument("--workload", choices=("decode", "prefill", "config4", "stack"), default="decode")
+    ap.add_argument("--layers", type=int, default=32, help="layers of the stack workload")
     ap.add_argument("--weights", choices=sorted(FORMATS), default="q4_k", help="GGML format of the expert matrices (decode workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
@@ -171,6 +259,12 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
+    if args.steps is None:
+        args.steps = 128 if args.workload == "stack" else 200
+    if args.workload == "stack":
+        if args.weights != "q4_k":
+            sys.exit("bench.py: --weights applies to the decode workload only")
+        return run_stack(args, np, torch, candle_amd)
     prefill = args.workload == "prefill"
     cfg4 = args.workload == "config4"
     B = args.batch or (4096 if prefill else 512 if cfg4 else 32)
