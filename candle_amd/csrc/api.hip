@@ -364,6 +364,13 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.rb.direct = direct ? 1 : 0;
     static const int force_tile = getenv("MOE_TILE_SLOTS") ? atoi(getenv("MOE_TILE_SLOTS")) : 0;
     fp.rb.tile_slots = force_tile == 64 || force_tile == 128 ? force_tile : T * L->k >= 96 * L->E ? 128 : 64;
+    // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
+    // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
+    // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches
+    // served without a dispatch pass only: a prefill's tens of millions of atomic adds cost more than its combine pass.
+    // MOE_COMBINE_PASS (read per call) keeps the separate pass.
+    const bool accumulate = direct && L->k == 2 && !shared && !L->has_rms && getenv("MOE_COMBINE_PASS") == nullptr;
+    if (accumulate) fp.y_zero = static_cast<float*>(d_y);
     MOE_MARK(ST_BEGIN);
     MOE_HIP_CHECK(launch_front(fp, s));
     MOE_MARK(ST_FRONT);
@@ -376,6 +383,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     ep.groups = L->groups.as<GroupWeights>();
     ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = L->hq.view(); ep.slot_origin = 0;
     ep.yw = L->yw.as<float>();
+    ep.y_acc = accumulate ? static_cast<float*>(d_y) : nullptr;
     ep.max_rows = T;
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
@@ -440,7 +448,7 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         MOE_HIP_CHECK(launch_expert_down(sp, s));
     }
     MOE_MARK(ST_SHARED);
-    MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    if (!accumulate) MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
     MOE_MARK(ST_COMBINE);
 #undef MOE_MARK
     L->last_direct = direct;

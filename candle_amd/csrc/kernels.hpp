@@ -43,6 +43,7 @@ struct FrontParams {
     int rms_serial = 0;                 // 1: the fast kernel adds the squares of a row term by term (checks the chunked evaluation)
     int vdt = MOE_GGML_Q8K;             // activation format
     ActBuf xq;                          // token-indexed quantised activations (output)
+    float* y_zero = nullptr;            // [T, H] or null: rows the kernel clears for the down kernels to accumulate into
     RouteBufs rb;
 };
 // rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token.
@@ -71,6 +72,8 @@ struct ExpertParams {
     ActBuf hq;                      // slot-indexed (row = slot - slot_origin), K = F
     int slot_origin = 0;
     float* yw = nullptr;            // [S, H] weighted expert outputs, slot-indexed (absolute)
+    float* y_acc = nullptr;         // when set: the down kernels add their weighted outputs to y_acc[token, :] (zeroed by the
+                                    // front kernel) instead of storing yw, and no combine pass runs
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
     int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1, 2 or, Q4K only, 4)
     int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)

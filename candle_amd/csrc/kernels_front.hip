@@ -298,6 +298,11 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     }
     __syncthreads();
 
+    // the row of x is in LDS by now (the output may be the input buffer): clear the token's output row if the down
+    // kernels are to accumulate into it
+    if (p.y_zero)
+        for (int h = tid * 4; h < H; h += FRONT_THREADS * 4) *reinterpret_cast<float4*>(p.y_zero + t * H + h) = make_float4(0.f, 0.f, 0.f, 0.f);
+
     // ---- one thread routes while the waves quantise the row
     if (tid == 0) route_one_token(probs, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
 
@@ -635,6 +640,10 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
             }
     }
     __syncthreads();
+    // every wave read the row of x at the start (the output may be the input buffer): clear the token's output row if
+    // the down kernels are to accumulate into it
+    if (p.y_zero)
+        for (int i = tid; i < H / 4; i += FAST_THREADS) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (wave == 0) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk,
                                         p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
 }

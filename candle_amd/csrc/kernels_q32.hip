@@ -303,7 +303,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_down_kernel(ExpertParams p) {
             const int pos = tg0 + tt * 16 + 4 * g + i;
             if (pos < gs.n) {
                 const int slot = gs.slot(pos);
-                p.yw[(int64_t)slot * H + rt * 16 + r] = acc[tt][i] * slot_weight(p, slot);
+                emit_expert_output(p, slot, rt * 16 + r, acc[tt][i] * slot_weight(p, slot));
             }
         }
 }
@@ -630,7 +630,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
             const int pos = tg0 + tt * 16 + 4 * g + i;
             if (pos < gs.n) {
                 const int slot = gs.slot(pos);
-                p.yw[(int64_t)slot * H + rt * 16 + r] = acc[0][tt][i] * slot_weight(p, slot);
+                emit_expert_output(p, slot, rt * 16 + r, acc[0][tt][i] * slot_weight(p, slot));
             }
         }
 }

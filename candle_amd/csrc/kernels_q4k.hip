@@ -720,7 +720,7 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
         const int pos = tg0 + tt * 16 + 4 * g + i;
         if (pos < gs.n && rt0 + j < n_rt) {
             const int slot = gs.slot(pos);
-            p.yw[(int64_t)slot * H + (rt0 + j) * 16 + r] = sum * slot_weight(p, slot);
+            emit_expert_output(p, slot, (rt0 + j) * 16 + r, sum * slot_weight(p, slot));
         }
     }
 }

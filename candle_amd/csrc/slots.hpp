@@ -78,4 +78,13 @@ __device__ inline float slot_weight(const ExpertParams& p, int slot) {
     return p.is_shared ? p.rb.shared_w[slot - p.rb.T * p.rb.k] : p.rb.topk_w[slot];
 }
 
+// Hands one weighted expert output to the layer's result.  With top-2 routing and nothing else to add, a token's result is
+// 0 + a + b (quantized_llama.rs:185-203 index_adds onto zeros in ascending expert order), and since a + b == b + a in
+// floating point the two terms may arrive in either order: they are added to the zeroed output row with device-scope
+// hardware float atomics and the combine pass is not needed.  Otherwise the output is stored per slot for that pass.
+__device__ inline void emit_expert_output(const ExpertParams& p, int slot, int col, float v) {
+    if (p.y_acc) unsafeAtomicAdd(p.y_acc + (int64_t)slot_token(p, slot) * p.H + col, v);
+    else p.yw[(int64_t)slot * p.H + col] = v;
+}
+
 }  // namespace moe

@@ -407,6 +407,31 @@ def test_rms_norm_sum_keeps_the_reference_order(H, monkeypatch):
     gpu.close()
 
 
+@pytest.mark.parametrize("dt,T", [(O.Q4K, 1), (O.Q4K, 7), (O.Q4K, 32), (O.Q4K, 100), (O.Q4_0, 16), (O.Q8_0, 300), (O.Q6K, 40), (O.Q5_1, 9)])
+def test_top2_outputs_accumulated_in_place_equal_the_combine_pass(dt, T, monkeypatch):
+    """With top-2 routing, no shared expert and no residual, the down kernels add a token's two terms into the zeroed
+    output row (either order gives the same float) and the combine pass is skipped; MOE_COMBINE_PASS keeps the pass.
+    Both must give the same bits, also when the output buffer held other values before the call."""
+    torch = pytest.importorskip("torch")
+    ref, gpu = make_pair(512, 1024, 8, 2, dt, seed=3)
+    xs = activations(T, 512, 31)
+    x = torch.from_numpy(xs).cuda()
+    out = torch.full_like(x, 7.0)
+    gpu.forward(x, out=out)
+    torch.cuda.synchronize()
+    acc = out.cpu().numpy()
+    monkeypatch.setenv("MOE_COMBINE_PASS", "1")
+    out2 = torch.full_like(x, -3.0)
+    gpu.forward(x, out=out2)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOE_COMBINE_PASS")
+    assert np.array_equal(bits(acc), bits(out2.cpu().numpy()))
+    want = ref.forward(xs, logits=gpu.last_logits(T))
+    kquant = dt in (O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K)   # Q8K activations: the bar of the Q4K blocks at this width
+    assert np.abs(acc - want).max() <= block_tol(O.Q4K if kquant else dt, 1024) * rms(want)
+    gpu.close()
+
+
 def test_long_inputs_go_through_in_several_passes(monkeypatch):
     # the kernels address quantised rows with 32-bit offsets, so a call carries a bounded number of tokens
     # and longer inputs are cut into passes; forced here at 48 tokens per pass on a 130-token input
