@@ -103,8 +103,10 @@ int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float*
  * after such a call the moe_layer_last_* hooks fail, since they describe one pass.) */
 
 /* Same computation on DEVICE pointers, enqueued on `hip_stream` (a hipStream_t, NULL = default
- * stream) without synchronising.  d_x and d_y must not alias.  This is the entry a caller that
- * already keeps activations on the GPU uses (no PCIe in the path). */
+ * stream) without synchronising.  d_x and d_y must not alias or overlap, and d_y is the call's to
+ * write from its first kernel on (top-2 layers clear it early and accumulate the two expert terms of
+ * a token in place), so nothing else may read or write it while the call runs.  This is the entry a
+ * caller that already keeps activations on the GPU uses (no PCIe in the path). */
 int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
 
 /* Measurement aid (no counterpart in the reference): one forward as moe_layer_forward_device with
