@@ -432,6 +432,23 @@ def test_top2_outputs_accumulated_in_place_equal_the_combine_pass(dt, T, monkeyp
     gpu.close()
 
 
+def test_top2_accumulation_keeps_denormal_terms(monkeypatch):
+    # activations of 1e-18 put most outputs below the smallest normal float: the float atomics must not flush them
+    torch = pytest.importorskip("torch")
+    _, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=3, want_gpu=True)
+    x = torch.from_numpy((activations(16, 512, 31) * 1e-18).astype(np.float32)).cuda()
+    acc, ref_pass = torch.full_like(x, 7.0), torch.full_like(x, 7.0)
+    gpu.forward(x, out=acc)
+    monkeypatch.setenv("MOE_COMBINE_PASS", "1")
+    gpu.forward(x, out=ref_pass)
+    torch.cuda.synchronize()
+    monkeypatch.delenv("MOE_COMBINE_PASS")
+    want = ref_pass.cpu().numpy()
+    assert ((np.abs(want) < np.finfo(np.float32).tiny) & (want != 0)).sum() > 100
+    assert np.array_equal(bits(acc.cpu().numpy()), bits(want))
+    gpu.close()
+
+
 def test_long_inputs_go_through_in_several_passes(monkeypatch):
     # the kernels address quantised rows with 32-bit offsets, so a call carries a bounded number of tokens
     # and longer inputs are cut into passes; forced here at 48 tokens per pass on a 130-token input
