@@ -26,29 +26,32 @@ def hipcc():
     return exe
 
 
-def _compile(src):
-    obj = os.path.join(OUT_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc()] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(src, out_dir=None, extra_flags=()):
+    obj = os.path.join(out_dir or OUT_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [hipcc()] + HIPCC_FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
     return obj, r.stderr
 
 
-def build_library(verbose=False):
-    os.makedirs(OUT_DIR, exist_ok=True)
+def build_library(verbose=False, out_dir=None, extra_flags=()):
+    """out_dir / extra_flags: a second build beside the product's (tuning experiments with -D macros)."""
+    out_dir = out_dir or OUT_DIR
+    lib_path = os.path.join(out_dir, os.path.basename(LIB_PATH))
+    os.makedirs(out_dir, exist_ok=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
-        results = list(ex.map(_compile, SOURCES))
+        results = list(ex.map(lambda src: _compile(src, out_dir, extra_flags), SOURCES))
     objs = [o for o, _ in results]
     if verbose:
         for _, err in results:
             if err.strip():
                 print(err)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
-    return LIB_PATH
+    return lib_path
 
 
 if __name__ == "__main__":

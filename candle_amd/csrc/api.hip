@@ -130,9 +130,152 @@ struct RouteStore {
     }
 };
 
+// A call's device workspace as one stretch of memory cut into 256-byte aligned pieces.  With base == nullptr the
+// cuts only measure: `off` ends up as the number of bytes the same cuts need.
+struct Carver {
+    uint8_t* base = nullptr;
+    size_t off = 0;
+    template <typename T>
+    T* take(size_t bytes) {
+        const size_t at = (off + 255) & ~(size_t)255;
+        off = at + bytes;
+        return base ? reinterpret_cast<T*>(base + at) : nullptr;
+    }
+    ActBuf take_act(int vdt, int64_t rows, int64_t k) {
+        ActBuf a;
+        a.qs = take<int8_t>(act_qs_bytes(rows, k));
+        a.d = take<float>(act_d_bytes(vdt, rows, k));
+        a.bsum = take<uint8_t>(act_bsum_bytes(vdt, rows, k));
+        return a;
+    }
+    RouteBufs take_route(int64_t T, int E, int k, bool shared, bool tile_tab) {
+        RouteBufs r;
+        const int64_t S = T * k + (shared ? T : 0);
+        r.logits = take<float>((size_t)T * E * 4);
+        r.topk_idx = take<int32_t>((size_t)T * k * 4);
+        r.topk_w = take<float>((size_t)T * k * 4);
+        r.shared_w = take<float>((size_t)T * 4);
+        r.offsets = take<int32_t>((size_t)(E + 2) * 4);
+        r.perm_token = take<int32_t>((size_t)S * 4);
+        r.perm_w = take<float>((size_t)S * 4);
+        r.tok_slots = take<int32_t>((size_t)T * (k + 1) * 4);
+        r.tile_tab = tile_tab ? take<int32_t>((size_t)(1 + 2 * max_gemm_tiles(S, E + 1)) * 4) : nullptr;
+        return r;
+    }
+};
+
+// A workspace that graph captures may have baked into their nodes: once `captured` is set, growing it keeps the old
+// memory alive until the owner goes (a replay of the capture still reads and writes it).
+struct GrowBuf {
+    void* p = nullptr;
+    size_t cap = 0;
+    bool captured = false;
+    std::vector<void*> retired;
+    GrowBuf() = default;
+    GrowBuf(const GrowBuf&) = delete;
+    GrowBuf& operator=(const GrowBuf&) = delete;
+    ~GrowBuf() {
+        if (p) (void)hipFree(p);
+        for (void* q : retired) (void)hipFree(q);
+    }
+    int reserve(size_t bytes) {
+        if (bytes <= cap) return MOE_OK;
+        void* fresh = nullptr;
+        const size_t want = std::max<size_t>(bytes, 256);
+        hipError_t e = hipMalloc(&fresh, want);
+        if (e != hipSuccess) return fail(MOE_E_NOMEM, std::string("hipMalloc(") + std::to_string(want) + "): " + hipGetErrorString(e));
+        if (p) {
+            if (captured) retired.push_back(p);
+            else MOE_HIP_CHECK(hipFree(p));   // waits for the work that still uses it
+        }
+        p = fresh;
+        cap = want;
+        return MOE_OK;
+    }
+};
+
+// Calls on one object share its workspace, so a call must not start before the previous one has finished.  On one
+// stream the stream's own order sees to that; the event is recorded (on the previous call's stream) only when a call
+// arrives on another stream or the host wants the results: an event record between every two calls costs a 5.6 us
+// bubble per step.
+struct CallOrder {
+    hipEvent_t done = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool pending = false;           // work enqueued on last_stream that `done` does not cover yet
+    int init() {
+        MOE_HIP_CHECK(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+        return MOE_OK;
+    }
+    void destroy() {
+        if (done) (void)hipEventDestroy(done);
+        done = nullptr;
+    }
+    // Marks the end of everything enqueued so far in `done`.  If the stream of the last call has gone (the caller
+    // destroyed it; its work completes all the same) the device is synchronised instead.
+    int close() {
+        if (!pending) return MOE_OK;
+        if (hipEventRecord(done, last_stream) != hipSuccess) {
+            (void)hipGetLastError();
+            MOE_HIP_CHECK(hipDeviceSynchronize());
+            MOE_HIP_CHECK(hipEventRecord(done, nullptr));
+        }
+        pending = false;
+        return MOE_OK;
+    }
+    // before the first launch of an eager call on stream s
+    int enter(hipStream_t s) {
+        if (pending && last_stream == s) return MOE_OK;
+        if (int rc = close()) return rc;
+        MOE_HIP_CHECK(hipStreamWaitEvent(s, done, 0));
+        return MOE_OK;
+    }
+    void leave(hipStream_t s) { last_stream = s; pending = true; }
+    // host side: wait for everything enqueued so far
+    int wait() {
+        if (int rc = close()) return rc;
+        MOE_HIP_CHECK(hipEventSynchronize(done));
+        return MOE_OK;
+    }
+};
+
+// ------------------------------------------------------------------ tuning / test switches
+static std::once_flag g_sw_once;
+static Switches g_sw;
+Switches& switches() {
+    std::call_once(g_sw_once, [] {
+        auto num = [](const char* name, long long dflt) {
+            const char* e = getenv(name);
+            return e ? atoll(e) : dflt;
+        };
+        g_sw.combine_pass = getenv("MOE_COMBINE_PASS") != nullptr;
+        g_sw.rms_serial = getenv("MOE_RMS_SERIAL") != nullptr;
+        g_sw.max_tokens_per_pass = num("MOE_MAX_TOKENS_PER_PASS", 0);
+        g_sw.no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+        g_sw.front_generic = getenv("MOE_FRONT_GENERIC") != nullptr;
+        g_sw.tile_slots = (int)num("MOE_TILE_SLOTS", 0);
+        g_sw.slot_tiles = (int)num("MOE_SLOT_TILES", 0);
+        g_sw.narrow = (int)num("MOE_NARROW", -1);
+    });
+    return g_sw;
+}
+
 }  // namespace moe
 
 using namespace moe;
+
+// The pieces of one forward's workspace (device pointers).
+struct Workspace {
+    RouteBufs rb;
+    ActBuf xq, hq, hq_shared;
+    float* yw = nullptr;
+    float* hbuf = nullptr;
+};
+
+// Which kernels a forward of T tokens takes.
+struct ForwardPlan {
+    bool tiled = false, tiled_down = false, direct = false, accumulate = false, narrow = false, hbuf = false;
+    int tile_slots = 128, slot_tiles = 1;
+};
 
 struct moe_layer {
     int64_t H = 0, F = 0, E = 0, k = 0, Fs = 0;
@@ -142,49 +285,15 @@ struct moe_layer {
     DevBuf weights;                 // all re-laid expert matrices
     DevBuf gate, gate_bias, shared_gate, rms_alpha, groups;
     std::vector<GroupWeights> host_groups;  // E routed (+1 shared)
-    // per-call workspace, grown on demand
     std::mutex mu;
-    int64_t cap_T = -1;
-    RouteStore route;
-    ActStore xq, hq, hq_shared;
-    DevBuf yw, x_dev, y_dev, hbuf;
+    GrowBuf ws;                     // per-call workspace, grown on demand, cut anew for every call
+    DevBuf x_dev, y_dev;            // staging of the host-pointer entry
     hipStream_t stream = nullptr;   // used by the host-pointer entry
-    // Calls share the workspace, so a call must not start before the previous one has finished.  On one stream the
-    // stream's own order sees to that; the event is recorded (on the previous call's stream) only when a call arrives on
-    // another stream or the host wants the results: an event record between every two forwards costs a 5.6 us bubble.
-    hipEvent_t done = nullptr;
-    hipStream_t last_stream = nullptr;
-    bool pending = false;           // work enqueued on last_stream that `done` does not cover yet
-    int64_t last_T = 0;
+    CallOrder order;
+    int64_t last_T = 0;             // -1: several passes, -2: a layer with top_k = 0 routes nothing
     bool last_direct = false;       // the last forward skipped the dispatch pass
+    Workspace last_ws;              // where the last forward left its logits and routing
 };
-
-// Marks the end of everything enqueued for the layer so far in L->done.  If the stream of the last call has gone
-// (the caller destroyed it; its work completes all the same) the device is synchronised instead.
-static int close_pending(moe_layer* L) {
-    if (!L->pending) return MOE_OK;
-    if (hipEventRecord(L->done, L->last_stream) != hipSuccess) {
-        (void)hipGetLastError();
-        MOE_HIP_CHECK(hipDeviceSynchronize());
-        MOE_HIP_CHECK(hipEventRecord(L->done, nullptr));
-    }
-    L->pending = false;
-    return MOE_OK;
-}
-
-static int reserve_workspace(moe_layer* L, int64_t T) {
-    if (T <= L->cap_T) return MOE_OK;
-    int rc;
-    const bool shared = L->Fs > 0;
-    const int64_t S = T * L->k + (shared ? T : 0);
-    if ((rc = L->route.reserve(T, (int)L->E, (int)L->k, shared))) return rc;
-    if ((rc = L->xq.reserve(L->vdt, T, L->H))) return rc;
-    if ((rc = L->hq.reserve(L->vdt, T * L->k, L->F))) return rc;
-    if (shared && (rc = L->hq_shared.reserve(L->vdt, T, L->Fs))) return rc;
-    if ((rc = L->yw.reserve((size_t)S * L->H * 4))) return rc;
-    L->cap_T = T;
-    return MOE_OK;
-}
 
 static int check_desc(const moe_desc* d) {
     if (!d) return fail(MOE_E_INVALID, "desc is NULL");
@@ -205,10 +314,11 @@ static int check_desc(const moe_desc* d) {
     if (d->hidden % 16 || d->ffn % 32) return fail(MOE_E_INVALID, "hidden must be a multiple of 16 and ffn of 32");
     if (d->hidden > 16384) return fail(MOE_E_INVALID, "hidden > 16384 is not supported");
     if (d->n_experts < 1 || d->n_experts > 256) return fail(MOE_E_INVALID, "n_experts must be in 1..256");
-    // top_k = 0 makes the reference return zeros (quantized_llama.rs:507-512 defaults the key to 0);
-    // that degenerate case is rejected here rather than silently reproduced
-    if (d->top_k < 1 || d->top_k > d->n_experts || d->top_k > 16)
-        return fail(MOE_E_INVALID, "top_k must be in 1..min(n_experts,16)");
+    // top_k = 0 is what the reference runs with when the file lacks llama.expert_used_count (quantized_llama.rs:507-512
+    // defaults the key to 0): `take(0)` at :167 selects nothing and the block returns zeros
+    if (d->top_k < 0 || d->top_k > d->n_experts || d->top_k > 16)
+        return fail(MOE_E_INVALID, "top_k must be in 0..min(n_experts,16)");
+    if (d->top_k == 0 && d->shared_ffn > 0) return fail(MOE_E_INVALID, "top_k = 0 with a shared expert is not supported");
     if (!d->gate || !d->w1 || !d->w2 || !d->w3) return fail(MOE_E_INVALID, "gate, w1, w2, w3 must be set");
     for (int64_t e = 0; e < d->n_experts; e++)
         if (!d->w1[e] || !d->w2[e] || !d->w3[e]) return fail(MOE_E_INVALID, "expert " + std::to_string(e) + " has a NULL matrix");
@@ -290,11 +400,11 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
     if ((rc = L->groups.reserve(L->host_groups.size() * sizeof(GroupWeights)))) return bail(rc);
     hipError_t e = hipMemcpy(L->groups.p, L->host_groups.data(), L->host_groups.size() * sizeof(GroupWeights), hipMemcpyHostToDevice);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&L->done, hipEventDisableTiming);
     if (e != hipSuccess) {
         fail(MOE_E_HIP, std::string("layer setup: ") + hipGetErrorString(e));
         return bail(MOE_E_HIP);
     }
+    if ((rc = L->order.init())) return bail(rc);
     *out = L;
     return MOE_OK;
 }
@@ -303,11 +413,10 @@ extern "C" void moe_layer_destroy(moe_layer* L) {
     if (!L) return;
     (void)hipDeviceSynchronize();
     if (L->stream) (void)hipStreamDestroy(L->stream);
-    if (L->done) (void)hipEventDestroy(L->done);
+    L->order.destroy();
     delete L;
 }
 
-// Enqueue one forward on `s`.  Caller holds L->mu.
 // Stage marks for moe_layer_forward_timed: events recorded between the launches.
 enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_REQUANT, ST_DOWN, ST_SHARED, ST_COMBINE, ST_COUNT };
 
@@ -315,27 +424,75 @@ enum { ST_BEGIN = 0, ST_FRONT, ST_DISPATCH, ST_UP, ST_REQUANT, ST_DOWN, ST_SHARE
 // at most this many tokens; longer inputs are cut into chunks (tokens are independent of each other).
 static int64_t max_tokens_per_pass(const moe_layer* L) {
     const int64_t widest = std::max(std::max(L->H, L->F), L->Fs);
-    int64_t limit = std::max<int64_t>(1, (((int64_t)1 << 31) - 1) / (L->k * widest));
-    if (const char* e = getenv("MOE_MAX_TOKENS_PER_PASS"))   // testing aid: force several passes on small inputs
-        if (atoll(e) > 0) limit = std::min<int64_t>(limit, atoll(e));
+    int64_t limit = std::max<int64_t>(1, (((int64_t)1 << 31) - 1) / (std::max<int64_t>(L->k, 1) * widest));
+    const int64_t forced = switches().max_tokens_per_pass;   // testing aid: force several passes on small inputs
+    if (forced > 0) limit = std::min(limit, forced);
     return limit;
 }
 
-static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
+static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
+    const Switches& sw = switches();
+    ForwardPlan pl;
+    const bool shared = L->Fs > 0;
+    // Q4K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
+    // multiple of 64, H of 128; those kernels address activation rows with 32-bit byte offsets), from ~64 rows per
+    // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
+    // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
+    // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
+    // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
+    pl.tiled = !sw.no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 38 * L->E;
+    pl.tiled_down = pl.tiled && L->dt_down == MOE_GGML_Q4K && T * L->k > 64 * L->E;
+    // small batches: slots are numbered t*k + r and no dispatch pass runs
+    pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
+    pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 96 * L->E ? 128 : 64;
+    // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
+    // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
+    // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches
+    // served without a dispatch pass only: a prefill's tens of millions of atomic adds cost more than its combine pass.
+    pl.accumulate = pl.direct && L->k == 2 && !shared && !L->has_rms && !sw.combine_pass;
+    // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
+    // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
+    // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
+    // tiles per pass up to ~34 rows per expert)
+    // (the 32-element kernels carry at most two tiles: three or four per pass measured slower at the Mixtral shape and
+    // 8 % faster at best where sixty small experts' weights exceed the caches)
+    pl.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    if (sw.slot_tiles) pl.slot_tiles = sw.slot_tiles;
+    // very small K-quant batches: at most half of the experts can be active, so the weights are cut
+    // into four times as many workgroups; those write f32 h and a small pass quantises it
+    pl.narrow = pl.direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && pl.slot_tiles == 1 &&
+                (sw.narrow >= 0 ? sw.narrow > 0 : T * L->k <= L->E);
+    pl.hbuf = pl.tiled || pl.narrow;
+    return pl;
+}
+
+// Cuts the workspace of a forward of T tokens out of `base`; returns the bytes it takes (base == nullptr: only that).
+static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& pl, uint8_t* base, Workspace* ws) {
+    Carver c;
+    c.base = base;
+    const bool shared = L->Fs > 0;
+    const int64_t S = T * L->k + (shared ? T : 0);
+    Workspace w;
+    w.rb = c.take_route(T, (int)L->E, (int)L->k, shared, true);
+    w.xq = c.take_act(L->vdt, T, L->H);
+    w.hq = c.take_act(L->vdt, T * L->k, L->F);
+    if (shared) w.hq_shared = c.take_act(L->vdt, T, L->Fs);
+    w.yw = c.take<float>((size_t)S * L->H * 4);
+    if (pl.hbuf) w.hbuf = c.take<float>((size_t)T * L->k * L->F * 4);
+    if (ws) *ws = w;
+    return c.off;
+}
+
+// Enqueues one forward of T tokens on `s` with the workspace `ws`.  Caller holds L->mu.
+static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace& ws, const float* d_x, int64_t T, float* d_y,
+                           hipStream_t s, hipEvent_t* marks = nullptr) {
 #define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
-    // Under stream capture (the caller records this forward into a HIP graph) nothing may be allocated, and
-    // the event that orders eager calls on different streams stays out of the graph.
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
-    const bool capturing = cap != hipStreamCaptureStatusNone;
-    const char* const capture_msg = "forward under stream capture needs its workspace: run one forward of the same number of tokens before capturing";
-    if (capturing && T > L->cap_T) return fail(MOE_E_INVALID, capture_msg);
-    int rc = reserve_workspace(L, T);
-    if (rc) return rc;
-    // a previous call may still be running on another stream and shares the workspace
-    if (!capturing && (!L->pending || L->last_stream != s)) {
-        if ((rc = close_pending(L))) return rc;
-        MOE_HIP_CHECK(hipStreamWaitEvent(s, L->done, 0));
+    if (L->k == 0) {
+        // nothing is selected: the block's output is zero (quantized_llama.rs:167 `take(0)`), plus the residual of a
+        // layer that carries the pre-norm
+        MOE_HIP_CHECK(launch_fill_or_copy(L->has_rms ? d_x : nullptr, d_y, T * L->H, s));
+        L->last_T = -2;
+        return MOE_OK;
     }
     const bool shared = L->Fs > 0;
     FrontParams fp;
@@ -345,68 +502,37 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
     fp.shared_gate = shared ? L->shared_gate.as<float>() : nullptr;
     fp.rms_alpha = L->has_rms ? L->rms_alpha.as<float>() : nullptr;
     fp.rms_eps = L->rms_eps;
+    fp.rms_serial = switches().rms_serial;
     fp.vdt = L->vdt;
-    fp.xq = L->xq.view();
-    fp.rb = L->route.view();
+    fp.xq = ws.xq;
+    fp.rb = ws.rb;
     fp.rb.T = (int)T; fp.rb.k = (int)L->k;
-    // Q4K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
-    // multiple of 64, H of 128; those kernels address activation rows with 32-bit byte offsets), from ~64 rows per
-    // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
-    // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
-    // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
-    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
-    // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
-    const bool tiled = !no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 &&
-                       T * L->k > 38 * L->E;
-    const bool tiled_down = tiled && L->dt_down == MOE_GGML_Q4K && T * L->k > 64 * L->E;
-    // small batches: slots are numbered t*k + r and no dispatch pass runs
-    const bool direct = !tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
-    fp.rb.direct = direct ? 1 : 0;
-    static const int force_tile = getenv("MOE_TILE_SLOTS") ? atoi(getenv("MOE_TILE_SLOTS")) : 0;
-    fp.rb.tile_slots = force_tile == 64 || force_tile == 128 ? force_tile : T * L->k >= 96 * L->E ? 128 : 64;
-    // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
-    // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
-    // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches
-    // served without a dispatch pass only: a prefill's tens of millions of atomic adds cost more than its combine pass.
-    // MOE_COMBINE_PASS (read per call) keeps the separate pass.
-    const bool accumulate = direct && L->k == 2 && !shared && !L->has_rms && getenv("MOE_COMBINE_PASS") == nullptr;
-    if (accumulate) fp.y_zero = static_cast<float*>(d_y);
+    fp.rb.direct = pl.direct ? 1 : 0;
+    fp.rb.tile_slots = pl.tile_slots;
+    if (pl.accumulate) fp.y_zero = d_y;
     MOE_MARK(ST_BEGIN);
     MOE_HIP_CHECK(launch_front(fp, s));
     MOE_MARK(ST_FRONT);
-    if (!direct) MOE_HIP_CHECK(launch_dispatch(fp.rb, T, (int)L->E, (int)L->k, shared, s));
+    if (!pl.direct) MOE_HIP_CHECK(launch_dispatch(fp.rb, T, (int)L->E, (int)L->k, shared, s));
     MOE_MARK(ST_DISPATCH);
 
     ExpertParams ep;
     ep.dt = L->dt; ep.dt_down = L->dt_down; ep.H = (int)L->H; ep.F = (int)L->F;
     ep.n_groups = (int)L->E; ep.group0 = 0;
     ep.groups = L->groups.as<GroupWeights>();
-    ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = L->hq.view(); ep.slot_origin = 0;
-    ep.yw = L->yw.as<float>();
-    ep.y_acc = accumulate ? static_cast<float*>(d_y) : nullptr;
+    ep.rb = fp.rb; ep.xq = fp.xq; ep.hq = ws.hq; ep.slot_origin = 0;
+    ep.yw = ws.yw;
+    ep.y_acc = pl.accumulate ? d_y : nullptr;
     ep.max_rows = T;
-    // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
-    // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
-    // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
-    // tiles per pass up to ~34 rows per expert)
-    ep.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
-    // (the 32-element kernels carry at most two tiles: three or four per pass measured slower at the Mixtral shape and
-    // 8 % faster at best where sixty small experts' weights exceed the caches)
-    static const int force_st = getenv("MOE_SLOT_TILES") ? atoi(getenv("MOE_SLOT_TILES")) : 0;
-    if (force_st) ep.slot_tiles = force_st;
-    static const int force_narrow = getenv("MOE_NARROW") ? atoi(getenv("MOE_NARROW")) : -1;
-    const bool narrow = direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && ep.slot_tiles == 1 &&
-                        (force_narrow >= 0 ? force_narrow > 0 : T * L->k <= L->E);
-    if (tiled) {
-        if (capturing && L->hbuf.cap < (size_t)T * L->k * L->F * 4) return fail(MOE_E_INVALID, capture_msg);
-        if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
-        ep.hbuf = L->hbuf.as<float>();
+    ep.slot_tiles = pl.slot_tiles;
+    if (pl.tiled) {
+        ep.hbuf = ws.hbuf;
         ep.n_slots = T * L->k;
         MOE_HIP_CHECK(launch_q4k_gemm_up(ep, s));
         MOE_MARK(ST_UP);
         MOE_HIP_CHECK(launch_quantize_rows(L->vdt, ep.hbuf, T * L->k, (int)L->F, ep.hq, s));
         MOE_MARK(ST_REQUANT);
-        if (tiled_down) {
+        if (pl.tiled_down) {
             MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
         } else {
             ExpertParams dp = ep;
@@ -414,12 +540,8 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
             MOE_HIP_CHECK(launch_expert_down(dp, s));
         }
         MOE_MARK(ST_DOWN);
-    } else if (narrow) {
-        // very small Q4K batches: at most half of the experts can be active, so the weights are cut
-        // into four times as many workgroups; those write f32 h and a small pass quantises it
-        if (capturing && L->hbuf.cap < (size_t)T * L->k * L->F * 4) return fail(MOE_E_INVALID, capture_msg);
-        if ((rc = L->hbuf.reserve((size_t)T * L->k * L->F * 4))) return rc;
-        ep.hbuf = L->hbuf.as<float>();
+    } else if (pl.narrow) {
+        ep.hbuf = ws.hbuf;
         ep.by_assignment = T * L->k <= L->E ? 1 : 0;   // one row of workgroups per assignment: none for idle experts
         MOE_HIP_CHECK(launch_expert_up(ep, s));
         MOE_MARK(ST_UP);
@@ -442,18 +564,48 @@ static int enqueue_forward(moe_layer* L, const float* d_x, int64_t T, float* d_y
         sp.hbuf = nullptr; sp.by_assignment = 0;
         sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
         sp.groups = L->groups.as<GroupWeights>() + L->E;
-        sp.hq = L->hq_shared.view(); sp.slot_origin = (int)(T * L->k);
+        sp.hq = ws.hq_shared; sp.slot_origin = (int)(T * L->k);
         sp.max_rows = T; sp.slot_tiles = T > 32 ? 4 : T > 16 ? 2 : 1;
         MOE_HIP_CHECK(launch_expert_up(sp, s));
         MOE_HIP_CHECK(launch_expert_down(sp, s));
     }
     MOE_MARK(ST_SHARED);
-    if (!accumulate) MOE_HIP_CHECK(launch_combine(L->yw.as<float>(), fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    if (!pl.accumulate) MOE_HIP_CHECK(launch_combine(ws.yw, fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
     MOE_MARK(ST_COMBINE);
 #undef MOE_MARK
-    L->last_direct = direct;
-    if (!capturing) { L->last_stream = s; L->pending = true; }
+    L->last_direct = pl.direct;
     L->last_T = T;
+    L->last_ws = ws;
+    L->last_ws.rb = fp.rb;
+    return MOE_OK;
+}
+
+// One pass (T within max_tokens_per_pass) on the layer's own workspace.  Under stream capture (the caller records the
+// forward into a HIP graph) nothing may be allocated, the event that orders eager calls on different streams stays out
+// of the graph, and the workspace is from then on never freed before the layer goes: a replay uses its addresses.
+static int forward_pass(moe_layer* L, const float* d_x, int64_t T, float* d_y, hipStream_t s, hipEvent_t* marks = nullptr) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    const ForwardPlan pl = plan_forward(L, T);
+    Workspace ws;
+    if (L->k > 0) {
+        const size_t need = carve_workspace(L, T, pl, nullptr, nullptr);
+        if (capturing && need > L->ws.cap)
+            return fail(MOE_E_INVALID, "forward under stream capture needs its workspace: run one forward of the same number of tokens before capturing");
+        if (need > L->ws.cap) {
+            // a call on another stream may still be using the old workspace
+            if (int rc = L->order.wait()) return rc;
+            if (int rc = L->ws.reserve(need)) return rc;
+        }
+        carve_workspace(L, T, pl, static_cast<uint8_t*>(L->ws.p), &ws);
+        if (capturing) L->ws.captured = true;
+    }
+    // a previous call may still be running on another stream and shares the workspace
+    if (!capturing)
+        if (int rc = L->order.enter(s)) return rc;
+    if (int rc = enqueue_forward(L, pl, ws, d_x, T, d_y, s, marks)) return rc;
+    if (!capturing) L->order.leave(s);
     return MOE_OK;
 }
 
@@ -465,11 +617,11 @@ extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T
     if (T == 0) { L->last_T = 0; return MOE_OK; }
     const int64_t step = max_tokens_per_pass(L);
     for (int64_t t0 = 0; t0 < T; t0 += step) {
-        const int rc = enqueue_forward(L, static_cast<const float*>(d_x) + t0 * L->H, std::min(step, T - t0),
-                                       static_cast<float*>(d_y) + t0 * L->H, static_cast<hipStream_t>(hip_stream));
+        const int rc = forward_pass(L, static_cast<const float*>(d_x) + t0 * L->H, std::min(step, T - t0),
+                                    static_cast<float*>(d_y) + t0 * L->H, static_cast<hipStream_t>(hip_stream));
         if (rc) return rc;
     }
-    if (T > step) L->last_T = -1;   // the routing hooks describe one pass only
+    if (T > step && L->k > 0) L->last_T = -1;   // the routing hooks describe one pass only
     return MOE_OK;
 }
 
@@ -477,13 +629,14 @@ extern "C" int moe_layer_forward_timed(moe_layer* L, const void* d_x, int64_t T,
     if (!L || T <= 0 || !d_x || !d_y || !stage_ms || d_x == d_y) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_timed");
     if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");
     std::lock_guard<std::mutex> lk(L->mu);
+    if (L->k == 0) return fail(MOE_E_INVALID, "moe_layer_forward_timed: the layer has top_k = 0 and launches no stages");
     if (T > max_tokens_per_pass(L)) return fail(MOE_E_INVALID, "moe_layer_forward_timed: more tokens than one pass carries (" + std::to_string(max_tokens_per_pass(L)) + ")");
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     hipEvent_t marks[ST_COUNT] = {};
     int rc = MOE_OK;
     for (int i = 0; i < ST_COUNT && !rc; i++)
         if (hipEventCreate(&marks[i]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventCreate failed");
-    if (!rc) rc = enqueue_forward(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s, marks);
+    if (!rc) rc = forward_pass(L, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s, marks);
     if (!rc && hipEventSynchronize(marks[ST_COMBINE]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventSynchronize failed");
     for (int i = 0; i + 1 < ST_COUNT && !rc; i++)
         if (hipEventElapsedTime(&stage_ms[i], marks[i], marks[i + 1]) != hipSuccess) rc = fail(MOE_E_HIP, "hipEventElapsedTime failed");
@@ -504,8 +657,8 @@ extern "C" int moe_layer_forward(moe_layer* L, const float* x, int64_t T, float*
     MOE_HIP_CHECK(hipMemcpyAsync(L->x_dev.p, x, bytes, hipMemcpyHostToDevice, L->stream));
     const int64_t step = max_tokens_per_pass(L);
     for (int64_t t0 = 0; t0 < T; t0 += step)
-        if ((rc = enqueue_forward(L, L->x_dev.as<float>() + t0 * L->H, std::min(step, T - t0), L->y_dev.as<float>() + t0 * L->H, L->stream))) return rc;
-    if (T > step) L->last_T = -1;   // the routing hooks describe one pass only
+        if ((rc = forward_pass(L, L->x_dev.as<float>() + t0 * L->H, std::min(step, T - t0), L->y_dev.as<float>() + t0 * L->H, L->stream))) return rc;
+    if (T > step && L->k > 0) L->last_T = -1;   // the routing hooks describe one pass only
     MOE_HIP_CHECK(hipMemcpyAsync(y, L->y_dev.p, bytes, hipMemcpyDeviceToHost, L->stream));
     MOE_HIP_CHECK(hipStreamSynchronize(L->stream));
     return MOE_OK;
@@ -517,36 +670,52 @@ static int d2h(void* dst, const void* src, size_t bytes) {
     return MOE_OK;
 }
 
+static int check_last(const moe_layer* L, int64_t T) {
+    if (L->last_T == -2) return fail(MOE_E_INVALID, "the layer has top_k = 0: its forward computes no logits and no routing");
+    if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
+    return MOE_OK;
+}
+
 extern "C" int moe_layer_last_logits(moe_layer* L, float* logits, int64_t T) {
     if (!L || !logits) return fail(MOE_E_INVALID, "bad argument to moe_layer_last_logits");
     std::lock_guard<std::mutex> lk(L->mu);
-    if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
-    if (int rc = close_pending(L)) return rc;
-    MOE_HIP_CHECK(hipEventSynchronize(L->done));
-    return d2h(logits, L->route.logits.p, (size_t)T * L->E * 4);
+    if (int rc = check_last(L, T)) return rc;
+    if (int rc = L->order.wait()) return rc;
+    return d2h(logits, L->last_ws.rb.logits, (size_t)T * L->E * 4);
 }
 
 extern "C" int moe_layer_last_routing(moe_layer* L, int64_t T, int32_t* topk_idx, float* topk_w, int32_t* offsets,
                                       int32_t* perm_token, float* perm_w) {
     if (!L) return fail(MOE_E_INVALID, "layer is NULL");
     std::lock_guard<std::mutex> lk(L->mu);
-    if (T != L->last_T) return fail(MOE_E_INVALID, "n_tokens differs from the last forward on this layer");
     int rc;
-    if ((rc = close_pending(L))) return rc;
-    MOE_HIP_CHECK(hipEventSynchronize(L->done));
+    if ((rc = check_last(L, T))) return rc;
+    if ((rc = L->order.wait())) return rc;
     const size_t A = (size_t)T * L->k;
+    const RouteBufs& rb = L->last_ws.rb;
     if (L->last_direct && T > 0) {  // the forward needed no lists; build them now for the caller
-        RouteBufs rb = L->route.view();
-        rb.T = (int)T; rb.k = (int)L->k;
         MOE_HIP_CHECK(launch_dispatch(rb, T, (int)L->E, (int)L->k, L->Fs > 0, nullptr));
         MOE_HIP_CHECK(hipDeviceSynchronize());
         L->last_direct = false;
     }
-    if ((rc = d2h(topk_idx, L->route.topk_idx.p, A * 4))) return rc;
-    if ((rc = d2h(topk_w, L->route.topk_w.p, A * 4))) return rc;
-    if ((rc = d2h(offsets, L->route.offsets.p, (size_t)(L->E + 1) * 4))) return rc;
-    if ((rc = d2h(perm_token, L->route.perm_token.p, A * 4))) return rc;
-    return d2h(perm_w, L->route.perm_w.p, A * 4);
+    if (T == 0) {
+        if (offsets) std::memset(offsets, 0, (size_t)(L->E + 1) * 4);
+        return MOE_OK;
+    }
+    if ((rc = d2h(topk_idx, rb.topk_idx, A * 4))) return rc;
+    if ((rc = d2h(topk_w, rb.topk_w, A * 4))) return rc;
+    if ((rc = d2h(offsets, rb.offsets, (size_t)(L->E + 1) * 4))) return rc;
+    if ((rc = d2h(perm_token, rb.perm_token, A * 4))) return rc;
+    return d2h(perm_w, rb.perm_w, A * 4);
+}
+
+extern "C" int moe_layer_shape(const moe_layer* L, int64_t* hidden, int64_t* ffn, int64_t* n_experts, int64_t* top_k) {
+    if (!L) return fail(MOE_E_INVALID, "layer is NULL");
+    if (hidden) *hidden = L->H;
+    if (ffn) *ffn = L->F;
+    if (n_experts) *n_experts = L->E;
+    if (top_k) *top_k = L->k;
+    return MOE_OK;
 }
 
 extern "C" int moe_layer_dequantize_weight(moe_layer* L, int64_t expert, int which, float* out, int64_t n_elems) {
@@ -570,9 +739,9 @@ extern "C" int moe_route(const float* logits, int64_t T, int64_t E, int64_t k, i
                          float* topk_w, int32_t* offsets, int32_t* perm_token, float* perm_w) {
     int rc = ensure_device();
     if (rc) return rc;
-    if (T < 0 || E < 1 || E > 256 || k < 1 || k > E || k > 16) return fail(MOE_E_INVALID, "moe_route: need 1<=E<=256, 1<=k<=min(E,16)");
+    if (T < 0 || E < 1 || E > 256 || k < 0 || k > E || k > 16) return fail(MOE_E_INVALID, "moe_route: need 1<=E<=256, 0<=k<=min(E,16)");
     if (T > 0 && !logits) return fail(MOE_E_INVALID, "logits is NULL");
-    if (T == 0) {
+    if (T == 0 || k == 0) {   // k = 0: `take(0)` selects nothing, every list is empty
         if (offsets) std::memset(offsets, 0, (size_t)(E + 1) * 4);
         return MOE_OK;
     }
@@ -640,9 +809,8 @@ struct moe_qlinear {
     int dt = 0, vdt = 0;
     DevBuf weights, group;
     std::mutex mu;
-    RouteStore route;
-    ActStore xq;
-    int64_t cap_m = -1;
+    GrowBuf ws;                     // quantised rows and the identity routing table, cut anew for every call
+    CallOrder order;
     int64_t routed_m = -1;          // row count the identity routing table currently describes (with routed_tile)
     int routed_tile = 0;
     bool routed_tab = false;
@@ -653,7 +821,9 @@ struct moe_qlinear {
 
 extern "C" void moe_qlinear_destroy(moe_qlinear* Q) {
     if (!Q) return;
-    if (Q->stream) { (void)hipStreamSynchronize(Q->stream); (void)hipStreamDestroy(Q->stream); }
+    (void)hipDeviceSynchronize();
+    if (Q->stream) (void)hipStreamDestroy(Q->stream);
+    Q->order.destroy();
     delete Q;
 }
 
@@ -680,41 +850,54 @@ extern "C" int moe_qlinear_create(int32_t dt, const void* w_blocks, int64_t n, i
     MOE_HIP_CHECK(hipMemcpy(Q->group.p, &g, sizeof g, hipMemcpyHostToDevice));
     MOE_HIP_CHECK(hipDeviceSynchronize());
     MOE_HIP_CHECK(hipStreamCreateWithFlags(&Q->stream, hipStreamNonBlocking));
+    if ((rc = Q->order.init())) return rc;
     *out = Q.release();
     return MOE_OK;
 }
 
+static size_t carve_qlinear(const moe_qlinear* Q, int64_t m, uint8_t* base, RouteBufs* rb, ActBuf* xq) {
+    Carver c;
+    c.base = base;
+    const RouteBufs r = c.take_route(m, 1, 1, false, true);
+    const ActBuf a = c.take_act(Q->vdt, m, Q->k);
+    if (rb) *rb = r;
+    if (xq) *xq = a;
+    return c.off;
+}
+
 // quantise the rows, then one pass over the matrix: streamed for short batches, tiled MFMA beyond
 static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d_y, hipStream_t s) {
-    int rc;
-    // under stream capture nothing may be allocated, and the graph carries its own copy of the routing table pass
+    // under stream capture nothing may be allocated, the graph carries its own copy of the routing table pass, and the
+    // workspace is never freed afterwards (a replay uses its addresses)
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
     const bool capturing = cap != hipStreamCaptureStatusNone;
-    if (capturing && m > Q->cap_m)
+    const size_t need = carve_qlinear(Q, m, nullptr, nullptr, nullptr);
+    if (capturing && need > Q->ws.cap)
         return fail(MOE_E_INVALID, "forward under stream capture needs its workspace: run one forward of the same number of rows before capturing");
-    if (capturing) Q->routed_m = -1;
-    if (m > Q->cap_m) {
-        if ((rc = Q->route.reserve(m, 1, 1, false))) return rc;
-        if ((rc = Q->xq.reserve(Q->vdt, m, Q->k))) return rc;
-        Q->cap_m = m;
-        Q->routed_m = -1;   // the table's buffers may have moved
+    if (need > Q->ws.cap) {
+        if (int rc = Q->order.wait()) return rc;   // a call on another stream may still be using the old workspace
+        if (int rc = Q->ws.reserve(need)) return rc;
+        Q->routed_m = -1;   // the table has moved
     }
-    static const bool no_gemm = getenv("MOE_NO_GEMM") != nullptr;
+    if (capturing) { Q->ws.captured = true; Q->routed_m = -1; }
+    RouteBufs rb;
+    ActBuf xq;
+    carve_qlinear(Q, m, static_cast<uint8_t*>(Q->ws.p), &rb, &xq);
+    // Calls share the quantised rows and the table: a call on another stream waits for the previous one.
+    if (!capturing)
+        if (int rc = Q->order.enter(s)) return rc;
     // The tiled MFMA kernel runs one workgroup per (128 weight rows, tile of 64 or 128 x rows): it pays
     // once that grid fills most of the 256 CUs; below, the streamed kernels split the matrix finer.
     const int64_t row_blocks = Q->n / 128;
     const int tile_slots = row_blocks * ((m + 127) / 128) >= 512 ? 128 : 64;
-    const bool tiled = !no_gemm && Q->dt == MOE_GGML_Q4K && Q->n % 128 == 0 && m >= 96 &&
+    const bool tiled = !switches().no_gemm && Q->dt == MOE_GGML_Q4K && Q->n % 128 == 0 && m >= 96 &&
                        row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192;
-    RouteBufs rb = Q->route.view();
     rb.T = (int)m; rb.k = 1;
     rb.tile_slots = tile_slots;
     if (!tiled) rb.tile_tab = nullptr;
-    MOE_HIP_CHECK(launch_quantize_rows(Q->vdt, d_x, m, (int)Q->k, Q->xq.view(), s));
+    MOE_HIP_CHECK(launch_quantize_rows(Q->vdt, d_x, m, (int)Q->k, xq, s));
     // the identity table depends on the row count only: a decode loop that calls with the same m finds it in place
-    // (calls on one object are serialised, and a call on another stream waits for nothing it did not enqueue itself:
-    // the table is rewritten whenever the previous call used another stream)
     if (Q->routed_m != m || Q->routed_tile != tile_slots || Q->routed_tab != tiled || Q->routed_stream != s) {
         MOE_HIP_CHECK(launch_identity_routing(rb, m, s));
         Q->routed_m = m; Q->routed_tile = tile_slots; Q->routed_tab = tiled; Q->routed_stream = s;
@@ -723,10 +906,11 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     ExpertParams ep;
     ep.dt = Q->dt; ep.H = (int)Q->n; ep.F = (int)Q->k; ep.n_groups = 1; ep.group0 = 0;
     ep.groups = Q->group.as<GroupWeights>();
-    ep.rb = rb; ep.hq = Q->xq.view(); ep.slot_origin = 0; ep.yw = d_y;
+    ep.rb = rb; ep.hq = xq; ep.slot_origin = 0; ep.yw = d_y;
     ep.max_rows = m; ep.n_slots = m; ep.slot_tiles = m > 32 ? 4 : m > 16 ? 2 : 1;
     if (tiled) MOE_HIP_CHECK(launch_q4k_gemm_down(ep, s));
     else MOE_HIP_CHECK(launch_expert_down(ep, s));
+    if (!capturing) Q->order.leave(s);
     return MOE_OK;
 }
 
@@ -823,6 +1007,59 @@ extern "C" int moe_quantize_weights(int32_t dt, const float* x, int64_t n, void*
     MOE_HIP_CHECK(launch_quantize_weights(dt, dx.as<float>(), n, dout.as<uint8_t>(), nullptr));
     MOE_HIP_CHECK(hipDeviceSynchronize());
     return d2h(out, dout.p, out_bytes);
+}
+
+// ------------------------------------------------------------------ rms-norm as an operation of its own
+static int check_rms_args(const void* x, const void* alpha, int64_t rows, int64_t hidden, const void* y, const char* who) {
+    if (rows < 0 || hidden <= 0 || hidden > 16256) return fail(MOE_E_INVALID, std::string(who) + ": need rows >= 0 and 0 < hidden <= 16256");
+    if (rows > 0 && (!x || !alpha || !y)) return fail(MOE_E_INVALID, std::string(who) + ": NULL pointer");
+    if (hidden % 4) return fail(MOE_E_INVALID, std::string(who) + ": hidden must be a multiple of 4");
+    return MOE_OK;
+}
+
+extern "C" int moe_add_rms_norm_device(const void* d_x, const void* d_residual, const void* d_alpha, float eps, int64_t rows, int64_t hidden,
+                                       void* d_sum, void* d_y, void* hip_stream) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if ((rc = check_rms_args(d_x, d_alpha, rows, hidden, d_y, "moe_add_rms_norm_device"))) return rc;
+    if (rows == 0) return MOE_OK;
+    if (d_residual && !d_sum) return fail(MOE_E_INVALID, "moe_add_rms_norm_device: d_sum must be given with d_residual");
+    MOE_HIP_CHECK(launch_add_rms_norm(static_cast<const float*>(d_x), static_cast<const float*>(d_residual), static_cast<const float*>(d_alpha), eps,
+                                      rows, (int)hidden, static_cast<float*>(d_sum), static_cast<float*>(d_y), static_cast<hipStream_t>(hip_stream)));
+    return MOE_OK;
+}
+
+extern "C" int moe_rms_norm(const float* x, const float* alpha, float eps, int64_t rows, int64_t hidden, float* y) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    if ((rc = check_rms_args(x, alpha, rows, hidden, y, "moe_rms_norm"))) return rc;
+    if (rows == 0) return MOE_OK;
+    DevBuf dx, da, dy;
+    const size_t bytes = (size_t)rows * hidden * 4;
+    if ((rc = dx.reserve(bytes))) return rc;
+    if ((rc = dy.reserve(bytes))) return rc;
+    if ((rc = da.reserve((size_t)hidden * 4))) return rc;
+    MOE_HIP_CHECK(hipMemcpy(dx.p, x, bytes, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(hipMemcpy(da.p, alpha, (size_t)hidden * 4, hipMemcpyHostToDevice));
+    MOE_HIP_CHECK(launch_add_rms_norm(dx.as<float>(), nullptr, da.as<float>(), eps, rows, (int)hidden, nullptr, dy.as<float>(), nullptr));
+    MOE_HIP_CHECK(hipDeviceSynchronize());
+    return d2h(y, dy.p, bytes);
+}
+
+extern "C" int moe_debug_set_switch(const char* name, int64_t value) {
+    if (!name) return fail(MOE_E_INVALID, "moe_debug_set_switch: name is NULL");
+    Switches& sw = switches();
+    const std::string n(name);
+    if (n == "combine_pass") sw.combine_pass = value != 0;
+    else if (n == "rms_serial") sw.rms_serial = value != 0;
+    else if (n == "max_tokens_per_pass") sw.max_tokens_per_pass = value;
+    else if (n == "no_gemm") sw.no_gemm = value != 0;
+    else if (n == "front_generic") sw.front_generic = value != 0;
+    else if (n == "tile_slots") sw.tile_slots = (int)value;
+    else if (n == "slot_tiles") sw.slot_tiles = (int)value;
+    else if (n == "narrow") sw.narrow = (int)value;
+    else return fail(MOE_E_INVALID, "moe_debug_set_switch: unknown switch '" + n + "'");
+    return MOE_OK;
 }
 
 extern "C" const char* moe_last_error(void) { return g_err.c_str(); }

@@ -344,7 +344,8 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     if (g->metadata.count("llama.expert_count") && moe_gguf_metadata_u64(g, "llama.expert_count", &n_expert)) return MOE_E_INVALID;
     if (g->metadata.count("llama.expert_used_count") && moe_gguf_metadata_u64(g, "llama.expert_used_count", &n_used)) return MOE_E_INVALID;
     if (n_expert <= 1) return fail(MOE_E_INVALID, "llama.expert_count is " + std::to_string(n_expert) + ": the file has dense feed-forward layers, no MoE block");
-    if (n_used == 0) return fail(MOE_E_INVALID, "llama.expert_used_count is 0 or absent (the reference would return all zeros)");
+    // n_used == 0 (key absent or zero): the reference builds the block all the same and its forward selects no expert
+    // (`take(0)`, quantized_llama.rs:167): a layer with top_k = 0 whose output is zero
     const std::string prefix = "blk." + std::to_string(layer_index);
 
     int dt = 0, nd = 0;
@@ -360,10 +361,17 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     else if (dt == 1) {
         const uint16_t* h = static_cast<const uint16_t*>(data);
         for (size_t i = 0; i < gate.size(); i++) gate[i] = half_bits_to_float(h[i]);
-    } else if (moe::weight_dtype_supported(dt)) {
-        if ((rc = moe_dequantize(dt, data, E * H, gate.data()))) return rc;   // on the GPU
+    } else if (dt == 30) {   // BF16: the upper half of an f32
+        const uint16_t* h = static_cast<const uint16_t*>(data);
+        for (size_t i = 0; i < gate.size(); i++) {
+            const uint32_t bits = (uint32_t)h[i] << 16;
+            memcpy(&gate[i], &bits, 4);
+        }
     } else
-        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: unsupported dtype " + std::to_string(dt) + " (supported: F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K)");
+        // QMatMul::from_arc (candle-core/src/quantized/mod.rs:429-443) dequantises F32, F16 and BF16 only; a quantised
+        // router would run as a quantised product over Q8-quantised activations, with other logits than an f32 gate
+        // gives.  llama.cpp never quantises this tensor; such a file is refused rather than routed differently.
+        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: dtype " + std::to_string(dt) + " is not supported for the router (supported: F32, F16, BF16)");
 
     std::vector<const void*> w1((size_t)E), w2((size_t)E), w3((size_t)E);
     int up_dt = -1, down_dt = -1;   // gate / up matrices share one dtype, down matrices one

@@ -4,6 +4,20 @@
 
 namespace moe {
 
+// Tuning and test switches of the whole process: read once from the MOE_* environment variables, changed afterwards
+// only through moe_debug_set_switch.  Nothing on a forward's path reads the environment.
+struct Switches {
+    int combine_pass = 0;             // MOE_COMBINE_PASS: keep the combine pass for top-2 layers
+    int rms_serial = 0;               // MOE_RMS_SERIAL: rms-norm sum of squares term by term
+    int64_t max_tokens_per_pass = 0;  // MOE_MAX_TOKENS_PER_PASS: lower the per-pass token bound (0 = the real bound)
+    int no_gemm = 0;                  // MOE_NO_GEMM: never take the tiled kernels
+    int front_generic = 0;            // MOE_FRONT_GENERIC: generic front kernel
+    int tile_slots = 0;               // MOE_TILE_SLOTS: 64 | 128 (0 = by batch size)
+    int slot_tiles = 0;               // MOE_SLOT_TILES: 16-slot tiles per streaming pass (0 = by batch size)
+    int narrow = -1;                  // MOE_NARROW: 0 | 1 (-1 = by batch size)
+};
+Switches& switches();
+
 // Routing state of one forward call (all device pointers).  "Groups" are the E routed experts
 // plus, when the layer has one, the always-on shared expert as group E.
 struct RouteBufs {
@@ -99,6 +113,13 @@ hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 // y[t] = sum over the token's slots (ascending expert index, shared expert last) of yw[slot] (+ residual[t]).
 hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,
                           int64_t T, int H, hipStream_t s);
+
+// y[i] = src ? src[i] : 0 for n floats (n % 4 == 0): the output of a layer that selects no expert.
+hipError_t launch_fill_or_copy(const float* src, float* y, int64_t n, hipStream_t s);
+// RmsNorm::forward (candle-nn/src/ops.rs:504-515) on rows of `hidden` floats: v = x (+ residual, stored to sum when
+// given), y = v / sqrt(sum(v^2) / hidden + eps) * alpha, the squares summed left to right as the reference does.
+hipError_t launch_add_rms_norm(const float* x, const float* residual, const float* alpha, float eps, int64_t rows, int hidden,
+                               float* sum, float* y, hipStream_t s);
 
 // Re-lay raw GGML blocks [rows, k] (device, standard layout) into the tiled device layout.
 hipError_t launch_relayout(int dt, const uint8_t* raw, uint8_t* tiled, int64_t rows, int64_t k, hipStream_t s);

@@ -648,6 +648,70 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
                                         p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
 }
 
+// RmsNorm::forward as a kernel of its own (candle-nn/src/ops.rs:504-515; the `(attn + residual)` that precedes the
+// ffn_norm at quantized_llama.rs:884-888 folded in when `residual` is given): one workgroup per row.
+template <int NCH>
+__global__ __launch_bounds__(FAST_THREADS) void rms_norm_fast_kernel(const float* x, const float* residual, const float* alpha, float eps,
+                                                                     float* sum, float* y, int serial) {
+    constexpr int H = NCH * 256;
+    __shared__ float row_lds[64 * (NCH * 4 + 1)];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t t = blockIdx.x;
+    float xr[NCH * 4];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        float4 v = *reinterpret_cast<const float4*>(x + t * H + i * 256 + lane * 4);
+        if (residual) {
+            const float4 r = *reinterpret_cast<const float4*>(residual + t * H + i * 256 + lane * 4);
+            v.x = v.x + r.x; v.y = v.y + r.y; v.z = v.z + r.z; v.w = v.w + r.w;
+            if ((i & 7) == wave) *reinterpret_cast<float4*>(sum + t * H + i * 256 + lane * 4) = v;
+        }
+        xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+    }
+    const float sum2 = ordered_sum_of_squares<NCH>(xr, tid, serial != 0, row_lds);
+    const float m = sqrtf(sum2 / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < NCH; i++)
+        if ((i & 7) == wave) {
+            const float4 a = *reinterpret_cast<const float4*>(alpha + i * 256 + lane * 4);
+            *reinterpret_cast<float4*>(y + t * H + i * 256 + lane * 4) =
+                make_float4(xr[4 * i] / m * a.x, xr[4 * i + 1] / m * a.y, xr[4 * i + 2] / m * a.z, xr[4 * i + 3] / m * a.w);
+        }
+}
+
+// any other row length: the row in LDS, one thread adds the squares
+__global__ __launch_bounds__(FRONT_THREADS) void rms_norm_generic_kernel(const float* x, const float* residual, const float* alpha, float eps,
+                                                                         float* sum, float* y, int H) {
+    extern __shared__ float xrow[];
+    __shared__ float mval;
+    const int tid = threadIdx.x;
+    const int64_t t = blockIdx.x;
+    for (int h = tid; h < H; h += FRONT_THREADS) {
+        float v = x[t * H + h];
+        if (residual) {
+            v = v + residual[t * H + h];
+            sum[t * H + h] = v;
+        }
+        xrow[h] = v;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float tot = 0.f;
+        for (int h = 0; h < H; h++) tot += xrow[h] * xrow[h];
+        mval = sqrtf(tot / (float)H + eps);
+    }
+    __syncthreads();
+    const float m = mval;
+    for (int h = tid; h < H; h += FRONT_THREADS) y[t * H + h] = xrow[h] / m * alpha[h];
+}
+
+__global__ __launch_bounds__(256) void fill_or_copy_kernel(const float* src, float* y, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    reinterpret_cast<float4*>(y)[i] = src ? reinterpret_cast<const float4*>(src)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const float* logits, int64_t T, int E, int k,
                                                                          int norm_topk, RouteBufs rb) {
     __shared__ float probs[FRONT_THREADS / 64][MAX_E];
@@ -740,11 +804,33 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
     return false;
 }
 
+hipError_t launch_fill_or_copy(const float* src, float* y, int64_t n, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    const int64_t n4 = n / 4;
+    hipLaunchKernelGGL(fill_or_copy_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, src, y, n4);
+    return hipGetLastError();
+}
+
+hipError_t launch_add_rms_norm(const float* x, const float* residual, const float* alpha, float eps, int64_t rows, int hidden,
+                               float* sum, float* y, hipStream_t s) {
+    if (rows == 0) return hipSuccess;
+    const int serial = switches().rms_serial;
+    dim3 grid((unsigned)rows), block(FAST_THREADS);
+#define MOE_RMS_CASE(N) case N: hipLaunchKernelGGL((rms_norm_fast_kernel<N>), grid, block, 0, s, x, residual, alpha, eps, sum, y, serial); return hipGetLastError();
+    if (hidden % 256 == 0 && !switches().front_generic) switch (hidden / 256) {
+        MOE_RMS_CASE(1) MOE_RMS_CASE(2) MOE_RMS_CASE(4) MOE_RMS_CASE(8) MOE_RMS_CASE(12) MOE_RMS_CASE(16)
+        MOE_RMS_CASE(20) MOE_RMS_CASE(24) MOE_RMS_CASE(28) MOE_RMS_CASE(32)
+    }
+#undef MOE_RMS_CASE
+    if ((size_t)hidden * 4 > 64 * 1024 - 512) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rms_norm_generic_kernel, grid, dim3(FRONT_THREADS), (size_t)hidden * sizeof(float), s, x, residual, alpha, eps, sum, y, hidden);
+    return hipGetLastError();
+}
+
 hipError_t launch_front(const FrontParams& p_in, hipStream_t s) {
     if (p_in.T == 0) return hipSuccess;
-    FrontParams p = p_in;
-    p.rms_serial = getenv("MOE_RMS_SERIAL") != nullptr;   // read per call: the tests compare the two evaluations in one process
-    static const bool no_fast = getenv("MOE_FRONT_GENERIC") != nullptr;
+    const FrontParams& p = p_in;
+    const bool no_fast = switches().front_generic != 0;
     const bool q8k = p.vdt == MOE_GGML_Q8K;
     if (!no_fast && (q8k ? launch_front_fast<MOE_GGML_Q8K>(p, s) : launch_front_fast<MOE_GGML_Q8_0>(p, s))) return hipGetLastError();
     size_t lds = (size_t)p.H * sizeof(float);

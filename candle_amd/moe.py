@@ -18,7 +18,8 @@ _BLOCK = {GGML_Q4_0: (32, 18), GGML_Q4_1: (32, 20), GGML_Q5_0: (32, 22), GGML_Q5
           GGML_Q8K: (256, 292)}
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "lib", "libcandle_amd_moe.so")
+# CANDLE_AMD_MOE_LIB points at another build of the library (a tuning experiment built beside the product's)
+_LIB_PATH = os.environ.get("CANDLE_AMD_MOE_LIB") or os.path.join(_HERE, "lib", "libcandle_amd_moe.so")
 _lib = None
 
 
@@ -65,6 +66,9 @@ def load_library():
     L.moe_layer_forward.argtypes = [vp, vp, i64, vp]
     L.moe_layer_forward_device.argtypes = [vp, vp, i64, vp, vp]
     L.moe_layer_forward_timed.argtypes = [vp, vp, i64, vp, vp, vp]
+    L.moe_rms_norm.argtypes = [vp, vp, C.c_float, i64, i64, vp]
+    L.moe_add_rms_norm_device.argtypes = [vp, vp, vp, C.c_float, i64, i64, vp, vp, vp]
+    L.moe_debug_set_switch.argtypes = [C.c_char_p, i64]
     L.moe_layer_last_logits.argtypes = [vp, vp, i64]
     L.moe_layer_last_routing.argtypes = [vp, i64, vp, vp, vp, vp, vp]
     L.moe_layer_dequantize_weight.argtypes = [vp, i64, C.c_int, vp, i64]
@@ -141,6 +145,41 @@ def device_arch():
 
 def debug_expf(x):
     return float(load_library().moe_debug_expf(float(x)))
+
+
+def set_switch(name, value):
+    """Test aid: sets a process-wide tuning switch of the library (see moe_debug_set_switch)."""
+    _check(load_library().moe_debug_set_switch(name.encode(), int(value)))
+
+
+def rms_norm(x, alpha, eps, residual=None):
+    """`RmsNorm::forward` (candle-transformers/src/quantized_nn.rs:100-126) on rows of f32.  numpy in -> numpy out
+    (host entry); torch CUDA tensors go through the device entry on torch's current stream.  With `residual`
+    (device tensors only) returns (x + residual, rms_norm(x + residual))."""
+    L = load_library()
+    if isinstance(x, np.ndarray):
+        if residual is not None:
+            raise MoeError("the host entry takes no residual")
+        x, alpha = _f32(x), _f32(alpha)
+        hidden = x.shape[-1]
+        if alpha.size != hidden:
+            raise MoeError("alpha must have %d elements" % hidden)
+        y = np.empty_like(x)
+        _check(L.moe_rms_norm(_p(x), _p(alpha), float(eps), x.size // hidden, hidden, _p(y)))
+        return y
+    import torch
+    ok = lambda t: isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+    if not ok(x) or not ok(alpha) or (residual is not None and not ok(residual)):
+        raise MoeError("rms_norm takes numpy arrays or contiguous f32 torch CUDA tensors")
+    hidden = x.shape[-1]
+    if alpha.numel() != hidden or (residual is not None and residual.shape != x.shape):
+        raise MoeError("shape mismatch")
+    y = torch.empty_like(x)
+    total = torch.empty_like(x) if residual is not None else None
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    _check(L.moe_add_rms_norm_device(x.data_ptr(), None if residual is None else residual.data_ptr(), alpha.data_ptr(), float(eps),
+                                     x.numel() // hidden, hidden, None if total is None else total.data_ptr(), y.data_ptr(), stream))
+    return y if residual is None else (total, y)
 
 
 def dequantize(dtype, blocks, n_elems):
@@ -345,7 +384,10 @@ class SparseMoeBlock:
             self.hidden, self.ffn, self.dtype = hdim, f, dt
             self.dtype_down = g.tensor(prefix + ".ffn_down.0.weight")[0]
             self.n_experts = g.metadata("llama.expert_count")
-            self.top_k = g.metadata("llama.expert_used_count")
+            try:
+                self.top_k = g.metadata("llama.expert_used_count")
+            except MoeError:
+                self.top_k = 0   # the reference's default for a missing key (quantized_llama.rs:510-512)
             self.shared_ffn = 0
             return self
         finally:

@@ -62,13 +62,16 @@ typedef struct {
     int64_t hidden;              /* H */
     int64_t ffn;                 /* F: per-expert intermediate size */
     int64_t n_experts;           /* E (1..256) */
-    int64_t top_k;               /* n_expert_used (1..min(E,16)) */
+    int64_t top_k;               /* n_expert_used (0..min(E,16)); 0 is what the reference runs with when the file lacks
+                                    llama.expert_used_count (quantized_llama.rs:507-512): `take(0)` at :167 selects no
+                                    expert and the block returns zeros (plus the residual when rms_alpha is set).  Not
+                                    accepted together with a shared expert. */
     int32_t ggml_dtype;          /* MOE_GGML_Q4_0 | Q4_1 | Q5_0 | Q5_1 | Q8_0 | Q2K | Q3K | Q4K | Q5K | Q6K: dtype of every w1 and w3 (and of w2
                                     unless ggml_dtype_down says otherwise) */
     int32_t norm_topk;           /* 1: weights renormalised over the selected experts (Mixtral,
                                     quantized_llama.rs:175-178); 0: raw softmax probability
                                     (qwen2_moe.rs:287 with norm_topk_prob=false) */
-    const float* gate;           /* [E, H] f32: the router is dequantised at load (mod.rs:430-436) */
+    const float* gate;           /* [E, H] f32: an F32 / F16 / BF16 router is dequantised at load (mod.rs:429-436) */
     const float* gate_bias;      /* optional [E], added to the logits; NULL for the reference's models */
     const void* const* w1;       /* E pointers */
     const void* const* w3;       /* E pointers */
@@ -93,12 +96,19 @@ typedef struct {
 int moe_layer_create(const moe_desc* desc, moe_layer** out);
 void moe_layer_destroy(moe_layer* layer);
 
+/* hidden, ffn, n_experts and top_k of a layer (what a caller that built it from a GGUF file needs for its shape
+ * checks; the reference reads the same from `feed_forward_gate_inp` / `n_expert_used`).  Any pointer may be NULL. */
+int moe_layer_shape(const moe_layer* layer, int64_t* hidden, int64_t* ffn, int64_t* n_experts, int64_t* top_k);
+
 /* `MlpOrMoe::forward`, quantized_llama.rs:143-211 (== CustomOp1::cpu_fwd for the drop-in op):
  * x and y are HOST f32 [n_tokens, hidden]; synchronous. */
 int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float* y);
 
 /* moe_layer_forward_device may be recorded into a HIP graph (stream capture): it then allocates nothing
- * and fails with a message if its workspace was not reserved by an earlier forward of the same size. */
+ * and fails with a message if its workspace was not reserved by an earlier forward of the same size.  The graph's
+ * nodes hold addresses inside the layer's workspace: from the first capture on, the layer never frees workspace
+ * memory before moe_layer_destroy (a later, larger eager forward moves to new memory and keeps the old alive), so a
+ * replay stays valid; a replay and another call on the same layer must not overlap in time (they share the layer). */
 /* (Both entries cut inputs of more than (2^31 - 1) / (top_k * max(hidden, ffn)) tokens into several passes;
  * after such a call the moe_layer_last_* hooks fail, since they describe one pass.) */
 
@@ -135,7 +145,10 @@ int moe_layer_dequantize_weight(moe_layer* layer, int64_t expert, int which, flo
 
 /* Parity hook: router + dispatch given logits (host pointers).  Restates softmax_last_dim
  * (candle-nn/src/ops.rs:313-351) + the host top-k loop (quantized_llama.rs:158-179) on the GPU.
- * Outputs as for moe_layer_last_routing. */
+ * Outputs as for moe_layer_last_routing.  The reference has no FFI for this step, so the signature is this
+ * library's own: it takes no layer handle (routing needs E, k and the renormalisation flag only) and also returns
+ * the per-slot weights perm_w that `selected_rws` holds (quantized_llama.rs:174-178).  A NaN probability is ranked as
+ * f32::total_cmp ranks it (:166): above every number when its sign bit is clear, below when set. */
 int moe_route(const float* logits, int64_t n_tokens, int64_t n_experts, int64_t top_k, int32_t norm_topk,
               int32_t* topk_idx, float* topk_w, int32_t* expert_offsets, int32_t* perm_token, float* perm_w);
 
@@ -161,7 +174,8 @@ int moe_qmatmul(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, 
  * size; Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K) and keeps it resident in the kernels' layout; forward quantises the m rows
  * of x as k_quants::matmul does (k_quants.rs:1893-1903) and writes y[m, n] = x . W^T.
  * forward takes host pointers and returns when y is filled; forward_device takes device pointers and
- * enqueues on hip_stream.  Calls on one object serialise; dequantize is QMatMul::dequantize
+ * enqueues on hip_stream.  Calls on one object serialise (a call on another stream waits for the previous call's
+ * kernels); captures into HIP graphs follow the rules given for moe_layer_forward_device.  dequantize is QMatMul::dequantize
  * (QTensor::dequantize, mod.rs:367-371) of the resident copy: [n, k] f32. */
 typedef struct moe_qlinear moe_qlinear;
 int moe_qlinear_create(int32_t ggml_dtype, const void* w_blocks, int64_t n, int64_t k, moe_qlinear** out);
@@ -170,6 +184,17 @@ int moe_qlinear_forward(moe_qlinear* q, const float* x, int64_t m, float* y);
 int moe_qlinear_forward_device(moe_qlinear* q, const void* d_x, int64_t m, void* d_y, void* hip_stream);
 int moe_qlinear_dequantize(moe_qlinear* q, float* out, int64_t n_elems);
 int moe_qlinear_shape(const moe_qlinear* q, int64_t* n, int64_t* k, int32_t* ggml_dtype);
+
+/* ---- rms-norm as an operation of its own --------------------------------------------------------
+ * RmsNorm::forward (candle-transformers/src/quantized_nn.rs:100-126 -> candle_nn::ops::rms_norm,
+ * candle-nn/src/ops.rs:504-515): y = x / sqrt(sum(x^2) / hidden + eps) * alpha per row, the squares summed left
+ * to right in f32 as the reference does (bit-identical divisor).  moe_add_rms_norm_device also folds in the
+ * `(attn + residual)` that precedes `ffn_norm` in the decoder layer (quantized_llama.rs:884-888): with d_residual
+ * set it stores v = x + residual to d_sum (the layer's new residual stream) and normalises v.  hidden % 4 == 0,
+ * hidden <= 16256.  (The norm + residual around the MoE block itself is fused into the layer: moe_desc.rms_alpha.) */
+int moe_rms_norm(const float* x, const float* alpha, float eps, int64_t rows, int64_t hidden, float* y);
+int moe_add_rms_norm_device(const void* d_x, const void* d_residual, const void* d_alpha, float eps, int64_t rows, int64_t hidden,
+                            void* d_sum, void* d_y, void* hip_stream);
 
 /* QTensor::quantize (candle-core/src/quantized/mod.rs:331-349) on the GPU: f32 [n_elems] -> raw
  * GGML blocks, bit-identical to GgmlType::from_float of k_quants.rs:188-224 (Q4_0), 605-634 (Q8_0)
@@ -201,8 +226,9 @@ int moe_gguf_metadata_array_len(const moe_gguf* file, const char* key, uint64_t*
 int moe_gguf_tensor(const moe_gguf* file, const char* name, int* ggml_dtype, int* n_dims, int64_t dims[8], const void** data,
                     uint64_t* nbytes);
 /* The MoE arm of `ModelWeights::from_gguf` for ONE layer (quantized_llama.rs:506-512, 553-578):
- * `llama.expert_count`, `llama.expert_used_count`, `blk.{l}.ffn_gate_inp.weight` (F32, F16 or a
- * supported quantized dtype) and `blk.{l}.ffn_{gate,down,up}.{i}.weight` as w1 / w2 / w3.  All gate / up
+ * `llama.expert_count`, `llama.expert_used_count` (0 when absent, as there: a layer that selects no expert),
+ * `blk.{l}.ffn_gate_inp.weight` (F32, F16 or BF16, the dtypes QMatMul::from_arc dequantises, quantized/mod.rs:429-443;
+ * a quantised router tensor is refused) and `blk.{l}.ffn_{gate,down,up}.{i}.weight` as w1 / w2 / w3.  All gate / up
  * matrices of the layer must share one supported dtype and all down matrices one (Q4K gate / up with
  * Q6K down, as Q4_K_M files have it, or Q5K with Q6K, is accepted).  Needs the GPU. */
 int moe_layer_create_from_gguf(const moe_gguf* file, int layer_index, int norm_topk, moe_layer** out);
@@ -216,6 +242,11 @@ const char* moe_last_error(void);
 
 /* Name of the device the library runs on, e.g. "gfx950"; NULL (and an error message) if none. */
 const char* moe_device_arch(void);
+
+/* Test aid (no counterpart in the reference): sets one of the process-wide tuning switches that are otherwise
+ * read once from the MOE_* environment variables: "combine_pass", "rms_serial", "max_tokens_per_pass", "no_gemm",
+ * "front_generic", "tile_slots", "slot_tiles", "narrow".  Not for use while forwards are in flight. */
+int moe_debug_set_switch(const char* name, int64_t value);
 
 /* Host restatement of the exp used by the device router (same source, compiled for the CPU), so
  * that its agreement with the platform's expf can be checked without a GPU. */

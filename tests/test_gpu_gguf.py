@@ -39,25 +39,46 @@ def test_layer_from_gguf_equals_layer_from_arrays(tmp_path, dt, version):
     direct.close(); loaded.close()
 
 
-def test_router_stored_as_f16_or_quantised(tmp_path):
+def test_router_stored_as_f16_bf16_or_quantised(tmp_path):
     H, F, E, k = 512, 1024, 8, 2
     gate, w1, w3, w2 = build(O.Q4K)
-    # F16 router: candle widens it (QMatMul::from_qtensor dequantises F16 tensors, quantized/mod.rs:430-436)
+    xs = activations(12, H, 5)
+    # F16 router: candle widens it (QMatMul::from_arc dequantises F32 / F16 / BF16 tensors, quantized/mod.rs:429-436)
     p16 = tmp_path / "f16.gguf"
     W.moe_layer_file(p16, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=1)
     a = candle_amd.SparseMoeBlock.from_gguf(str(p16), 0)
     b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, gate.astype(np.float16).astype(np.float32), w1, w3, w2)
-    xs = activations(12, H, 5)
     assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
     a.close(); b.close()
-    # Q8_0 router: the layer uses to_float of the blocks
+    # BF16 router (GgmlDType 30): the upper half of the f32 bits
+    gb = (bits(gate) >> 16).astype(np.uint16)
+    pb = tmp_path / "bf16.gguf"
+    W.moe_layer_file(pb, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=30, gate_blocks=gb)
+    a = candle_amd.SparseMoeBlock.from_gguf(str(pb), 0)
+    b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, (gb.astype(np.uint32) << 16).view(np.float32).reshape(E, H), w1, w3, w2)
+    assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
+    a.close(); b.close()
+    # Q8_0 router: the reference would run it as a quantised product over Q8_0-quantised activations (QMatMul::QTensor
+    # arm), which gives other logits than the f32 gate; llama.cpp never quantises this tensor.  Refused, not approximated.
     gq = O.quantize(O.Q8_0, gate.reshape(-1))
     pq = tmp_path / "q8.gguf"
     W.moe_layer_file(pq, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=O.Q8_0, gate_blocks=gq)
-    a = candle_amd.SparseMoeBlock.from_gguf(str(pq), 0)
-    b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, O.dequantize(O.Q8_0, gq, E * H).reshape(E, H), w1, w3, w2)
-    assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
-    a.close(); b.close()
+    with pytest.raises(candle_amd.MoeError, match="not supported for the router"):
+        candle_amd.SparseMoeBlock.from_gguf(str(pq), 0)
+
+
+def test_missing_expert_used_count_gives_the_reference_zeros(tmp_path):
+    # `llama.expert_used_count` absent -> n_expert_used = 0 (quantized_llama.rs:507-512): the block selects nothing and
+    # returns zeros (:167)
+    H, F, E, k = 512, 1024, 8, 2
+    gate, w1, w3, w2 = build(O.Q4K)
+    p = tmp_path / "no_used.gguf"
+    W.moe_layer_file(p, 0, gate, w1, w3, w2, O.Q4K, k, expert_keys=False, extra_metadata=[("llama.expert_count", W.U32, E)])
+    layer = candle_amd.SparseMoeBlock.from_gguf(str(p), 0)
+    assert layer.top_k == 0
+    xs = activations(5, H, 6)
+    assert not layer.forward(xs).any()
+    layer.close()
 
 
 def test_loader_errors(tmp_path):

@@ -372,7 +372,7 @@ def test_block_rms_residual_chain():
 def test_rms_norm_sum_keeps_the_reference_order(H, monkeypatch):
     """rms_norm folds the squares of a row left to right in f32 (candle-nn/src/ops.rs:504-515).  The fast front kernel
     evaluates that fold in chunks (per-chunk significand increments, exact while the running sum stays in one binade);
-    MOE_RMS_SERIAL makes it add term by term instead.  Logits and outputs of the two must agree bit for bit on rows
+    the `rms_serial` switch makes it add term by term instead.  Logits and outputs of the two must agree bit for bit on rows
     chosen to stress the chunked form: many exact rounding ties (few mantissa bits), outliers that jump binades, tiny
     terms under a large sum, an all-zero row, a row that overflows to infinity.  The term-by-term form itself is held
     to the oracle by the tolerance tests of the rms-norm layers."""
@@ -394,10 +394,12 @@ def test_rms_norm_sum_keeps_the_reference_order(H, monkeypatch):
     with np.errstate(all="ignore"):
         fast = gpu.forward(xs)
         fast_logits = gpu.last_logits(T)
-        monkeypatch.setenv("MOE_RMS_SERIAL", "1")
-        serial = gpu.forward(xs)
-        serial_logits = gpu.last_logits(T)
-        monkeypatch.delenv("MOE_RMS_SERIAL")
+        candle_amd.set_switch("rms_serial", 1)
+        try:
+            serial = gpu.forward(xs)
+            serial_logits = gpu.last_logits(T)
+        finally:
+            candle_amd.set_switch("rms_serial", 0)
     assert np.array_equal(bits(fast_logits), bits(serial_logits))
     assert np.array_equal(bits(fast), bits(serial))
     finite = np.isfinite(serial).all(axis=1)
@@ -410,7 +412,7 @@ def test_rms_norm_sum_keeps_the_reference_order(H, monkeypatch):
 @pytest.mark.parametrize("dt,T", [(O.Q4K, 1), (O.Q4K, 7), (O.Q4K, 32), (O.Q4K, 100), (O.Q4_0, 16), (O.Q8_0, 300), (O.Q6K, 40), (O.Q5_1, 9)])
 def test_top2_outputs_accumulated_in_place_equal_the_combine_pass(dt, T, monkeypatch):
     """With top-2 routing, no shared expert and no residual, the down kernels add a token's two terms into the zeroed
-    output row (either order gives the same float) and the combine pass is skipped; MOE_COMBINE_PASS keeps the pass.
+    output row (either order gives the same float) and the combine pass is skipped; the `combine_pass` switch keeps the pass.
     Both must give the same bits, also when the output buffer held other values before the call."""
     torch = pytest.importorskip("torch")
     ref, gpu = make_pair(512, 1024, 8, 2, dt, seed=3)
@@ -420,11 +422,13 @@ def test_top2_outputs_accumulated_in_place_equal_the_combine_pass(dt, T, monkeyp
     gpu.forward(x, out=out)
     torch.cuda.synchronize()
     acc = out.cpu().numpy()
-    monkeypatch.setenv("MOE_COMBINE_PASS", "1")
-    out2 = torch.full_like(x, -3.0)
-    gpu.forward(x, out=out2)
-    torch.cuda.synchronize()
-    monkeypatch.delenv("MOE_COMBINE_PASS")
+    candle_amd.set_switch("combine_pass", 1)
+    try:
+        out2 = torch.full_like(x, -3.0)
+        gpu.forward(x, out=out2)
+        torch.cuda.synchronize()
+    finally:
+        candle_amd.set_switch("combine_pass", 0)
     assert np.array_equal(bits(acc), bits(out2.cpu().numpy()))
     want = ref.forward(xs, logits=gpu.last_logits(T))
     kquant = dt in (O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K)   # Q8K activations: the bar of the Q4K blocks at this width
@@ -439,10 +443,12 @@ def test_top2_accumulation_keeps_denormal_terms(monkeypatch):
     x = torch.from_numpy((activations(16, 512, 31) * 1e-18).astype(np.float32)).cuda()
     acc, ref_pass = torch.full_like(x, 7.0), torch.full_like(x, 7.0)
     gpu.forward(x, out=acc)
-    monkeypatch.setenv("MOE_COMBINE_PASS", "1")
-    gpu.forward(x, out=ref_pass)
-    torch.cuda.synchronize()
-    monkeypatch.delenv("MOE_COMBINE_PASS")
+    candle_amd.set_switch("combine_pass", 1)
+    try:
+        gpu.forward(x, out=ref_pass)
+        torch.cuda.synchronize()
+    finally:
+        candle_amd.set_switch("combine_pass", 0)
     want = ref_pass.cpu().numpy()
     assert ((np.abs(want) < np.finfo(np.float32).tiny) & (want != 0)).sum() > 100
     assert np.array_equal(bits(acc.cpu().numpy()), bits(want))
@@ -455,14 +461,16 @@ def test_long_inputs_go_through_in_several_passes(monkeypatch):
     ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
     xs = activations(130, 512, 21)
     whole = gpu.forward(xs)
-    monkeypatch.setenv("MOE_MAX_TOKENS_PER_PASS", "48")
-    pieces = gpu.forward(xs)
-    with pytest.raises(candle_amd.MoeError):
-        gpu.last_logits(130)          # the hooks describe one pass only
-    import torch
-    dev = gpu.forward(torch.from_numpy(xs).cuda())
-    torch.cuda.synchronize()
-    monkeypatch.delenv("MOE_MAX_TOKENS_PER_PASS")
+    candle_amd.set_switch("max_tokens_per_pass", 48)
+    try:
+        pieces = gpu.forward(xs)
+        with pytest.raises(candle_amd.MoeError):
+            gpu.last_logits(130)          # the hooks describe one pass only
+        import torch
+        dev = gpu.forward(torch.from_numpy(xs).cuda())
+        torch.cuda.synchronize()
+    finally:
+        candle_amd.set_switch("max_tokens_per_pass", 0)
     assert np.array_equal(bits(pieces), bits(dev.cpu().numpy()))
     # a token's result does not depend on which other tokens share its pass, up to the kernel chosen for the
     # pass size (130 tokens: tiled; 48: streamed), hence the tolerance rather than bit equality
@@ -505,7 +513,77 @@ def test_forward_recorded_into_a_hip_graph(T):
             gpu.forward(big, out=out)
     torch.cuda.synchronize()
     assert torch.equal(gpu.forward(xs[0]), eager[0])
+    # A larger eager forward grows the workspace.  The graph's nodes hold addresses in the old one, which the layer
+    # keeps alive from the first capture on: replays after the growth still equal the eager results.
+    want_big = gpu.forward(big).clone()
+    for x, want in zip(xs, eager):
+        x_in.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_out, want)
+        assert torch.equal(gpu.forward(big), want_big)
     gpu.close()
+
+
+def test_top_k_zero_returns_zeros_as_the_reference_does():
+    # llama.expert_used_count absent -> n_expert_used = 0 (quantized_llama.rs:507-512): `take(0)` selects nothing
+    # (:167) and the block returns zeros; with the fused pre-norm + residual the layer returns its input
+    torch = pytest.importorskip("torch")
+    for rms_norm in (False, True):
+        ref, gpu = make_pair(256, 512, 4, 0, O.Q4K, seed=2, rms=rms_norm)
+        xs = activations(9, 256, 4)
+        want = ref.forward(xs)
+        assert np.array_equal(bits(want), bits(xs if rms_norm else np.zeros_like(xs)))
+        assert np.array_equal(bits(gpu.forward(xs)), bits(want))
+        out = torch.full((9, 256), 5.0, device="cuda")
+        gpu.forward(torch.from_numpy(xs).cuda(), out=out)
+        assert np.array_equal(bits(out.cpu().numpy()), bits(want))
+        with pytest.raises(candle_amd.MoeError, match="top_k = 0"):
+            gpu.last_logits(9)
+        gpu.close()
+    idx, w, off, perm, pw = candle_amd.route(activations(5, 8, 1), 0)
+    assert idx.shape == (5, 0) and not off.any()
+
+
+@pytest.mark.parametrize("E,k", [(8, 2), (60, 4), (160, 6)])
+def test_nan_probabilities_are_ranked_as_total_cmp_ranks_them(E, k):
+    """`sort_by(total_cmp)` (quantized_llama.rs:166) puts a NaN with a clear sign bit above every number and one with
+    the sign bit set below.  One NaN logit makes the whole softmax row NaN (the sum is NaN), so every key of the row
+    is equal and the stable sort keeps index order: experts 0..k-1, with NaN weights."""
+    rng = np.random.default_rng(E)
+    logits = rng.standard_normal((6, E)).astype(np.float32)
+    logits[1, E // 2] = np.float32(np.nan)
+    logits[3, 0] = -np.float32(np.nan)
+    logits[4, E - 1] = np.float32(np.inf)     # exp(inf - inf) = NaN at that position, exp(-inf) = 0 elsewhere
+    with np.errstate(all="ignore"):
+        probs = O.softmax_last_dim(logits)
+        ri, rw, roff, rperm, rpw = O.route(probs, k)
+    gi, gw, goff, gperm, gpw = candle_amd.route(logits, k)
+    assert np.array_equal(gi, ri) and np.array_equal(goff, roff) and np.array_equal(gperm, rperm)
+    assert np.array_equal(np.isnan(gw), np.isnan(rw))
+    ok = ~np.isnan(rw)
+    assert np.array_equal(bits(gw)[ok], bits(rw)[ok])
+    assert np.isnan(gw[1]).all() and np.array_equal(gi[1], np.arange(k))
+
+
+@pytest.mark.parametrize("H", [256, 1024, 4096, 1000, 5120])
+def test_rms_norm_as_an_operation_of_its_own(H):
+    """RmsNorm::forward (quantized_nn.rs:100-126, candle-nn/src/ops.rs:504-515): bit-exact against the oracle, which adds
+    the squares left to right as the reference does; with a residual, the sum x + residual is returned as well."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(H)
+    x = (rng.standard_normal((11, H)) * np.exp(rng.standard_normal((11, 1)))).astype(np.float32)
+    alpha = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    want = O.rms_norm(x, alpha, 1e-5)
+    assert np.array_equal(bits(candle_amd.rms_norm(x, alpha, 1e-5)), bits(want))
+    xd, ad = torch.from_numpy(x).cuda(), torch.from_numpy(alpha).cuda()
+    assert np.array_equal(bits(candle_amd.rms_norm(xd, ad, 1e-5).cpu().numpy()), bits(want))
+    res = (rng.standard_normal((11, H)) * 3).astype(np.float32)
+    total, y = candle_amd.rms_norm(xd, ad, 1e-5, residual=torch.from_numpy(res).cuda())
+    assert np.array_equal(bits(total.cpu().numpy()), bits(x + res))
+    assert np.array_equal(bits(y.cpu().numpy()), bits(O.rms_norm(x + res, alpha, 1e-5)))
+    with pytest.raises(candle_amd.MoeError):
+        candle_amd.rms_norm(x[:, :H - 1], alpha[:H - 1], 1e-5)
 
 
 def test_empty_and_shape_errors():

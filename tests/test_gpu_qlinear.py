@@ -132,3 +132,44 @@ def test_projection_recorded_into_a_hip_graph():
             # eager calls with other row counts in between rewrite the routing table; the graph carries its own pass
             lin.forward(torch.from_numpy(activations(3, k, seed=1)).cuda())
             torch.cuda.synchronize()
+    # a larger eager call moves the workspace to new memory; the graph's nodes keep using the old, which stays alive
+    big = torch.from_numpy(activations(m + 300, k, seed=2)).cuda()
+    want_big = O.matmul(dt, big.cpu().numpy(), w, n)
+    check(dt, lin.forward(big).cpu().numpy(), want_big)
+    for x, want in zip(xs, eager):
+        x_in.copy_(x)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_out, want)
+        check(dt, lin.forward(big).cpu().numpy(), want_big)
+    lin.close()
+
+
+def test_projection_called_from_alternating_streams():
+    # Calls on one object share the quantised rows and the routing table: a call on another stream has to wait for
+    # the previous call's kernels, or its quantiser overwrites rows the previous product is still reading.
+    torch = pytest.importorskip("torch")
+    dt, n, k = O.Q4K, 4096, 4096
+    w = O.fill_normal_quantized(9, dt, n, k, 0.02)
+    lin = candle_amd.QMatMul(dt, w, n, k)
+    xs = [torch.from_numpy(activations(m, k, seed=80 + i)).cuda() for i, m in enumerate((64, 3, 200, 17, 64, 5))]
+    want = [lin.forward(x).cpu().numpy() for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.current_stream()]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        outs = []
+        for i, x in enumerate(xs):
+            st = streams[(i + rep) % 3]
+            with torch.cuda.stream(st):
+                outs.append((st, lin.forward(x)))
+        for (st, y), wnt in zip(outs, want):
+            st.synchronize()
+            assert np.array_equal(bits(y.cpu().numpy()), bits(wnt))
+    # the host entry (the object's own stream) after device calls on another stream
+    with torch.cuda.stream(streams[0]):
+        y = lin.forward(xs[2])
+    host = lin.forward(xs[3].cpu().numpy())
+    assert np.array_equal(bits(host), bits(want[3]))
+    streams[0].synchronize()
+    assert np.array_equal(bits(y.cpu().numpy()), bits(want[2]))
+    lin.close()
