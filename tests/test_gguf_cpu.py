@@ -189,3 +189,53 @@ def test_reader_survives_mutated_files_under_sanitizers(tmp_path):
     r = subprocess.run([str(exe), str(good), str(tmp_path / "mut.gguf"), "2000", "7"], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0, (r.stdout[-500:], r.stderr[-3000:])
     assert "2000 mutants survived" in r.stdout
+
+
+# ---------------------------------------------------------------------------------------------
+# Hand-assembled byte fixtures (tests/golden/gguf_v*.hex.txt): one field per line with the width Content::read takes
+# for it (gguf_file.rs:34-46, 135-150, 318-357, 402-420, 443-505), written without tests/gguf_writer.py, so that a
+# misreading shared by the library's reader and the test's own writer cannot hide.
+def _fixture_bytes(version):
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gguf_v%d.hex.txt" % version)
+    out = bytearray()
+    for line in open(path, encoding="utf-8"):
+        if line.startswith("#"):
+            continue
+        out += bytes.fromhex(line.split("#", 1)[0].strip())
+    return bytes(out)
+
+
+@pytest.mark.parametrize("version,alignment,data_start", [(1, 32, 384), (2, 64, 576), (3, 128, 640)])
+def test_hand_assembled_fixture(tmp_path, version, alignment, data_start):
+    raw = _fixture_bytes(version)
+    # what the reference's field widths give for v3: header 24 bytes, thirteen typed entries up to byte 342,
+    # llama.expert_count (8 + 18 + 4 + 4) to 376, general.alignment (8 + 17 + 4 + 4) to 409, tensor infos
+    # (8 + 23 + 4 + 16 + 4 + 8 = 63) to 472 and (8 + 9 + 4 + 8 + 4 + 8 = 41) to 513 -> next multiple of 128 = 640;
+    # data: 288 bytes, the second tensor at +384, its 16 bytes end the file at 1040
+    if version == 3:
+        assert len(raw) == 1040
+    path = tmp_path / ("fixture_v%d.gguf" % version)
+    path.write_bytes(raw)
+    with candle_amd.GgufFile(str(path)) as g:
+        assert g.version == version
+        assert g.tensor_data_offset == data_start and data_start % alignment == 0
+        assert g.tensor_names() == ["blk.0.ffn_gate.0.weight", "small.f32"]
+        assert g.metadata("t.u8") == 200 and g.metadata("t.i8") == -100
+        assert g.metadata("t.u16") == 50000 and g.metadata("t.i16") == -20000
+        assert g.metadata("t.u32") == 4000000000 and g.metadata("t.i32") == -2000000000
+        assert g.metadata("t.f32") == 0.5 and g.metadata("t.bool") is True
+        assert g.metadata("t.str") == "héllo"
+        assert g.metadata("t.arr") == ("array", 3, 8)
+        assert g.metadata("t.u64") == 2 ** 63 + 5 and g.metadata("t.i64") == -(2 ** 62) and g.metadata("t.f64") == -1.25
+        assert g.metadata("llama.expert_count") == 8
+        if version > 1:
+            assert g.metadata("general.alignment") == alignment
+        dt, shape, data = g.tensor("blk.0.ffn_gate.0.weight")
+        assert dt == 12 and shape == (2, 256)          # outermost first: the on-disk order is reversed
+        assert bytes(data) == bytes((7 * i + 3) & 0xFF for i in range(288))
+        dt, shape, data = g.tensor("small.f32")
+        assert dt == 0 and shape == (4,)
+        assert np.array_equal(np.frombuffer(bytes(data), dtype="<f4"), np.array([1.0, -2.5, 0.0, 1e-3], dtype=np.float32))
+        # the second tensor sits at the first multiple of the alignment past the 288 bytes of the first
+        second = data_start + (288 + alignment - 1) // alignment * alignment
+        assert raw[second:second + 16] == bytes(data)
