@@ -625,6 +625,58 @@ extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T
     return MOE_OK;
 }
 
+// ------------------------------------------------------------------ the entry point that allocates nothing
+// Its workspace is this array instead of memory from hipMalloc.  The name below is a host-side stand-in: the device
+// address comes from hipGetSymbolAddress, once per device, and only that address is handed to kernels.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)MOE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[MAX_DEVICES] = {};
+
+static int static_scratch(uint8_t** out) {
+    int dev = 0;
+    MOE_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(MOE_E_INVALID, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        MOE_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(MOE_E_HIP, "hipGetSymbolAddress returned no address for the static scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = static_cast<uint8_t*>(g_scratch_ptr[dev]);
+    return MOE_OK;
+}
+
+extern "C" int64_t moe_static_scratch_bytes(void) { return (int64_t)STATIC_SCRATCH_BYTES; }
+
+extern "C" int moe_layer_forward_device_noalloc(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream) {
+    if (!L || T < 0 || (T > 0 && (!d_x || !d_y))) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_device_noalloc");
+    if (d_x == d_y && T > 0) return fail(MOE_E_INVALID, "d_x and d_y must not alias");
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (T == 0) { L->last_T = 0; return MOE_OK; }
+    if (T > max_tokens_per_pass(L))
+        return fail(MOE_E_INVALID, "moe_layer_forward_device_noalloc: " + std::to_string(T) + " tokens are more than one pass carries");
+    const ForwardPlan pl = plan_forward(L, T);
+    const size_t need = L->k > 0 ? carve_workspace(L, T, pl, nullptr, nullptr) : 0;
+    if (need > STATIC_SCRATCH_BYTES)
+        return fail(MOE_E_INVALID, "moe_layer_forward_device_noalloc: " + std::to_string(T) + " tokens need a workspace of " + std::to_string(need) +
+                                       " bytes, the static scratch array holds " + std::to_string(STATIC_SCRATCH_BYTES) +
+                                       "; use moe_layer_forward_device for batches of this size");
+    uint8_t* base = nullptr;
+    if (int rc = static_scratch(&base)) return rc;
+    Workspace ws;
+    if (L->k > 0) carve_workspace(L, T, pl, base, &ws);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    if (int rc = enqueue_forward(L, pl, ws, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s)) return rc;
+    // the hooks that read the last call's logits and routing wait for this stream
+    if (cap == hipStreamCaptureStatusNone) L->order.leave(s);
+    return MOE_OK;
+}
+
 extern "C" int moe_layer_forward_timed(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream, float* stage_ms) {
     if (!L || T <= 0 || !d_x || !d_y || !stage_ms || d_x == d_y) return fail(MOE_E_INVALID, "bad argument to moe_layer_forward_timed");
     if (T > (1 << 20)) return fail(MOE_E_INVALID, "n_tokens > 2^20 is not supported");

@@ -65,6 +65,8 @@ def load_library():
     L.moe_layer_destroy.restype = None
     L.moe_layer_forward.argtypes = [vp, vp, i64, vp]
     L.moe_layer_forward_device.argtypes = [vp, vp, i64, vp, vp]
+    L.moe_layer_forward_device_noalloc.argtypes = [vp, vp, i64, vp, vp]
+    L.moe_static_scratch_bytes.restype = i64
     L.moe_layer_forward_timed.argtypes = [vp, vp, i64, vp, vp, vp]
     L.moe_rms_norm.argtypes = [vp, vp, C.c_float, i64, i64, vp]
     L.moe_add_rms_norm_device.argtypes = [vp, vp, vp, C.c_float, i64, i64, vp, vp, vp]
@@ -150,6 +152,10 @@ def debug_expf(x):
 def set_switch(name, value):
     """Test aid: sets a process-wide tuning switch of the library (see moe_debug_set_switch)."""
     _check(load_library().moe_debug_set_switch(name.encode(), int(value)))
+
+
+def static_scratch_bytes():
+    return int(load_library().moe_static_scratch_bytes())
 
 
 def rms_norm(x, alpha, eps, residual=None):
@@ -401,11 +407,15 @@ class SparseMoeBlock:
 
     __del__ = close
 
-    def forward(self, xs, out=None):
+    def forward(self, xs, out=None, noalloc=False):
+        """noalloc (device tensors only): the entry point that allocates nothing (workspace in the library's static
+        device array; fails for batches beyond it)."""
         L = load_library()
         if self._h is None:
             raise MoeError("layer is closed")
         if isinstance(xs, np.ndarray):
+            if noalloc:
+                raise MoeError("noalloc applies to device tensors")
             x = _f32(xs)
             if x.ndim not in (2, 3) or x.shape[-1] != self.hidden:
                 raise MoeError("expected [b, seq, %d] or [tokens, %d], got %s" % (self.hidden, self.hidden, x.shape))
@@ -423,7 +433,8 @@ class SparseMoeBlock:
         T = xs.numel() // self.hidden
         y = torch.empty_like(xs) if out is None else out
         stream = torch.cuda.current_stream(xs.device).cuda_stream
-        _check(L.moe_layer_forward_device(self._h, xs.data_ptr(), T, y.data_ptr(), stream))
+        entry = L.moe_layer_forward_device_noalloc if noalloc else L.moe_layer_forward_device
+        _check(entry(self._h, xs.data_ptr(), T, y.data_ptr(), stream))
         return y
 
     __call__ = forward

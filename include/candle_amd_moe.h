@@ -119,6 +119,18 @@ int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float*
  * caller that already keeps activations on the GPU uses (no PCIe in the path). */
 int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory while they run: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The same forward as
+ * moe_layer_forward_device (same kernels, same results), but its workspace (routing lists, quantised activations,
+ * the experts' weighted outputs) is a file-scope device array of MOE_STATIC_SCRATCH_BYTES bytes that every GPU the
+ * library runs on holds until the process ends; the call makes no hipMalloc / hipFree.  A batch whose workspace
+ * exceeds the array is rejected with MOE_E_INVALID and a message (Mixtral-8x7B shape: batches of up to 119 tokens fit; the
+ * need grows with n_tokens * top_k * (ffn + 4 hidden)).  All layers and all calls on one GPU share the array: calls
+ * that overlap in time on one GPU race (same-stream calls are ordered by the stream). */
+#define MOE_STATIC_SCRATCH_BYTES (8 * 1024 * 1024)
+int moe_layer_forward_device_noalloc(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
+int64_t moe_static_scratch_bytes(void);
+
 /* Measurement aid (no counterpart in the reference): one forward as moe_layer_forward_device with
  * HIP events recorded on `hip_stream` between the launches; waits for completion and returns the
  * elapsed milliseconds of the seven stages in stage_ms[0..6]: front (router + activation quantiser),

@@ -64,6 +64,8 @@ pub mod ffi {
         pub fn moe_layer_shape(layer: *const MoeLayer, hidden: *mut i64, ffn: *mut i64, n_experts: *mut i64, top_k: *mut i64) -> i32;
         pub fn moe_layer_forward(layer: *mut MoeLayer, x: *const f32, n_tokens: i64, y: *mut f32) -> i32;
         pub fn moe_layer_forward_device(layer: *mut MoeLayer, d_x: *const c_void, n_tokens: i64, d_y: *mut c_void, hip_stream: *mut c_void) -> i32;
+        pub fn moe_layer_forward_device_noalloc(layer: *mut MoeLayer, d_x: *const c_void, n_tokens: i64, d_y: *mut c_void, hip_stream: *mut c_void) -> i32;
+        pub fn moe_static_scratch_bytes() -> i64;
         pub fn moe_qmatmul(ggml_dtype: i32, w_blocks: *const c_void, n: i64, k: i64, x: *const f32, m: i64, y: *mut f32) -> i32;
         pub fn moe_qlinear_create(ggml_dtype: i32, w_blocks: *const c_void, n: i64, k: i64, out: *mut *mut MoeQLinear) -> i32;
         pub fn moe_qlinear_destroy(q: *mut MoeQLinear);
@@ -301,9 +303,15 @@ impl HipSparseMoe {
     }
 
     /// The forward on device pointers (HIP memory the caller owns), enqueued on `hip_stream` (null = default
-    /// stream) without synchronising: for hosts that keep activations on the GPU.
-    pub unsafe fn forward_device(&self, d_x: *const c_void, n_tokens: usize, d_y: *mut c_void, hip_stream: *mut c_void) -> Result<()> {
-        check(ffi::moe_layer_forward_device(self.handle, d_x, n_tokens as i64, d_y, hip_stream))
+    /// stream) without synchronising: for hosts that keep activations on the GPU.  `no_alloc` selects the entry
+    /// point that allocates nothing (workspace in the library's static device array, batches up to what it holds).
+    pub unsafe fn forward_device(&self, d_x: *const c_void, n_tokens: usize, d_y: *mut c_void, hip_stream: *mut c_void, no_alloc: bool) -> Result<()> {
+        let rc = if no_alloc {
+            ffi::moe_layer_forward_device_noalloc(self.handle, d_x, n_tokens as i64, d_y, hip_stream)
+        } else {
+            ffi::moe_layer_forward_device(self.handle, d_x, n_tokens as i64, d_y, hip_stream)
+        };
+        check(rc)
     }
 }
 
