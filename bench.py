@@ -1,23 +1,29 @@
 #!/usr/bin/env python3
-"""Benchmark of the quantized sparse-MoE block on one MI355X.
+"""Benchmark of the quantized sparse-MoE block on one MI355X.  Prints ONE JSON line.
 
-Workload (BASELINE config 2): one Mixtral-8x7B-shape MoE layer, hidden 4096, expert FFN 14336,
-8 experts, top-2, Q4_K weights (N(0, 0.02) quantised with candle's algorithm), f32 router gate,
-decode batch of 32 tokens of N(0, 1) activations.  A "step" is one forward of the layer with the
-activations already resident in HBM.  Prints ONE JSON line.
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|decode|prefill|config4|stack] ...
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 32] [--no-cpu-baseline]
+The line's `value` / `roofline` are BASELINE config 2 at decode batch 32: one Mixtral-8x7B-shape MoE layer (hidden
+4096, expert FFN 14336, 8 experts, top-2, Q4_K weights drawn N(0, 0.02) and quantised with candle's algorithm, f32
+router gate), N(0, 1) activations already resident in HBM; a "step" is one forward of the layer.  BASELINE's metric names
+three quantities (tokens/s; decode HBM share of peak; prefill MFMA share of peak), so the default run (`--workload all`)
+measures the other regimes in the same process and reports them as sub-objects of `config`:
 
-`--workload prefill` measures BASELINE config 3 instead (same layer, 4096 tokens, router bias that makes
-the expert load follow Zipf(1)); its roofline object is the int8-MFMA one of the tiled up kernel.
-`--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with
-another GGML format (random block payloads with small finite scales: timing does not depend on the values).
-`--workload config4` measures BASELINE config 4 (hidden 2048, 60 experts of FFN 1408, top-4, one always-on
-shared expert of FFN 5632 behind a sigmoid gate, Q8_0 weights, 512 tokens); its line carries the time of the
-dispatch (histogram, scan, permutation) beside the other stages.
-`--workload stack` measures BASELINE config 5: 32 such layers chained on one GPU (26 GB of Q4_K blocks resident),
-each y = x + moe(rms_norm(x)), a 32-token batch run for `--steps` (default 128) consecutive steps, each step
-feeding the previous output plus N(0, 0.1) noise; a "step" is one pass through all 32 layers.
+  config.prefill  BASELINE config 3: the same layer, 4096 tokens, router bias that makes the expert load follow Zipf(1);
+                  tokens/s, the tiled up kernel's int8 TOP/s against the dense int8 MFMA peak, the whole step's share.
+  config.cfg4     BASELINE config 4: hidden 2048, 60 experts of FFN 1408, top-4, one always-on shared expert of FFN 5632
+                  behind a sigmoid gate, Q8_0 weights, 512 tokens.
+  config.stack    BASELINE config 5: 32 such Mixtral layers chained on one GPU (26 GB of Q4_K blocks resident), each
+                  y = x + moe(rms_norm(x)), a 32-token batch for 128 consecutive steps, each step fed the previous output
+                  plus N(0, 0.1) noise; end-to-end tokens/s.
+
+`--workload decode|prefill|config4|stack` measures one of them alone as the line's `value`.
+`--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with another
+GGML format (random block payloads with small finite scales: timing does not depend on the values).
+
+Timing.  Every measurement first runs forwards for at least 0.5 s (clocks and caches settle; `--warmup` steps are run
+on top), then times max(K, 200) steps (decode, config 4) in one region bracketed by HIP events on the launch stream and
+host synchronisation: `steps` repeats K as given, `timed_steps` says how many were timed, `ms_per_step` is their mean.
 """
 import argparse
 import re
@@ -42,6 +48,8 @@ HBM_PEAK_GBS = 8000.0                          # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0                        # MI355X dense int8 MFMA, published
 # per-expert logit biases under which top-2 routing of N(0, 1.28^2) logits gives Zipf(1) loads (shares 1/i)
 ZIPF_BIAS = [0.0, -1.158, -1.581, -1.845, -2.033, -2.186, -2.299, -2.398]
+MIN_WARM_SECONDS = 0.5
+MIN_TIMED_STEPS = 200
 
 
 def random_blocks(np, rng, fmt, n_elems):
@@ -55,13 +63,12 @@ def random_blocks(np, rng, fmt, n_elems):
     return raw.reshape(-1)
 
 
-def build_layer(torch, candle_amd, seed=0, gate_bias=None, cfg4=False, fmt="q4_k"):
-    """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel
-    (bit-identical to candle's CPU quantiser), kept as host bytes for the CPU baseline too."""
-    h, f, e_n, k, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, TOPK, Q4K, 0)
+def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k"):
+    """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel (bit-identical to candle's
+    CPU quantiser), returned as host bytes (the CPU baseline runs on the same bytes)."""
+    h, f, e_n, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, Q4K, 0)
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
-
     if fmt != "q4_k" and not cfg4:
         import numpy as np
         dt = FORMATS[fmt][0]
@@ -73,21 +80,25 @@ def build_layer(torch, candle_amd, seed=0, gate_bias=None, cfg4=False, fmt="q4_k
         x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
         return candle_amd.quantize_weights(dt, x).cpu().numpy()
 
-    w = {"w1": [], "w3": [], "w2": []}
+    w = {"w1": [], "w3": [], "w2": [], "dt": dt}
     for e in range(e_n):
         for name, shape in (("w1", (f, h)), ("w3", (f, h)), ("w2", (h, f))):
             w[name].append(draw(shape))
-    kw = {}
     if fs:
         w["shared"] = (draw((fs, h)), draw((fs, h)), draw((h, fs)))
     g.manual_seed(seed + 1)
-    gate = (torch.randn((e_n, h), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
+    w["gate"] = (torch.randn((e_n, h), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
     if fs:
         w["shared_gate"] = (torch.randn((h,), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
-        kw = dict(shared_ffn=fs, shared_w1=w["shared"][0], shared_w3=w["shared"][1], shared_w2=w["shared"][2],
-                  shared_gate=w["shared_gate"])
-    layer = candle_amd.SparseMoeBlock(h, f, e_n, k, dt, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias, **kw)
-    return layer, gate, w
+    return w
+
+
+def make_layer(candle_amd, w, gate_bias=None, cfg4=False):
+    if cfg4:
+        c = CFG4
+        return candle_amd.SparseMoeBlock(c["H"], c["F"], c["E"], c["k"], Q8_0, w["gate"], w["w1"], w["w3"], w["w2"], shared_ffn=c["Fs"],
+                                         shared_w1=w["shared"][0], shared_w3=w["shared"][1], shared_w2=w["shared"][2], shared_gate=w["shared_gate"])
+    return candle_amd.SparseMoeBlock(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
 
 
 def hip_events():
@@ -100,20 +111,65 @@ def hip_events():
     return hip
 
 
-def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=False, dt=Q4K):
-    """candle's CPU path restated (the oracle: serial rows, columns threaded, AVX2 inner loops of
-    candle's x86 build) on all host cores: the same batch, same weight bytes, same routing,
-    repeated until `min_seconds` of wall time have passed."""
+class Timer:
+    """Times a callable `step(i)` on a torch stream: warm-up by time, then n steps between two HIP events recorded on
+    that stream, bracketed by host synchronisation."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.hip = hip_events()
+        self.stream = torch.cuda.Stream()
+        self.ev = [C.c_void_p() for _ in range(2)]
+        for e in self.ev:
+            self.hip.hipEventCreate(C.byref(e))
+
+    def run(self, step, n_steps, warmup, min_warm_seconds=MIN_WARM_SECONDS):
+        torch = self.torch
+        with torch.cuda.stream(self.stream):
+            i, t0 = 0, time.perf_counter()
+            while i < warmup or time.perf_counter() - t0 < min_warm_seconds:
+                step(i)
+                i += 1
+                if i % 16 == 0:
+                    self.stream.synchronize()   # the clock above is the host's: keep it honest
+            self.stream.synchronize()
+            sh = C.c_void_p(self.stream.cuda_stream)
+            torch.cuda.synchronize()
+            w0 = time.perf_counter()
+            self.hip.hipEventRecord(self.ev[0], sh)
+            for j in range(n_steps):
+                step(i + j)
+            self.hip.hipEventRecord(self.ev[1], sh)
+            self.hip.hipEventSynchronize(self.ev[1])
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - w0
+            ms = C.c_float()
+            self.hip.hipEventElapsedTime(C.byref(ms), self.ev[0], self.ev[1])
+        return ms.value / n_steps, wall * 1e3 / n_steps, i
+
+    def stages(self, layer, xs, ys, iters):
+        """Per-stage durations: HIP events recorded by the library between its launches, on this stream."""
+        stage = {k: 0.0 for k in layer.STAGES}
+        with self.torch.cuda.stream(self.stream):
+            for i in range(iters):
+                for k, v in layer.forward_timed(xs[i % len(xs)], ys[i % len(ys)]).items():
+                    stage[k] += v / iters
+        return stage
+
+
+def cpu_baseline(w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=False):
+    """candle's CPU path restated (the oracle: serial rows, columns threaded, AVX2 inner loops of candle's x86 build) on
+    all host cores: the same batch, same weight bytes, same routing, repeated until `min_seconds` of wall time have passed."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import pyoracle as O
 
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
     if cfg4:
-        layer = O.Layer(CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, gate, w["w1"], w["w3"], w["w2"], Fs=CFG4["Fs"],
+        layer = O.Layer(CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, w["gate"], w["w1"], w["w3"], w["w2"], Fs=CFG4["Fs"],
                         sw1=w["shared"][0], sw3=w["shared"][1], sw2=w["shared"][2], shared_gate=w["shared_gate"])
     else:
-        layer = O.Layer(H, F, E, TOPK, dt, gate, w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+        layer = O.Layer(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
     layer.forward(xs_host[:1], logits=logits_host[:1], simd=True, threads=cores)  # warm the pages
     reps, t0 = 0, time.perf_counter()
     while True:
@@ -127,10 +183,11 @@ def cpu_baseline(gate, w, xs_host, logits_host, min_seconds, gate_bias=None, cfg
                       "(AVX2 vec_dot, %d threads over output columns)" % (reps, xs_host.shape[0], dt, cores)}
 
 
-def measured_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
-    """HBM bytes per launch of the up kernel from the committed rocprofv3 counter summary (FETCH_SIZE +
-    WRITE_SIZE, scaled by the copy kernel), or None when the summary does not cover this batch size."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", name)
+def profiled_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
+    """HBM bytes per launch of the dominant kernel as the committed rocprofv3 counter summary gives them (FETCH_SIZE +
+    WRITE_SIZE, scaled by the copy kernel): a figure from that profile, not a reading of this run; None when the summary
+    does not cover this batch size."""
+    path = os.path.join(ROOT, "profiles", name)
     key = key or "batch=%d" % batch
     try:
         for line in open(path):
@@ -142,16 +199,102 @@ def measured_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
     return None
 
 
-def run_stack(args, np, torch, candle_amd):
-    """BASELINE config 5: `--layers` Mixtral-shape MoE layers chained, each with its own resident copy of its
-    weights and its own gate; layer l's experts are the drawn eight rotated by l places (timing does not depend on
-    the values, and drawing 26 GB of distinct blocks would only lengthen the set-up)."""
-    B = args.batch or 32
-    _, gate0, w = build_layer(torch, candle_amd)
+def activations(torch, B, hid, seed=2, n=4):
+    """Several distinct activation batches, rotated, so that no step repeats the previous one's input."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    xs = [torch.randn((B, hid), generator=g, device="cuda", dtype=torch.float32) for _ in range(n)]
+    return xs, [torch.empty_like(x) for x in xs]
+
+
+def measure_decode(args, np, torch, timer, layer, B, fmt="q4_k"):
+    xs, ys = activations(torch, B, H)
+    n_steps = max(args.steps, MIN_TIMED_STEPS)
+    ms, wall_ms, warmed = timer.run(lambda i: layer.forward(xs[i % 4], out=ys[i % 4]), n_steps, args.warmup)
+    loads = np.diff(layer.last_routing(B)[2])[:E]
+    n_active = int((loads > 0).sum())
+    stage = timer.stages(layer, xs, ys, args.stage_iters)
+    stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
+    fmt_dt, fmt_be, fmt_bb, _ = FORMATS[fmt]
+    expert_bytes = 3 * H * F * fmt_bb // fmt_be
+    step_bytes = n_active * expert_bytes + E * H * 4 + 2 * B * H * 4
+    # Roofline of the dominant kernel, the up projection (w1, w3 + SiLU): it streams w1 and w3 of every active expert
+    # exactly once per launch; algorithmic bytes = the blocks of those matrices plus the quantised activations it reads
+    # and the quantised intermediate it writes.
+    act = 36 / 256 if fmt_be == 256 else 8 / 32    # bytes of scales and sums per quantised activation element
+    up_bytes = n_active * (2 * H * F * fmt_bb // fmt_be) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
+    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+    q4k = fmt == "q4_k"
+    traffic = profiled_traffic(B) if q4k else None
+    roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)" if q4k else "up projection (w1, w3, SiLU, re-quantisation), %s" % fmt,
+                "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "traffic_source": "profiles/q4k_up_decode_hbm_traffic.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
+                "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+    return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
+            "batch": B, "active_experts": n_active, "stage_us": stage_us, "empty_stage_us": min(stage_us.values()),
+            "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "roofline": roofline, "xs": xs, "ys": ys}
+
+
+def measure_prefill(args, np, torch, timer, layer, B):
+    xs, ys = activations(torch, B, H, n=2)
+    n_steps = max(20, min(args.steps, 50))
+    ms, wall_ms, warmed = timer.run(lambda i: layer.forward(xs[i % 2], out=ys[i % 2]), n_steps, min(args.warmup, 5))
+    loads = np.diff(layer.last_routing(B)[2])[:E]
+    stage = timer.stages(layer, xs, ys, max(3, min(args.stage_iters, 10)))
+    stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
+    # Roofline of the dominant kernel, the tiled up projection: 2 * slots * 2 * H * F integer multiply-adds (w1 and w3)
+    # per launch against the dense int8 MFMA peak.
+    up_ops = 2.0 * B * TOPK * 2 * H * F
+    achieved = up_ops / (stage["up"] * 1e-3) / 1e12
+    step_ops = 2.0 * B * TOPK * 3 * H * F
+    roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, two scale planes)",
+                "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": achieved / INT8_PEAK_TOPS,
+                "traffic": None, "algorithmic_ops_per_launch": up_ops, "launch_us": stage_us["up"],
+                # every algorithmic multiply-add is issued twice (the 6-bit scale is split over two pre-scaled int8
+                # planes so that the integer sums stay exact): share of the peak the MFMA pipe is actually kept busy
+                # with, slot tiles padded to 64 / 128 not counted
+                "mfma_issued_frac": 2.0 * achieved / INT8_PEAK_TOPS}
+    return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
+            "tokens": B, "expert_loads": [int(v) for v in loads], "stage_us": stage_us, "step_int8_ops": step_ops,
+            "step_mfma_frac": step_ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, "roofline": roofline, "xs": xs, "ys": ys}
+
+
+def measure_cfg4(args, np, torch, timer, layer, B):
+    c = CFG4
+    xs, ys = activations(torch, B, c["H"])
+    n_steps = max(args.steps, MIN_TIMED_STEPS)
+    ms, wall_ms, warmed = timer.run(lambda i: layer.forward(xs[i % 4], out=ys[i % 4]), n_steps, args.warmup)
+    loads = np.diff(layer.last_routing(B)[2])[:c["E"]]
+    n_active = int((loads > 0).sum())
+    stage = timer.stages(layer, xs, ys, args.stage_iters)
+    stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
+    # Weights are Q8_0 (34 bytes per 32 elements); every routed expert with a token and the shared expert are read at
+    # least once per step.  The up kernel (w1, w3 of the routed experts) is the longest launch.
+    expert_bytes = 3 * c["H"] * c["F"] * 34 // 32
+    shared_bytes = 3 * c["H"] * c["Fs"] * 34 // 32
+    step_bytes = n_active * expert_bytes + shared_bytes + c["E"] * c["H"] * 4 + 2 * B * c["H"] * 4
+    up_bytes = n_active * (2 * c["H"] * c["F"] * 34 // 32)
+    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+    traffic = profiled_traffic(B, "q32s_config4_kernel_trace.md", "config4") if B == 512 else None
+    roofline = {"bound": "hbm", "kernel": "routed up projection (w1, w3, SiLU, Q8_0 re-quantisation)",
+                "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                "traffic_source": "profiles/q32s_config4_kernel_trace.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
+                "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+    return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
+            "tokens": B, "active_experts": n_active, "max_expert_load": int(loads.max()), "stage_us": stage_us, "dispatch_us": stage_us["dispatch"],
+            "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "step_int8_ops": 2.0 * B * 3 * c["H"] * (c["k"] * c["F"] + c["Fs"]), "roofline": roofline, "xs": xs, "ys": ys}
+
+
+def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32):
+    """BASELINE config 5: `n_layers` Mixtral-shape MoE layers chained, each with its own resident copy of its weights and its
+    own gate; layer l's experts are the drawn eight rotated by l places (timing does not depend on the values, and drawing
+    26 GB of distinct blocks would only lengthen the set-up)."""
     g = torch.Generator(device="cuda")
     g.manual_seed(5)
     layers = []
-    for l in range(args.layers):
+    for l in range(n_layers):
         r = l % E
         gate = (torch.randn((E, H), generator=g, device="cuda", dtype=torch.float32) * 0.02).cpu().numpy()
         alpha = (1.0 + 0.1 * torch.randn((H,), generator=g, device="cuda", dtype=torch.float32)).cpu().numpy()
@@ -159,42 +302,23 @@ def run_stack(args, np, torch, candle_amd):
                                                 w["w2"][r:] + w["w2"][:r], rms_alpha=alpha, rms_eps=1e-5))
     x0 = torch.randn((B, H), generator=g, device="cuda", dtype=torch.float32)
     bufs = [torch.empty_like(x0) for _ in range(2)]
-    noise, x_next = torch.empty_like(x0), torch.empty_like(x0)
+    noise, state = torch.empty_like(x0), {"h": x0}
+    x_next = torch.empty_like(x0)
 
-    def step(h):
+    def step(_):
+        h = state["h"]
         for i, layer in enumerate(layers):
             layer.forward(h, out=bufs[i & 1])
             h = bufs[i & 1]
         noise.normal_(0.0, 0.1, generator=g)
-        return torch.add(h, noise, out=x_next)   # the next step's input
+        state["h"] = torch.add(h, noise, out=x_next)   # the next step's input
 
-    stream = torch.cuda.Stream()
-    hip = hip_events()
-    with torch.cuda.stream(stream):
-        h = x0
-        for _ in range(args.warmup):
-            h = step(h)
-        stream.synchronize()
-        ev = [C.c_void_p() for _ in range(2)]
-        for e in ev:
-            hip.hipEventCreate(C.byref(e))
-        sh = C.c_void_p(stream.cuda_stream)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        hip.hipEventRecord(ev[0], sh)
-        for _ in range(args.steps):
-            h = step(h)
-        hip.hipEventRecord(ev[1], sh)
-        hip.hipEventSynchronize(ev[1])
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        ms = C.c_float()
-        hip.hipEventElapsedTime(C.byref(ms), ev[0], ev[1])
-        ms_per_step = ms.value / args.steps
-        finite = bool(torch.isfinite(h).all())
-        # stage times of a mid-stack layer, measured right after its predecessors ran (its weights and gate are cold)
-        mid = len(layers) // 2
-        stage = {k: 0.0 for k in layers[mid].STAGES}
+    ms, wall_ms, warmed = timer.run(step, n_steps, min(args.warmup, 3), min_warm_seconds=0.3)
+    finite = bool(torch.isfinite(state["h"]).all())
+    # stage times of a mid-stack layer, measured right after its predecessors ran (its weights and gate are cold)
+    mid = len(layers) // 2
+    stage = {k: 0.0 for k in layers[mid].STAGES}
+    with torch.cuda.stream(timer.stream):
         for _ in range(5):
             hh = x0
             for i, layer in enumerate(layers[:mid]):
@@ -208,32 +332,31 @@ def run_stack(args, np, torch, candle_amd):
     up_bytes = n_active * (2 * H * F * 144 // 256) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
     achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
     step_bytes = len(layers) * (n_active * EXPERT_BYTES + E * H * 4 + 3 * B * H * 4)
-    out = {
-        "metric": "MoE stack tokens/s end to end (%d Mixtral-8x7B MoE layers, Q4_K, decode)" % len(layers),
-        "value": B / (ms_per_step * 1e-3), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8", "data": "synthetic",
-        "config": {"workload": "BASELINE config 5: %d chained MoE layers (hidden 4096, ffn 14336, 8 experts, top-2, Q4_K, %.1f GB "
-                               "resident), y = x + moe(rms_norm(x)) per layer, %d-token batch, each step fed the previous output "
-                               "plus N(0, 0.1) noise" % (len(layers), len(layers) * E * EXPERT_BYTES / 1e9, B),
-                   "layers": len(layers), "us_per_layer": ms_per_step * 1e3 / len(layers), "wall_ms_per_step": wall * 1e3 / args.steps,
-                   "mid_stack_stage_us": stage_us, "output_finite": finite,
-                   "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        "roofline": {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation), layer %d of the stack" % mid,
-                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]},
-    }
-    print(json.dumps(out))
+    for layer in layers:
+        layer.close()
+    return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
+            "layers": n_layers, "batch": B, "resident_gb": n_layers * E * EXPERT_BYTES / 1e9, "us_per_layer": ms * 1e3 / n_layers,
+            "mid_stack_stage_us": stage_us, "output_finite": finite, "step_algorithmic_bytes": step_bytes,
+            "step_hbm_frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+            "roofline": {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation), layer %d of the stack" % mid,
+                         "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                         "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}}
+
+
+def sub(m):
+    """A measurement as a sub-object of `config`: everything but the tensors."""
+    return {k: v for k, v in m.items() if k not in ("xs", "ys")}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 200; 128 for the stack workload)")
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=200, help="timed steps K (at least 200 are timed; the stack times its own 128)")
+    ap.add_argument("--warmup", type=int, default=20, help="warm-up steps, on top of the 0.5 s every measurement warms up for")
     ap.add_argument("--batch", type=int, default=None, help="tokens per step (default 32 for decode, 4096 for prefill, 512 for config4)")
-    ap.add_argument("--workload", choices=("decode", "prefill", "config4", "stack"), default="decode")
+    ap.add_argument("--workload", choices=("all", "decode", "prefill", "config4", "stack"), default="all")
     ap.add_argument("--layers", type=int, default=32, help="layers of the stack workload")
+    ap.add_argument("--stack-steps", type=int, default=128, help="consecutive steps of the stack workload")
     ap.add_argument("--weights", choices=sorted(FORMATS), default="q4_k", help="GGML format of the expert matrices (decode workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
@@ -259,135 +382,94 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
-    if args.steps is None:
-        args.steps = 128 if args.workload == "stack" else 200
-    if args.workload == "stack":
-        if args.weights != "q4_k":
-            sys.exit("bench.py: --weights applies to the decode workload only")
-        return run_stack(args, np, torch, candle_amd)
-    prefill = args.workload == "prefill"
-    cfg4 = args.workload == "config4"
-    B = args.batch or (4096 if prefill else 512 if cfg4 else 32)
-    bias = np.array(ZIPF_BIAS, dtype=np.float32) if prefill else None
-    if args.weights != "q4_k" and args.workload != "decode":
+    wl = args.workload
+    if args.weights != "q4_k" and wl not in ("decode", "all"):
         sys.exit("bench.py: --weights applies to the decode workload only")
-    layer, gate, w = build_layer(torch, candle_amd, gate_bias=bias, cfg4=cfg4, fmt=args.weights)
-    fmt_dt, fmt_be, fmt_bb, _ = FORMATS[args.weights]
-    n_exp, hid = (CFG4["E"], CFG4["H"]) if cfg4 else (E, H)
-    g = torch.Generator(device="cuda")
-    g.manual_seed(2)
-    # several distinct activation batches, rotated, so that no step repeats the previous one's input
-    xs = [torch.randn((B, hid), generator=g, device="cuda", dtype=torch.float32) for _ in range(4)]
-    ys = [torch.empty_like(x) for x in xs]
+    if args.weights != "q4_k":
+        wl = "decode"
+    timer = Timer(torch)
+    out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "i8", "data": "synthetic", "unit": "tokens/s"}
+    bias = np.array(ZIPF_BIAS, dtype=np.float32)
+    cpu = None
 
-    stream = torch.cuda.Stream()
-    hip = hip_events()
-    with torch.cuda.stream(stream):
-        for i in range(args.warmup):
-            layer.forward(xs[i % 4], out=ys[i % 4])
-        stream.synchronize()
-        loads = np.diff(layer.last_routing(B)[2])[:n_exp]
-        n_active = int((loads > 0).sum())
-        ev = [C.c_void_p() for _ in range(2)]
-        for e in ev:
-            hip.hipEventCreate(C.byref(e))
-        sh = C.c_void_p(stream.cuda_stream)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        hip.hipEventRecord(ev[0], sh)
-        for i in range(args.steps):
-            layer.forward(xs[i % 4], out=ys[i % 4])
-        hip.hipEventRecord(ev[1], sh)
-        hip.hipEventSynchronize(ev[1])
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        ms = C.c_float()
-        hip.hipEventElapsedTime(C.byref(ms), ev[0], ev[1])
-        ms_per_step = ms.value / args.steps
-        tokens_per_s = B / (ms_per_step * 1e-3)
-
-        # per-stage durations: HIP events recorded by the library between its launches, same stream
-        stage = {k: 0.0 for k in layer.STAGES}
-        for i in range(args.stage_iters):
-            for k, v in layer.forward_timed(xs[i % 4], ys[i % 4]).items():
-                stage[k] += v / args.stage_iters
-    stage_us = {k: round(v * 1e3, 2) for k, v in stage.items()}
-
-    expert_bytes = 3 * H * F * fmt_bb // fmt_be
-    step_bytes = n_active * expert_bytes + E * H * 4 + 2 * B * H * 4
-    metric = "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, %s)" % args.workload
-    if cfg4:
-        # Weights are Q8_0 (34 bytes per 32 elements); every routed expert with a token and the shared expert are
-        # read at least once per step.  The up kernel (w1, w3 of the routed experts) is the longest launch.
-        c = CFG4
-        expert_bytes = 3 * c["H"] * c["F"] * 34 // 32
-        shared_bytes = 3 * c["H"] * c["Fs"] * 34 // 32
-        step_bytes = n_active * expert_bytes + shared_bytes + c["E"] * c["H"] * 4 + 2 * B * c["H"] * 4
-        up_bytes = n_active * (2 * c["H"] * c["F"] * 34 // 32)
-        achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
-        step_ops = 2.0 * B * 3 * c["H"] * (c["k"] * c["F"] + c["Fs"])
-        roofline = {"bound": "hbm", "kernel": "q32s_up (routed w1, w3, SiLU, Q8_0 re-quantisation; lists beyond 32 rows re-read the weights from L2)",
-                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                    "traffic": measured_traffic(B, "q32s_config4_kernel_trace.md", "config4") if B == 512 else None,
-                    "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
-        workload = ("BASELINE config 4: hidden 2048, 60 experts of ffn 1408, top-4 renormalised, shared expert of ffn 5632 "
-                    "with sigmoid gate, Q8_0 weights, %d tokens" % B)
-        extra = {"step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                 "step_int8_ops": step_ops, "dispatch_us": stage_us["dispatch"], "max_expert_load": int(loads.max())}
-        metric = "MoE layer tokens/s (Qwen-MoE shape, Q8_0, 512-token batch)"
-    elif prefill:
-        # Roofline of the dominant kernel, the tiled up projection: 2 * slots * 2 * H * F integer
-        # multiply-adds (w1 and w3) per launch against the dense int8 MFMA peak.
-        up_ops = 2.0 * B * TOPK * 2 * H * F
-        achieved = up_ops / (stage["up"] * 1e-3) / 1e12
-        step_ops = 2.0 * B * TOPK * 3 * H * F
-        roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, two scale planes)",
-                    "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": achieved / INT8_PEAK_TOPS,
-                    "traffic": None, "algorithmic_ops_per_launch": up_ops, "launch_us": stage_us["up"],
-                    # every algorithmic multiply-add is issued twice (the 6-bit scale is split over two
-                    # pre-scaled int8 planes so that the integer sums stay exact): share of the peak the
-                    # MFMA pipe is actually kept busy with, slot tiles padded to 64 / 128 not counted
-                    "mfma_issued_frac": 2.0 * achieved / INT8_PEAK_TOPS}
-        workload = ("BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, prefill of %d tokens, "
-                    "Zipf(1) expert load" % B)
-        extra = {"expert_loads": [int(v) for v in loads], "step_int8_ops": step_ops,
-                 "step_mfma_frac": step_ops / (ms_per_step * 1e-3) / 1e12 / INT8_PEAK_TOPS}
+    if wl == "config4":
+        w4 = draw_weights(torch, candle_amd, cfg4=True)
+        layer = make_layer(candle_amd, w4, cfg4=True)
+        B = args.batch or 512
+        m = measure_cfg4(args, np, torch, timer, layer, B)
+        out.update(metric="MoE layer tokens/s (Qwen-MoE shape, Q8_0, 512-token batch)", value=m["tokens_per_s"], ms_per_step=m["ms_per_step"],
+                   timed_steps=m["timed_steps"], roofline=m["roofline"],
+                   config=dict({"workload": "BASELINE config 4: hidden 2048, 60 experts of ffn 1408, top-4 renormalised, shared expert of ffn 5632 "
+                                            "with sigmoid gate, Q8_0 weights, %d tokens" % B}, **{k: v for k, v in sub(m).items() if k != "roofline"}))
+        if not args.no_cpu_baseline:
+            n_cpu = min(B, 64)
+            layer.forward(m["xs"][0], out=m["ys"][0])
+            torch.cuda.synchronize()
+            cpu = cpu_baseline(w4, m["xs"][0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu], args.cpu_seconds, cfg4=True)
+    elif wl == "stack":
+        w = draw_weights(torch, candle_amd)
+        m = measure_stack(args, np, torch, candle_amd, timer, w, args.layers, args.stack_steps, args.batch or 32)
+        out.update(metric="MoE stack tokens/s end to end (%d Mixtral-8x7B MoE layers, Q4_K, decode)" % args.layers, value=m["tokens_per_s"],
+                   ms_per_step=m["ms_per_step"], timed_steps=m["timed_steps"], roofline=m["roofline"],
+                   config=dict({"workload": "BASELINE config 5: %d chained MoE layers (hidden 4096, ffn 14336, 8 experts, top-2, Q4_K, %.1f GB resident), "
+                                            "y = x + moe(rms_norm(x)) per layer, %d-token batch, each step fed the previous output plus N(0, 0.1) noise"
+                                            % (args.layers, m["resident_gb"], m["batch"])}, **{k: v for k, v in m.items() if k != "roofline"}))
+    elif wl == "prefill":
+        w = draw_weights(torch, candle_amd)
+        layer = make_layer(candle_amd, w, gate_bias=bias)
+        B = args.batch or 4096
+        m = measure_prefill(args, np, torch, timer, layer, B)
+        out.update(metric="MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, prefill)", value=m["tokens_per_s"], ms_per_step=m["ms_per_step"],
+                   timed_steps=m["timed_steps"], roofline=m["roofline"],
+                   config=dict({"workload": "BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, prefill of %d tokens, "
+                                            "Zipf(1) expert load" % B}, **{k: v for k, v in sub(m).items() if k != "roofline"}))
+        if not args.no_cpu_baseline:
+            n_cpu = min(B, 64)   # a bounded sample: the CPU path does ~1 k tokens/s
+            cpu = cpu_baseline(w, m["xs"][0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu], args.cpu_seconds, gate_bias=bias)
     else:
-        # Roofline of the dominant kernel, the up projection (w1, w3 + SiLU): it streams w1 and w3 of
-        # every active expert exactly once per launch; algorithmic bytes = Q4_K bytes of those matrices
-        # plus the quantised activations it reads and the quantised intermediate it writes.
-        act = 36 / 256 if fmt_be == 256 else 8 / 32    # bytes of scales and sums per quantised activation element
-        up_bytes = n_active * (2 * H * F * fmt_bb // fmt_be) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
-        achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
-        q4k = args.weights == "q4_k"
-        roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)" if q4k else "up projection (w1, w3, SiLU, re-quantisation), %s" % args.weights,
-                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                    "traffic": measured_traffic(B) if q4k else None,
-                    "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
+        fmt = args.weights
+        w = draw_weights(torch, candle_amd, fmt=fmt)
+        layer = make_layer(candle_amd, w)
+        B = args.batch or 32
+        m = measure_decode(args, np, torch, timer, layer, B, fmt)
+        q4k = fmt == "q4_k"
         workload = "BASELINE config 2: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, decode batch %d" % B
+        metric = "MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, decode)"
         if not q4k:
-            workload = "BASELINE config 2's layer with %s weights (random block payloads), decode batch %d" % (args.weights, B)
-            metric = "MoE layer tokens/s (Mixtral-8x7B shape, %s, decode)" % args.weights
-        extra = {"step_algorithmic_bytes": step_bytes,
-                 "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS}
-    out = {
-        "metric": metric, "value": tokens_per_s, "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "i8",
-        "data": "synthetic",
-        "config": dict({"workload": workload, "active_experts": n_active,
-                        "wall_ms_per_step": wall * 1e3 / args.steps, "stage_us": stage_us,
-                        # a stage that launches nothing still reads what its pair of event records costs
-                        "empty_stage_us": min(stage_us.values())}, **extra),
-        "roofline": roofline,
-    }
-    if not args.no_cpu_baseline:
-        layer.forward(xs[0], out=ys[0])
-        torch.cuda.synchronize()
-        # a bounded sample: the CPU path does ~1 k tokens/s, so a prefill batch is cut to its first 64 tokens
-        n_cpu = min(B, 64)
-        out["cpu_baseline"] = cpu_baseline(gate, w, xs[0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu],
-                                           args.cpu_seconds, gate_bias=bias, cfg4=cfg4, dt=fmt_dt)
+            workload = "BASELINE config 2's layer with %s weights (random block payloads), decode batch %d" % (fmt, B)
+            metric = "MoE layer tokens/s (Mixtral-8x7B shape, %s, decode)" % fmt
+        cfg = dict({"workload": workload}, **{k: v for k, v in sub(m).items() if k != "roofline"})
+        out.update(metric=metric, value=m["tokens_per_s"], ms_per_step=m["ms_per_step"], timed_steps=m["timed_steps"], roofline=m["roofline"], config=cfg)
+        if not args.no_cpu_baseline:
+            layer.forward(m["xs"][0], out=m["ys"][0])
+            torch.cuda.synchronize()
+            cpu = cpu_baseline(w, m["xs"][0].cpu().numpy(), layer.last_logits(B), args.cpu_seconds)
+        if wl == "all":
+            out["metric"] = "MoE layer tokens/s; decode HBM GB/s %peak; prefill MFMA util, Mixtral-8x7B Q4_K"
+            # prefill on the same weights, with the router bias that skews the load
+            pl = make_layer(candle_amd, w, gate_bias=bias)
+            mp = measure_prefill(args, np, torch, timer, pl, 4096)
+            cfg["prefill"] = dict({"workload": "BASELINE config 3: the same layer, prefill of 4096 tokens, Zipf(1) expert load"}, **sub(mp))
+            pl.close()
+            del mp
+            w4 = draw_weights(torch, candle_amd, cfg4=True)
+            l4 = make_layer(candle_amd, w4, cfg4=True)
+            m4 = measure_cfg4(args, np, torch, timer, l4, 512)
+            cfg["cfg4"] = dict({"workload": "BASELINE config 4: hidden 2048, 60 experts of ffn 1408, top-4, shared expert of ffn 5632, Q8_0, 512 tokens"}, **sub(m4))
+            l4.close()
+            del m4, w4
+            layer.close()
+            ms_ = measure_stack(args, np, torch, candle_amd, timer, w, args.layers, args.stack_steps)
+            cfg["stack"] = dict({"workload": "BASELINE config 5: %d chained layers, y = x + moe(rms_norm(x)), 32-token batch, %d steps"
+                                             % (args.layers, args.stack_steps)}, **ms_)
+            # the three quantities the metric names, side by side
+            cfg["summary"] = {"decode_tokens_per_s": m["tokens_per_s"], "decode_step_hbm_frac": m["step_hbm_frac"],
+                              "decode_up_kernel_hbm_frac": m["roofline"]["frac"], "prefill_tokens_per_s": cfg["prefill"]["tokens_per_s"],
+                              "prefill_up_kernel_int8_frac": cfg["prefill"]["roofline"]["frac"], "prefill_step_int8_frac": cfg["prefill"]["step_mfma_frac"],
+                              "cfg4_tokens_per_s": cfg["cfg4"]["tokens_per_s"], "stack_tokens_per_s": cfg["stack"]["tokens_per_s"]}
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 
