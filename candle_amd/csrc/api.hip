@@ -273,7 +273,7 @@ struct Workspace {
 
 // Which kernels a forward of T tokens takes.
 struct ForwardPlan {
-    bool tiled = false, tiled_down = false, direct = false, accumulate = false, narrow = false, hbuf = false;
+    bool tiled = false, tiled_down = false, tiled32 = false, direct = false, accumulate = false, narrow = false, hbuf = false;
     int tile_slots = 128, slot_tiles = 1;
 };
 
@@ -289,6 +289,10 @@ struct moe_layer {
     GrowBuf ws;                     // per-call workspace, grown on demand, cut anew for every call
     DevBuf x_dev, y_dev;            // staging of the host-pointer entry
     hipStream_t stream = nullptr;   // used by the host-pointer entry
+    // layers with a shared expert: its two kernels run on this stream beside the routed experts' (fork after the front
+    // kernels, join before the combine pass); nothing but the workspace pieces of its own is shared with them
+    hipStream_t side = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
     CallOrder order;
     int64_t last_T = 0;             // -1: several passes, -2: a layer with top_k = 0 routes nothing
     bool last_direct = false;       // the last forward skipped the dispatch pass
@@ -405,6 +409,15 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
         return bail(MOE_E_HIP);
     }
     if ((rc = L->order.init())) return bail(rc);
+    if (L->Fs > 0) {
+        e = hipStreamCreateWithFlags(&L->side, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->fork, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->join, hipEventDisableTiming);
+        if (e != hipSuccess) {
+            fail(MOE_E_HIP, std::string("layer setup: ") + hipGetErrorString(e));
+            return bail(MOE_E_HIP);
+        }
+    }
     *out = L;
     return MOE_OK;
 }
@@ -413,6 +426,9 @@ extern "C" void moe_layer_destroy(moe_layer* L) {
     if (!L) return;
     (void)hipDeviceSynchronize();
     if (L->stream) (void)hipStreamDestroy(L->stream);
+    if (L->side) (void)hipStreamDestroy(L->side);
+    if (L->fork) (void)hipEventDestroy(L->fork);
+    if (L->join) (void)hipEventDestroy(L->join);
     L->order.destroy();
     delete L;
 }
@@ -463,6 +479,10 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     pl.narrow = pl.direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && pl.slot_tiles == 1 &&
                 (sw.narrow >= 0 ? sw.narrow > 0 : T * L->k <= L->E);
     pl.hbuf = pl.tiled || pl.narrow;
+    // Q8_0 layers whose slots are grouped by expert (more than DIRECT_MAX_SLOTS assignments): the tiled kernels of
+    // kernels_q32.hip read an expert's weights once for up to 64 of its slots
+    pl.tiled32 = !sw.no_gemm && !pl.direct && q8_0_gemm_usable(L->dt, L->dt_down, L->H, L->F) && T * L->k > 20 * L->E;
+    if (pl.tiled32) pl.tile_slots = 64;
     return pl;
 }
 
@@ -525,6 +545,32 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
     ep.y_acc = pl.accumulate ? d_y : nullptr;
     ep.max_rows = T;
     ep.slot_tiles = pl.slot_tiles;
+    // The always-on expert reads the quantised activations and writes its own slots of yw: independent of the routed
+    // experts until the combine pass, so its kernels go to the side stream and fill the CUs the routed launches leave idle
+    // (the timed entry keeps one stream: its stage marks would mean nothing otherwise).
+    const bool overlap_shared = shared && !marks;
+    hipStream_t ss = overlap_shared ? L->side : s;
+    auto run_shared = [&]() -> int {
+        ExpertParams sp = ep;
+        // the always-on expert takes the regular kernels (which quantise its intermediate in their epilogue) also when
+        // the routed experts of a tiny batch took the narrow ones with their separate quantisation pass
+        sp.hbuf = nullptr; sp.by_assignment = 0;
+        sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
+        sp.groups = L->groups.as<GroupWeights>() + L->E;
+        sp.hq = ws.hq_shared; sp.slot_origin = (int)(T * L->k);
+        sp.max_rows = T; sp.slot_tiles = T > 32 ? 4 : T > 16 ? 2 : 1;
+        // (measured at the Qwen-MoE shape, 512 tokens: the streaming kernels take 112 us for the always-on expert, the
+        // 64-slot tiled ones 183 us: its eight tiles by sixteen row blocks leave half of the CUs without a down workgroup)
+        MOE_HIP_CHECK(launch_expert_up(sp, ss));
+        MOE_HIP_CHECK(launch_expert_down(sp, ss));
+        return MOE_OK;
+    };
+    if (overlap_shared) {
+        MOE_HIP_CHECK(hipEventRecord(L->fork, s));
+        MOE_HIP_CHECK(hipStreamWaitEvent(ss, L->fork, 0));
+        if (int rc = run_shared()) return rc;
+        MOE_HIP_CHECK(hipEventRecord(L->join, ss));
+    }
     if (pl.tiled) {
         ep.hbuf = ws.hbuf;
         ep.n_slots = T * L->k;
@@ -539,6 +585,13 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
             dp.hbuf = nullptr;
             MOE_HIP_CHECK(launch_expert_down(dp, s));
         }
+        MOE_MARK(ST_DOWN);
+    } else if (pl.tiled32) {
+        ep.n_slots = T * L->k;
+        MOE_HIP_CHECK(launch_q8_0_gemm_up(ep, s));   // quantises the intermediate in its epilogue
+        MOE_MARK(ST_UP);
+        MOE_MARK(ST_REQUANT);
+        MOE_HIP_CHECK(launch_q8_0_gemm_down(ep, s));
         MOE_MARK(ST_DOWN);
     } else if (pl.narrow) {
         ep.hbuf = ws.hbuf;
@@ -557,18 +610,9 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
         MOE_HIP_CHECK(launch_expert_down(ep, s));
         MOE_MARK(ST_DOWN);
     }
-    if (shared) {
-        ExpertParams sp = ep;
-        // the always-on expert takes the regular kernels (which quantise its intermediate in their epilogue) also when
-        // the routed experts of a tiny batch took the narrow ones with their separate quantisation pass
-        sp.hbuf = nullptr; sp.by_assignment = 0;
-        sp.F = (int)L->Fs; sp.n_groups = 1; sp.group0 = (int)L->E; sp.is_shared = 1;
-        sp.groups = L->groups.as<GroupWeights>() + L->E;
-        sp.hq = ws.hq_shared; sp.slot_origin = (int)(T * L->k);
-        sp.max_rows = T; sp.slot_tiles = T > 32 ? 4 : T > 16 ? 2 : 1;
-        MOE_HIP_CHECK(launch_expert_up(sp, s));
-        MOE_HIP_CHECK(launch_expert_down(sp, s));
-    }
+    if (overlap_shared) MOE_HIP_CHECK(hipStreamWaitEvent(s, L->join, 0));
+    else if (shared)
+        if (int rc = run_shared()) return rc;
     MOE_MARK(ST_SHARED);
     if (!pl.accumulate) MOE_HIP_CHECK(launch_combine(ws.yw, fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
     MOE_MARK(ST_COMBINE);

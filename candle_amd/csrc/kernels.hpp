@@ -110,6 +110,14 @@ hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 
+// Tiled products for Q8_0 layers whose slots are grouped by expert (tiles of 64 slots, rb.tile_slots == 64; F a multiple
+// of 128 for the reduction of w2 and of 64 for the row blocks of w1 / w3, H a multiple of 128): up quantises the
+// intermediate into p.hq in its epilogue, down writes yw.  With p.is_shared the launch covers the always-on expert
+// (one group of p.max_rows tokens) and needs no tile list.
+bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F);
+hipError_t launch_q8_0_gemm_up(const ExpertParams& p, hipStream_t s);
+hipError_t launch_q8_0_gemm_down(const ExpertParams& p, hipStream_t s);
+
 // y[t] = sum over the token's slots (ascending expert index, shared expert last) of yw[slot] (+ residual[t]).
 hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,
                           int64_t T, int H, hipStream_t s);

@@ -691,6 +691,235 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Tiled grouped products for Q8_0 weights (batches whose slots are grouped by expert): one pass over an expert's
+// weights for up to 64 of its slots, where the streaming kernels above take a pass per 32.
+//
+// Same arithmetic and the same order of additions as q32s_mac (bit-identical results): one
+// v_mfma_i32_16x16x32_i8 per 32-element block, its four integers per lane turned into
+// ((isum as f32) * d_w) * d_x and added in ascending block order.  Three vector instructions per result and
+// block is what exactness costs, so these kernels are bound by the vector ALU, not by HBM; what the tiled
+// form buys is one read of the weights per 64 slots and enough independent work per wave to keep that ALU busy.
+//
+// Work split: a workgroup (8 waves) owns one tile of up to 64 slots of one group (from the dispatch kernel's tile
+// list; the always-on expert's tiles follow from the token count) and eight 16-row weight operands, one per wave
+// (MODE 0: four of w1 and the same rows of w3; MODE 1: eight of w2).  Per K step of 128 (four blocks, one super-tile
+// per wave) the tile's quants go from global memory straight into LDS as 16-byte pieces ([operand][piece][slot], piece
+// p = bytes 16p .. 16p+15 of the step: the two dwords of a lane's MFMA operand are 256 bytes apart), with the scales
+// of the step's four blocks per slot beside them; both double-buffered, one barrier per step.  16-slot operands past
+// the end of the list are skipped, so the work follows the list length in steps of 16.
+constexpr int QG_NOP = 4;
+constexpr int QG_THREADS = 512;
+struct alignas(16) QGemmLds {
+    alignas(16) uint8_t q[2][QG_NOP][8][256];       // [buffer][operand][piece][slot m] 16 bytes
+    alignas(16) float yd[2][QG_NOP * 16][4];          // [buffer][slot][block of the step]
+};
+__device__ __forceinline__ uint32_t qg_lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+// direct global -> LDS load: lane i of the wave writes 16 bytes at lds + 16 i (the issuing wave waits for it with vmcnt)
+__device__ __forceinline__ void qg_dma16(const void* gbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbase), "s"(lds));
+}
+
+template <int MODE>
+__global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q8_0_gemm_kernel(ExpertParams p) {
+    constexpr int DT = MOE_GGML_Q8_0;
+    constexpr size_t STB = Q32SFmt<DT>::STB;
+    __shared__ QGemmLds L;
+    __shared__ float hx[MODE == 0 ? QG_NOP * 16 : 1][MODE == 0 ? 65 : 1];   // MODE 0: h of the tile's slots x the workgroup's 64 rows
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // workgroup -> (row block, slot tile): 8 x 8 patches per XCD, as in q4k_gemm_kernel
+    const int n_rb = MODE == 0 ? p.F / 64 : p.H / 128;
+    const int RG = (n_rb + 7) / 8;
+    const int xcd = blockIdx.x & 7, qq = blockIdx.x >> 3;
+    const int st = (qq >> 6) * 8 + xcd, within = qq & 63;
+    const int rblk = (st % RG) * 8 + (within & 7);
+    const int tile = (st / RG) * 8 + (within >> 3);
+    if (rblk >= n_rb) return;
+    int gi, pos0;
+    if (p.is_shared) {   // one group holding every token: its tiles need no list
+        gi = p.group0; pos0 = tile * (QG_NOP * 16);
+        if (pos0 >= p.rb.T) return;
+    } else {
+        if (tile >= p.rb.tile_tab[0]) return;
+        gi = p.rb.tile_tab[1 + 2 * tile]; pos0 = p.rb.tile_tab[2 + 2 * tile];
+        if (gi < p.group0 || gi >= p.group0 + p.n_groups) return;
+    }
+    const int grp = gi - p.group0;
+    const int s_begin = p.rb.offsets[gi], n_g = p.rb.offsets[gi + 1] - s_begin;
+    const int n_here = n_g - pos0 < QG_NOP * 16 ? n_g - pos0 : QG_NOP * 16;   // slots of this tile
+    const int n_op = __builtin_amdgcn_readfirstlane((n_here + 15) >> 4);       // live 16-slot operands
+    const int K = MODE == 0 ? p.H : p.F;
+    const int N = MODE == 0 ? p.F : p.H;
+    const int nks = K / 128, nkb = K / 32;
+    const size_t step_stride = (size_t)(N / 16) * STB;
+    const ActBuf& ab = MODE == 0 ? p.xq : p.hq;
+
+    auto act_row = [&](int r) {   // positions past the list repeat its last row (read, never stored)
+        const int pos = pos0 + r;
+        const int slot = s_begin + (pos < n_g ? pos : n_g - 1);
+        return MODE == 0 ? p.rb.perm_token[slot] : slot - p.slot_origin;
+    };
+    // transfers of a step: wave w stages half w % 2 (pieces 4 (w % 2) .. +3) of operand w / 2; wave 0 also the scales
+    const uint32_t q_src = (uint32_t)act_row(16 * (wave >> 1) + (lane & 15)) * (uint32_t)K + (uint32_t)((4 * (wave & 1) + (lane >> 4)) * 16);
+    const uint32_t d_src = (uint32_t)act_row(lane) * (uint32_t)nkb * 4u;
+    auto stage = [&](int ks, int buf) {
+        qg_dma16(ab.qs, q_src + (uint32_t)(ks * 128), qg_lds_address(&L.q[buf][wave >> 1][4 * (wave & 1)][0]));
+        if (wave == 0) qg_dma16(ab.d, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.yd[buf][0][0]));
+    };
+
+    const GroupWeights gw = p.groups[grp];
+    const uint8_t* wp;
+    int row0;
+    if (MODE == 0) {
+        row0 = rblk * 64 + (wave & 3) * 16;
+        wp = (wave < 4 ? gw.w1 : gw.w3) + (size_t)(row0 / 16) * STB;
+    } else {
+        row0 = rblk * 128 + wave * 16;
+        wp = gw.w2 + (size_t)(row0 / 16) * STB;
+    }
+    const int m = lane & 15, g = lane >> 4;
+    float acc[QG_NOP][4];
+#pragma unroll
+    for (int o = 0; o < QG_NOP; o++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[o][i] = 0.f;
+
+    stage(0, 0);
+    Q32SRaw<DT> cur = load_q32s<DT, false>(wp, lane);
+    Q32SRaw<DT> nxt = load_q32s<DT, false>(wp + (size_t)(1 < nks ? 1 : 0) * step_stride, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    __syncthreads();
+    const v4i magic = {Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS};
+    for (int ks = 0; ks < nks; ks++) {
+        const int buf = ks & 1;
+        const int ks1 = ks + 1 < nks ? ks + 1 : ks, ks2 = ks + 2 < nks ? ks + 2 : nks - 1;
+        stage(ks1, buf ^ 1);
+        const Q32SRaw<DT> w = cur;
+        cur = nxt;
+        nxt = load_q32s<DT, false>(wp + (size_t)ks2 * step_stride, lane);
+        const Q32Tile<DT> w0 = q32s_block<DT, 0>(w, g), w1 = q32s_block<DT, 1>(w, g), w2 = q32s_block<DT, 2>(w, g), w3 = q32s_block<DT, 3>(w, g);
+        const float dwv[4] = {w0.d, w1.d, w2.d, w3.d};
+        const uint2 wq[4] = {w0.q, w1.q, w2.q, w3.q};
+        float cneg[4];
+#pragma unroll
+        for (int b = 0; b < 4; b++) cneg[b] = -(Q32S_MAGIC * dwv[b]);
+#pragma unroll
+        for (int o = 0; o < QG_NOP; o++) {
+            if (o < n_op) {   // wave-uniform
+                f32x4g ydv[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) ydv[i] = *reinterpret_cast<const f32x4g*>(&L.yd[buf][o * 16 + 4 * g + i][0]);
+                v4i D[4];
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const uint8_t* ap = &L.q[buf][o][2 * b][0] + m * 16 + 4 * g;
+                    const uint32_t alo = *reinterpret_cast<const uint32_t*>(ap), ahi = *reinterpret_cast<const uint32_t*>(ap + 256);
+                    const long av = (long)(((uint64_t)ahi << 32) | alo);
+                    const long bv = (long)(((uint64_t)wq[b].y << 32) | wq[b].x);
+                    D[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, magic, 0, 0, 0);
+                }
+                // ascending block order per (row, slot), every product rounded where the reference rounds it
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        float t = __builtin_fmaf(__int_as_float(D[b][i]), dwv[b], cneg[b]);
+                        t = t * ydv[i][b];
+                        acc[o][i] += t;
+                    }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // the next step's transfers (and tiles) have landed
+        __syncthreads();
+    }
+
+    // epilogue: lane holds weight row n = lane % 16 and slots 16 o + 4 (lane / 16) + i
+    const int n = lane & 15;
+    if (MODE == 0) {
+        // w3 waves (4-7) park their sums in LDS (the staging buffers are free now), w1 waves combine
+        float* xch = reinterpret_cast<float*>(&L.q[0][0][0][0]);   // [4 waves][QG_NOP][4 i][64 lanes] floats
+        static_assert(4 * QG_NOP * 4 * 64 * 4 <= sizeof(L.q), "exchange area");
+        if (wave >= 4) {
+#pragma unroll
+            for (int o = 0; o < QG_NOP; o++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) xch[(((wave - 4) * QG_NOP + o) * 4 + i) * 64 + lane] = acc[o][i];
+        }
+        __syncthreads();
+        if (wave < 4) {
+#pragma unroll
+            for (int o = 0; o < QG_NOP; o++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float up = xch[((wave * QG_NOP + o) * 4 + i) * 64 + lane];
+                    hx[o * 16 + 4 * g + i][wave * 16 + n] = silu_ref32(acc[o][i]) * up;
+                }
+        }
+        __syncthreads();
+        // Q8_0 blocks of h (BlockQ8_0::from_float, k_quants.rs:605-634): the workgroup's 64 rows are two blocks per slot;
+        // half a wave quantises one (slot, block)
+        const int nfb = p.F / 32;
+#pragma unroll
+        for (int it = 0; it < QG_NOP * 16 * 2 / 16; it++) {
+            const int pair = (wave * (QG_NOP * 2) + it) * 2 + (lane >> 5);
+            const int slot_in_tile = pair >> 1, blk = pair & 1, e = lane & 31;
+            const float x = hx[slot_in_tile][blk * 32 + e];
+            float amax = fabsf(x);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const float d = amax / 127.0f;
+            const float id = (d != 0.f) ? 1.0f / d : 0.f;
+            const int q = sat_i8(roundf(x * id));
+            int sum = q;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+            if (slot_in_tile < n_here) {
+                const int64_t hrow = s_begin + pos0 + slot_in_tile - p.slot_origin;
+                p.hq.qs[hrow * p.F + rblk * 64 + blk * 32 + e] = (int8_t)q;
+                if (e == 0) {
+                    const float dh = __half2float(__float2half_rn(d));
+                    p.hq.d[hrow * nfb + rblk * 2 + blk] = dh;
+                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + rblk * 2 + blk] = q8_block_word(MOE_GGML_Q8_0, sum, dh);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int o = 0; o < QG_NOP; o++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int pos = o * 16 + g * 4 + i;
+                if (pos >= n_here) continue;
+                const int slot = s_begin + pos0 + pos;
+                p.yw[(int64_t)slot * p.H + row0 + n] = acc[o][i] * p.rb.perm_w[slot];
+            }
+    }
+}
+
+bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F) {
+    return dt == MOE_GGML_Q8_0 && (dt_down == 0 || dt_down == MOE_GGML_Q8_0) && H % 128 == 0 && F % 128 == 0;
+}
+static unsigned qg_grid(int n_rb, int64_t tiles) {
+    const int64_t RG = (n_rb + 7) / 8, TG = (tiles + 7) / 8;
+    return (unsigned)((RG * TG + 7) / 8 * 8 * 64);
+}
+static int64_t qg_tiles(const ExpertParams& p) {
+    return p.is_shared ? (p.max_rows + QG_NOP * 16 - 1) / (QG_NOP * 16) : max_gemm_tiles(p.n_slots, p.n_groups + 1, QG_NOP * 16);
+}
+hipError_t launch_q8_0_gemm_up(const ExpertParams& p, hipStream_t s) {
+    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
+    hipLaunchKernelGGL((q8_0_gemm_kernel<0>), dim3(qg_grid(p.F / 64, qg_tiles(p))), dim3(QG_THREADS), 0, s, p);
+    return hipGetLastError();
+}
+hipError_t launch_q8_0_gemm_down(const ExpertParams& p, hipStream_t s) {
+    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
+    hipLaunchKernelGGL((q8_0_gemm_kernel<1>), dim3(qg_grid(p.H / 128, qg_tiles(p))), dim3(QG_THREADS), 0, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s);
 

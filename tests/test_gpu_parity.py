@@ -586,6 +586,30 @@ def test_rms_norm_as_an_operation_of_its_own(H):
         candle_amd.rms_norm(x[:, :H - 1], alpha[:H - 1], 1e-5)
 
 
+def test_shared_expert_layer_recorded_into_a_hip_graph():
+    # The always-on expert's kernels run on a side stream of the layer, forked after the front kernels and joined before
+    # the combine pass: under stream capture the fork and the join become edges of the graph.
+    torch = pytest.importorskip("torch")
+    ref, gpu = make_pair(256, 512, 12, 4, O.Q8_0, seed=36, Fs=1024)
+    xs = [torch.from_numpy(activations(40, 256, 80 + i)).cuda() for i in range(3)]
+    eager = [gpu.forward(x).clone() for x in xs]
+    gpu.forward(xs[0])
+    assert np.abs(eager[0].cpu().numpy() - ref.forward(xs[0].cpu().numpy(), logits=gpu.last_logits(40))).max() <= 2e-3 * rms(eager[0].cpu().numpy())
+    x_in, y_out = xs[0].clone(), torch.empty_like(xs[0])
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        gpu.forward(x_in, out=y_out)
+    for rep in range(3):
+        for x, w in zip(xs, eager):
+            x_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_out, w)
+            assert torch.equal(gpu.forward(x), w)
+    gpu.close()
+
+
 def test_empty_and_shape_errors():
     ref, gpu = make_pair(256, 256, 4, 2, O.Q4_0, seed=6)
     assert gpu.forward(np.zeros((0, 256), np.float32)).shape == (0, 256)
