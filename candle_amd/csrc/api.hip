@@ -455,9 +455,9 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
     // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
     // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
-    // (a Q6K w2 beside Q4K w1 / w3 keeps the tiled up kernel and streams the down projection)
+    // (a Q6K w2 beside Q4K w1 / w3, as mixed files carry, takes the tiled down kernel's Q6K variant)
     pl.tiled = !sw.no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 38 * L->E;
-    pl.tiled_down = pl.tiled && L->dt_down == MOE_GGML_Q4K && T * L->k > 64 * L->E;
+    pl.tiled_down = pl.tiled && (L->dt_down == MOE_GGML_Q4K || L->dt_down == MOE_GGML_Q6K) && T * L->k > 64 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 96 * L->E ? 128 : 64;

@@ -19,6 +19,12 @@
 // The 16-row operand keeps a wave below 128 VGPRs, so four waves share a SIMD: a single wave issues
 // at most one vector instruction every ~5 cycles and stalls on every MFMA result, and it takes that
 // many waves to keep the MFMA pipe and the vector ALU busy at the same time.
+//
+// Q6K weights (the w2 of mixed files) take the same kernel for the down projection.  BlockQ6K::vec_dot
+// (k_quants.rs:1613-1671) is d * y.d * sum_j sc_j * ((code_j - 32) . q8_j) with an i8 scale per 16 elements; the
+// products W = sc * (code - 32) (|W| <= 4096) are formed in packed 16-bit arithmetic and cut into two signed bytes,
+// W = 256 * H + L with L in [-128, 127], which are the two planes: 256 * acc_H + acc_L is the reference's integer, and
+// no term over the block sums is left.
 #include <type_traits>
 #include "act_quant.hpp"
 #include "kernels.hpp"
@@ -107,14 +113,23 @@ __device__ __forceinline__ void stage_piece(const ActBuf& ab, const StageRows& r
 // One wave's weights for one super-block: the 16 rows of one tile of the device layout.  Lane
 // (n = l%16, g = l/16) owns row n and k-chunk g of every sub-block: exactly the tile's own lane order.
 struct BRegs {
-    u32x4 c[2];   // plane pl: (x,y) = 8 bytes of pair 2pl, chunk g; (z,w) = pair 2pl+1
-    u32x4 hdr;    // d, dmin, 12 scale bytes of row n
+    u32x4 c[2];   // plane pl: (x,y) = 8 bytes of pair 2pl, chunk g; (z,w) = pair 2pl+1 (Q6K: the codes' low nibbles)
+    u32x4 hdr;    // Q4K: d, dmin, 12 scale bytes of row n; Q6K: the row's sixteen i8 scales
+    u32x4 qh;     // Q6K: the codes' top two bits, word P for pair P
+    uint32_t d16; // Q6K: d (f16 bits)
 };
+template <int FMT>
 __device__ __forceinline__ BRegs b_load(const uint8_t* tile, int lane) {
     BRegs b;
     b.c[0] = gld<u32x4>(tile, (uint32_t)(lane * 16));
     b.c[1] = gld<u32x4>(tile, (uint32_t)(1024 + lane * 16));
-    b.hdr = gld<u32x4>(tile, (uint32_t)(2048 + (lane & 15) * 16));
+    if (FMT == MOE_GGML_Q6K) {
+        b.qh = gld<u32x4>(tile, (uint32_t)(2048 + lane * 16));
+        b.hdr = gld<u32x4>(tile, (uint32_t)(3072 + (lane & 15) * 16));
+        b.d16 = gld<uint16_t>(tile, (uint32_t)(3328 + (lane & 15) * 2));
+    } else {
+        b.hdr = gld<u32x4>(tile, (uint32_t)(2048 + (lane & 15) * 16));
+    }
     return b;
 }
 
@@ -160,9 +175,54 @@ __device__ __forceinline__ BPlanes b_prepare(const BRegs& b, int lane) {
     return o;
 }
 
+// Q6K: both planes of W = sc * (code - 32).  A word of four codes is spread over two registers of two 16-bit lanes
+// (even and odd bytes), each multiplied and offset in one packed multiply-add: W + 128 = code * sc + (128 - 32 sc).
+// The high bytes of W + 128 are H = floor((W + 128) / 256); its low bytes, with the top bit flipped, are W - 256 H as a
+// signed byte.
+__device__ __forceinline__ uint32_t pk_mad_u16(uint32_t a, uint32_t b, uint32_t c) {
+    return __builtin_bit_cast(uint32_t, (u16x2)(__builtin_bit_cast(u16x2, a) * __builtin_bit_cast(u16x2, b) + __builtin_bit_cast(u16x2, c)));
+}
+__device__ __forceinline__ void q6k_planes(uint32_t codes, uint32_t s2, uint32_t add2, int& lo, int& hi) {
+    const uint32_t ev = codes & 0x00ff00ffu;
+    const uint32_t od = __builtin_amdgcn_perm(0u, codes, 0x0c030c01u);
+    const uint32_t we = pk_mad_u16(ev, s2, add2), wo = pk_mad_u16(od, s2, add2);
+    lo = (int)(__builtin_amdgcn_perm(wo, we, 0x06020400u) ^ 0x80808080u);
+    hi = (int)__builtin_amdgcn_perm(wo, we, 0x07030501u);
+}
+__device__ __forceinline__ BPlanes b_prepare_q6k(const BRegs& b, int lane) {
+    const int g = lane >> 4;
+    const uint32_t M4 = 0x0f0f0f0fu, M2H = 0x30303030u;
+    BPlanes o;
+    o.d = __half2float(__ushort_as_half((unsigned short)b.d16));
+    o.dmin = 0.f;
+    o.mB = v4h{0, 0, 0, 0};
+    const uint32_t sel = (uint32_t)(g >> 1) * 8u;   // elements 8g .. 8g+7 of a 32-element stretch: its first or second 16
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const u32x4 c = b.c[P >> 1];
+        const uint32_t w0 = (P & 1) ? c.z : c.x, w1 = (P & 1) ? c.w : c.y;
+        const uint32_t h = b.qh[P], sw = b.hdr[P];
+        // i8 scales of sub-blocks 4P + g/2 (first stretch of the pair) and 4P + 2 + g/2 (second), in both 16-bit lanes
+        const int sa = __builtin_amdgcn_sbfe(sw, sel, 8), sb = __builtin_amdgcn_sbfe(sw, sel + 16u, 8);
+        const uint32_t sa2 = __builtin_amdgcn_perm((uint32_t)sa, (uint32_t)sa, 0x05040100u);
+        const uint32_t sb2 = __builtin_amdgcn_perm((uint32_t)sb, (uint32_t)sb, 0x05040100u);
+        const uint32_t aa2 = pk_mad_u16(sa2, 0xffe0ffe0u, 0x00800080u), ab2 = pk_mad_u16(sb2, 0xffe0ffe0u, 0x00800080u);
+        const uint32_t c0 = (w0 & M4) | ((h << 4) & M2H), c1 = (w1 & M4) | ((h << 2) & M2H);
+        const uint32_t c2 = ((w0 >> 4) & M4) | (h & M2H), c3 = ((w1 >> 4) & M4) | ((h >> 2) & M2H);
+        int l0, l1, l2, l3, h0, h1, h2, h3;
+        q6k_planes(c0, sa2, aa2, l0, h0);
+        q6k_planes(c1, sa2, aa2, l1, h1);
+        q6k_planes(c2, sb2, ab2, l2, h2);
+        q6k_planes(c3, sb2, ab2, l3, h3);
+        o.lo[P] = v4i{l0, l1, l2, l3};
+        o.hi[P] = v4i{h0, h1, h2, h3};
+    }
+    return o;
+}
+
 // one super-block of the wave's 16 weight rows against 16-slot operand o of the staged tile
 // `while_busy` runs right after the MFMAs are issued: this is where the next super-block's loads go.
-template <int NOP, typename Fill>
+template <int FMT, int NOP, typename Fill>
 __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP>& L, int buf, int o, int lane, v4f& facc, Fill while_busy) {
     const int m = lane & 15, g = lane >> 4;
     const v4i zero4 = {0, 0, 0, 0};
@@ -174,17 +234,27 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
         acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.lo[P], P == 0 ? zero4 : acc_lo, 0, 0, 0);
         acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.hi[P], P == 0 ? zero4 : acc_hi, 0, 0, 0);
     }
-    const v4h mA = *reinterpret_cast<const v4h*>(&L.bs[buf][o][g >> 1][m][(g & 1) * 4]);
-    const v4f zf = {0.f, 0.f, 0.f, 0.f};
-    const v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(mA, B.mB, zf, 0, 0, 0);
     // D[i] belongs to slot 16 o + 4 g + i, weight row n = lane%16
-    const v4f yd = *reinterpret_cast<const v4f*>(&L.yd[buf][o * 16 + g * 4]);
-    while_busy();
+    if constexpr (FMT == MOE_GGML_Q6K) {
+        const v4f yd = *reinterpret_cast<const v4f*>(&L.yd[buf][o * 16 + g * 4]);
+        while_busy();
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int isum = (acc_hi[i] << 3) + acc_lo[i];
-        const float v = __builtin_fmaf(B.d, (float)isum, -(B.dmin * Dm[i]));
-        facc[i] = __builtin_fmaf(yd[i], v, facc[i]);
+        for (int i = 0; i < 4; i++) {
+            const int isum = (acc_hi[i] << 8) + acc_lo[i];
+            facc[i] = __builtin_fmaf(B.d * yd[i], (float)isum, facc[i]);
+        }
+    } else {
+        const v4h mA = *reinterpret_cast<const v4h*>(&L.bs[buf][o][g >> 1][m][(g & 1) * 4]);
+        const v4f zf = {0.f, 0.f, 0.f, 0.f};
+        const v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(mA, B.mB, zf, 0, 0, 0);
+        const v4f yd = *reinterpret_cast<const v4f*>(&L.yd[buf][o * 16 + g * 4]);
+        while_busy();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int isum = (acc_hi[i] << 3) + acc_lo[i];
+            const float v = __builtin_fmaf(B.d, (float)isum, -(B.dmin * Dm[i]));
+            facc[i] = __builtin_fmaf(yd[i], v, facc[i]);
+        }
     }
 }
 
@@ -197,9 +267,13 @@ __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-template <int MODE, int NOP>
+// FMT: the weights' format (Q4K; Q6K for MODE 1 only).
+template <int FMT, int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
+    static_assert(FMT == MOE_GGML_Q4K || (FMT == MOE_GGML_Q6K && MODE == 1), "formats of the tiled kernel");
     constexpr int NB = NOP / 2;
+    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : Q4K_TILE_BYTES;
+    constexpr bool kSums = FMT != MOE_GGML_Q6K;   // block sums staged (the mins term)
     __shared__ GemmLds<NOP> L;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -222,7 +296,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     const int K = MODE == 0 ? p.H : p.F;        // reduction length
     const int N = MODE == 0 ? p.F : p.H;        // weight rows of the matrix
     const int nsb = K / 256;
-    const size_t sb_stride = (size_t)(N / 16) * Q4K_TILE_BYTES;
+    const size_t sb_stride = (size_t)(N / 16) * TILE_BYTES;
     const ActBuf& ab = MODE == 0 ? p.xq : p.hq;
 
     // activation row behind position r of the tile (positions past the expert's list repeat its last row)
@@ -242,45 +316,52 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     int row0;
     if (MODE == 0) {
         row0 = rblk * 64 + (wave & 3) * 16;
-        wp = (wave < 4 ? gw.w1 : gw.w3) + (size_t)(row0 / 16) * Q4K_TILE_BYTES;
+        wp = (wave < 4 ? gw.w1 : gw.w3) + (size_t)(row0 / 16) * TILE_BYTES;
     } else {
         row0 = rblk * 128 + wave * 16;
-        wp = gw.w2 + (size_t)(row0 / 16) * Q4K_TILE_BYTES;
+        wp = gw.w2 + (size_t)(row0 / 16) * TILE_BYTES;
     }
     v4f facc[NOP];
 #pragma unroll
     for (int o = 0; o < NOP; o++) facc[o] = v4f{0.f, 0.f, 0.f, 0.f};
 
     // transfer t of the wave's share (quant stretches, sums, scales), then the weight tile
-    auto stage = [&](auto I, int sb, int buf) { stage_piece<decltype(I)::value, NOP>(ab, rows, nsb, sb, L, buf, wave, lane); };
+    auto stage = [&](auto I, int sb, int buf) {
+        if constexpr (!kSums && decltype(I)::value == NB) return;
+        stage_piece<decltype(I)::value, NOP>(ab, rows, nsb, sb, L, buf, wave, lane);
+    };
+    auto prepare = [&](const BRegs& r) {
+        if constexpr (FMT == MOE_GGML_Q6K) return b_prepare_q6k(r, lane);
+        else return b_prepare(r, lane);
+    };
     using std::integral_constant;
     stage(integral_constant<int, 0>{}, 0, 0);
     stage(integral_constant<int, 1>{}, 0, 0);
     stage(integral_constant<int, NB>{}, 0, 0);
     stage(integral_constant<int, NB + 1>{}, 0, 0);
     if constexpr (NB == 4) { stage(integral_constant<int, 2>{}, 0, 0); stage(integral_constant<int, 3>{}, 0, 0); }
-    BRegs raw = b_load(wp, lane);
+    BRegs raw = b_load<FMT>(wp, lane);
     wait_all_loads();
     __syncthreads();
     for (int sb = 0; sb < nsb; sb++) {
         const int buf = sb & 1, nb = buf ^ 1;
         const int sbn = sb + 1 < nsb ? sb + 1 : sb;
-        const BPlanes B = b_prepare(raw, lane);
+        const BPlanes B = prepare(raw);
         // the next super-block's activations and weights are requested while the operands' MFMAs drain
         if constexpr (NOP == 8) {
-            gemm_operand(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, 1>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 2, lane, facc[2], [&] { stage(integral_constant<int, 2>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 3, lane, facc[3], [&] { stage(integral_constant<int, 3>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 4, lane, facc[4], [&] { stage(integral_constant<int, 4>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 5, lane, facc[5], [&] { stage(integral_constant<int, 5>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 6, lane, facc[6], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
-            gemm_operand(B, L, buf, 7, lane, facc[7], [&] {});
+            gemm_operand<FMT>(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, 1>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 2, lane, facc[2], [&] { stage(integral_constant<int, 2>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 3, lane, facc[3], [&] { stage(integral_constant<int, 3>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 4, lane, facc[4], [&] { stage(integral_constant<int, 4>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 5, lane, facc[5], [&] { stage(integral_constant<int, 5>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 6, lane, facc[6], [&] { raw = b_load<FMT>(wp + (size_t)sbn * sb_stride, lane); });
+            gemm_operand<FMT>(B, L, buf, 7, lane, facc[7], [&] {});
         } else {
-            gemm_operand(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); stage(integral_constant<int, 1>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, NB>{}, sbn, nb); stage(integral_constant<int, NB + 1>{}, sbn, nb); });
-            gemm_operand(B, L, buf, 2, lane, facc[2], [&] { raw = b_load(wp + (size_t)sbn * sb_stride, lane); });
-            gemm_operand(B, L, buf, 3, lane, facc[3], [&] {});
+            gemm_operand<FMT>(B, L, buf, 0, lane, facc[0], [&] { stage(integral_constant<int, 0>{}, sbn, nb); stage(integral_constant<int, 1>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 1, lane, facc[1], [&] { stage(integral_constant<int, NB>{}, sbn, nb); stage(integral_constant<int, NB + 1>{}, sbn, nb); });
+            gemm_operand<FMT>(B, L, buf, 2, lane, facc[2], [&] { raw = b_load<FMT>(wp + (size_t)sbn * sb_stride, lane); });
+            gemm_operand<FMT>(B, L, buf, 3, lane, facc[3], [&] {});
         }
         wait_all_loads();
         __syncthreads();
@@ -330,14 +411,17 @@ static unsigned gemm_grid(int n_rb, int64_t max_tiles) {
 }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s) {
     dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
-    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<0, 4>), grid, dim3(G_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((q4k_gemm_kernel<0, 8>), grid, dim3(G_THREADS), 0, s, p);
+    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 0, 4>), grid, dim3(G_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 0, 8>), grid, dim3(G_THREADS), 0, s, p);
     return hipGetLastError();
 }
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s) {
     dim3 grid(gemm_grid(p.H / 128, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
-    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<1, 4>), grid, dim3(G_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((q4k_gemm_kernel<1, 8>), grid, dim3(G_THREADS), 0, s, p);
+    if (p.dt_down == MOE_GGML_Q6K) {
+        if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q6K, 1, 4>), grid, dim3(G_THREADS), 0, s, p);
+        else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q6K, 1, 8>), grid, dim3(G_THREADS), 0, s, p);
+    } else if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 1, 4>), grid, dim3(G_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 1, 8>), grid, dim3(G_THREADS), 0, s, p);
     return hipGetLastError();
 }
 

@@ -174,6 +174,38 @@ def test_cfg3_prefill_zipf(mixtral_layer, request):
     gpu.close()
 
 
+def test_cfg3_prefill_q4k_up_q6k_down(mixtral_layer, request):
+    """The arrangement of Q4_K_M files (Q4K w1 / w3, Q6K w2) at the Mixtral shape, 2048 tokens with the Zipf load: the
+    tiled kernels serve both projections, the down one in its Q6K variant.  Same bars as the all-Q4K prefill."""
+    ref, _ = mixtral_layer
+    T = 2048
+    w2 = [O.fill_normal_quantized(900 + e, O.Q6K, 4096, 14336, 0.02, threads=CORES) for e in range(8)]
+    gpu = candle_amd.SparseMoeBlock(4096, 14336, 8, 2, O.Q4K, ref.gate, ref.w1, ref.w3, w2, gate_bias=ZIPF_BIAS, ggml_dtype_down=O.Q6K)
+    ref_b = O.Layer(4096, 14336, 8, 2, O.Q4K, ref.gate, ref.w1, ref.w3, w2, gate_bias=ZIPF_BIAS, dtype_down=O.Q6K)
+    xs = acts(T, 4096, 21)
+    ys = gpu.forward(xs)
+    logits = gpu.last_logits(T)
+    gi, gw, goff, gperm, gpw = gpu.last_routing(T)
+    ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), 2)
+    assert np.array_equal(gi, ri) and np.array_equal(bits(gw), bits(rw))
+    assert np.array_equal(goff, roff) and np.array_equal(gperm, rperm) and np.array_equal(bits(gpw), bits(rpw))
+    want = ref_b.forward(xs, logits=logits, simd=True, threads=CORES)
+    r = rms(want)
+    e_max, e_share, e_rms = tail_stats(ys, want, r)
+    say(request.config, " [Q4K up / Q6K down vs AVX2: max %.2e, share > 2e-3 %.1e, rms %.1e]" % (e_max, e_share, e_rms))
+    assert e_rms <= 2e-4 and e_share <= 5e-5 and e_max <= 3 * TOL, (e_max, e_share, e_rms)
+    n = 512
+    want_s = ref_b.forward(xs[:n], logits=logits[:n], simd=False, threads=CORES)
+    g_max, g_share, _ = tail_stats(ys[:n], want[:n], r)
+    s_max, s_share, _ = tail_stats(want_s, want[:n], r)
+    say(request.config, " [first %d tokens: HIP vs AVX2 max %.2e share %.1e; scalar vs AVX2 max %.2e share %.1e]" % (n, g_max, g_share, s_max, s_share))
+    assert g_max <= max(2 * TOL, 1.5 * s_max) and g_share <= 1.5 * s_share + 2e-5, (g_max, g_share, s_max, s_share)
+    # one weight matrix back out of the device layout, bit for bit
+    got = gpu.dequantize_weight(5, 2)
+    assert np.array_equal(bits(got).reshape(-1), bits(O.dequantize(O.Q6K, w2[5], got.size)))
+    gpu.close()
+
+
 def test_cfg4_fine_grained_q8_0_shared_expert():
     ref, gpu = build(2048, 1408, 60, 4, O.Q8_0, seed=4, Fs=5632)
     check(ref, gpu, acts(512, 2048, 12))

@@ -270,9 +270,10 @@ def test_block_q6k_and_mixed_down_dtype(dt, dt_down):
     # all-Q6K and all-Q5K experts, the Q4_K_M arrangement (Q4K gate / up with Q6K down), its reverse, and
     # the Q5_K_M arrangement (Q5K with Q6K down).
     # T = 1, 3: narrow workgroups; 8, 33: one and two slot tiles per pass; 70: dispatched lists;
-    # 200, 500: the Q4K up projection switches to the tiled kernel while a Q6K down keeps streaming
+    # 200: the Q4K up projection switches to the tiled kernel; 300, 500: so does a Q4K or Q6K down projection (64-slot
+    # and 128-slot tiles)
     ref, gpu = make_pair(512, 1024, 8, 2, dt, seed=12, dt_down=dt_down)
-    for T in (1, 3, 8, 33, 70, 200, 500):
+    for T in (1, 3, 8, 33, 70, 200, 300, 500):
         check_block(ref, gpu, T, tol=block_tol(O.Q4K, 1024))
     for e, which, wdt in ((0, 1, dt), (7, 3, dt), (5, 2, dt_down or dt)):
         want = O.dequantize(wdt, getattr(ref, "w%d" % which)[e], 512 * 1024)
