@@ -1077,10 +1077,15 @@ extern "C" int moe_qmatmul(int32_t dt, const void* w_blocks, int64_t n, int64_t 
     return rc;
 }
 
+static bool weight_quantiser_exists(int dt) {
+    return dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K ||
+           dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K;
+}
+
 extern "C" int moe_quantize_weights_device(int32_t dt, const void* d_x, int64_t n, void* d_out, void* hip_stream) {
     int rc = ensure_device();
     if (rc) return rc;
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
+    if (!weight_quantiser_exists(dt)) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
     if (n < 0 || n % block_elems(dt)) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
     if (n == 0) return MOE_OK;
     if (!d_x || !d_out) return fail(MOE_E_INVALID, "NULL pointer");
@@ -1091,7 +1096,7 @@ extern "C" int moe_quantize_weights_device(int32_t dt, const void* d_x, int64_t 
 extern "C" int moe_quantize_weights(int32_t dt, const float* x, int64_t n, void* out) {
     int rc = ensure_device();
     if (rc) return rc;
-    if (dt != MOE_GGML_Q4_0 && dt != MOE_GGML_Q8_0 && dt != MOE_GGML_Q4K) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
+    if (!weight_quantiser_exists(dt)) return fail(MOE_E_INVALID, "moe_quantize_weights: unsupported dtype");
     if (n < 0 || n % block_elems(dt)) return fail(MOE_E_INVALID, "n_elems must be a non-negative multiple of the block size");
     if (n == 0) return MOE_OK;
     if (!x || !out) return fail(MOE_E_INVALID, "NULL pointer");

@@ -209,8 +209,9 @@ int moe_add_rms_norm_device(const void* d_x, const void* d_residual, const void*
                             void* d_sum, void* d_y, void* hip_stream);
 
 /* QTensor::quantize (candle-core/src/quantized/mod.rs:331-349) on the GPU: f32 [n_elems] -> raw
- * GGML blocks, bit-identical to GgmlType::from_float of k_quants.rs:188-224 (Q4_0), 605-634 (Q8_0)
- * and 1287-1345 (Q4K).  Host pointers / device pointers (the latter enqueued on hip_stream). */
+ * GGML blocks, bit-identical to GgmlType::from_float of k_quants.rs:188-224 (Q4_0), 605-634 (Q8_0), 808-870 (Q2K),
+ * 1049-1129 (Q3K), 1287-1345 (Q4K), 1484-1561 (Q5K) and 1675-1751 (Q6K); other formats are refused.  Host pointers /
+ * device pointers (the latter enqueued on hip_stream). */
 int moe_quantize_weights(int32_t ggml_dtype, const float* x, int64_t n_elems, void* out_blocks);
 int moe_quantize_weights_device(int32_t ggml_dtype, const void* d_x, int64_t n_elems, void* d_out_blocks, void* hip_stream);
 

@@ -58,7 +58,7 @@ def test_to_float_bit_exact(dt):
     assert candle_amd.dequantize(dt, raw[:0], 0).size == 0
 
 
-@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q4K])
+@pytest.mark.parametrize("dt", [O.Q4_0, O.Q8_0, O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K])
 def test_weight_quantiser_bit_exact(dt, golden):
     n = 256 * 2048
     x = O.fill_normal(40 + dt, n, 0.0, 0.02)
