@@ -245,10 +245,14 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
 }
 
 // ---------------------------------------------------------------------------------------------
+__device__ inline void route_one_token_wave(float logit, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out);
+__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel);
+
 template <int VDT>
 __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     extern __shared__ float xrow[];  // [H]
     __shared__ float probs[MAX_E];
+    __shared__ int sel_lds[MAX_K];
     __shared__ float red[FRONT_THREADS / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t t = blockIdx.x;
@@ -303,8 +307,11 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     if (p.y_zero)
         for (int h = tid * 4; h < H; h += FRONT_THREADS * 4) *reinterpret_cast<float4*>(p.y_zero + t * H + h) = make_float4(0.f, 0.f, 0.f, 0.f);
 
-    // ---- one thread routes while the waves quantise the row
-    if (tid == 0) route_one_token(probs, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+    // ---- wave 0 routes, then joins the others in quantising the row
+    if (wave == 0) {
+        if (E <= 64) route_one_token_wave(lane < E ? probs[lane] : 0.f, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+        else route_one_token_wave_lds(probs, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds);
+    }
 
     if (VDT == MOE_GGML_Q8K) {
         const int nb = H / 256;
@@ -380,6 +387,66 @@ __device__ inline void route_one_token_wave(float logit, int lane, int E, int k,
     if (lane < k) {
         idx_out[lane] = my_e;
         w_out[lane] = norm_topk ? my_p / sum : my_p;
+    }
+}
+
+// Wave-parallel routing for 64 < E <= 256, the logits in LDS (`p`, overwritten with the probabilities): lane l holds
+// experts l, l + 64, l + 128, l + 192.  Same arithmetic and order as route_one_token: the maximum (any order gives the
+// same float), the exp values summed as vec_sum_ref_order sums them (lane j < 32 carries accumulator j over the blocks
+// of 32, then the tree, then the tail left to right), the rank of an expert = the number of experts that precede it in
+// the (total_cmp key descending, index ascending) order.  `sel` (LDS, k ints) receives the experts in rank order.
+// Call with all 64 lanes of one wave active; p and sel belong to that wave.
+__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel) {
+    float mx = -__builtin_inff();
+    bool any = false;   // fmaxf skips NaNs; with nothing but NaNs the serial loop is left with one
+    for (int e = lane; e < E; e += 64) {
+        const float v = p[e];
+        if (v == v) { mx = fmaxf(mx, v); any = true; }
+    }
+    mx = wave_max_f(mx);
+    if (__ballot(any) == 0ull) mx = p[0];
+    for (int e = lane; e < E; e += 64) p[e] = expf_glibc(p[e] - mx);
+    __builtin_amdgcn_wave_barrier();
+    const int np = E & ~31;
+    float acc = 0.f;
+    for (int b = 0; b < np; b += 32) acc = acc + p[b + (lane & 31)];
+    const int l8 = lane & 7;
+    const float x0 = (__shfl(acc, l8, 64) + __shfl(acc, 8 + l8, 64)) + (__shfl(acc, 16 + l8, 64) + __shfl(acc, 24 + l8, 64));
+    const float t0 = lane_bcast(x0, 0) + lane_bcast(x0, 4);
+    const float t1 = lane_bcast(x0, 1) + lane_bcast(x0, 5);
+    const float t2 = lane_bcast(x0, 2) + lane_bcast(x0, 6);
+    const float t3 = lane_bcast(x0, 3) + lane_bcast(x0, 7);
+    float s = (t0 + t1) + (t2 + t3);
+    for (int i = np; i < E; i++) s += p[i];
+    float pr[4];
+    int key[4], rank[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int e = lane + 64 * q;
+        pr[q] = e < E ? p[e] / s : 0.f;
+        key[q] = total_key(pr[q]);
+        rank[q] = 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        if (lane + 64 * q < E) p[lane + 64 * q] = pr[q];
+    __builtin_amdgcn_wave_barrier();
+    for (int i = 0; i < E; i++) {
+        const int ki = total_key(p[i]);
+#pragma unroll
+        for (int q = 0; q < 4; q++) rank[q] += (ki > key[q] || (ki == key[q] && i < lane + 64 * q)) ? 1 : 0;
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        if (lane + 64 * q < E && rank[q] < k) sel[rank[q]] = lane + 64 * q;
+    __builtin_amdgcn_wave_barrier();
+    float sum = 0.f;
+    for (int r = 0; r < k; r++) sum += p[sel[r]];
+    if (lane < k) {
+        const int e = sel[lane];
+        idx_out[lane] = e;
+        w_out[lane] = norm_topk ? p[e] / sum : p[e];
     }
 }
 
@@ -715,8 +782,9 @@ __global__ __launch_bounds__(256) void fill_or_copy_kernel(const float* src, flo
 __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const float* logits, int64_t T, int E, int k,
                                                                          int norm_topk, RouteBufs rb) {
     __shared__ float probs[FRONT_THREADS / 64][MAX_E];
+    __shared__ int sel_lds[FRONT_THREADS / 64][MAX_K];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // one wave per token (4 tokens per workgroup); lane 0 routes
+    // one wave per token (4 tokens per workgroup)
     int64_t t = (int64_t)blockIdx.x * (FRONT_THREADS / 64) + wave;
     if (t < T) {
         for (int e = lane; e < E; e += 64) {
@@ -728,8 +796,8 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
     __syncthreads();
     if (E <= 64) {
         if (t < T) route_one_token_wave(lane < E ? probs[wave][lane] : 0.f, lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
-    } else if (t < T && lane == 0) {
-        route_one_token(probs[wave], E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
+    } else if (t < T) {
+        route_one_token_wave_lds(probs[wave], lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k, sel_lds[wave]);
     }
 }
 

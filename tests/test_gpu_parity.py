@@ -100,7 +100,8 @@ def test_activation_quantiser_bit_exact(vdt):
 
 
 @pytest.mark.parametrize("T,E,k,norm", [(16, 8, 2, True), (1, 8, 2, True), (333, 60, 4, True), (4096, 8, 2, True),
-                                         (65, 64, 6, False), (7, 3, 3, True), (50, 160, 8, True), (9, 1, 1, True)])
+                                         (65, 64, 6, False), (7, 3, 3, True), (50, 160, 8, True), (9, 1, 1, True),
+                                         (33, 256, 16, True), (12, 65, 3, False), (20, 100, 5, True), (40, 224, 1, True)])
 def test_route_bit_exact_given_logits(T, E, k, norm):
     logits = O.fill_normal(T * 31 + E, T * E, 0.0, 1.5).reshape(T, E)
     if T > 4:
@@ -358,6 +359,15 @@ def test_block_no_renorm_and_bias():
     gpu.close()
 
 
+@pytest.mark.parametrize("E,k", [(96, 6), (200, 8)])
+def test_block_more_than_64_experts(E, k):
+    # the front kernel's routing holds up to four experts per lane
+    ref, gpu = make_pair(256, 256, E, k, O.Q4K, seed=30 + E)
+    for T in (1, 9, 150):
+        check_block(ref, gpu, T, tol=block_tol(O.Q4K, 256))
+    gpu.close()
+
+
 def test_block_rms_residual_chain():
     ref, gpu = make_pair(512, 512, 4, 2, O.Q4K, seed=5, rms=True)
     xs = activations(6, 512, 9)
@@ -546,7 +556,7 @@ def test_top_k_zero_returns_zeros_as_the_reference_does():
     assert idx.shape == (5, 0) and not off.any()
 
 
-@pytest.mark.parametrize("E,k", [(8, 2), (60, 4), (160, 6)])
+@pytest.mark.parametrize("E,k", [(8, 2), (60, 4), (160, 6), (256, 16), (97, 3)])
 def test_nan_probabilities_are_ranked_as_total_cmp_ranks_them(E, k):
     """`sort_by(total_cmp)` (quantized_llama.rs:166) puts a NaN with a clear sign bit above every number and one with
     the sign bit set below.  One NaN logit makes the whole softmax row NaN (the sum is NaN), so every key of the row
