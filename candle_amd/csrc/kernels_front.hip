@@ -15,6 +15,7 @@
 //   top-k + lists     candle-transformers/src/models/quantized_llama.rs:158-179
 //   combine           quantized_llama.rs:200-202 (index_add in ascending expert order)
 //   rms_norm          candle-nn/src/ops.rs:504-515;  sigmoid candle-nn/src/ops.rs:59-61
+#include <algorithm>
 #include <cstdlib>
 
 #include "act_quant.hpp"
@@ -823,8 +824,6 @@ __global__ void identity_routing_kernel(RouteBufs rb, int64_t rows) {
 __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs rb, int shared, const float* residual,
                                                       float* y, int64_t T, int H) {
     const int64_t t = blockIdx.x;
-    const int h = (blockIdx.y * 256 + threadIdx.x) * 4;
-    if (h >= H) return;
     const int k = rb.k;
     int slots[MAX_K + 1];
     int n = k + (shared ? 1 : 0);
@@ -840,16 +839,45 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs
     } else {
         for (int j = 0; j < n; j++) slots[j] = rb.tok_slots[t * n + j];
     }
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int j = 0; j < n; j++) {
-        float4 v = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h);
-        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    // a workgroup walks the token's row in steps of 1024 floats, two steps' loads in flight
+    const int h0 = (blockIdx.y * 256 + threadIdx.x) * 4, hstep = gridDim.y * 1024;
+    for (int h = h0; h < H; h += 2 * hstep) {
+        const int h2 = h + hstep;
+        const bool two = h2 < H;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f), acc2 = acc;
+        if (n == 2) {   // the common case: both terms of both steps requested before the first add
+            const float4 a0 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[0] * H + h);
+            const float4 a1 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[1] * H + h);
+            float4 b0 = acc, b1 = acc;
+            if (two) {
+                b0 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[0] * H + h2);
+                b1 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[1] * H + h2);
+            }
+            acc.x += a0.x; acc.y += a0.y; acc.z += a0.z; acc.w += a0.w;
+            acc.x += a1.x; acc.y += a1.y; acc.z += a1.z; acc.w += a1.w;
+            acc2.x += b0.x; acc2.y += b0.y; acc2.z += b0.z; acc2.w += b0.w;
+            acc2.x += b1.x; acc2.y += b1.y; acc2.z += b1.z; acc2.w += b1.w;
+        } else {
+            for (int j = 0; j < n; j++) {
+                const float4 v = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h);
+                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+                if (two) {
+                    const float4 u = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h2);
+                    acc2.x += u.x; acc2.y += u.y; acc2.z += u.z; acc2.w += u.w;
+                }
+            }
+        }
+        if (residual) {
+            const float4 r = *reinterpret_cast<const float4*>(residual + t * H + h);
+            acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w;
+            if (two) {
+                const float4 r2 = *reinterpret_cast<const float4*>(residual + t * H + h2);
+                acc2.x += r2.x; acc2.y += r2.y; acc2.z += r2.z; acc2.w += r2.w;
+            }
+        }
+        *reinterpret_cast<float4*>(y + t * H + h) = acc;
+        if (two) *reinterpret_cast<float4*>(y + t * H + h2) = acc2;
     }
-    if (residual) {
-        float4 r = *reinterpret_cast<const float4*>(residual + t * H + h);
-        acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w;
-    }
-    *reinterpret_cast<float4*>(y + t * H + h) = acc;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -933,7 +961,10 @@ hipError_t launch_dispatch(const RouteBufs& rb, int64_t T, int E, int k, bool sh
 hipError_t launch_combine(const float* yw, const RouteBufs& rb, bool shared, const float* residual, float* y,
                           int64_t T, int H, hipStream_t s) {
     if (T == 0) return hipSuccess;
-    dim3 grid((unsigned)T, (unsigned)((H / 4 + 255) / 256));
+    // few tokens: one workgroup per 1024 floats of a row; many: one or two per row, each walking it
+    const unsigned per_row = (unsigned)((H / 4 + 255) / 256);
+    const unsigned split = T >= 2048 ? 1u : T >= 512 ? std::min(per_row, 2u) : per_row;
+    dim3 grid((unsigned)T, split);
     hipLaunchKernelGGL(combine_kernel, grid, dim3(256), 0, s, yw, rb, shared ? 1 : 0, residual, y, T, H);
     return hipGetLastError();
 }

@@ -453,11 +453,26 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const float* x, int6
     const float* xr = x + row * k;
     if (VDT == MOE_GGML_Q8K) {
         // blocks of a row are dealt to the waves of gridDim.y workgroups (few rows: many workgroups per row)
+        // (four blocks of a wave side by side: their loads, wave reductions and divisions overlap)
         const int nb = k / 256;
-        for (int b = blockIdx.y * 4 + wave; b < nb; b += 4 * gridDim.y) {
-            float4 v = *reinterpret_cast<const float4*>(xr + b * 256 + lane * 4);
-            quantize_q8k_block(v, lane, out.qs + row * k + b * 256, out.d + row * nb + b,
-                               reinterpret_cast<__half*>(out.bsum) + (row * nb + b) * 16);
+        constexpr int NQ = 4;
+        const int stride = 4 * gridDim.y;
+        for (int b0 = blockIdx.y * 4 + wave; b0 < nb; b0 += NQ * stride) {
+            float4 v[NQ];
+            bool valid[NQ];
+            int8_t* qs_out[NQ];
+            float* d_out[NQ];
+            __half* bs_out[NQ];
+#pragma unroll
+            for (int n = 0; n < NQ; n++) {
+                valid[n] = b0 + n * stride < nb;
+                const int b = valid[n] ? b0 + n * stride : b0;
+                v[n] = *reinterpret_cast<const float4*>(xr + b * 256 + lane * 4);
+                qs_out[n] = out.qs + row * k + b * 256;
+                d_out[n] = out.d + row * nb + b;
+                bs_out[n] = reinterpret_cast<__half*>(out.bsum) + (row * nb + b) * 16;
+            }
+            quantize_q8k_blocks<NQ>(v, valid, lane, qs_out, d_out, bs_out);
         }
     } else {
         const int nb = k / 32;
