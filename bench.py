@@ -18,6 +18,7 @@ measures the other regimes in the same process and reports them as sub-objects o
                   plus N(0, 0.1) noise; end-to-end tokens/s.
 
 `--workload decode|prefill|config4|stack` measures one of them alone as the line's `value`.
+`--workload prefill --weights-down q6_k` measures the prefill with w2 stored as Q6_K (what Q4_K_M files do).
 `--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with another
 GGML format (random block payloads with small finite scales: timing does not depend on the values).
 
@@ -63,7 +64,7 @@ def random_blocks(np, rng, fmt, n_elems):
     return raw.reshape(-1)
 
 
-def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k"):
+def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k", fmt_down=None):
     """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel (bit-identical to candle's
     CPU quantiser), returned as host bytes (the CPU baseline runs on the same bytes)."""
     h, f, e_n, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, Q4K, 0)
@@ -74,16 +75,18 @@ def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k"):
         dt = FORMATS[fmt][0]
         rng = np.random.default_rng(seed)
 
-    def draw(shape):
+    dt_down = FORMATS[fmt_down][0] if fmt_down else dt
+
+    def draw(shape, dtype=None):
         if fmt != "q4_k" and not cfg4:
             return random_blocks(np, rng, fmt, shape[0] * shape[1])
         x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
-        return candle_amd.quantize_weights(dt, x).cpu().numpy()
+        return candle_amd.quantize_weights(dtype or dt, x).cpu().numpy()
 
-    w = {"w1": [], "w3": [], "w2": [], "dt": dt}
+    w = {"w1": [], "w3": [], "w2": [], "dt": dt, "dt_down": dt_down}
     for e in range(e_n):
         for name, shape in (("w1", (f, h)), ("w3", (f, h)), ("w2", (h, f))):
-            w[name].append(draw(shape))
+            w[name].append(draw(shape, dt_down if name == "w2" else None))
     if fs:
         w["shared"] = (draw((fs, h)), draw((fs, h)), draw((h, fs)))
     g.manual_seed(seed + 1)
@@ -98,7 +101,8 @@ def make_layer(candle_amd, w, gate_bias=None, cfg4=False):
         c = CFG4
         return candle_amd.SparseMoeBlock(c["H"], c["F"], c["E"], c["k"], Q8_0, w["gate"], w["w1"], w["w3"], w["w2"], shared_ffn=c["Fs"],
                                          shared_w1=w["shared"][0], shared_w3=w["shared"][1], shared_w2=w["shared"][2], shared_gate=w["shared_gate"])
-    return candle_amd.SparseMoeBlock(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+    return candle_amd.SparseMoeBlock(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias,
+                                     ggml_dtype_down=w.get("dt_down", w["dt"]))
 
 
 def hip_events():
@@ -169,7 +173,7 @@ def cpu_baseline(w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=Fals
         layer = O.Layer(CFG4["H"], CFG4["F"], CFG4["E"], CFG4["k"], Q8_0, w["gate"], w["w1"], w["w3"], w["w2"], Fs=CFG4["Fs"],
                         sw1=w["shared"][0], sw3=w["shared"][1], sw2=w["shared"][2], shared_gate=w["shared_gate"])
     else:
-        layer = O.Layer(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias)
+        layer = O.Layer(H, F, E, TOPK, w["dt"], w["gate"], w["w1"], w["w3"], w["w2"], gate_bias=gate_bias, dtype_down=w.get("dt_down", w["dt"]))
     layer.forward(xs_host[:1], logits=logits_host[:1], simd=True, threads=cores)  # warm the pages
     reps, t0 = 0, time.perf_counter()
     while True:
@@ -276,10 +280,10 @@ def measure_cfg4(args, np, torch, timer, layer, B):
     step_bytes = n_active * expert_bytes + shared_bytes + c["E"] * c["H"] * 4 + 2 * B * c["H"] * 4
     up_bytes = n_active * (2 * c["H"] * c["F"] * 34 // 32)
     achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
-    traffic = profiled_traffic(B, "q32s_config4_kernel_trace.md", "config4") if B == 512 else None
-    roofline = {"bound": "hbm", "kernel": "routed up projection (w1, w3, SiLU, Q8_0 re-quantisation)",
+    traffic = profiled_traffic(B, "q8_0_gemm_config4_kernel_trace.md", "config4") if B == 512 else None
+    roofline = {"bound": "hbm", "kernel": "q8_0_gemm<0>: routed up projection (w1, w3, SiLU, Q8_0 re-quantisation), 64-slot tiles",
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                "traffic_source": "profiles/q32s_config4_kernel_trace.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
+                "traffic_source": "profiles/q8_0_gemm_config4_kernel_trace.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
                 "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "tokens": B, "active_experts": n_active, "max_expert_load": int(loads.max()), "stage_us": stage_us, "dispatch_us": stage_us["dispatch"],
@@ -358,6 +362,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="layers of the stack workload")
     ap.add_argument("--stack-steps", type=int, default=128, help="consecutive steps of the stack workload")
     ap.add_argument("--weights", choices=sorted(FORMATS), default="q4_k", help="GGML format of the expert matrices (decode workload)")
+    ap.add_argument("--weights-down", choices=("q6_k",), default=None,
+                    help="prefill workload: w2 in this format beside Q4_K w1 / w3 (the arrangement of Q4_K_M files)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
@@ -387,6 +393,8 @@ def main():
         sys.exit("bench.py: --weights applies to the decode workload only")
     if args.weights != "q4_k":
         wl = "decode"
+    if args.weights_down and wl != "prefill":
+        sys.exit("bench.py: --weights-down applies to the prefill workload only")
     timer = Timer(torch)
     out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "i8", "data": "synthetic", "unit": "tokens/s"}
@@ -416,14 +424,15 @@ def main():
                                             "y = x + moe(rms_norm(x)) per layer, %d-token batch, each step fed the previous output plus N(0, 0.1) noise"
                                             % (args.layers, m["resident_gb"], m["batch"])}, **{k: v for k, v in m.items() if k != "roofline"}))
     elif wl == "prefill":
-        w = draw_weights(torch, candle_amd)
+        w = draw_weights(torch, candle_amd, fmt_down=args.weights_down)
         layer = make_layer(candle_amd, w, gate_bias=bias)
         B = args.batch or 4096
         m = measure_prefill(args, np, torch, timer, layer, B)
+        wdesc = "Q4_K weights" if not args.weights_down else "Q4_K w1 / w3 with %s w2" % args.weights_down
         out.update(metric="MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, prefill)", value=m["tokens_per_s"], ms_per_step=m["ms_per_step"],
                    timed_steps=m["timed_steps"], roofline=m["roofline"],
-                   config=dict({"workload": "BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, Q4_K weights, prefill of %d tokens, "
-                                            "Zipf(1) expert load" % B}, **{k: v for k, v in sub(m).items() if k != "roofline"}))
+                   config=dict({"workload": "BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, %s, prefill of %d tokens, "
+                                            "Zipf(1) expert load" % (wdesc, B)}, **{k: v for k, v in sub(m).items() if k != "roofline"}))
         if not args.no_cpu_baseline:
             n_cpu = min(B, 64)   # a bounded sample: the CPU path does ~1 k tokens/s
             cpu = cpu_baseline(w, m["xs"][0][:n_cpu].cpu().numpy(), layer.last_logits(B)[:n_cpu], args.cpu_seconds, gate_bias=bias)
