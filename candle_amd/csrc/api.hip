@@ -472,7 +472,10 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     // tiles per pass up to ~34 rows per expert)
     // (the 32-element kernels carry at most two tiles: three or four per pass measured slower at the Mixtral shape and
     // 8 % faster at best where sixty small experts' weights exceed the caches)
-    pl.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > 9 * L->E) ? 2 : 1;
+    // (K-quants, Mixtral shape: one tile with a second pass for the lists beyond 16 rows beats two tiles up to ~13 rows per
+    // expert on average: 48 tokens 168 against 181 us per step, 64 tokens 214 against 185)
+    const int64_t two_from = (L->vdt == MOE_GGML_Q8K ? 13 : 9) * L->E;
+    pl.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > two_from) ? 2 : 1;
     if (sw.slot_tiles) pl.slot_tiles = sw.slot_tiles;
     // very small K-quant batches: at most half of the experts can be active, so the weights are cut
     // into four times as many workgroups; those write f32 h and a small pass quantises it
