@@ -18,7 +18,8 @@ measures the other regimes in the same process and reports them as sub-objects o
                   plus N(0, 0.1) noise; end-to-end tokens/s.
 
 `--workload decode|prefill|config4|stack` measures one of them alone as the line's `value`.
-`--workload prefill --weights-down q6_k` measures the prefill with w2 stored as Q6_K (what Q4_K_M files do).
+`--workload prefill [--weights q5_k] [--weights-down q5_k|q6_k]` measures the prefill with Q5_K w1 / w3 and / or w2 stored
+in another K-quant (Q4_K_M and Q5_K_M files store part of w2 as Q6_K).
 `--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with another
 GGML format (random block payloads with small finite scales: timing does not depend on the values).
 
@@ -64,12 +65,13 @@ def random_blocks(np, rng, fmt, n_elems):
     return raw.reshape(-1)
 
 
-def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k", fmt_down=None):
+def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k", fmt_down=None, quantise=False):
     """Weights drawn on the GPU, quantised there with the library's QTensor::quantize kernel (bit-identical to candle's
     CPU quantiser), returned as host bytes (the CPU baseline runs on the same bytes)."""
     h, f, e_n, dt, fs = (CFG4["H"], CFG4["F"], CFG4["E"], Q8_0, CFG4["Fs"]) if cfg4 else (H, F, E, Q4K, 0)
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
+    random_payload = fmt != "q4_k" and not cfg4 and not quantise
     if fmt != "q4_k" and not cfg4:
         import numpy as np
         dt = FORMATS[fmt][0]
@@ -78,7 +80,7 @@ def draw_weights(torch, candle_amd, seed=0, cfg4=False, fmt="q4_k", fmt_down=Non
     dt_down = FORMATS[fmt_down][0] if fmt_down else dt
 
     def draw(shape, dtype=None):
-        if fmt != "q4_k" and not cfg4:
+        if random_payload:
             return random_blocks(np, rng, fmt, shape[0] * shape[1])
         x = torch.randn(shape, generator=g, device="cuda", dtype=torch.float32) * 0.02
         return candle_amd.quantize_weights(dtype or dt, x).cpu().numpy()
@@ -362,8 +364,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="layers of the stack workload")
     ap.add_argument("--stack-steps", type=int, default=128, help="consecutive steps of the stack workload")
     ap.add_argument("--weights", choices=sorted(FORMATS), default="q4_k", help="GGML format of the expert matrices (decode workload)")
-    ap.add_argument("--weights-down", choices=("q6_k",), default=None,
-                    help="prefill workload: w2 in this format beside Q4_K w1 / w3 (the arrangement of Q4_K_M files)")
+    ap.add_argument("--weights-down", choices=("q5_k", "q6_k"), default=None,
+                    help="prefill workload: w2 in this format beside the w1 / w3 of --weights (Q4_K_M and Q5_K_M files store part of w2 as Q6_K)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
@@ -389,9 +391,9 @@ def main():
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
     wl = args.workload
-    if args.weights != "q4_k" and wl not in ("decode", "all"):
-        sys.exit("bench.py: --weights applies to the decode workload only")
-    if args.weights != "q4_k":
+    if args.weights != "q4_k" and wl not in ("decode", "all") and not (wl == "prefill" and args.weights == "q5_k"):
+        sys.exit("bench.py: --weights applies to the decode workload (and q5_k to the prefill workload) only")
+    if args.weights != "q4_k" and wl != "prefill":
         wl = "decode"
     if args.weights_down and wl != "prefill":
         sys.exit("bench.py: --weights-down applies to the prefill workload only")
@@ -424,11 +426,11 @@ def main():
                                             "y = x + moe(rms_norm(x)) per layer, %d-token batch, each step fed the previous output plus N(0, 0.1) noise"
                                             % (args.layers, m["resident_gb"], m["batch"])}, **{k: v for k, v in m.items() if k != "roofline"}))
     elif wl == "prefill":
-        w = draw_weights(torch, candle_amd, fmt_down=args.weights_down)
+        w = draw_weights(torch, candle_amd, fmt=args.weights, fmt_down=args.weights_down, quantise=True)
         layer = make_layer(candle_amd, w, gate_bias=bias)
         B = args.batch or 4096
         m = measure_prefill(args, np, torch, timer, layer, B)
-        wdesc = "Q4_K weights" if not args.weights_down else "Q4_K w1 / w3 with %s w2" % args.weights_down
+        wdesc = "%s weights" % args.weights if not args.weights_down else "%s w1 / w3 with %s w2" % (args.weights, args.weights_down)
         out.update(metric="MoE layer tokens/s (Mixtral-8x7B shape, Q4_K, prefill)", value=m["tokens_per_s"], ms_per_step=m["ms_per_step"],
                    timed_steps=m["timed_steps"], roofline=m["roofline"],
                    config=dict({"workload": "BASELINE config 3: hidden 4096, ffn 14336, 8 experts, top-2, %s, prefill of %d tokens, "

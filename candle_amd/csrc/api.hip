@@ -450,14 +450,14 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     const Switches& sw = switches();
     ForwardPlan pl;
     const bool shared = L->Fs > 0;
-    // Q4K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
+    // Q4K / Q5K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
     // multiple of 64, H of 128; those kernels address activation rows with 32-bit byte offsets), from ~64 rows per
     // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
     // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
     // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
-    // (a Q6K w2 beside Q4K w1 / w3, as mixed files carry, takes the tiled down kernel's Q6K variant)
-    pl.tiled = !sw.no_gemm && L->dt == MOE_GGML_Q4K && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 38 * L->E;
-    pl.tiled_down = pl.tiled && (L->dt_down == MOE_GGML_Q4K || L->dt_down == MOE_GGML_Q6K) && T * L->k > 64 * L->E;
+    // (w2 may be Q4K, Q5K or Q6K whatever w1 / w3 are: mixed files store part of it as Q6K)
+    pl.tiled = !sw.no_gemm && q4k_gemm_up_format(L->dt) && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 38 * L->E;
+    pl.tiled_down = pl.tiled && q4k_gemm_down_format(L->dt_down) && T * L->k > 64 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
     pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 96 * L->E ? 128 : 64;
@@ -990,7 +990,7 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     // once that grid fills most of the 256 CUs; below, the streamed kernels split the matrix finer.
     const int64_t row_blocks = Q->n / 128;
     const int tile_slots = row_blocks * ((m + 127) / 128) >= 512 ? 128 : 64;
-    const bool tiled = !switches().no_gemm && Q->dt == MOE_GGML_Q4K && Q->n % 128 == 0 && m >= 96 &&
+    const bool tiled = !switches().no_gemm && q4k_gemm_down_format(Q->dt) && Q->n % 128 == 0 && m >= 96 &&
                        row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192;
     rb.T = (int)m; rb.k = 1;
     rb.tile_slots = tile_slots;

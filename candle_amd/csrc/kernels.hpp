@@ -107,6 +107,8 @@ hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
 // Tiled (prefill) variants for Q4K in dispatched mode: activations staged through LDS, weights
 // unpacked and pre-scaled per wave, v_mfma_i32_32x32x32_i8.  up writes f32 h into p.hbuf (the
 // caller re-quantises it), down writes yw.
+bool q4k_gemm_up_format(int dt);
+bool q4k_gemm_down_format(int dt);
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 

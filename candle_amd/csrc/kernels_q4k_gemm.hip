@@ -1,5 +1,5 @@
-// Tiled grouped expert products for large batches (prefill): Q4K weights x Q8K activations on
-// v_mfma_i32_16x16x64_i8, a full-rate int8 MFMA shape of gfx950.
+// Tiled grouped expert products for large batches (prefill): Q4K (also Q5K, and Q6K for the down projection) weights x
+// Q8K activations on v_mfma_i32_16x16x64_i8, a full-rate int8 MFMA shape of gfx950.
 //
 // Same integers as BlockQ4K::vec_dot (candle-core/src/quantized/k_quants.rs:1205-1285):
 //     sum_j sc_j * (q4_j . q8_j)      and      sum_j m_j * (bsum_2j + bsum_2j+1).
@@ -116,6 +116,7 @@ struct BRegs {
     u32x4 c[2];   // plane pl: (x,y) = 8 bytes of pair 2pl, chunk g; (z,w) = pair 2pl+1 (Q6K: the codes' low nibbles)
     u32x4 hdr;    // Q4K: d, dmin, 12 scale bytes of row n; Q6K: the row's sixteen i8 scales
     u32x4 qh;     // Q6K: the codes' top two bits, word P for pair P
+    u32x2 q5;     // Q5K: the lane's fifth bits (pairs 0,1 / 2,3; four bits per byte and pair)
     uint32_t d16; // Q6K: d (f16 bits)
 };
 template <int FMT>
@@ -129,6 +130,7 @@ __device__ __forceinline__ BRegs b_load(const uint8_t* tile, int lane) {
         b.d16 = gld<uint16_t>(tile, (uint32_t)(3328 + (lane & 15) * 2));
     } else {
         b.hdr = gld<u32x4>(tile, (uint32_t)(2048 + (lane & 15) * 16));
+        if (FMT == MOE_GGML_Q5K) b.q5 = gld<u32x2>(tile, (uint32_t)(Q4K_TILE_BYTES + lane * 8));
     }
     return b;
 }
@@ -220,6 +222,44 @@ __device__ __forceinline__ BPlanes b_prepare_q6k(const BRegs& b, int lane) {
     return o;
 }
 
+// Q5K (BlockQ5K::vec_dot, k_quants.rs:1394-1485): the Q4K sums on 5-bit codes.  A 3-bit digit times a code of up to 31
+// no longer fits a signed byte, so the planes are the two bytes of W = sc * code (<= 1953), formed and cut as for Q6K
+// (no offset: the minimum leaves through the block sums, as for Q4K).
+__device__ __forceinline__ BPlanes b_prepare_q5k(const BRegs& b, int lane) {
+    const int g = lane >> 4;
+    const uint32_t M4 = 0x0f0f0f0fu, M1H = 0x10101010u;
+    const uint32_t u0 = b.hdr.y, u1 = b.hdr.z, u2 = b.hdr.w;
+    BPlanes o;
+    o.d = __half2float(__ushort_as_half((unsigned short)(b.hdr.x & 0xffffu)));
+    o.dmin = __half2float(__ushort_as_half((unsigned short)(b.hdr.x >> 16)));
+    const uint32_t sc03 = u0 & 0x3f3f3f3fu;
+    const uint32_t sc47 = (u2 & M4) | (((u0 >> 6) & 0x03030303u) << 4);
+    const uint32_t m03 = u1 & 0x3f3f3f3fu;
+    const uint32_t m47 = ((u2 >> 4) & M4) | (((u1 >> 6) & 0x03030303u) << 4);
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const u32x4 c = b.c[P >> 1];
+        const uint32_t w0 = (P & 1) ? c.z : c.x, w1 = (P & 1) ? c.w : c.y;
+        const uint32_t h = ((P < 2) ? b.q5.x : b.q5.y) >> (4 * (P & 1));
+        const uint32_t scw = (P < 2) ? sc03 : sc47;
+        const uint32_t sa = (scw >> (16 * (P & 1))) & 0xffu, sb = (scw >> (16 * (P & 1) + 8)) & 0xffu;
+        const uint32_t sa2 = sa | (sa << 16), sb2 = sb | (sb << 16);
+        const uint32_t c0 = (w0 & M4) | ((h << 4) & M1H), c1 = (w1 & M4) | ((h << 3) & M1H);
+        const uint32_t c2 = ((w0 >> 4) & M4) | ((h << 2) & M1H), c3 = ((w1 >> 4) & M4) | ((h << 1) & M1H);
+        int l0, l1, l2, l3, h0, h1, h2, h3;
+        q6k_planes(c0, sa2, 0x00800080u, l0, h0);
+        q6k_planes(c1, sa2, 0x00800080u, l1, h1);
+        q6k_planes(c2, sb2, 0x00800080u, l2, h2);
+        q6k_planes(c3, sb2, 0x00800080u, l3, h3);
+        o.lo[P] = v4i{l0, l1, l2, l3};
+        o.hi[P] = v4i{h0, h1, h2, h3};
+    }
+    const uint32_t mw = (g < 2) ? m03 : m47;
+    const uint32_t ma = (mw >> (16 * (g & 1))) & 0xffu, mb = (mw >> (16 * (g & 1) + 8)) & 0xffu;
+    o.mB = v4h{(_Float16)(int)ma, (_Float16)(int)ma, (_Float16)(int)mb, (_Float16)(int)mb};
+    return o;
+}
+
 // one super-block of the wave's 16 weight rows against 16-slot operand o of the staged tile
 // `while_busy` runs right after the MFMAs are issued: this is where the next super-block's loads go.
 template <int FMT, int NOP, typename Fill>
@@ -251,7 +291,7 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
         while_busy();
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int isum = (acc_hi[i] << 3) + acc_lo[i];
+            const int isum = (acc_hi[i] << (FMT == MOE_GGML_Q5K ? 8 : 3)) + acc_lo[i];
             const float v = __builtin_fmaf(B.d, (float)isum, -(B.dmin * Dm[i]));
             facc[i] = __builtin_fmaf(yd[i], v, facc[i]);
         }
@@ -267,12 +307,12 @@ __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-// FMT: the weights' format (Q4K; Q6K for MODE 1 only).
+// FMT: the weights' format (Q4K, Q5K; Q6K for MODE 1 only).
 template <int FMT, int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
-    static_assert(FMT == MOE_GGML_Q4K || (FMT == MOE_GGML_Q6K && MODE == 1), "formats of the tiled kernel");
+    static_assert(FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || (FMT == MOE_GGML_Q6K && MODE == 1), "formats of the tiled kernel");
     constexpr int NB = NOP / 2;
-    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : Q4K_TILE_BYTES;
+    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : Q4K_TILE_BYTES;
     constexpr bool kSums = FMT != MOE_GGML_Q6K;   // block sums staged (the mins term)
     __shared__ GemmLds<NOP> L;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -332,6 +372,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     };
     auto prepare = [&](const BRegs& r) {
         if constexpr (FMT == MOE_GGML_Q6K) return b_prepare_q6k(r, lane);
+        else if constexpr (FMT == MOE_GGML_Q5K) return b_prepare_q5k(r, lane);
         else return b_prepare(r, lane);
     };
     using std::integral_constant;
@@ -409,19 +450,27 @@ static unsigned gemm_grid(int n_rb, int64_t max_tiles) {
     const int64_t RG = (n_rb + 7) / 8, TG = (max_tiles + 7) / 8;
     return (unsigned)((RG * TG + 7) / 8 * 8 * 64);
 }
+template <int FMT, int MODE>
+static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
+    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 4>), grid, dim3(G_THREADS), 0, s, p);
+    else hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 8>), grid, dim3(G_THREADS), 0, s, p);
+}
+bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K; }
+bool q4k_gemm_down_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s) {
     dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
-    if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 0, 4>), grid, dim3(G_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 0, 8>), grid, dim3(G_THREADS), 0, s, p);
+    if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
+    else if (p.dt == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 0>(p, grid, s);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s) {
     dim3 grid(gemm_grid(p.H / 128, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
-    if (p.dt_down == MOE_GGML_Q6K) {
-        if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q6K, 1, 4>), grid, dim3(G_THREADS), 0, s, p);
-        else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q6K, 1, 8>), grid, dim3(G_THREADS), 0, s, p);
-    } else if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 1, 4>), grid, dim3(G_THREADS), 0, s, p);
-    else hipLaunchKernelGGL((q4k_gemm_kernel<MOE_GGML_Q4K, 1, 8>), grid, dim3(G_THREADS), 0, s, p);
+    const int dtd = p.dt_down ? p.dt_down : p.dt;
+    if (dtd == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 1>(p, grid, s);
+    else if (dtd == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 1>(p, grid, s);
+    else if (dtd == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 1>(p, grid, s);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 
