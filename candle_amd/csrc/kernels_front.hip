@@ -603,8 +603,8 @@ __device__ inline float ordered_sum_of_squares(const float* xr, int tid, bool se
     return result;
 }
 
-template <int VDT, int NCH>
-__global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p) {
+template <int VDT, int NCH, bool LEAN>
+__device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     __shared__ float logit_lds[64];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -635,9 +635,9 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
     };
     // (only with an rms-norm ahead: without one the early request measured 0.9 us slower on a gate that is still in the
     // L2; and not for rows beyond 4096, where two gate rows and the token's row exceed the registers)
-    const bool early_gate = NCH <= 16 && p.rms_alpha != nullptr;
+    const bool early_gate = !LEAN && NCH <= 16 && p.rms_alpha != nullptr;
     if (early_gate && wave < 4 && wave < n_dot) load_gate_pair(wave);
-    if (p.rms_alpha) {
+    if (!LEAN && p.rms_alpha) {
         // rms_norm (candle-nn/src/ops.rs:504-515) sums the squares left to right in f32.  A different
         // order changes the divisor in the last ulp, which flips quantised activations now and then
         // and moves a whole output row by 1e-3 of its rms, so the sum keeps the reference's order.
@@ -660,18 +660,61 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
             xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
         }
     }
-    if (wave < 4) {
-        // gate products
-        for (int e0 = wave; e0 < n_dot; e0 += 8) {
-            const int e1 = e0 + 4 < n_dot ? e0 + 4 : e0;
-            if (!early_gate || e0 != wave) load_gate_pair(e0);
-            float acc0 = 0.f, acc1 = 0.f;
+    // rows of 4096 and more leave no registers for a second buffer (and few experts per wave to run ahead over)
+    // gate products: waves 0..3 while waves 4..7 quantise (all eight waves on the products with the quantisation shared
+    // out afterwards measured no better at 61 products per token and worse at 8)
+    constexpr int GW = 4;
+    constexpr bool LEAN_PIPE = NCH < 16;
+    constexpr int LEAN_PIECE = LEAN_PIPE ? 2 : 4, LEAN_NP = LEAN ? NCH / LEAN_PIECE : 2;
+    static_assert(!LEAN || (NCH % LEAN_PIECE == 0 && LEAN_NP % 2 == 0), "the pieces alternate between two buffers");
+    float4 qa[2][LEAN_PIECE], qb[2][LEAN_PIECE];
+    auto load_piece = [&](int e0, int pc, int buf) {
+        const int e1 = e0 + GW < n_dot ? e0 + GW : e0;
+        const float* w0 = (e0 < E) ? p.gate + (int64_t)e0 * H : p.shared_gate;
+        const float* w1 = (e1 < E) ? p.gate + (int64_t)e1 * H : p.shared_gate;
 #pragma unroll
-            for (int i = 0; i < NCH; i++) {
-                acc0 = __builtin_fmaf(wa[i].x, xr[4 * i], acc0);     acc1 = __builtin_fmaf(wb[i].x, xr[4 * i], acc1);
-                acc0 = __builtin_fmaf(wa[i].y, xr[4 * i + 1], acc0); acc1 = __builtin_fmaf(wb[i].y, xr[4 * i + 1], acc1);
-                acc0 = __builtin_fmaf(wa[i].z, xr[4 * i + 2], acc0); acc1 = __builtin_fmaf(wb[i].z, xr[4 * i + 2], acc1);
-                acc0 = __builtin_fmaf(wa[i].w, xr[4 * i + 3], acc0); acc1 = __builtin_fmaf(wb[i].w, xr[4 * i + 3], acc1);
+        for (int j = 0; j < LEAN_PIECE; j++) {
+            qa[buf][j] = *reinterpret_cast<const float4*>(w0 + (pc * LEAN_PIECE + j) * 256 + lane * 4);
+            qb[buf][j] = *reinterpret_cast<const float4*>(w1 + (pc * LEAN_PIECE + j) * 256 + lane * 4);
+        }
+    };
+    if (wave < GW) {
+        // gate products
+        if (LEAN && LEAN_PIPE && wave < n_dot) load_piece(wave, 0, 0);
+        for (int e0 = wave; e0 < n_dot; e0 += 2 * GW) {
+            const int e1 = e0 + GW < n_dot ? e0 + GW : e0;
+            float acc0 = 0.f, acc1 = 0.f;
+            if constexpr (LEAN) {
+                // the gate rows pass through in pieces of two or four chunks (same products, same order; a quarter of
+                // the registers, so that two workgroups fit a CU); short rows: each piece is requested while the one before
+                // it is multiplied, across the wave's experts too
+#pragma unroll
+                for (int pc = 0; pc < LEAN_NP; pc++) {
+                    if (!LEAN_PIPE) load_piece(e0, pc, 0);
+                    else if (pc + 1 < LEAN_NP) load_piece(e0, pc + 1, (pc + 1) & 1);
+                    else if (e0 + 2 * GW < n_dot) load_piece(e0 + 2 * GW, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int buf = LEAN_PIPE ? (pc & 1) : 0;
+#pragma unroll
+                    for (int j = 0; j < LEAN_PIECE; j++) {
+                        const int i = pc * LEAN_PIECE + j;
+                        const float4 a = qa[buf][j], b = qb[buf][j];
+                        acc0 = __builtin_fmaf(a.x, xr[4 * i], acc0);     acc1 = __builtin_fmaf(b.x, xr[4 * i], acc1);
+                        acc0 = __builtin_fmaf(a.y, xr[4 * i + 1], acc0); acc1 = __builtin_fmaf(b.y, xr[4 * i + 1], acc1);
+                        acc0 = __builtin_fmaf(a.z, xr[4 * i + 2], acc0); acc1 = __builtin_fmaf(b.z, xr[4 * i + 2], acc1);
+                        acc0 = __builtin_fmaf(a.w, xr[4 * i + 3], acc0); acc1 = __builtin_fmaf(b.w, xr[4 * i + 3], acc1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                if (!early_gate || e0 != wave) load_gate_pair(e0);
+#pragma unroll
+                for (int i = 0; i < NCH; i++) {
+                    acc0 = __builtin_fmaf(wa[i].x, xr[4 * i], acc0);     acc1 = __builtin_fmaf(wb[i].x, xr[4 * i], acc1);
+                    acc0 = __builtin_fmaf(wa[i].y, xr[4 * i + 1], acc0); acc1 = __builtin_fmaf(wb[i].y, xr[4 * i + 1], acc1);
+                    acc0 = __builtin_fmaf(wa[i].z, xr[4 * i + 2], acc0); acc1 = __builtin_fmaf(wb[i].z, xr[4 * i + 2], acc1);
+                    acc0 = __builtin_fmaf(wa[i].w, xr[4 * i + 3], acc0); acc1 = __builtin_fmaf(wb[i].w, xr[4 * i + 3], acc1);
+                }
             }
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) {
@@ -697,9 +740,10 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
                 }
             }
         }
-    } else {
+    }
+    if (wave >= GW) {
         // quantise: wave 4+q owns chunks q, q+4, ...; the branches are wave-uniform
-        const int q = wave - 4;
+        const int q = wave - GW;
 #pragma unroll
         for (int i = 0; i < NCH; i++)
             if ((i & 3) == q) {
@@ -714,6 +758,16 @@ __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p)
         for (int i = tid; i < H / 4; i += FAST_THREADS) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (wave == 0) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk,
                                         p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+}
+template <int VDT, int NCH>
+__global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p) {
+    front_fast_body<VDT, NCH, false>(p);
+}
+// The same for large batches: at most 128 registers, so that two workgroups share a CU (a batch of thousands of tokens
+// is bound by how many of these latency chains run at once, a decode batch by the length of one).
+template <int VDT, int NCH>
+__global__ __launch_bounds__(FAST_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void front_fast_kernel_dense(FrontParams p) {
+    front_fast_body<VDT, NCH, true>(p);   // layers without the pre-norm only
 }
 
 // RmsNorm::forward as a kernel of its own (candle-nn/src/ops.rs:504-515; the `(attn + residual)` that precedes the
@@ -889,9 +943,15 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
         case 1: hipLaunchKernelGGL((front_fast_kernel<VDT, 1>), grid, block, 0, s, p); return true;
         case 2: hipLaunchKernelGGL((front_fast_kernel<VDT, 2>), grid, block, 0, s, p); return true;
         case 4: hipLaunchKernelGGL((front_fast_kernel<VDT, 4>), grid, block, 0, s, p); return true;
-        case 8: hipLaunchKernelGGL((front_fast_kernel<VDT, 8>), grid, block, 0, s, p); return true;
+        case 8:
+            if (p.T >= 256 && !p.rms_alpha) hipLaunchKernelGGL((front_fast_kernel_dense<VDT, 8>), grid, block, 0, s, p);
+            else hipLaunchKernelGGL((front_fast_kernel<VDT, 8>), grid, block, 0, s, p);
+            return true;
         case 12: hipLaunchKernelGGL((front_fast_kernel<VDT, 12>), grid, block, 0, s, p); return true;
-        case 16: hipLaunchKernelGGL((front_fast_kernel<VDT, 16>), grid, block, 0, s, p); return true;
+        case 16:
+            if (p.T >= 1024 && !p.rms_alpha) hipLaunchKernelGGL((front_fast_kernel_dense<VDT, 16>), grid, block, 0, s, p);
+            else hipLaunchKernelGGL((front_fast_kernel<VDT, 16>), grid, block, 0, s, p);
+            return true;
         case 20: hipLaunchKernelGGL((front_fast_kernel<VDT, 20>), grid, block, 0, s, p); return true;
         case 24: hipLaunchKernelGGL((front_fast_kernel<VDT, 24>), grid, block, 0, s, p); return true;
         case 28: hipLaunchKernelGGL((front_fast_kernel<VDT, 28>), grid, block, 0, s, p); return true;
