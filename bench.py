@@ -189,6 +189,18 @@ def cpu_baseline(w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=Fals
                       "(AVX2 vec_dot, %d threads over output columns)" % (reps, xs_host.shape[0], dt, cores)}
 
 
+def profiled_value(name, label, key):
+    """A `label[key]: value` line of a committed profile summary (a float), or None."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            m = re.match(r"%s\[([^\]]+)\]:\s*([0-9.eE+-]+)" % re.escape(label), line.strip())
+            if m and m.group(1) == key:
+                return float(m.group(2))
+    except OSError:
+        pass
+    return None
+
+
 def profiled_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
     """HBM bytes per launch of the dominant kernel as the committed rocprofv3 counter summary gives them (FETCH_SIZE +
     WRITE_SIZE, scaled by the copy kernel): a figure from that profile, not a reading of this run; None when the summary
@@ -260,7 +272,11 @@ def measure_prefill(args, np, torch, timer, layer, B):
                 # every algorithmic multiply-add is issued twice (the 6-bit scale is split over two pre-scaled int8
                 # planes so that the integer sums stay exact): share of the peak the MFMA pipe is actually kept busy
                 # with, slot tiles padded to 64 / 128 not counted
-                "mfma_issued_frac": 2.0 * achieved / INT8_PEAK_TOPS}
+                "mfma_issued_frac": 2.0 * achieved / INT8_PEAK_TOPS,
+                # share of the cycles the matrix pipe is busy (SQ_VALU_MFMA_BUSY_CYCLES over the kernel's SIMD cycles)
+                # as the committed rocprofv3 counter summary gives it: a figure of that profile, not a reading of this run
+                "mfma_pipe_busy_frac": profiled_value("q4k_gemm_prefill_4096_kernel_trace.md", "mfma_busy_frac", "prefill_up") if B == 4096 else None,
+                "mfma_pipe_busy_source": "profiles/q4k_gemm_prefill_4096_kernel_trace.md (rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES, SQ_CYCLES)"}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "tokens": B, "expert_loads": [int(v) for v in loads], "stage_us": stage_us, "step_int8_ops": step_ops,
             "step_mfma_frac": step_ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, "roofline": roofline, "xs": xs, "ys": ys}
