@@ -1,4 +1,4 @@
-// Tiled grouped expert products for large batches (prefill): Q4K (also Q5K, and Q6K for the down projection) weights x
+// Tiled grouped expert products for large batches (prefill): Q4K (also Q5K and Q6K) weights x
 // Q8K activations on v_mfma_i32_16x16x64_i8, a full-rate int8 MFMA shape of gfx950.
 //
 // Same integers as BlockQ4K::vec_dot (candle-core/src/quantized/k_quants.rs:1205-1285):
@@ -307,10 +307,10 @@ __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-// FMT: the weights' format (Q4K, Q5K; Q6K for MODE 1 only).
+// FMT: the weights' format (Q4K, Q5K, Q6K).
 template <int FMT, int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
-    static_assert(FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || (FMT == MOE_GGML_Q6K && MODE == 1), "formats of the tiled kernel");
+    static_assert(FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || FMT == MOE_GGML_Q6K, "formats of the tiled kernel");
     constexpr int NB = NOP / 2;
     constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : Q4K_TILE_BYTES;
     constexpr bool kSums = FMT != MOE_GGML_Q6K;   // block sums staged (the mins term)
@@ -455,11 +455,12 @@ static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
     if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 4>), grid, dim3(G_THREADS), 0, s, p);
     else hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 8>), grid, dim3(G_THREADS), 0, s, p);
 }
-bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K; }
+bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
 bool q4k_gemm_down_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s) {
     dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
-    if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
+    if (p.dt == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 0>(p, grid, s);
+    else if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 0>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
