@@ -47,7 +47,8 @@ def build_library(verbose=False, out_dir=None, extra_flags=()):
         for _, err in results:
             if err.strip():
                 print(err)
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path] + objs
+    # -Wl,--no-undefined: a launcher that a source file no longer defines fails the link here, not the first dlopen
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", "-o", lib_path] + objs
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))

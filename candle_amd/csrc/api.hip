@@ -482,8 +482,8 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     pl.narrow = pl.direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && pl.slot_tiles == 1 &&
                 (sw.narrow >= 0 ? sw.narrow > 0 : T * L->k <= L->E);
     pl.hbuf = pl.tiled || pl.narrow;
-    // Q8_0 layers whose slots are grouped by expert (more than DIRECT_MAX_SLOTS assignments): the tiled kernels of
-    // kernels_q32.hip read an expert's weights once for up to 64 of its slots
+    // Q8_0 / Q4_0 / Q5_0 layers whose slots are grouped by expert (more than DIRECT_MAX_SLOTS assignments): the tiled
+    // kernels of kernels_q32.hip read an expert's weights once for up to 64 of its slots
     pl.tiled32 = !sw.no_gemm && !pl.direct && q8_0_gemm_usable(L->dt, L->dt_down, L->H, L->F) && T * L->k > 20 * L->E;
     if (pl.tiled32) pl.tile_slots = 64;
     return pl;
@@ -591,7 +591,11 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
         MOE_MARK(ST_DOWN);
     } else if (pl.tiled32) {
         ep.n_slots = T * L->k;
-        MOE_HIP_CHECK(launch_q8_0_gemm_up(ep, s));   // quantises the intermediate in its epilogue
+        // (Q4_0 w1 / w3 stay with the streaming kernel: its nibble unpacking and offset addends per block put the tiled
+        // up kernel 3 % behind it at the Mixtral shape, 4832 against 4683 us for 4096 tokens; both quantise the
+        // intermediate in their epilogue)
+        if (L->dt == MOE_GGML_Q4_0) MOE_HIP_CHECK(launch_expert_up(ep, s));
+        else MOE_HIP_CHECK(launch_q8_0_gemm_up(ep, s));
         MOE_MARK(ST_UP);
         MOE_MARK(ST_REQUANT);
         MOE_HIP_CHECK(launch_q8_0_gemm_down(ep, s));

@@ -692,7 +692,7 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Tiled grouped products for Q8_0 weights (batches whose slots are grouped by expert): one pass over an expert's
+// Tiled grouped products for Q8_0 weights, and for Q4_0 / Q5_0 (batches whose slots are grouped by expert): one pass over an expert's
 // weights for up to 64 of its slots, where the streaming kernels above take a pass per 32.
 //
 // Same arithmetic and the same order of additions as q32s_mac (bit-identical results): one
@@ -713,6 +713,7 @@ constexpr int QG_THREADS = 512;
 struct alignas(16) QGemmLds {
     alignas(16) uint8_t q[2][QG_NOP][8][256];       // [buffer][operand][piece][slot m] 16 bytes
     alignas(16) float yd[2][QG_NOP * 16][4];          // [buffer][slot][block of the step]
+    alignas(16) int bs[2][QG_NOP * 16][4];            // the blocks' sums of quants (formats with a code offset)
 };
 __device__ __forceinline__ uint32_t qg_lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
@@ -722,9 +723,10 @@ __device__ __forceinline__ void qg_dma16(const void* gbase, uint32_t voff, uint3
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbase), "s"(lds));
 }
 
-template <int MODE>
+template <int DT, int MODE>
 __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q8_0_gemm_kernel(ExpertParams p) {
-    constexpr int DT = MOE_GGML_Q8_0;
+    static_assert(DT == MOE_GGML_Q8_0 || DT == MOE_GGML_Q4_0 || DT == MOE_GGML_Q5_0, "formats with Q8_0 activations and no minimum");
+    constexpr int OFFSET = Q32Fmt<DT>::OFFSET;
     constexpr size_t STB = Q32SFmt<DT>::STB;
     __shared__ QGemmLds L;
     __shared__ float hx[MODE == 0 ? QG_NOP * 16 : 1][MODE == 0 ? 65 : 1];   // MODE 0: h of the tile's slots x the workgroup's 64 rows
@@ -768,6 +770,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     auto stage = [&](int ks, int buf) {
         qg_dma16(ab.qs, q_src + (uint32_t)(ks * 128), qg_lds_address(&L.q[buf][wave >> 1][4 * (wave & 1)][0]));
         if (wave == 0) qg_dma16(ab.d, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.yd[buf][0][0]));
+        if (OFFSET && wave == 1) qg_dma16(ab.bsum, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.bs[buf][0][0]));
     };
 
     const GroupWeights gw = p.groups[grp];
@@ -819,7 +822,12 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                     const uint32_t alo = *reinterpret_cast<const uint32_t*>(ap), ahi = *reinterpret_cast<const uint32_t*>(ap + 256);
                     const long av = (long)(((uint64_t)ahi << 32) | alo);
                     const long bv = (long)(((uint64_t)wq[b].y << 32) | wq[b].x);
-                    D[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, magic, 0, 0, 0);
+                    v4i addend = magic;
+                    if (OFFSET) {   // stored code = value + OFFSET: the block's sum of quants leaves through the addend
+#pragma unroll
+                        for (int i = 0; i < 4; i++) addend[i] = Q32S_MAGIC_BITS - OFFSET * L.bs[buf][o * 16 + 4 * g + i][b];
+                    }
+                    D[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, addend, 0, 0, 0);
                 }
                 // ascending block order per (row, slot), every product rounded where the reference rounds it
 #pragma unroll
@@ -899,8 +907,9 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 }
 
+static bool qg_format(int dt) { return dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q5_0; }
 bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F) {
-    return dt == MOE_GGML_Q8_0 && (dt_down == 0 || dt_down == MOE_GGML_Q8_0) && H % 128 == 0 && F % 128 == 0;
+    return qg_format(dt) && (dt_down == 0 || qg_format(dt_down)) && H % 128 == 0 && F % 128 == 0;
 }
 static unsigned qg_grid(int n_rb, int64_t tiles) {
     const int64_t RG = (n_rb + 7) / 8, TG = (tiles + 7) / 8;
@@ -909,15 +918,23 @@ static unsigned qg_grid(int n_rb, int64_t tiles) {
 static int64_t qg_tiles(const ExpertParams& p) {
     return p.is_shared ? (p.max_rows + QG_NOP * 16 - 1) / (QG_NOP * 16) : max_gemm_tiles(p.n_slots, p.n_groups + 1, QG_NOP * 16);
 }
+template <int MODE>
+static hipError_t qg_launch(int dt, const ExpertParams& p, dim3 grid, hipStream_t s) {
+    switch (dt) {
+        case MOE_GGML_Q8_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q8_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q4_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q4_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q5_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q5_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
 hipError_t launch_q8_0_gemm_up(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    hipLaunchKernelGGL((q8_0_gemm_kernel<0>), dim3(qg_grid(p.F / 64, qg_tiles(p))), dim3(QG_THREADS), 0, s, p);
-    return hipGetLastError();
+    return qg_launch<0>(p.dt, p, dim3(qg_grid(p.F / 64, qg_tiles(p))), s);
 }
 hipError_t launch_q8_0_gemm_down(const ExpertParams& p, hipStream_t s) {
     if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    hipLaunchKernelGGL((q8_0_gemm_kernel<1>), dim3(qg_grid(p.H / 128, qg_tiles(p))), dim3(QG_THREADS), 0, s, p);
-    return hipGetLastError();
+    return qg_launch<1>(p.dt_down ? p.dt_down : p.dt, p, dim3(qg_grid(p.H / 128, qg_tiles(p))), s);
 }
 
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s);

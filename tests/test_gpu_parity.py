@@ -133,7 +133,7 @@ def test_route_zipf_bias_lists():
                                        (O.Q5K, 64, 512, 5), (O.Q5K, 1040, 1024, 33), (O.Q5K, 256, 2304, 150),
                                        (O.Q6K, 64, 512, 5), (O.Q6K, 1040, 1024, 33), (O.Q6K, 256, 2304, 150),
                                        (O.Q4K, 4096, 1024, 700), (O.Q5K, 4096, 1024, 700), (O.Q6K, 4096, 1024, 700),
-                                       (O.Q8_0, 4096, 1024, 1100), (O.Q8_0, 2048, 1408, 2100),
+                                       (O.Q8_0, 4096, 1024, 1100), (O.Q8_0, 2048, 1408, 2100), (O.Q4_0, 4096, 1024, 1100), (O.Q5_0, 2048, 1408, 2100),
                                        (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70),
                                        (O.Q5_0, 48, 96, 3), (O.Q5_0, 256, 1408, 40), (O.Q5_0, 128, 1024, 70),
                                        (O.Q4_1, 48, 96, 3), (O.Q4_1, 256, 1408, 40), (O.Q4_1, 128, 1024, 70),
@@ -341,6 +341,19 @@ def test_block_32_element_formats_ragged_row_tiles(dt):
         w = O.fill_normal_quantized(n + k, dt, n, k, 0.02)
         x = activations(m, k, seed=n)
         assert np.array_equal(bits(candle_amd.qmatmul(dt, w, n, k, x)), bits(O.matmul(dt, x, w, n)))
+
+
+@pytest.mark.parametrize("dt,dt_down", [(O.Q4_0, None), (O.Q5_0, None), (O.Q8_0, None), (O.Q4_0, O.Q8_0), (O.Q5_0, O.Q4_0)])
+def test_block_32_element_formats_tiled_kernels(dt, dt_down):
+    # beyond 1024 assignments the slots are grouped by expert and the Q8_0-activation formats take the tiled kernels
+    # (64-slot tiles): lists of ~300 and ~650 rows, a last tile of every length, and a shared expert beside them
+    ref, gpu = make_pair(256, 384, 4, 2, dt, seed=50, dt_down=dt_down)
+    for T in (600, 1301):
+        check_block(ref, gpu, T, tol=TOL)
+    gpu.close()
+    ref, gpu = make_pair(128, 256, 6, 3, dt, seed=51, dt_down=dt_down, Fs=384)
+    check_block(ref, gpu, 700, tol=TOL)
+    gpu.close()
 
 
 def test_mixed_dtypes_need_one_activation_format():
