@@ -17,6 +17,12 @@ struct GroupSlots {
 template <int NTHREADS>
 __device__ inline GroupSlots group_slots(const ExpertParams& p, int grp, int* list_lds, int* wtot_lds) {
     GroupSlots gs;
+    if (p.is_shared) {   // every token, in order, at slots T*k ..: needs nothing of the routing (nor of the dispatch pass)
+        gs.s_begin = p.rb.T * p.rb.k;
+        gs.n = p.rb.T;
+        gs.list = nullptr;
+        return gs;
+    }
     if (!p.rb.direct) {
         gs.s_begin = p.rb.offsets[p.group0 + grp];
         gs.n = p.rb.offsets[p.group0 + grp + 1] - gs.s_begin;
@@ -27,12 +33,6 @@ __device__ inline GroupSlots group_slots(const ExpertParams& p, int grp, int* li
     const int A = p.rb.T * p.rb.k;
     gs.s_begin = 0;
     gs.list = list_lds;
-    if (p.is_shared) {  // every token, in order
-        for (int i = tid; i < p.rb.T; i += NTHREADS) list_lds[i] = A + i;
-        __syncthreads();
-        gs.n = p.rb.T;
-        return gs;
-    }
     const int e = p.group0 + grp;
     int base = 0;
     const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -70,12 +70,12 @@ __device__ inline int group_of_row(const ExpertParams& p, int row) {
 
 // token row / routing weight of a slot
 __device__ inline int slot_token(const ExpertParams& p, int slot) {
-    if (!p.rb.direct) return p.rb.perm_token[slot];
-    return p.is_shared ? slot - p.rb.T * p.rb.k : slot / p.rb.k;
+    if (p.is_shared) return slot - p.rb.T * p.rb.k;
+    return p.rb.direct ? slot / p.rb.k : p.rb.perm_token[slot];
 }
 __device__ inline float slot_weight(const ExpertParams& p, int slot) {
-    if (!p.rb.direct) return p.rb.perm_w[slot];
-    return p.is_shared ? p.rb.shared_w[slot - p.rb.T * p.rb.k] : p.rb.topk_w[slot];
+    if (p.is_shared) return p.rb.shared_w[slot - p.rb.T * p.rb.k];
+    return p.rb.direct ? p.rb.topk_w[slot] : p.rb.perm_w[slot];
 }
 
 // Hands one weighted expert output to the layer's result.  With top-2 routing and nothing else to add, a token's result is
