@@ -569,10 +569,18 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
         sp.groups = L->groups.as<GroupWeights>() + L->E;
         sp.hq = ws.hq_shared; sp.slot_origin = (int)(T * L->k);
         sp.max_rows = T; sp.slot_tiles = T > 32 ? 4 : T > 16 ? 2 : 1;
-        // (measured at the Qwen-MoE shape, 512 tokens: the streaming kernels take 112 us for the always-on expert, the
-        // 64-slot tiled ones 183 us: its eight tiles by sixteen row blocks leave half of the CUs without a down workgroup)
-        MOE_HIP_CHECK(launch_expert_up(sp, ss));
-        MOE_HIP_CHECK(launch_expert_down(sp, ss));
+        // Tiled kernels for the always-on expert too once its up projection fills the chip twice over.  (Qwen-MoE shape,
+        // 512 tokens: alone on the GPU the tiled pair takes 132 us against 116 us streamed -- its down projection has
+        // 8 tiles x 16 row blocks = 128 workgroups -- but beside the routed launches the step takes 291 against 300 us:
+        // the tiled kernels read the expert's weights once, the streaming ones 16 times out of the caches.)
+        const bool shared_tiled = pl.tiled32 && L->Fs % 128 == 0 && (L->Fs / 64) * ((T + 63) / 64) >= 512;
+        if (shared_tiled) {
+            MOE_HIP_CHECK(launch_q8_0_gemm_up(sp, ss));
+            MOE_HIP_CHECK(launch_q8_0_gemm_down(sp, ss));
+        } else {
+            MOE_HIP_CHECK(launch_expert_up(sp, ss));
+            MOE_HIP_CHECK(launch_expert_down(sp, ss));
+        }
         return MOE_OK;
     };
     if (overlap_shared) {
@@ -1001,9 +1009,9 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     const int tile_slots = row_blocks * ((m + 127) / 128) >= 512 ? 128 : 64;
     const bool tiled = !switches().no_gemm && q4k_gemm_down_format(Q->dt) && Q->n % 128 == 0 && m >= 96 &&
                        row_blocks * ((m + tile_slots - 1) / tile_slots) >= 192;
-    // Q8_0 matrices: the tiled kernel of the 32-element formats (64-row tiles of the one group, no tile list) once its grid
-    // holds two workgroups per CU (4096 x 4096: 87 against 112 us at 1024 rows, 82 against 65 us at 512)
-    const bool tiled32 = !switches().no_gemm && q8_0_gemm_usable(Q->dt, 0, Q->n, Q->k) && row_blocks * ((m + 63) / 64) >= 512;
+    // Q8_0 / Q4_0 / Q5_0 matrices: the tiled kernel of the 32-element formats (64-row tiles of the one group, no tile list)
+    // once its grid holds a workgroup per CU (Q8_0, 4096 x 4096: 58 against 65 us at 512 rows, 53 against 42 us at 256)
+    const bool tiled32 = !switches().no_gemm && q8_0_gemm_usable(Q->dt, 0, Q->n, Q->k) && row_blocks * ((m + 63) / 64) >= 256;
     rb.T = (int)m; rb.k = 1;
     rb.tile_slots = tiled32 ? 64 : tile_slots;
     if (!tiled) rb.tile_tab = nullptr;

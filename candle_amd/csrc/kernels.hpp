@@ -45,6 +45,28 @@ constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a 
 constexpr int GEMM_MIN_TILE_SLOTS = 64;  // smallest tile of the tiled expert kernels
 inline int64_t max_gemm_tiles(int64_t slots, int64_t groups, int tile_slots = GEMM_MIN_TILE_SLOTS) { return slots / tile_slots + groups + 1; }
 
+// Tiled kernels: workgroup id -> (row block, slot tile).  Hardware hands consecutive workgroup ids to the eight XCDs in
+// turn, each with its own L2; the ids that land on one XCD are walked in patches of edge x edge (row blocks x tiles), so
+// that the workgroups an XCD runs at a time share their weight rows and their activation tiles through that L2.  The
+// edge is 8 when that still gives every XCD at least two patches, else 4 or 2: a grid of a few hundred workgroups cut
+// into 8 x 8 patches would leave XCDs without work.
+struct PatchPos { int rblk, tile; };
+__host__ __device__ inline PatchPos patch_position(int block, int n_rb, int edge) {
+    const int per = edge * edge, RG = (n_rb + edge - 1) / edge;
+    const int xcd = block & 7, q = block >> 3;
+    const int st = (q / per) * 8 + xcd, within = q % per;
+    return PatchPos{(st % RG) * edge + within % edge, (st / RG) * edge + within / edge};
+}
+inline int patch_edge(int64_t n_rb, int64_t tiles) {
+    for (int e = 8; e > 2; e >>= 1)
+        if (((n_rb + e - 1) / e) * ((tiles + e - 1) / e) >= 16) return e;
+    return 2;
+}
+inline unsigned patch_grid(int64_t n_rb, int64_t tiles, int edge) {
+    const int64_t RG = (n_rb + edge - 1) / edge, TG = (tiles + edge - 1) / edge;
+    return (unsigned)((RG * TG + 7) / 8 * 8 * edge * edge);
+}
+
 struct FrontParams {
     const float* x = nullptr;       // [T, H]
     int64_t T = 0;
@@ -91,6 +113,7 @@ struct ExpertParams {
     int64_t max_rows = 0;           // upper bound of rows in any group of this launch
     int slot_tiles = 1;             // 16-slot tiles a workgroup carries per pass over the weights (1, 2 or, Q4K only, 4)
     int is_shared = 0;              // this launch is the always-on shared expert (one group, all tokens)
+    int patch = 8;                  // tiled kernels: edge of the (row block x tile) patches dealt to the XCDs (set by the launchers)
     // Narrow launches of tiny batches (direct slot numbering, T*k <= E): the grid's y dimension counts assignments
     // instead of experts, workgroup row y serves the expert of assignment y unless an earlier assignment names the
     // same expert.  No workgroups (and no weight prefetches) for experts without tokens.

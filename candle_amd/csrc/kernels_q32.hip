@@ -732,13 +732,10 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     __shared__ float hx[MODE == 0 ? QG_NOP * 16 : 1][MODE == 0 ? 65 : 1];   // MODE 0: h of the tile's slots x the workgroup's 64 rows
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // workgroup -> (row block, slot tile): 8 x 8 patches per XCD, as in q4k_gemm_kernel
+    // workgroup -> (row block, slot tile), in patches per XCD (patch_position)
     const int n_rb = MODE == 0 ? p.F / 64 : p.H / 128;
-    const int RG = (n_rb + 7) / 8;
-    const int xcd = blockIdx.x & 7, qq = blockIdx.x >> 3;
-    const int st = (qq >> 6) * 8 + xcd, within = qq & 63;
-    const int rblk = (st % RG) * 8 + (within & 7);
-    const int tile = (st / RG) * 8 + (within >> 3);
+    const PatchPos pp = patch_position((int)blockIdx.x, n_rb, p.patch);
+    const int rblk = pp.rblk, tile = pp.tile;
     if (rblk >= n_rb) return;
     int gi, pos0;
     if (p.is_shared) {   // one group holding every token: its tiles need no list
@@ -911,10 +908,6 @@ static bool qg_format(int dt) { return dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_
 bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F) {
     return qg_format(dt) && (dt_down == 0 || qg_format(dt_down)) && H % 128 == 0 && F % 128 == 0;
 }
-static unsigned qg_grid(int n_rb, int64_t tiles) {
-    const int64_t RG = (n_rb + 7) / 8, TG = (tiles + 7) / 8;
-    return (unsigned)((RG * TG + 7) / 8 * 8 * 64);
-}
 static int64_t qg_tiles(const ExpertParams& p) {
     return p.is_shared ? (p.max_rows + QG_NOP * 16 - 1) / (QG_NOP * 16) : max_gemm_tiles(p.n_slots, p.n_groups + 1, QG_NOP * 16);
 }
@@ -928,13 +921,17 @@ static hipError_t qg_launch(int dt, const ExpertParams& p, dim3 grid, hipStream_
     }
     return hipGetLastError();
 }
-hipError_t launch_q8_0_gemm_up(const ExpertParams& p, hipStream_t s) {
-    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    return qg_launch<0>(p.dt, p, dim3(qg_grid(p.F / 64, qg_tiles(p))), s);
+hipError_t launch_q8_0_gemm_up(const ExpertParams& p_in, hipStream_t s) {
+    if (p_in.max_rows == 0 || p_in.n_groups == 0) return hipSuccess;
+    ExpertParams p = p_in;
+    p.patch = patch_edge(p.F / 64, qg_tiles(p));
+    return qg_launch<0>(p.dt, p, dim3(patch_grid(p.F / 64, qg_tiles(p), p.patch)), s);
 }
-hipError_t launch_q8_0_gemm_down(const ExpertParams& p, hipStream_t s) {
-    if (p.max_rows == 0 || p.n_groups == 0) return hipSuccess;
-    return qg_launch<1>(p.dt_down ? p.dt_down : p.dt, p, dim3(qg_grid(p.H / 128, qg_tiles(p))), s);
+hipError_t launch_q8_0_gemm_down(const ExpertParams& p_in, hipStream_t s) {
+    if (p_in.max_rows == 0 || p_in.n_groups == 0) return hipSuccess;
+    ExpertParams p = p_in;
+    p.patch = patch_edge(p.H / 128, qg_tiles(p));
+    return qg_launch<1>(p.dt_down ? p.dt_down : p.dt, p, dim3(patch_grid(p.H / 128, qg_tiles(p), p.patch)), s);
 }
 
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s);

@@ -318,16 +318,10 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_tiles = p.rb.tile_tab[0];
-    // Workgroup -> (row block, slot tile).  Hardware hands consecutive workgroup ids to the eight XCDs
-    // in turn, each with its own L2; the ids that land on one XCD are therefore walked in 8 x 8
-    // super-tiles (8 row blocks x 8 slot tiles), so that the ~64 workgroups an XCD runs at a time share
-    // their weight rows and their activation tiles through that L2.
+    // workgroup -> (row block, slot tile), in patches per XCD (patch_position)
     const int n_rb = MODE == 0 ? p.F / 64 : p.H / 128;
-    const int RG = (n_rb + 7) / 8;
-    const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-    const int st = (q >> 6) * 8 + xcd, within = q & 63;
-    const int rblk = (st % RG) * 8 + (within & 7);
-    const int tile = (st / RG) * 8 + (within >> 3);
+    const PatchPos pos = patch_position((int)blockIdx.x, n_rb, p.patch);
+    const int rblk = pos.rblk, tile = pos.tile;
     if (tile >= n_tiles || rblk >= n_rb) return;
     const int gi = p.rb.tile_tab[1 + 2 * tile], pos0 = p.rb.tile_tab[2 + 2 * tile];
     if (gi < p.group0 || gi >= p.group0 + p.n_groups) return;
@@ -445,11 +439,6 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     }
 }
 
-static unsigned gemm_grid(int n_rb, int64_t max_tiles) {
-    // patches of 8 row blocks x 8 tiles, dealt round-robin to the eight XCDs: a whole number of rounds
-    const int64_t RG = (n_rb + 7) / 8, TG = (max_tiles + 7) / 8;
-    return (unsigned)((RG * TG + 7) / 8 * 8 * 64);
-}
 template <int FMT, int MODE>
 static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
     if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 4>), grid, dim3(G_THREADS), 0, s, p);
@@ -457,16 +446,22 @@ static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
 }
 bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
 bool q4k_gemm_down_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
-hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s) {
-    dim3 grid(gemm_grid(p.F / 64, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
+hipError_t launch_q4k_gemm_up(const ExpertParams& p_in, hipStream_t s) {
+    ExpertParams p = p_in;
+    const int64_t tiles = max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots);
+    p.patch = patch_edge(p.F / 64, tiles);
+    dim3 grid(patch_grid(p.F / 64, tiles, p.patch));
     if (p.dt == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 0>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
-hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s) {
-    dim3 grid(gemm_grid(p.H / 128, max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots)));
+hipError_t launch_q4k_gemm_down(const ExpertParams& p_in, hipStream_t s) {
+    ExpertParams p = p_in;
+    const int64_t tiles = max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots);
+    p.patch = patch_edge(p.H / 128, tiles);
+    dim3 grid(patch_grid(p.H / 128, tiles, p.patch));
     const int dtd = p.dt_down ? p.dt_down : p.dt;
     if (dtd == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 1>(p, grid, s);
     else if (dtd == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 1>(p, grid, s);

@@ -133,7 +133,7 @@ def test_route_zipf_bias_lists():
                                        (O.Q5K, 64, 512, 5), (O.Q5K, 1040, 1024, 33), (O.Q5K, 256, 2304, 150),
                                        (O.Q6K, 64, 512, 5), (O.Q6K, 1040, 1024, 33), (O.Q6K, 256, 2304, 150),
                                        (O.Q4K, 4096, 1024, 700), (O.Q5K, 4096, 1024, 700), (O.Q6K, 4096, 1024, 700),
-                                       (O.Q8_0, 4096, 1024, 1100), (O.Q8_0, 2048, 1408, 2100), (O.Q4_0, 4096, 1024, 1100), (O.Q5_0, 2048, 1408, 2100),
+                                       (O.Q8_0, 4096, 1024, 1100), (O.Q8_0, 2048, 1408, 1100), (O.Q4_0, 4096, 1024, 600), (O.Q5_0, 2048, 1408, 2100),
                                        (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70),
                                        (O.Q5_0, 48, 96, 3), (O.Q5_0, 256, 1408, 40), (O.Q5_0, 128, 1024, 70),
                                        (O.Q4_1, 48, 96, 3), (O.Q4_1, 256, 1408, 40), (O.Q4_1, 128, 1024, 70),
@@ -353,6 +353,10 @@ def test_block_32_element_formats_tiled_kernels(dt, dt_down):
     gpu.close()
     ref, gpu = make_pair(128, 256, 6, 3, dt, seed=51, dt_down=dt_down, Fs=384)
     check_block(ref, gpu, 700, tol=TOL)
+    gpu.close()
+    # a shared expert wide enough for the tiled kernels itself (its tiles follow from the token count, no list)
+    ref, gpu = make_pair(128, 256, 6, 3, dt, seed=52, dt_down=dt_down, Fs=1024)
+    check_block(ref, gpu, 2100, tol=TOL)
     gpu.close()
 
 
