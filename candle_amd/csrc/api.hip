@@ -450,17 +450,19 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     const Switches& sw = switches();
     ForwardPlan pl;
     const bool shared = L->Fs > 0;
-    // Q4K / Q5K batches with more than ~40 rows per expert take the tiled MFMA kernel for the up projection (F a
+    // K-quant batches with more than 34 rows per expert take the tiled MFMA kernel for the up projection (F a
     // multiple of 64, H of 128; those kernels address activation rows with 32-bit byte offsets), from ~64 rows per
-    // expert on for the down projection too (measured at the Mixtral shape: 48 rows per expert, up 198 us tiled
+    // expert on for the down projection too (measured at the Mixtral shape: 36 rows per expert, 316 against 326 us per
+    // step, 32 rows 310 against 296; 48 rows per expert, up 198 us tiled
     // against 230 us streamed with four slot tiles, down 170 against 120 us; 64 rows: down 177 against 170).
-    // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~96 rows per expert.
+    // Their tiles hold 64 slots while the lists are short (less padding), 128 beyond ~72 rows per expert (Mixtral shape:
+    // 64 rows per expert 449 against 485 us per step, 80 rows 531 against 498).
     // (w2 may be Q4K, Q5K or Q6K whatever w1 / w3 are: mixed files store part of it as Q6K)
-    pl.tiled = !sw.no_gemm && q4k_gemm_up_format(L->dt) && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 38 * L->E;
+    pl.tiled = !sw.no_gemm && q4k_gemm_up_format(L->dt) && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 34 * L->E;
     pl.tiled_down = pl.tiled && q4k_gemm_down_format(L->dt_down) && T * L->k > 64 * L->E;
     // small batches: slots are numbered t*k + r and no dispatch pass runs
     pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
-    pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 96 * L->E ? 128 : 64;
+    pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 72 * L->E ? 128 : 64;
     // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
     // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
     // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches

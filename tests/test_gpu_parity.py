@@ -257,12 +257,12 @@ def test_block_q4k_shared_expert_slot_tiles(T):
 
 
 def test_block_q4k_tile_sizes_and_paths():
-    # two slot tiles per streamed pass with a second pass for lists beyond 32 rows (T = 104, 130); four slot tiles from
-    # 35 rows per expert (T = 140, 150); from 39 rows the tiled kernel for the up projection with the down projection
-    # still streamed (T = 160, 200, 250), from 65 rows for both: 64-slot tiles (T = 300) up to ~96 rows per expert,
-    # 128 beyond (T = 400, 600)
+    # two slot tiles per streamed pass with a second pass for lists beyond 32 rows (T = 104, 130); from 35 rows per
+    # expert the tiled kernel for the up projection with the down projection still streamed, four slot tiles per pass
+    # (T = 140, 150, 160, 200, 250), from 65 rows for both: 64-slot tiles (T = 270) up to ~72 rows per expert,
+    # 128 beyond (T = 300, 400, 600)
     ref, gpu = make_pair(512, 1024, 8, 2, O.Q4K, seed=1)
-    for T in (104, 130, 140, 150, 160, 200, 250, 300, 400, 600):
+    for T in (104, 130, 140, 150, 160, 200, 250, 270, 300, 400, 600):
         check_block(ref, gpu, T)
     gpu.close()
 
