@@ -206,6 +206,32 @@ def test_cfg3_prefill_q4k_up_q6k_down(mixtral_layer, request):
     gpu.close()
 
 
+def test_cfg3_prefill_q5k_experts(request):
+    """Q5_K experts (what Q5_K_M files hold) at the Mixtral shape, 2048 tokens with the Zipf load: the tiled kernels in
+    their Q5K variant for both projections.  Same bars as the Q4K prefill."""
+    T = 2048
+    ref, gpu = build(4096, 14336, 8, 2, O.Q5K, seed=3, bias=ZIPF_BIAS)
+    xs = acts(T, 4096, 23)
+    ys = gpu.forward(xs)
+    logits = gpu.last_logits(T)
+    gi, gw, goff, gperm, gpw = gpu.last_routing(T)
+    ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), 2)
+    assert np.array_equal(gi, ri) and np.array_equal(bits(gw), bits(rw))
+    assert np.array_equal(goff, roff) and np.array_equal(gperm, rperm) and np.array_equal(bits(gpw), bits(rpw))
+    want = ref.forward(xs, logits=logits, simd=True, threads=CORES)
+    r = rms(want)
+    e_max, e_share, e_rms = tail_stats(ys, want, r)
+    say(request.config, " [Q5K vs AVX2: max %.2e, share > 2e-3 %.1e, rms %.1e]" % (e_max, e_share, e_rms))
+    assert e_rms <= 2e-4 and e_share <= 5e-5 and e_max <= 3 * TOL, (e_max, e_share, e_rms)
+    n = 512
+    want_s = ref.forward(xs[:n], logits=logits[:n], simd=False, threads=CORES)
+    g_max, g_share, _ = tail_stats(ys[:n], want[:n], r)
+    s_max, s_share, _ = tail_stats(want_s, want[:n], r)
+    say(request.config, " [first %d tokens: HIP vs AVX2 max %.2e share %.1e; scalar vs AVX2 max %.2e share %.1e]" % (n, g_max, g_share, s_max, s_share))
+    assert g_max <= max(2 * TOL, 1.5 * s_max) and g_share <= 1.5 * s_share + 2e-5, (g_max, g_share, s_max, s_share)
+    gpu.close()
+
+
 def test_cfg4_fine_grained_q8_0_shared_expert():
     ref, gpu = build(2048, 1408, 60, 4, O.Q8_0, seed=4, Fs=5632)
     check(ref, gpu, acts(512, 2048, 12))
