@@ -813,6 +813,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
                 for (int i = 0; i < 4; i++) ydv[i] = *reinterpret_cast<const f32x4g*>(&L.yd[buf][o * 16 + 4 * g + i][0]);
                 v4i D[4];
+                __builtin_amdgcn_s_setprio(2);   // issue priority while the matrix instructions go out (as in q4k_gemm_kernel)
 #pragma unroll
                 for (int b = 0; b < 4; b++) {
                     const uint8_t* ap = &L.q[buf][o][2 * b][0] + m * 16 + 4 * g;
@@ -826,6 +827,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                     }
                     D[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, addend, 0, 0, 0);
                 }
+                __builtin_amdgcn_s_setprio(0);
                 // ascending block order per (row, slot), every product rounded where the reference rounds it
 #pragma unroll
                 for (int b = 0; b < 4; b++)

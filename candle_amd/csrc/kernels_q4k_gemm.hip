@@ -268,12 +268,16 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
     const v4i zero4 = {0, 0, 0, 0};
     v4i acc_lo, acc_hi;
     const uint8_t* arow = L.q[buf] + o * 4096 + lane * 16;
+    // the wave takes issue priority while its matrix instructions go out: they keep the matrix pipe fed while the other
+    // waves of the SIMD work through their result steps (2 % on the kernel)
+    __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int P = 0; P < 4; P++) {
         const v4i a = *reinterpret_cast<const v4i*>(arow + P * 1024);
         acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.lo[P], P == 0 ? zero4 : acc_lo, 0, 0, 0);
         acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.hi[P], P == 0 ? zero4 : acc_hi, 0, 0, 0);
     }
+    __builtin_amdgcn_s_setprio(0);
     // D[i] belongs to slot 16 o + 4 g + i, weight row n = lane%16
     if constexpr (FMT == MOE_GGML_Q6K) {
         const v4f yd = *reinterpret_cast<const v4f*>(&L.yd[buf][o * 16 + g * 4]);
