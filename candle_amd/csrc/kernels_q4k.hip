@@ -217,6 +217,7 @@ __device__ inline void q4k_mac_planes(const Q4KPlanes& pl, const Q8KOperand& A, 
         acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.hi[P], acc_hi, 0, 0, 0);
         acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, pl.lo[P], acc_lo, 0, 0, 0);
     }
+
     const v4f zf = {0.f, 0.f, 0.f, 0.f};
     v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, pl.mB, zf, 0, 0, 0);
 #pragma unroll
@@ -529,7 +530,11 @@ __device__ inline void q4k_engine(const uint8_t* const tp[NT], size_t sb_stride,
                 const int jn = ahead % NT;
                 int sbn = sb0 + ahead / NT;
                 sbn = sbn < sb_hi ? sbn : sb_hi - 1;
+                // (issue priority for the refill: the sooner the request leaves, the longer the memory system has for it;
+                // 1 % at batch 64, 0.3 % at batch 32)
+                __builtin_amdgcn_s_setprio(3);
                 t[idx % RING] = FMT::load(tp[jn] + (size_t)sbn * sb_stride, lane);
+                __builtin_amdgcn_s_setprio(0);
                 __builtin_amdgcn_sched_barrier(0);
                 const auto prep = FMT::prepare(w, g);   // what of the tile's unpacking serves every slot tile
 #pragma unroll
