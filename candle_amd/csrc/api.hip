@@ -255,6 +255,7 @@ Switches& switches() {
         g_sw.tile_slots = (int)num("MOE_TILE_SLOTS", 0);
         g_sw.slot_tiles = (int)num("MOE_SLOT_TILES", 0);
         g_sw.narrow = (int)num("MOE_NARROW", -1);
+        g_sw.fused_rows = (int)num("MOE_FUSED_ROWS", 0);
     });
     return g_sw;
 }
@@ -985,6 +986,17 @@ static size_t carve_qlinear(const moe_qlinear* Q, int64_t m, uint8_t* base, Rout
 
 // quantise the rows, then one pass over the matrix: streamed for short batches, tiled MFMA beyond
 static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d_y, hipStream_t s) {
+    // One or two rows of a K-quant matrix (single-stream decoding): one launch that quantises the rows itself; no workspace,
+    // nothing shared between calls.  Every workgroup repeats the quantisation, which costs a wave ~0.5 us per block and
+    // row, so the two passes win from three rows on and for the widest matrices (measured inside a HIP graph, Q4_K,
+    // fused / two passes: 4096 x 4096: 5.8 / 12.6 us at one row, 7.8 / 13.0 at two, 11.6 / 13.4 at four -- the graph's two
+    // passes carry a table kernel that eager calls skip, ~2.5 us; 4096 x 14336: 16.9 / 28.0 at one row; 16384 x 4096:
+    // 10.7 / 14.5; 32000 x 4096: 21.2 / 19.5).  fused_rows: 1 = never, 2 = whenever the kernel can (test aid).
+    const int fr = switches().fused_rows;
+    if (fr != 1 && qlinear_fused_usable(Q->dt, m, Q->n, Q->k) && (fr == 2 || (m <= 2 && Q->n <= 16384))) {
+        MOE_HIP_CHECK(launch_qlinear_fused(Q->dt, d_x, m, Q->n, Q->k, Q->weights.as<uint8_t>(), d_y, s));
+        return MOE_OK;
+    }
     // under stream capture nothing may be allocated, the graph carries its own copy of the routing table pass, and the
     // workspace is never freed afterwards (a replay uses its addresses)
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -1190,6 +1202,7 @@ extern "C" int moe_debug_set_switch(const char* name, int64_t value) {
     else if (n == "tile_slots") sw.tile_slots = (int)value;
     else if (n == "slot_tiles") sw.slot_tiles = (int)value;
     else if (n == "narrow") sw.narrow = (int)value;
+    else if (n == "fused_rows") sw.fused_rows = (int)value;
     else return fail(MOE_E_INVALID, "moe_debug_set_switch: unknown switch '" + n + "'");
     return MOE_OK;
 }

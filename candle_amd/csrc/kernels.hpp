@@ -15,6 +15,7 @@ struct Switches {
     int tile_slots = 0;               // MOE_TILE_SLOTS: 64 | 128 (0 = by batch size)
     int slot_tiles = 0;               // MOE_SLOT_TILES: 16-slot tiles per streaming pass (0 = by batch size)
     int narrow = -1;                  // MOE_NARROW: 0 | 1 (-1 = by batch size)
+    int fused_rows = 0;               // MOE_FUSED_ROWS: dense products of a few rows in one launch: 1 = never, 2 = whenever possible (0 = by size)
 };
 Switches& switches();
 
@@ -132,6 +133,9 @@ hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
 // caller re-quantises it), down writes yw.
 bool q4k_gemm_up_format(int dt);
 bool q4k_gemm_down_format(int dt);
+// Dense K-quant matrix [n, k] (device layout) times m <= 4 rows of f32 in one launch (the rows are quantised in the kernel).
+bool qlinear_fused_usable(int dt, int64_t m, int64_t n, int64_t k);
+hipError_t launch_qlinear_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s);
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 

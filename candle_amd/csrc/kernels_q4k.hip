@@ -54,6 +54,13 @@ __device__ inline uint4 gload<uint4>(const void* uniform_base, uint32_t off) {
     return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+template <>
+__device__ inline float4 gload<float4>(const void* uniform_base, uint32_t off) {
+    f32x4 v = *reinterpret_cast<const __attribute__((address_space(1))) f32x4*>((gbytes)uniform_base + off);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 // weight tiles are read once per launch: non-temporal loads keep them from displacing the activations
 // and routing lists in the caches
 __device__ inline uint4 gload_stream(const void* uniform_base, uint32_t off) {
@@ -800,6 +807,172 @@ DEF_UP(q6k_up_t2, FmtQ6K, 2, 4, 2, 2)
 DEF_DOWN(q6k_down_t1, FmtQ6K, 1, 4, 2, 2)
 DEF_DOWN_NARROW(q6k_down_t1_narrow, FmtQ6K, 8, 2, 2)
 DEF_DOWN(q6k_down_t2, FmtQ6K, 2, 4, 2, 2)
+
+// ---------------------------------------------------------------------------------------------
+// Dense matrix times a few rows (single-stream decoding: attention projections, output head) in one launch: the rows
+// are quantised to Q8K inside the kernel.  A wave multiplies super-blocks w, w + 4, ... of its workgroup's row tiles, as
+// the streaming down kernel's waves do; just before each of them it quantises that block of every row (the wave-level
+// BlockQ8K::from_float of act_quant.hpp, 64 lanes x 4 elements) into a few hundred bytes of LDS of its own and reads
+// its MFMA operand back from there.  Every workgroup repeats the quantisation of the rows -- ~80 instructions per block
+// and row -- which is why this pays for a handful of rows only: against it stand a kernel launch and a round trip of the
+// quantised rows through memory.  Same blocks, same products, partial sums added in the same order as quantize_rows_kernel
+// followed by the streaming down kernel: the results carry the same bits.
+constexpr int FUSED_MAX_ROWS = 4;
+constexpr int XQ_BSUM = 256, XQ_D = 288, XQ_BYTES = 320;   // one quantised block in LDS: 256 quants, 16 f16 sums, f32 scale
+constexpr int FUSED_NW = 4;
+constexpr size_t FUSED_MAX_LDS = 44 * 1024;   // beside the 16 KiB at most of partial sums: below the 64 KiB a workgroup gets without asking
+// LDS for the quantised rows: every wave keeps its own super-blocks of every row
+__host__ __device__ inline int fused_blocks_per_wave(int K) { return (K / 256 + FUSED_NW - 1) / FUSED_NW; }
+static size_t fused_lds_bytes(int64_t m, int64_t K) { return (size_t)FUSED_NW * (size_t)fused_blocks_per_wave((int)K) * (size_t)m * XQ_BYTES; }
+
+template <class FMT, int NTD>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qlinear_fused_kernel(const float* x, int m, int n, int K,
+                                                                                                         const uint8_t* w, float* y) {
+    constexpr int NW = FUSED_NW;
+    constexpr int RING = 4, U = RING / NTD;   // tiles in flight per wave; super-blocks per trip of the loop
+    static_assert(RING % NTD == 0, "the ring holds whole super-blocks");
+    __shared__ float part[NW][NTD * 4][64];
+    extern __shared__ __align__(16) uint8_t xq_all[];   // [wave][block of the wave][row][XQ_BYTES]
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nsb = K / 256, n_rt = n / 16;
+    const int rt0 = blockIdx.x * NTD;
+    const int mine = wave < nsb ? (nsb - wave + NW - 1) / NW : 0;   // super-blocks wave, wave + NW, ...
+    const size_t sb_stride = (size_t)n_rt * FMT::TILE_BYTES * NW;
+    const uint8_t* tp[NTD];
+#pragma unroll
+    for (int j = 0; j < NTD; j++) {
+        const int rt = rt0 + j < n_rt ? rt0 + j : n_rt - 1;   // tiles past the last row are computed and dropped
+        tp[j] = w + (size_t)rt * FMT::TILE_BYTES + (size_t)(mine ? wave : 0) * (size_t)n_rt * FMT::TILE_BYTES;
+    }
+    float acc[NTD][4];
+#pragma unroll
+    for (int j = 0; j < NTD; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[j][i] = 0.f;
+    if (mine > 0) {
+        // the first weight tiles are requested before anything else: the rows are quantised while they travel
+        typename FMT::Tile ring[RING];
+#pragma unroll
+        for (int q = 0; q < RING; q++) {
+            const int it = q / NTD < mine ? q / NTD : mine - 1;
+            ring[q] = FMT::load(tp[q % NTD] + (size_t)it * sb_stride, lane);
+        }
+        uint8_t* xq = xq_all + (size_t)wave * fused_blocks_per_wave(K) * m * XQ_BYTES;
+        {
+            // the wave's blocks of all rows, numbered b = it * m + row, four at a time side by side (their loads, wave
+            // reductions and divisions overlap); 32-bit byte offsets: m * K * 4 < 2^31
+            constexpr int NQ = 4;
+            const int n_blk = mine * m;
+            auto x_offset = [&](int b) {
+                const int bb = b < n_blk ? b : n_blk - 1;
+                const int it = bb / m, row = bb - it * m;
+                return ((uint32_t)row * (uint32_t)K + (uint32_t)((wave + it * NW) * 256 + lane * 4)) * 4u;
+            };
+            float4 v[NQ];
+#pragma unroll
+            for (int i = 0; i < NQ; i++) v[i] = gload<float4>(x, x_offset(i));
+            for (int b0 = 0; b0 < n_blk; b0 += NQ) {
+                bool valid[NQ];
+                int8_t* qs_out[NQ];
+                float* d_out[NQ];
+                __half* bs_out[NQ];
+                float4 cur[NQ];
+#pragma unroll
+                for (int i = 0; i < NQ; i++) {
+                    valid[i] = b0 + i < n_blk;
+                    uint8_t* blk = xq + (size_t)(valid[i] ? b0 + i : 0) * XQ_BYTES;
+                    qs_out[i] = reinterpret_cast<int8_t*>(blk);
+                    bs_out[i] = reinterpret_cast<__half*>(blk + XQ_BSUM);
+                    d_out[i] = reinterpret_cast<float*>(blk + XQ_D);
+                    cur[i] = v[i];
+                }
+#pragma unroll
+                for (int i = 0; i < NQ; i++) v[i] = gload<float4>(x, x_offset(b0 + NQ + i));
+                quantize_q8k_blocks<NQ>(cur, valid, lane, qs_out, d_out, bs_out);
+            }
+        }
+        // the wave reads what its other lanes have written: LDS serves a wave's requests in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int my_row = r < m ? r : m - 1;
+        for (int it0 = 0; it0 < mine; it0 += U) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int it = it0 + u;
+                if (it < mine) {   // uniform
+                    const uint8_t* blk = xq + (size_t)it * m * XQ_BYTES;
+                    Q8KOperand A;
+#pragma unroll
+                    for (int P = 0; P < 4; P++) A.a[P] = *reinterpret_cast<const uint4*>(blk + my_row * XQ_BYTES + P * 64 + g * 16);
+                    A.bs = *reinterpret_cast<const v4h*>(blk + my_row * XQ_BYTES + XQ_BSUM + g * 8);
+                    float yd[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int row = 4 * g + i;
+                        yd[i] = *reinterpret_cast<const float*>(blk + (row < m ? row : m - 1) * XQ_BYTES + XQ_D);
+                    }
+                    A.yd = yd[0];
+                    __builtin_amdgcn_sched_barrier(0);   // (the fences bound the live ranges: one tile's arithmetic at a time)
+#pragma unroll
+                    for (int j = 0; j < NTD; j++) {
+                        const int q = u * NTD + j;
+                        const typename FMT::Tile wt = ring[q];
+                        int ita = it0 + U + u;               // the super-block that takes this ring place
+                        ita = ita < mine ? ita : mine - 1;
+                        ring[q] = FMT::load(tp[j] + (size_t)ita * sb_stride, lane);
+                        __builtin_amdgcn_sched_barrier(0);
+                        const auto prep = FMT::prepare(wt, g);
+                        FMT::mac(prep, A, yd, g, acc[j]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NTD; j++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) part[wave][j * 4 + i][lane] = acc[j][i];
+    __syncthreads();
+    for (int v2 = wave; v2 < NTD * 4; v2 += NW) {
+        float sum = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < NW; ww++) sum += part[ww][v2][lane];
+        const int j = v2 / 4, i = v2 % 4;
+        const int row = 4 * g + i;
+        if (row < m && rt0 + j < n_rt) y[(size_t)row * n + (size_t)(rt0 + j) * 16 + r] = sum;
+    }
+}
+
+bool qlinear_fused_usable(int dt, int64_t m, int64_t n, int64_t k) {
+    return vecdot_dtype(dt) == MOE_GGML_Q8K && m >= 1 && m <= FUSED_MAX_ROWS && n % 16 == 0 && k % 256 == 0 && k >= 256 &&
+           m * k < ((int64_t)1 << 29) && fused_lds_bytes(m, k) <= FUSED_MAX_LDS;
+}
+
+template <class FMT>
+static void launch_fused_fmt(const float* x, int m, int n, int k, const uint8_t* w, float* y, hipStream_t s) {
+    // enough workgroups for two per CU where the matrix has the rows for it
+    const int n_rt = n / 16;
+    const size_t lds = fused_lds_bytes(m, k);
+    if (n_rt >= 2048) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 4>), dim3((unsigned)((n_rt + 3) / 4)), dim3(256), lds, s, x, m, n, k, w, y);
+    else if (n_rt >= 1024) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 2>), dim3((unsigned)((n_rt + 1) / 2)), dim3(256), lds, s, x, m, n, k, w, y);
+    else hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 1>), dim3((unsigned)n_rt), dim3(256), lds, s, x, m, n, k, w, y);
+}
+
+hipError_t launch_qlinear_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s) {
+    if (!qlinear_fused_usable(dt, m, n, k)) return hipErrorInvalidValue;
+    switch (dt) {
+        case MOE_GGML_Q2K: launch_fused_fmt<FmtQ2K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        case MOE_GGML_Q3K: launch_fused_fmt<FmtQ3K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        case MOE_GGML_Q4K: launch_fused_fmt<FmtQ4K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        case MOE_GGML_Q5K: launch_fused_fmt<FmtQ5K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        case MOE_GGML_Q6K: launch_fused_fmt<FmtQ6K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
 
 // ---------------------------------------------------------------------------------------------
 static int variant(const char* name, int dflt) {

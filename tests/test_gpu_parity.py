@@ -160,6 +160,36 @@ def test_q4_0_matmul_known_answers(golden):
     assert np.round(got).reshape(-1).tolist() == golden["q4_0_matmul_3_64_4"]["expected_rounded"]
 
 
+@pytest.mark.parametrize("dt", [O.Q2K, O.Q3K, O.Q4K, O.Q5K, O.Q6K])
+def test_few_rows_quantised_inside_the_kernel_equal_the_two_pass_path(dt):
+    # up to four rows of a K-quant matrix can take one launch that quantises the rows itself (one or two do by default): same blocks, same products, same
+    # order of the partial sums as the row quantiser followed by the streaming kernel -- the same bits -- and the oracle's
+    # values.  Shapes: K of 1, 5 and 16 super-blocks (waves with no, one and several blocks), row counts that are not
+    # multiples of the workgroups' 32 and 64 rows; rows with an all-zero block and with ties for the largest magnitude.
+    for n, k in ((48, 256), (1040, 1280), (16416, 512), (32784, 256), (4096, 4096)):
+        w = O.fill_normal_quantized(n + k + dt, dt, n, k, 0.02)
+        q = candle_amd.QMatMul(dt, w, n, k)
+        try:
+            for m in (1, 2, 3, 4):
+                x = activations(m, k, seed=100 + m)
+                x[0, :256] = 0.0
+                if k > 256:
+                    x[m - 1, 256:512] = np.where(np.arange(256) % 2 == 0, 1.5, -1.5)   # +-max: the first one sets the sign
+                try:
+                    candle_amd.set_switch("fused_rows", 2)   # whenever the kernel can: by default three rows take two passes
+                    fused = q.forward(x)
+                    candle_amd.set_switch("fused_rows", 1)   # never
+                    two_pass = q.forward(x)
+                finally:
+                    candle_amd.set_switch("fused_rows", 0)
+                assert np.array_equal(bits(fused), bits(two_pass)), (dt, n, k, m)
+                if n * k <= 1040 * 1280:
+                    want = O.matmul(dt, x, w, n)
+                    assert np.abs(fused - want).max() <= 1e-5 * rms(want) * 10, (dt, n, k, m)
+        finally:
+            q.close()
+
+
 def test_batch_invariance():
     # qmm_batch, candle-core/tests/quantized_tests.rs:221-256
     n, k = 256, 512
