@@ -27,6 +27,23 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, n) is not None, n
 
 
+def test_header_is_plain_c(tmp_path):
+    # the boundary is a C ABI: the header has to compile as C99 (no C++ in the signatures), and a C caller has to link
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no gcc")
+    src = tmp_path / "caller.c"
+    src.write_text('#include "candle_amd_moe.h"\n'
+                   'int main(void) { moe_desc d; (void)d; return moe_static_scratch_bytes() > 0 && moe_last_error() ? 0 : 1; }\n')
+    lib = candle_amd.lib_path()
+    exe = tmp_path / "caller"
+    subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                    "-L", os.path.dirname(lib), "-lcandle_amd_moe", "-Wl,-rpath," + os.path.dirname(lib)], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
+
+
 def test_debug_expf_equals_platform_expf():
     libm = ctypes.CDLL("libm.so.6")
     libm.expf.restype = ctypes.c_float
