@@ -765,6 +765,16 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
         q4k_down_body<FMT, TT, NW, RING>(p, part, list_lds, wtot_lds);                                      \
     }
 
+// Down-projection workgroups of one row tile (16 rows) instead of four: dense matrices of a few thousand rows, whose
+// 64-row workgroups would leave most CUs without work.
+#define DEF_DOWN_FINE(NAME, FMT, TT, NW, RING, WPE)                                                         \
+    __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) void NAME(ExpertParams p) { \
+        __shared__ float part[NW][1 * TT * 4][64];                                                          \
+        __shared__ int list_lds[DIRECT_MAX_SLOTS];                                                          \
+        __shared__ int wtot_lds[NW];                                                                        \
+        q4k_down_body<FMT, TT, NW, RING, 1>(p, part, list_lds, wtot_lds);                                   \
+    }
+
 // One 16-slot tile per pass (small batches): variant 1 (default) 4 waves, 168 VGPRs, three workgroups
 // per CU; variant 0 8 waves, 128 VGPRs.  Two and four tiles per pass (up to 32 / 64 rows per expert
 // without streaming its weights twice) need the registers of a two-waves-per-SIMD launch.
@@ -807,6 +817,18 @@ DEF_UP(q6k_up_t2, FmtQ6K, 2, 4, 2, 2)
 DEF_DOWN(q6k_down_t1, FmtQ6K, 1, 4, 2, 2)
 DEF_DOWN_NARROW(q6k_down_t1_narrow, FmtQ6K, 8, 2, 2)
 DEF_DOWN(q6k_down_t2, FmtQ6K, 2, 4, 2, 2)
+
+DEF_DOWN_FINE(q4k_down_t1_fine, FmtQ4K, 1, 4, 4, 3)
+DEF_DOWN_FINE(q4k_down_t2_fine, FmtQ4KP, 2, 4, 4, 2)
+DEF_DOWN_FINE(q4k_down_t4_fine, FmtQ4KP, 4, 8, 2, 2)
+DEF_DOWN_FINE(q2k_down_t1_fine, FmtQ2K, 1, 4, 4, 3)
+DEF_DOWN_FINE(q2k_down_t2_fine, FmtQ2K, 2, 4, 4, 2)
+DEF_DOWN_FINE(q3k_down_t1_fine, FmtQ3K, 1, 4, 4, 3)
+DEF_DOWN_FINE(q3k_down_t2_fine, FmtQ3K, 2, 4, 4, 2)
+DEF_DOWN_FINE(q5k_down_t1_fine, FmtQ5K, 1, 4, 4, 3)
+DEF_DOWN_FINE(q5k_down_t2_fine, FmtQ5K, 2, 4, 4, 2)
+DEF_DOWN_FINE(q6k_down_t1_fine, FmtQ6K, 1, 4, 4, 2)
+DEF_DOWN_FINE(q6k_down_t2_fine, FmtQ6K, 2, 4, 4, 2)
 
 // ---------------------------------------------------------------------------------------------
 // Dense matrix times a few rows (single-stream decoding: attention projections, output head) in one launch: the rows
@@ -985,15 +1007,21 @@ typedef void (*ExpertKernel)(ExpertParams);
 struct KernelFamily {
     ExpertKernel up_t1, up_narrow, up_t2, up_t4;
     ExpertKernel down_t1, down_narrow, down_t2, down_t4;
+    ExpertKernel down_t1_fine, down_t2_fine, down_t4_fine;
 };
 static const KernelFamily* kernel_family(int dt) {
     static const int uv = variant("MOE_UP_VARIANT", 1), dv = variant("MOE_DOWN_VARIANT", 1);
     static const KernelFamily q4k = {uv == 0 ? q4k_up_t1_v0 : q4k_up_t1_v1, q4k_up_t1_narrow, q4k_up_t2, q4k_up_t4,
-                                     dv == 0 ? q4k_down_t1_v0 : q4k_down_t1_v1, q4k_down_t1_narrow, q4k_down_t2, q4k_down_t4};
-    static const KernelFamily q2k = {q2k_up_t1, q2k_up_t1_narrow, q2k_up_t2, nullptr, q2k_down_t1, q2k_down_t1_narrow, q2k_down_t2, nullptr};
-    static const KernelFamily q3k = {q3k_up_t1, q3k_up_t1_narrow, q3k_up_t2, nullptr, q3k_down_t1, q3k_down_t1_narrow, q3k_down_t2, nullptr};
-    static const KernelFamily q5k = {q5k_up_t1, q5k_up_t1_narrow, q5k_up_t2, nullptr, q5k_down_t1, q5k_down_t1_narrow, q5k_down_t2, nullptr};
-    static const KernelFamily q6k = {q6k_up_t1, q6k_up_t1_narrow, q6k_up_t2, nullptr, q6k_down_t1, q6k_down_t1_narrow, q6k_down_t2, nullptr};
+                                     dv == 0 ? q4k_down_t1_v0 : q4k_down_t1_v1, q4k_down_t1_narrow, q4k_down_t2, q4k_down_t4,
+                                     q4k_down_t1_fine, q4k_down_t2_fine, q4k_down_t4_fine};
+    static const KernelFamily q2k = {q2k_up_t1, q2k_up_t1_narrow, q2k_up_t2, nullptr, q2k_down_t1, q2k_down_t1_narrow, q2k_down_t2, nullptr,
+                                     q2k_down_t1_fine, q2k_down_t2_fine, nullptr};
+    static const KernelFamily q3k = {q3k_up_t1, q3k_up_t1_narrow, q3k_up_t2, nullptr, q3k_down_t1, q3k_down_t1_narrow, q3k_down_t2, nullptr,
+                                     q3k_down_t1_fine, q3k_down_t2_fine, nullptr};
+    static const KernelFamily q5k = {q5k_up_t1, q5k_up_t1_narrow, q5k_up_t2, nullptr, q5k_down_t1, q5k_down_t1_narrow, q5k_down_t2, nullptr,
+                                     q5k_down_t1_fine, q5k_down_t2_fine, nullptr};
+    static const KernelFamily q6k = {q6k_up_t1, q6k_up_t1_narrow, q6k_up_t2, nullptr, q6k_down_t1, q6k_down_t1_narrow, q6k_down_t2, nullptr,
+                                     q6k_down_t1_fine, q6k_down_t2_fine, nullptr};
     switch (dt) {
         case MOE_GGML_Q2K: return &q2k;
         case MOE_GGML_Q3K: return &q3k;
@@ -1037,7 +1065,23 @@ hipError_t launch_q4k_down(const ExpertParams& p_in, hipStream_t s) {
         hipLaunchKernelGGL(f->down_narrow, ngrid, dim3(512), 0, s, p);
         return hipGetLastError();
     }
-    dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)((p.max_rows + tt * 16 - 1) / (tt * 16)));
+    // one group whose 64-row workgroups would not fill the chip (a dense matrix of a few thousand rows): 16-row workgroups
+    const int64_t passes = (p.max_rows + tt * 16 - 1) / (tt * 16);
+    static const int fine_sw = variant("MOE_DOWN_FINE", -1);
+    // (measured in a HIP graph, us per call, 64-row / 16-row workgroups: Q4_K 4096 x 4096: 13.1 / 9.7 at 3 rows, 18.2 / 13.6 at
+    // 32, 24.6 / 19.2 at 64, 25.8 / 27.7 at 90; 8192 x 4096: 13.9 / 11.7 at 3 rows, 18.7 / 20.4 at 32; 4096 x 14336: 41.0 / 31.9
+    // at 32 rows; 32000 x 4096: 20.4 / 29.2 at 3 rows; Q6_K 4096 x 4096: 25.3 / 14.6 at 32 rows, 25.4 / 19.8 at 48 (two passes
+    // of two slot tiles), 8192 x 4096: 25.6 / 22.4 at 32 rows)
+    const int64_t n_rt = p.H / 16;
+    const bool fine = fine_sw >= 0 ? fine_sw > 0 : (p.n_groups == 1 && (n_rt * passes <= (dtd == MOE_GGML_Q6K ? 512 : 256) || (n_rt <= 512 && tt == 1)));
+    if (fine) {
+        dim3 fgrid((unsigned)(p.H / 16), (unsigned)p.n_groups, (unsigned)passes);
+        if (tt == 4) hipLaunchKernelGGL(f->down_t4_fine, fgrid, dim3(512), 0, s, p);
+        else if (tt == 2) hipLaunchKernelGGL(f->down_t2_fine, fgrid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(f->down_t1_fine, fgrid, dim3(256), 0, s, p);
+        return hipGetLastError();
+    }
+    dim3 grid((unsigned)((p.H / 16 + 3) / 4), (unsigned)p.n_groups, (unsigned)passes);
     if (tt == 4) hipLaunchKernelGGL(f->down_t4, grid, dim3(512), 0, s, p);
     else if (tt == 2) hipLaunchKernelGGL(f->down_t2, grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL(f->down_t1, grid, dim3(dtd == MOE_GGML_Q4K && dv == 0 ? 512 : 256), 0, s, p);
