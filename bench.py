@@ -18,7 +18,7 @@ measures the other regimes in the same process and reports them as sub-objects o
                   plus N(0, 0.1) noise; end-to-end tokens/s.
 
 `--workload decode|prefill|config4|stack` measures one of them alone as the line's `value`.
-`--workload prefill [--weights q5_k|q6_k] [--weights-down q5_k|q6_k]` measures the prefill with Q5_K / Q6_K w1 / w3 and / or w2 stored
+`--workload prefill [--weights q2_k|q5_k|q6_k] [--weights-down q5_k|q6_k]` measures the prefill with Q2_K / Q5_K / Q6_K w1 / w3 and / or w2 stored
 in another K-quant (Q4_K_M and Q5_K_M files store part of w2 as Q6_K).
 `--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with another
 GGML format (random block payloads with small finite scales: timing does not depend on the values).
@@ -266,16 +266,18 @@ def measure_prefill(args, np, torch, timer, layer, B):
     up_ops = 2.0 * B * TOPK * 2 * H * F
     achieved = up_ops / (stage["up"] * 1e-3) / 1e12
     step_ops = 2.0 * B * TOPK * 3 * H * F
-    roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, two scale planes)",
+    one_plane = args.weights == "q2_k"   # a 4-bit scale times a 2-bit code fits a byte: one plane, every multiply-add issued once
+    q4k = args.weights == "q4_k"
+    roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, %s)" % ("one plane of scaled codes" if one_plane else "two scale planes"),
                 "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": achieved / INT8_PEAK_TOPS,
                 "traffic": None, "algorithmic_ops_per_launch": up_ops, "launch_us": stage_us["up"],
                 # every algorithmic multiply-add is issued twice (the 6-bit scale is split over two pre-scaled int8
                 # planes so that the integer sums stay exact): share of the peak the MFMA pipe is actually kept busy
                 # with, slot tiles padded to 64 / 128 not counted
-                "mfma_issued_frac": 2.0 * achieved / INT8_PEAK_TOPS,
+                "mfma_issued_frac": (1.0 if one_plane else 2.0) * achieved / INT8_PEAK_TOPS,
                 # share of the cycles the matrix pipe is busy (SQ_VALU_MFMA_BUSY_CYCLES over the kernel's SIMD cycles)
                 # as the committed rocprofv3 counter summary gives it: a figure of that profile, not a reading of this run
-                "mfma_pipe_busy_frac": profiled_value("q4k_gemm_prefill_4096_kernel_trace.md", "mfma_busy_frac", "prefill_up") if B == 4096 else None,
+                "mfma_pipe_busy_frac": profiled_value("q4k_gemm_prefill_4096_kernel_trace.md", "mfma_busy_frac", "prefill_up") if B == 4096 and q4k else None,
                 "mfma_pipe_busy_source": "profiles/q4k_gemm_prefill_4096_kernel_trace.md (rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES, SQ_CYCLES)"}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "tokens": B, "expert_loads": [int(v) for v in loads], "stage_us": stage_us, "step_int8_ops": step_ops,
@@ -407,8 +409,8 @@ def main():
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
     wl = args.workload
-    if args.weights != "q4_k" and wl not in ("decode", "all") and not (wl == "prefill" and args.weights in ("q5_k", "q6_k")):
-        sys.exit("bench.py: --weights applies to the decode workload (and q5_k / q6_k to the prefill workload) only")
+    if args.weights != "q4_k" and wl not in ("decode", "all") and not (wl == "prefill" and args.weights in ("q2_k", "q5_k", "q6_k")):
+        sys.exit("bench.py: --weights applies to the decode workload (and q2_k / q5_k / q6_k to the prefill workload) only")
     if args.weights != "q4_k" and wl != "prefill":
         wl = "decode"
     if args.weights_down and wl != "prefill":

@@ -300,10 +300,8 @@ __device__ inline void q2k_mac(const Q2KTile& w, const Q8KOperand& A, const floa
     const v4f zf = {0.f, 0.f, 0.f, 0.f};
     v4f Dm = __builtin_amdgcn_mfma_f32_16x16x16f16(A.bs, mB, zf, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        acc[i] += (d * yd[i]) * (float)isum[i];
-        acc[i] -= (dmin * yd[i]) * Dm[i];
-    }
+    for (int i = 0; i < 4; i++)   // sumf += dall * isum - dmin * summs, rounded where the reference rounds (k_quants.rs:772-773, 801)
+        acc[i] += (yd[i] * d) * (float)isum[i] - (yd[i] * dmin) * Dm[i];
 }
 
 struct Q6KTile {

@@ -1,4 +1,4 @@
-// Tiled grouped expert products for large batches (prefill): Q4K (also Q5K and Q6K) weights x
+// Tiled grouped expert products for large batches (prefill): Q4K (also Q2K, Q5K and Q6K) weights x
 // Q8K activations on v_mfma_i32_16x16x64_i8, a full-rate int8 MFMA shape of gfx950.
 //
 // Same integers as BlockQ4K::vec_dot (candle-core/src/quantized/k_quants.rs:1205-1285):
@@ -25,6 +25,10 @@
 // products W = sc * (code - 32) (|W| <= 4096) are formed in packed 16-bit arithmetic and cut into two signed bytes,
 // W = 256 * H + L with L in [-128, 127], which are the two planes: 256 * acc_H + acc_L is the reference's integer, and
 // no term over the block sums is left.
+//
+// Q2K weights (BlockQ2K::vec_dot, k_quants.rs:755-805) need one plane only: a 4-bit scale times a 2-bit code is at most 45,
+// so the scaled codes are the weight operand as they are and a super-block takes four int8 MFMAs per operand instead of
+// eight; the minimums leave through the sixteen block sums as for Q4K.
 #include <type_traits>
 #include "act_quant.hpp"
 #include "kernels.hpp"
@@ -117,12 +121,17 @@ struct BRegs {
     u32x4 hdr;    // Q4K: d, dmin, 12 scale bytes of row n; Q6K: the row's sixteen i8 scales
     u32x4 qh;     // Q6K: the codes' top two bits, word P for pair P
     u32x2 q5;     // Q5K: the lane's fifth bits (pairs 0,1 / 2,3; four bits per byte and pair)
-    uint32_t d16; // Q6K: d (f16 bits)
+    uint32_t d16; // Q6K: d (f16 bits); Q2K: d | dmin << 16
 };
 template <int FMT>
 __device__ __forceinline__ BRegs b_load(const uint8_t* tile, int lane) {
     BRegs b;
     b.c[0] = gld<u32x4>(tile, (uint32_t)(lane * 16));
+    if (FMT == MOE_GGML_Q2K) {   // word P of the lane: the 2-bit codes of pair P; then the row's 16 (scale | min << 4) bytes and d | dmin << 16
+        b.hdr = gld<u32x4>(tile, (uint32_t)(1024 + (lane & 15) * 16));
+        b.d16 = gld<uint32_t>(tile, (uint32_t)(1280 + (lane & 15) * 4));
+        return b;
+    }
     b.c[1] = gld<u32x4>(tile, (uint32_t)(1024 + lane * 16));
     if (FMT == MOE_GGML_Q6K) {
         b.qh = gld<u32x4>(tile, (uint32_t)(2048 + lane * 16));
@@ -260,6 +269,28 @@ __device__ __forceinline__ BPlanes b_prepare_q5k(const BRegs& b, int lane) {
     return o;
 }
 
+// Q2K: the one plane sc * code (<= 45).  A lane's eight elements of a 32-element stretch lie in one 16-element sub-block
+// (the first for chunks 0 and 1, the second for chunks 2 and 3), so each half of an MFMA operand takes one scale.
+__device__ __forceinline__ BPlanes b_prepare_q2k(const BRegs& b, int lane) {
+    const int g = lane >> 4;
+    const uint32_t M3 = 0x03030303u;
+    BPlanes o;
+    o.d = __half2float(__ushort_as_half((unsigned short)(b.d16 & 0xffffu)));
+    o.dmin = __half2float(__ushort_as_half((unsigned short)(b.d16 >> 16)));
+    const int sel = 8 * (g >> 1);
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t q = b.c[0][P], sw = b.hdr[P];
+        const uint32_t s_a = (sw >> sel) & 0xFu, s_b = (sw >> (16 + sel)) & 0xFu;
+        o.lo[P] = v4i{(int)scale_bytes(q & M3, s_a), (int)scale_bytes((q >> 2) & M3, s_a),
+                      (int)scale_bytes((q >> 4) & M3, s_b), (int)scale_bytes((q >> 6) & M3, s_b)};
+    }
+    // mins: the f16 MFMA's k = 4g + j is block sum 4g + j = sub-block 4g + j
+    const uint32_t mg = (b.hdr[g] >> 4) & 0x0f0f0f0fu;
+    o.mB = v4h{(_Float16)(int)(mg & 0xffu), (_Float16)(int)((mg >> 8) & 0xffu), (_Float16)(int)((mg >> 16) & 0xffu), (_Float16)(int)(mg >> 24)};
+    return o;
+}
+
 // one super-block of the wave's 16 weight rows against 16-slot operand o of the staged tile
 // `while_busy` runs right after the MFMAs are issued: this is where the next super-block's loads go.
 template <int FMT, int NOP, typename Fill>
@@ -275,7 +306,7 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
     for (int P = 0; P < 4; P++) {
         const v4i a = *reinterpret_cast<const v4i*>(arow + P * 1024);
         acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.lo[P], P == 0 ? zero4 : acc_lo, 0, 0, 0);
-        acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.hi[P], P == 0 ? zero4 : acc_hi, 0, 0, 0);
+        if constexpr (FMT != MOE_GGML_Q2K) acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.hi[P], P == 0 ? zero4 : acc_hi, 0, 0, 0);
     }
     __builtin_amdgcn_s_setprio(0);
     // D[i] belongs to slot 16 o + 4 g + i, weight row n = lane%16
@@ -295,9 +326,17 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
         while_busy();
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int isum = (acc_hi[i] << (FMT == MOE_GGML_Q5K ? 8 : 3)) + acc_lo[i];
-            const float v = __builtin_fmaf(B.d, (float)isum, -(B.dmin * Dm[i]));
-            facc[i] = __builtin_fmaf(yd[i], v, facc[i]);
+            if constexpr (FMT == MOE_GGML_Q2K) {
+                // the reference's own order, every product and the difference rounded (k_quants.rs:772-773, 801): with unsigned
+                // 2-bit codes the two terms are large and nearly cancel, and the scalar path's sum has one order only -- a
+                // wave walks K in that order, so the up projection repeats vec_dot_unopt bit for bit
+                const float dall = yd[i] * B.d, dminy = yd[i] * B.dmin;
+                facc[i] += dall * (float)acc_lo[i] - dminy * Dm[i];
+            } else {
+                const int isum = (acc_hi[i] << (FMT == MOE_GGML_Q5K ? 8 : 3)) + acc_lo[i];
+                const float v = __builtin_fmaf(B.d, (float)isum, -(B.dmin * Dm[i]));
+                facc[i] = __builtin_fmaf(yd[i], v, facc[i]);
+            }
         }
     }
 }
@@ -311,12 +350,12 @@ __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-// FMT: the weights' format (Q4K, Q5K, Q6K).
+// FMT: the weights' format (Q2K, Q4K, Q5K, Q6K).
 template <int FMT, int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
-    static_assert(FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || FMT == MOE_GGML_Q6K, "formats of the tiled kernel");
+    static_assert(FMT == MOE_GGML_Q2K || FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || FMT == MOE_GGML_Q6K, "formats of the tiled kernel");
     constexpr int NB = NOP / 2;
-    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : Q4K_TILE_BYTES;
+    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : FMT == MOE_GGML_Q2K ? Q2K_TILE_BYTES : Q4K_TILE_BYTES;
     constexpr bool kSums = FMT != MOE_GGML_Q6K;   // block sums staged (the mins term)
     __shared__ GemmLds<NOP> L;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -370,6 +409,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     };
     auto prepare = [&](const BRegs& r) {
         if constexpr (FMT == MOE_GGML_Q6K) return b_prepare_q6k(r, lane);
+        else if constexpr (FMT == MOE_GGML_Q2K) return b_prepare_q2k(r, lane);
         else if constexpr (FMT == MOE_GGML_Q5K) return b_prepare_q5k(r, lane);
         else return b_prepare(r, lane);
     };
@@ -448,8 +488,8 @@ static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
     if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 4>), grid, dim3(G_THREADS), 0, s, p);
     else hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 8>), grid, dim3(G_THREADS), 0, s, p);
 }
-bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
-bool q4k_gemm_down_format(int dt) { return dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
+bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q2K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
+bool q4k_gemm_down_format(int dt) { return q4k_gemm_up_format(dt); }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p_in, hipStream_t s) {
     ExpertParams p = p_in;
     const int64_t tiles = max_gemm_tiles(p.n_slots, p.n_groups + 1, p.rb.tile_slots);
@@ -458,6 +498,7 @@ hipError_t launch_q4k_gemm_up(const ExpertParams& p_in, hipStream_t s) {
     if (p.dt == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 0>(p, grid, s);
+    else if (p.dt == MOE_GGML_Q2K) launch_gemm<MOE_GGML_Q2K, 0>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -470,6 +511,7 @@ hipError_t launch_q4k_gemm_down(const ExpertParams& p_in, hipStream_t s) {
     if (dtd == MOE_GGML_Q6K) launch_gemm<MOE_GGML_Q6K, 1>(p, grid, s);
     else if (dtd == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 1>(p, grid, s);
     else if (dtd == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 1>(p, grid, s);
+    else if (dtd == MOE_GGML_Q2K) launch_gemm<MOE_GGML_Q2K, 1>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -206,11 +206,12 @@ def test_cfg3_prefill_q4k_up_q6k_down(mixtral_layer, request):
     gpu.close()
 
 
-def test_cfg3_prefill_q5k_experts(request):
-    """Q5_K experts (what Q5_K_M files hold) at the Mixtral shape, 2048 tokens with the Zipf load: the tiled kernels in
-    their Q5K variant for both projections.  Same bars as the Q4K prefill."""
+@pytest.mark.parametrize("dt,name", [(O.Q5K, "Q5K"), (O.Q2K, "Q2K")])
+def test_cfg3_prefill_other_kquant_experts(request, dt, name):
+    """Q5_K experts (what Q5_K_M files hold) and Q2_K experts (the one-plane variant) at the Mixtral shape, 2048 tokens with
+    the Zipf load: the tiled kernels in their variant of the format for both projections.  Same bars as the Q4K prefill."""
     T = 2048
-    ref, gpu = build(4096, 14336, 8, 2, O.Q5K, seed=3, bias=ZIPF_BIAS)
+    ref, gpu = build(4096, 14336, 8, 2, dt, seed=3, bias=ZIPF_BIAS)
     xs = acts(T, 4096, 23)
     ys = gpu.forward(xs)
     logits = gpu.last_logits(T)
@@ -221,7 +222,7 @@ def test_cfg3_prefill_q5k_experts(request):
     want = ref.forward(xs, logits=logits, simd=True, threads=CORES)
     r = rms(want)
     e_max, e_share, e_rms = tail_stats(ys, want, r)
-    say(request.config, " [Q5K vs AVX2: max %.2e, share > 2e-3 %.1e, rms %.1e]" % (e_max, e_share, e_rms))
+    say(request.config, " [%s vs AVX2: max %.2e, share > 2e-3 %.1e, rms %.1e]" % (name, e_max, e_share, e_rms))
     assert e_rms <= 2e-4 and e_share <= 5e-5 and e_max <= 3 * TOL, (e_max, e_share, e_rms)
     n = 512
     want_s = ref.forward(xs[:n], logits=logits[:n], simd=False, threads=CORES)
