@@ -18,7 +18,7 @@ measures the other regimes in the same process and reports them as sub-objects o
                   plus N(0, 0.1) noise; end-to-end tokens/s.
 
 `--workload decode|prefill|config4|stack` measures one of them alone as the line's `value`.
-`--workload prefill [--weights q2_k|q5_k|q6_k] [--weights-down q5_k|q6_k]` measures the prefill with Q2_K / Q5_K / Q6_K w1 / w3 and / or w2 stored
+`--workload prefill [--weights q2_k|q3_k|q5_k|q6_k] [--weights-down q5_k|q6_k]` measures the prefill with Q2_K / Q3_K / Q5_K / Q6_K w1 / w3 and / or w2 stored
 in another K-quant (Q4_K_M and Q5_K_M files store part of w2 as Q6_K).
 `--weights q4_0|q4_1|q5_0|q5_1|q8_0|q2_k|q3_k|q5_k|q6_k` runs the decode workload on the same layer shape with another
 GGML format (random block payloads with small finite scales: timing does not depend on the values).
@@ -409,8 +409,8 @@ def main():
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
         return
     wl = args.workload
-    if args.weights != "q4_k" and wl not in ("decode", "all") and not (wl == "prefill" and args.weights in ("q2_k", "q5_k", "q6_k")):
-        sys.exit("bench.py: --weights applies to the decode workload (and q2_k / q5_k / q6_k to the prefill workload) only")
+    if args.weights != "q4_k" and wl not in ("decode", "all") and not (wl == "prefill" and args.weights in ("q2_k", "q3_k", "q5_k", "q6_k")):
+        sys.exit("bench.py: --weights applies to the decode workload (and the other K-quants to the prefill workload) only")
     if args.weights != "q4_k" and wl != "prefill":
         wl = "decode"
     if args.weights_down and wl != "prefill":

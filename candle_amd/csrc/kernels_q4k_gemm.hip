@@ -1,4 +1,4 @@
-// Tiled grouped expert products for large batches (prefill): Q4K (also Q2K, Q5K and Q6K) weights x
+// Tiled grouped expert products for large batches (prefill): Q4K (also Q2K, Q3K, Q5K and Q6K) weights x
 // Q8K activations on v_mfma_i32_16x16x64_i8, a full-rate int8 MFMA shape of gfx950.
 //
 // Same integers as BlockQ4K::vec_dot (candle-core/src/quantized/k_quants.rs:1205-1285):
@@ -120,13 +120,19 @@ struct BRegs {
     u32x4 c[2];   // plane pl: (x,y) = 8 bytes of pair 2pl, chunk g; (z,w) = pair 2pl+1 (Q6K: the codes' low nibbles)
     u32x4 hdr;    // Q4K: d, dmin, 12 scale bytes of row n; Q6K: the row's sixteen i8 scales
     u32x4 qh;     // Q6K: the codes' top two bits, word P for pair P
-    u32x2 q5;     // Q5K: the lane's fifth bits (pairs 0,1 / 2,3; four bits per byte and pair)
-    uint32_t d16; // Q6K: d (f16 bits); Q2K: d | dmin << 16
+    u32x2 q5;     // Q5K: the lane's fifth bits (pairs 0,1 / 2,3; four bits per byte and pair); Q3K: the codes' third bits, placed alike
+    uint32_t d16; // Q6K, Q3K: d (f16 bits); Q2K: d | dmin << 16
 };
 template <int FMT>
 __device__ __forceinline__ BRegs b_load(const uint8_t* tile, int lane) {
     BRegs b;
     b.c[0] = gld<u32x4>(tile, (uint32_t)(lane * 16));
+    if (FMT == MOE_GGML_Q3K) {   // the codes' low two bits (placed as Q2K's codes), their high bits, the row's sixteen i8 scales, d
+        b.q5 = gld<u32x2>(tile, (uint32_t)(1024 + lane * 8));
+        b.hdr = gld<u32x4>(tile, (uint32_t)(1536 + (lane & 15) * 16));
+        b.d16 = gld<uint16_t>(tile, (uint32_t)(1792 + (lane & 15) * 2));
+        return b;
+    }
     if (FMT == MOE_GGML_Q2K) {   // word P of the lane: the 2-bit codes of pair P; then the row's 16 (scale | min << 4) bytes and d | dmin << 16
         b.hdr = gld<u32x4>(tile, (uint32_t)(1024 + (lane & 15) * 16));
         b.d16 = gld<uint32_t>(tile, (uint32_t)(1280 + (lane & 15) * 4));
@@ -269,6 +275,38 @@ __device__ __forceinline__ BPlanes b_prepare_q5k(const BRegs& b, int lane) {
     return o;
 }
 
+// Q3K (BlockQ3K::vec_dot, k_quants.rs:923-1047): d * y.d * sum_j sc_j * ((code_j - 4) . q8_j) with a signed 6-bit scale per
+// 16 elements.  W = sc * (code - 4) lies in [-124, 128] -- one too many for a signed byte -- so it is formed and cut into two
+// signed bytes exactly as the Q6K products are, W + 128 = code * sc + (128 - 4 sc); the high plane is zero but where W = 128.
+__device__ __forceinline__ BPlanes b_prepare_q3k(const BRegs& b, int lane) {
+    const int g = lane >> 4;
+    const uint32_t M3 = 0x03030303u, M1H = 0x04040404u;
+    BPlanes o;
+    o.d = __half2float(__ushort_as_half((unsigned short)b.d16));
+    o.dmin = 0.f;
+    o.mB = v4h{0, 0, 0, 0};
+    const uint32_t sel = (uint32_t)(g >> 1) * 8u;   // elements 8g .. 8g+7 of a 32-element stretch: its first or second 16
+#pragma unroll
+    for (int P = 0; P < 4; P++) {
+        const uint32_t q = b.c[0][P], sw = b.hdr[P];
+        const uint32_t h = ((P < 2) ? b.q5.x : b.q5.y) >> (4 * (P & 1));
+        const int sa = __builtin_amdgcn_sbfe(sw, sel, 8), sb = __builtin_amdgcn_sbfe(sw, sel + 16u, 8);
+        const uint32_t sa2 = __builtin_amdgcn_perm((uint32_t)sa, (uint32_t)sa, 0x05040100u);
+        const uint32_t sb2 = __builtin_amdgcn_perm((uint32_t)sb, (uint32_t)sb, 0x05040100u);
+        const uint32_t aa2 = pk_mad_u16(sa2, 0xfffcfffcu, 0x00800080u), ab2 = pk_mad_u16(sb2, 0xfffcfffcu, 0x00800080u);
+        const uint32_t c0 = (q & M3) | ((h << 2) & M1H), c1 = ((q >> 2) & M3) | ((h << 1) & M1H);
+        const uint32_t c2 = ((q >> 4) & M3) | (h & M1H), c3 = ((q >> 6) & M3) | ((h >> 1) & M1H);
+        int l0, l1, l2, l3, h0, h1, h2, h3;
+        q6k_planes(c0, sa2, aa2, l0, h0);
+        q6k_planes(c1, sa2, aa2, l1, h1);
+        q6k_planes(c2, sb2, ab2, l2, h2);
+        q6k_planes(c3, sb2, ab2, l3, h3);
+        o.lo[P] = v4i{l0, l1, l2, l3};
+        o.hi[P] = v4i{h0, h1, h2, h3};
+    }
+    return o;
+}
+
 // Q2K: the one plane sc * code (<= 45).  A lane's eight elements of a 32-element stretch lie in one 16-element sub-block
 // (the first for chunks 0 and 1, the second for chunks 2 and 3), so each half of an MFMA operand takes one scale.
 __device__ __forceinline__ BPlanes b_prepare_q2k(const BRegs& b, int lane) {
@@ -310,7 +348,7 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
     }
     __builtin_amdgcn_s_setprio(0);
     // D[i] belongs to slot 16 o + 4 g + i, weight row n = lane%16
-    if constexpr (FMT == MOE_GGML_Q6K) {
+    if constexpr (FMT == MOE_GGML_Q6K || FMT == MOE_GGML_Q3K) {
         const v4f yd = *reinterpret_cast<const v4f*>(&L.yd[buf][o * 16 + g * 4]);
         while_busy();
 #pragma unroll
@@ -350,13 +388,13 @@ __device__ __forceinline__ float silu_gemm(float v) { return v / (1.0f + __expf(
 //                 rows of w3; the w3 waves hand their sums over through LDS and the w1 waves write
 //                 h = silu(a) * b (f32).
 // MODE 1: down -- a workgroup owns 128 rows of H of w2, one 16-row operand per wave; writes yw.
-// FMT: the weights' format (Q2K, Q4K, Q5K, Q6K).
+// FMT: the weights' format (Q2K ... Q6K).
 template <int FMT, int MODE, int NOP>
 __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q4k_gemm_kernel(ExpertParams p) {
-    static_assert(FMT == MOE_GGML_Q2K || FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || FMT == MOE_GGML_Q6K, "formats of the tiled kernel");
+    static_assert(FMT == MOE_GGML_Q2K || FMT == MOE_GGML_Q3K || FMT == MOE_GGML_Q4K || FMT == MOE_GGML_Q5K || FMT == MOE_GGML_Q6K, "formats of the tiled kernel");
     constexpr int NB = NOP / 2;
-    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : FMT == MOE_GGML_Q2K ? Q2K_TILE_BYTES : Q4K_TILE_BYTES;
-    constexpr bool kSums = FMT != MOE_GGML_Q6K;   // block sums staged (the mins term)
+    constexpr int TILE_BYTES = FMT == MOE_GGML_Q6K ? Q6K_TILE_BYTES : FMT == MOE_GGML_Q5K ? Q5K_TILE_BYTES : FMT == MOE_GGML_Q2K ? Q2K_TILE_BYTES : FMT == MOE_GGML_Q3K ? Q3K_TILE_BYTES : Q4K_TILE_BYTES;
+    constexpr bool kSums = FMT != MOE_GGML_Q6K && FMT != MOE_GGML_Q3K;   // block sums staged (the mins term)
     __shared__ GemmLds<NOP> L;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -410,6 +448,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
     auto prepare = [&](const BRegs& r) {
         if constexpr (FMT == MOE_GGML_Q6K) return b_prepare_q6k(r, lane);
         else if constexpr (FMT == MOE_GGML_Q2K) return b_prepare_q2k(r, lane);
+        else if constexpr (FMT == MOE_GGML_Q3K) return b_prepare_q3k(r, lane);
         else if constexpr (FMT == MOE_GGML_Q5K) return b_prepare_q5k(r, lane);
         else return b_prepare(r, lane);
     };
@@ -488,7 +527,7 @@ static void launch_gemm(const ExpertParams& p, dim3 grid, hipStream_t s) {
     if (p.rb.tile_slots == 64) hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 4>), grid, dim3(G_THREADS), 0, s, p);
     else hipLaunchKernelGGL((q4k_gemm_kernel<FMT, MODE, 8>), grid, dim3(G_THREADS), 0, s, p);
 }
-bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q2K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
+bool q4k_gemm_up_format(int dt) { return dt == MOE_GGML_Q2K || dt == MOE_GGML_Q3K || dt == MOE_GGML_Q4K || dt == MOE_GGML_Q5K || dt == MOE_GGML_Q6K; }
 bool q4k_gemm_down_format(int dt) { return q4k_gemm_up_format(dt); }
 hipError_t launch_q4k_gemm_up(const ExpertParams& p_in, hipStream_t s) {
     ExpertParams p = p_in;
@@ -499,6 +538,7 @@ hipError_t launch_q4k_gemm_up(const ExpertParams& p_in, hipStream_t s) {
     else if (p.dt == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 0>(p, grid, s);
     else if (p.dt == MOE_GGML_Q2K) launch_gemm<MOE_GGML_Q2K, 0>(p, grid, s);
+    else if (p.dt == MOE_GGML_Q3K) launch_gemm<MOE_GGML_Q3K, 0>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -512,6 +552,7 @@ hipError_t launch_q4k_gemm_down(const ExpertParams& p_in, hipStream_t s) {
     else if (dtd == MOE_GGML_Q5K) launch_gemm<MOE_GGML_Q5K, 1>(p, grid, s);
     else if (dtd == MOE_GGML_Q4K) launch_gemm<MOE_GGML_Q4K, 1>(p, grid, s);
     else if (dtd == MOE_GGML_Q2K) launch_gemm<MOE_GGML_Q2K, 1>(p, grid, s);
+    else if (dtd == MOE_GGML_Q3K) launch_gemm<MOE_GGML_Q3K, 1>(p, grid, s);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }

@@ -206,9 +206,9 @@ def test_cfg3_prefill_q4k_up_q6k_down(mixtral_layer, request):
     gpu.close()
 
 
-@pytest.mark.parametrize("dt,name", [(O.Q5K, "Q5K"), (O.Q2K, "Q2K")])
+@pytest.mark.parametrize("dt,name", [(O.Q5K, "Q5K"), (O.Q2K, "Q2K"), (O.Q3K, "Q3K")])
 def test_cfg3_prefill_other_kquant_experts(request, dt, name):
-    """Q5_K experts (what Q5_K_M files hold) and Q2_K experts (the one-plane variant) at the Mixtral shape, 2048 tokens with
+    """Q5_K experts (what Q5_K_M files hold), Q2_K experts (the one-plane variant) and Q3_K experts at the Mixtral shape, 2048 tokens with
     the Zipf load: the tiled kernels in their variant of the format for both projections.  Same bars as the Q4K prefill."""
     T = 2048
     ref, gpu = build(4096, 14336, 8, 2, dt, seed=3, bias=ZIPF_BIAS)

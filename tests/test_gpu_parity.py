@@ -132,7 +132,7 @@ def test_route_zipf_bias_lists():
                                        (O.Q3K, 64, 512, 5), (O.Q3K, 1040, 1024, 33), (O.Q3K, 256, 2304, 150),
                                        (O.Q5K, 64, 512, 5), (O.Q5K, 1040, 1024, 33), (O.Q5K, 256, 2304, 150),
                                        (O.Q6K, 64, 512, 5), (O.Q6K, 1040, 1024, 33), (O.Q6K, 256, 2304, 150),
-                                       (O.Q4K, 4096, 1024, 700), (O.Q5K, 4096, 1024, 700), (O.Q6K, 4096, 1024, 700), (O.Q2K, 4096, 1024, 700),
+                                       (O.Q4K, 4096, 1024, 700), (O.Q5K, 4096, 1024, 700), (O.Q6K, 4096, 1024, 700), (O.Q2K, 4096, 1024, 700), (O.Q3K, 4096, 1024, 700),
                                        (O.Q8_0, 4096, 1024, 1100), (O.Q8_0, 2048, 1408, 1100), (O.Q4_0, 4096, 1024, 600), (O.Q5_0, 2048, 1408, 2100),
                                        (O.Q8_0, 256, 1408, 40), (O.Q4_0, 32, 64, 16), (O.Q4_0, 128, 1024, 70),
                                        (O.Q5_0, 48, 96, 3), (O.Q5_0, 256, 1408, 40), (O.Q5_0, 128, 1024, 70),
@@ -303,7 +303,7 @@ def test_block_q6k_and_mixed_down_dtype(dt, dt_down):
     # all-Q6K and all-Q5K experts, the Q4_K_M arrangement (Q4K gate / up with Q6K down), its reverse, and
     # the Q5_K_M arrangement (Q5K with Q6K down).
     # T = 1, 3: narrow workgroups; 8, 33: one and two slot tiles per pass; 70: dispatched lists;
-    # 200: a Q2K, Q4K, Q5K or Q6K up projection switches to the tiled kernel; 300, 500: so does such a down projection
+    # 200: a K-quant up projection switches to the tiled kernel; 300, 500: so does such a down projection
     # behind it (64-slot and 128-slot tiles)
     ref, gpu = make_pair(512, 1024, 8, 2, dt, seed=12, dt_down=dt_down)
     for T in (1, 3, 8, 33, 70, 200, 300, 500):
