@@ -111,9 +111,11 @@ def test_projection_from_gguf(tmp_path):
     check(O.Q4_0, lin.forward(x[:3]), O.matmul(O.Q4_0, x[:3], blocks["output.weight"], 1024))
 
 
-def test_projection_recorded_into_a_hip_graph():
+@pytest.mark.parametrize("m", [8, 1])
+def test_projection_recorded_into_a_hip_graph(m):
+    # m = 8: quantiser, table and product recorded; m = 1: the single launch that quantises the row itself
     torch = pytest.importorskip("torch")
-    dt, n, k, m = O.Q4K, 512, 1024, 8
+    dt, n, k = O.Q4K, 512, 1024
     w = O.fill_normal_quantized(6, dt, n, k, 0.02)
     lin = candle_amd.QMatMul(dt, w, n, k)
     xs = [torch.from_numpy(activations(m, k, seed=60 + i)).cuda() for i in range(3)]
