@@ -997,6 +997,13 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
         MOE_HIP_CHECK(launch_qlinear_fused(Q->dt, d_x, m, Q->n, Q->k, Q->weights.as<uint8_t>(), d_y, s));
         return MOE_OK;
     }
+    // the 32-element formats: the same, with the block values added in the reference's order by one wave (in a graph,
+    // Q8_0, fused / two passes: 4096 x 4096: 9.3 / 22.1 us at one row, 13.6 / 22.4 at two, 21.4 / 22.8 at four; 4096 x 14336:
+    // 27.6 / 57.0 at one row; 8192 x 4096: 11.4 / 22.7; 32000 x 4096: 33.1 / 30.3)
+    if (fr != 1 && q32_rows_fused_usable(Q->dt, m, Q->n, Q->k) && (fr == 2 || (m <= 3 && Q->n <= 16384))) {
+        MOE_HIP_CHECK(launch_q32_rows_fused(Q->dt, d_x, m, Q->n, Q->k, Q->weights.as<uint8_t>(), d_y, s));
+        return MOE_OK;
+    }
     // under stream capture nothing may be allocated, the graph carries its own copy of the routing table pass, and the
     // workspace is never freed afterwards (a replay uses its addresses)
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

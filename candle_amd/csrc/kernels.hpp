@@ -135,6 +135,9 @@ bool q4k_gemm_up_format(int dt);
 bool q4k_gemm_down_format(int dt);
 // Dense K-quant matrix [n, k] (device layout) times m <= 4 rows of f32 in one launch (the rows are quantised in the kernel).
 bool qlinear_fused_usable(int dt, int64_t m, int64_t n, int64_t k);
+// The same for the 32-element formats (super-tile layout): bit-identical to the streaming kernel's results.
+bool q32_rows_fused_usable(int dt, int64_t m, int64_t n, int64_t k);
+hipError_t launch_q32_rows_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s);
 hipError_t launch_qlinear_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s);
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);

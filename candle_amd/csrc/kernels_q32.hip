@@ -936,6 +936,177 @@ hipError_t launch_q8_0_gemm_down(const ExpertParams& p_in, hipStream_t s) {
     return qg_launch<1>(p.dt_down ? p.dt_down : p.dt, p, dim3(patch_grid(p.H / 128, qg_tiles(p), p.patch)), s);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Dense matrix (super-tile layout) times one to four rows in one launch, for single-stream decoding.  The streaming down
+// kernel gives a row tile to one wave, which walks all of K -- 256 waves for a matrix of 4096 rows -- because the
+// reference adds a row's block values in ascending block order and the results have to carry the same bits.  Here the four
+// waves of a workgroup share a row tile's K all the same: they compute the block values ((isum as f32) * d_w) * d_x
+// (+ m_w * s_x) in parallel, 64 blocks at a time, and park them in LDS; one wave then adds them to the running sums in
+// block order.  The rows are quantised inside the kernel (BlockQ8_0 / BlockQ8_1::from_float, k_quants.rs:605-634, 700-729:
+// the arithmetic of quantize_q8_0_block, eight pairs of blocks side by side), each wave the blocks it multiplies.
+// Maximum / sum over the 32 lanes that hold one block, left in all of them: four rotations inside the rows of 16 lanes
+// (DPP: no LDS traffic, no address arithmetic) and one exchange between the two rows.
+__device__ __forceinline__ float block32_max(float v) {
+#define GV_ROR_MAX(n) v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + (n), 0xf, 0xf, false)))
+    GV_ROR_MAX(8); GV_ROR_MAX(4); GV_ROR_MAX(2); GV_ROR_MAX(1);
+#undef GV_ROR_MAX
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401f)));   // lane ^ 16
+}
+__device__ __forceinline__ int block32_sum(int v) {
+#define GV_ROR_ADD(n) v += __builtin_amdgcn_update_dpp(0, v, 0x120 + (n), 0xf, 0xf, false)
+    GV_ROR_ADD(8); GV_ROR_ADD(4); GV_ROR_ADD(2); GV_ROR_ADD(1);
+#undef GV_ROR_ADD
+    return v + __builtin_amdgcn_ds_swizzle(v, 0x401f);
+}
+
+constexpr int GV_MAX_ROWS = 4;
+constexpr int GV_STEPS = 4;                     // K steps (of four blocks) a wave takes per chunk
+constexpr int GV_BLOCKS = 4 * GV_STEPS;         // blocks per wave and chunk
+constexpr int GV_CHUNK = 4 * GV_BLOCKS;         // blocks per workgroup and chunk
+
+template <int DT>
+__global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int m, int n, int K, const uint8_t* w, float* y) {
+    typedef Q32Fmt<DT> F;
+    constexpr size_t STB = Q32SFmt<DT>::STB;
+    constexpr int VDT = F::HAS_M ? MOE_GGML_Q8_1 : MOE_GGML_Q8_0;
+    __shared__ float terms[2][GV_CHUNK][4][16];                       // [buffer][block of the chunk][row of x][weight row]
+    __shared__ __align__(16) int8_t xq[4][GV_BLOCKS][GV_MAX_ROWS][32];  // [wave][block][row]: quants
+    __shared__ float xd[4][GV_BLOCKS][GV_MAX_ROWS];
+    __shared__ int32_t xw[4][GV_BLOCKS][GV_MAX_ROWS];
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_rt = n / 16, nks = K / 128, nkb = K / 32;
+    const int rt = blockIdx.x;
+    const uint8_t* tp = w + (size_t)rt * STB;
+    const size_t step_stride = (size_t)n_rt * STB;
+    const int n_chunks = (nks + 4 * GV_STEPS - 1) / (4 * GV_STEPS);
+    const int my_row = r < m ? r : m - 1;
+    float acc = 0.f;   // wave 0: lane (weight row r, row g of x)
+    // weights of the wave's steps of a chunk: requested a chunk ahead, the rows are quantised while they travel
+    Q32SRaw<DT> raw[GV_STEPS];
+    auto request = [&](int c) {
+#pragma unroll
+        for (int st = 0; st < GV_STEPS; st++) {
+            int ks = c * 4 * GV_STEPS + wave * GV_STEPS + st;
+            ks = ks < nks ? ks : nks - 1;
+            raw[st] = load_q32s<DT, true>(tp + (size_t)ks * step_stride, lane);
+        }
+    };
+    request(0);
+    float xnext[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const int e = wave * GV_STEPS * 128 + j * 64 + lane;
+        xnext[j] = ldg<float>(x, (uint32_t)(e < K ? e : K - 1) * 4u);
+    }
+    for (int c = 0; c < n_chunks; c++) {
+        const int ks0 = c * 4 * GV_STEPS + wave * GV_STEPS;       // this wave's first K step of the chunk
+        const int n_steps = nks - ks0 < GV_STEPS ? (nks - ks0 < 0 ? 0 : nks - ks0) : GV_STEPS;
+        // the rows' blocks of these steps: 512 elements per row, lane l holds elements l, l + 64, ... (pair of blocks j)
+        for (int row = 0; row < m; row++) {
+            float xv[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) xv[j] = xnext[j];
+            {   // the values of the next row (after the last one: of row 0 of the next chunk) are requested a turn ahead
+                const int nrow = row + 1 < m ? row + 1 : 0;
+                const int nks0 = row + 1 < m ? ks0 : ks0 + 4 * GV_STEPS;
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int e = nks0 * 128 + j * 64 + lane;
+                    xnext[j] = ldg<float>(x, ((uint32_t)nrow * (uint32_t)K + (uint32_t)(e < K ? e : K - 1)) * 4u);
+                }
+            }
+            float amax[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) amax[j] = fabsf(xv[j]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) amax[j] = block32_max(amax[j]);
+            int q[8], sum[8];
+            float d[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                d[j] = amax[j] / 127.0f;
+                const float id = (d[j] != 0.f) ? 1.0f / d[j] : 0.f;
+                q[j] = sat_i8(roundf(xv[j] * id));
+                sum[j] = q[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) sum[j] = block32_sum(sum[j]);
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int blk = 2 * j + (lane >> 5);
+                xq[wave][blk][row][lane & 31] = (int8_t)q[j];
+                if ((lane & 31) == 0) {
+                    const float dh = __half2float(__float2half_rn(d[j]));
+                    xd[wave][blk][row] = dh;
+                    xw[wave][blk][row] = q8_block_word(VDT, sum[j], dh);
+                }
+            }
+        }
+        // the wave reads what its other lanes have written: LDS serves a wave's requests in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int buf = c & 1;
+#pragma unroll
+        for (int st = 0; st < GV_STEPS; st++) {
+            if (st < n_steps) {   // uniform
+                const Q32Tile<DT> wb[4] = {q32s_block<DT, 0>(raw[st], g), q32s_block<DT, 1>(raw[st], g), q32s_block<DT, 2>(raw[st], g),
+                                           q32s_block<DT, 3>(raw[st], g)};
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    const int blk = st * 4 + b;
+                    const int8_t* ap = &xq[wave][blk][my_row][0];
+                    const uint32_t alo = *reinterpret_cast<const uint32_t*>(ap + 4 * g), ahi = *reinterpret_cast<const uint32_t*>(ap + 16 + 4 * g);
+                    const long av = (long)(((uint64_t)ahi << 32) | alo);
+                    const long bv = (long)(((uint64_t)wb[b].q.y << 32) | wb[b].q.x);
+                    const v4i zero = {0, 0, 0, 0};
+                    const v4i D = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, zero, 0, 0, 0);
+                    if (g == 0) {   // D[i]: row i of x, weight row r
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            if (i >= m) break;   // uniform
+                            const int xr = i;
+                            const int word = xw[wave][blk][xr];
+                            int isum = D[i];
+                            if (F::OFFSET) isum -= F::OFFSET * word;
+                            float t = (float)isum * wb[b].d;
+                            t = t * xd[wave][blk][xr];
+                            if (F::HAS_M) t = t + wb[b].m * __int_as_float(word);   // the word holds the activation block's s
+                            terms[buf][wave * GV_BLOCKS + blk][i][r] = t;
+                        }
+                    }
+                }
+            }
+        }
+        if (c + 1 < n_chunks) request(c + 1);
+        __syncthreads();
+        if (wave == 0) {   // the chunk's block values join the running sums in ascending block order
+            const int nb = nkb - c * GV_CHUNK < GV_CHUNK ? nkb - c * GV_CHUNK : GV_CHUNK;
+            for (int b = 0; b < nb; b++) acc += terms[buf][b][g][r];
+        }
+    }
+    if (wave == 0 && g < m) y[(size_t)g * n + (size_t)rt * 16 + r] = acc;
+}
+
+bool q32_rows_fused_usable(int dt, int64_t m, int64_t n, int64_t k) {
+    const bool fmt = dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_1;
+    return fmt && m >= 1 && m <= GV_MAX_ROWS && n % 16 == 0 && q32_super_layout(k) && k >= 128 && m * k < ((int64_t)1 << 29);
+}
+hipError_t launch_q32_rows_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s) {
+    if (!q32_rows_fused_usable(dt, m, n, k)) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)(n / 16)), block(256);
+    switch (dt) {
+        case MOE_GGML_Q8_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q8_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        case MOE_GGML_Q4_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q4_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        case MOE_GGML_Q5_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q5_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        case MOE_GGML_Q4_1: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q4_1>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        case MOE_GGML_Q5_1: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q5_1>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_q4k_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_down(const ExpertParams& p, hipStream_t s);
 

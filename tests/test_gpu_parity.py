@@ -190,6 +190,32 @@ def test_few_rows_quantised_inside_the_kernel_equal_the_two_pass_path(dt):
             q.close()
 
 
+@pytest.mark.parametrize("dt", [O.Q8_0, O.Q4_0, O.Q5_0, O.Q4_1, O.Q5_1])
+def test_few_rows_of_the_32_element_formats_in_one_launch(dt):
+    # the four waves of a workgroup share a row tile's K and one of them adds the block values in ascending block order:
+    # the bits of the streaming kernel (one wave per row tile) and of the scalar reference loop.  K of 1, 10, 18 and 32
+    # steps of 128 (a wave without blocks, a partial second chunk); a row with an all-zero block.
+    for n, k in ((48, 128), (1040, 1280), (256, 2304), (4096, 4096)):
+        w = O.fill_normal_quantized(n + k + dt, dt, n, k, 0.02)
+        q = candle_amd.QMatMul(dt, w, n, k)
+        try:
+            for m in (1, 2, 3, 4):
+                x = activations(m, k, seed=200 + m)
+                x[0, :32] = 0.0
+                try:
+                    candle_amd.set_switch("fused_rows", 2)
+                    fused = q.forward(x)
+                    candle_amd.set_switch("fused_rows", 1)
+                    two_pass = q.forward(x)
+                finally:
+                    candle_amd.set_switch("fused_rows", 0)
+                assert np.array_equal(bits(fused), bits(two_pass)), (dt, n, k, m)
+                if n * k <= 1040 * 1280:
+                    assert np.array_equal(bits(fused), bits(O.matmul(dt, x, w, n))), (dt, n, k, m)
+        finally:
+            q.close()
+
+
 def test_batch_invariance():
     # qmm_batch, candle-core/tests/quantized_tests.rs:221-256
     n, k = 256, 512
