@@ -9,9 +9,21 @@
 
 namespace moe {
 
+// Maximum over the wave, in every lane: four rotations inside the rows of 16 lanes (DPP: no LDS traffic, no address
+// arithmetic), one exchange between neighbouring rows, and the two halves' values read back as scalars.
 __device__ inline float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+#define MOE_ROR_MAX(n) v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + (n), 0xf, 0xf, false)))
+    MOE_ROR_MAX(8); MOE_ROR_MAX(4); MOE_ROR_MAX(2); MOE_ROR_MAX(1);
+#undef MOE_ROR_MAX
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401f)));   // lane ^ 16
+    const float lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    return fmaxf(lo, hi);
+}
+// v + (lane ^ 1's v) + (lane ^ 2's) + (lane ^ 3's): the sum over a quad, in each of its lanes
+__device__ inline int quad_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false);   // quad_perm [1, 0, 3, 2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
     return v;
 }
 
@@ -46,14 +58,12 @@ __device__ inline void quantize_q8k_block(float4 v, int lane, int8_t* qs_block, 
     uint32_t packed = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        float r = roundf(iscale * e[i]);
-        int q = sat_i8(fminf(r, 127.f));
+        int q = round_min127_as_i8(iscale * e[i]);
         sum += q;
         packed |= (uint32_t)(uint8_t)q << (8 * i);
     }
     *reinterpret_cast<uint32_t*>(qs_block + q8k_act_offset(4 * lane)) = packed;
-    sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
+    sum = quad_sum(sum);
     if ((lane & 3) == 0) bs_out[lane >> 2] = __int2half_rn(sum);
     if (lane == 0) *d_out = 1.0f / iscale;
 }
@@ -92,13 +102,11 @@ __device__ inline void quantize_q8k_blocks(const float4 (&v)[N], const bool (&va
         uint32_t packed = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float r = roundf(iscale[n] * e[i]);
-            const int q = sat_i8(fminf(r, 127.f));
+            const int q = round_min127_as_i8(iscale[n] * e[i]);
             sum += q;
             packed |= (uint32_t)(uint8_t)q << (8 * i);
         }
-        sum += __shfl_xor(sum, 1, 64);
-        sum += __shfl_xor(sum, 2, 64);
+        sum = quad_sum(sum);
         if (valid[n]) {
             *reinterpret_cast<uint32_t*>(qs_block[n] + q8k_act_offset(4 * lane)) = packed;
             if ((lane & 3) == 0) bs_out[n][lane >> 2] = __int2half_rn(sum);
@@ -125,7 +133,7 @@ __device__ inline void quantize_q8_0_block(int vdt, float x, int lane, int8_t* q
     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
     float d = amax / 127.0f;
     float id = (d != 0.f) ? 1.0f / d : 0.f;
-    int q = sat_i8(roundf(x * id));
+    int q = round_as_i8(x * id);
     *q_out = (int8_t)q;
     int sum = q;
 #pragma unroll

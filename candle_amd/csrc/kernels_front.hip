@@ -479,7 +479,7 @@ __device__ inline void quantize_chunk(const FrontParams& p, int64_t t, int H, in
         int sum = 0;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            int qv = sat_i8(roundf(e[j] * id));
+            int qv = round_as_i8(e[j] * id);
             sum += qv;
             packed |= (uint32_t)(uint8_t)qv << (8 * j);
         }

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(Q32_THREADS) void q32_up_kernel(ExpertParams p) {
             for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
             float d = amax / 127.0f;
             float id = (d != 0.f) ? 1.0f / d : 0.f;
-            int q0 = sat_i8(roundf(h0 * id)), q1 = sat_i8(roundf(h1 * id));
+            int q0 = round_as_i8(h0 * id), q1 = round_as_i8(h1 * id);
             int sum = q0 + q1;
 #pragma unroll
             for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
@@ -571,7 +571,7 @@ __global__ __launch_bounds__(Q32_THREADS) __attribute__((amdgpu_waves_per_eu(WPE
             for (int o = 8; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
             float d = amax / 127.0f;
             float id = (d != 0.f) ? 1.0f / d : 0.f;
-            int q0 = sat_i8(roundf(h0 * id)), q1 = sat_i8(roundf(h1 * id));
+            int q0 = round_as_i8(h0 * id), q1 = round_as_i8(h1 * id);
             int sum = q0 + q1;
 #pragma unroll
             for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
@@ -879,7 +879,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
             for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
             const float d = amax / 127.0f;
             const float id = (d != 0.f) ? 1.0f / d : 0.f;
-            const int q = sat_i8(roundf(x * id));
+            const int q = round_as_i8(x * id);
             int sum = q;
 #pragma unroll
             for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
@@ -1027,7 +1027,7 @@ __global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int
             for (int j = 0; j < 8; j++) {
                 d[j] = amax[j] / 127.0f;
                 const float id = (d[j] != 0.f) ? 1.0f / d[j] : 0.f;
-                q[j] = sat_i8(roundf(xv[j] * id));
+                q[j] = round_as_i8(xv[j] * id);
                 sum[j] = q[j];
             }
 #pragma unroll

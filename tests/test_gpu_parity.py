@@ -93,6 +93,14 @@ def test_activation_quantiser_bit_exact(vdt):
     x[7, ::2] = 0.5                 # exact .5 ties after scaling
     x[8, :32] = 3.0                 # block sum 32 * 127 = 4064 is not representable in f16 (Q8_1's s rounds it)
     x[9] *= 1e-7                    # Q8_1: s = f16(sum) * d falls among the f16 subnormals
+    # scale 1 (the largest magnitude is 128 for Q8K, 127 for Q8_0 / Q8_1): every product is the value itself; halves
+    # and their float neighbours on both sides, positive and negative (round() is half away from zero)
+    big = 128.0 if vdt == O.Q8K else 127.0
+    halves = (np.arange(k) % 120).astype(np.float32) + 0.5
+    for row, vals in ((10, halves), (11, -halves), (12, np.nextafter(halves, np.float32(0))), (13, np.nextafter(halves, np.float32(200))),
+                      (14, -np.nextafter(halves, np.float32(0))), (15, -np.nextafter(halves, np.float32(200)))):
+        x[row] = vals
+        x[row, ::32] = -big         # the first element of every block sets the scale (and, for Q8K, the sign)
     got = candle_amd.quantize_act(vdt, x)
     want = O.quantize(vdt, x)
     assert np.array_equal(got, want)
