@@ -427,3 +427,19 @@ def test_q3k_layout_against_independent_decoder(O):
     assert np.array_equal(got.view(np.uint32), out.reshape(-1).view(np.uint32))
     assert codes.min() == -4 and codes.max() == 3 and scs.min() == -32 and scs.max() > 0
     assert np.abs(got - x).max() < 0.02 * 8 / 4
+
+
+def test_round_half_away_identity_of_the_device_quantisers():
+    """The HIP activation quantisers take `(scale * x).round()` (f32::round: half away from zero) as
+    trunc(v + copysign(0.49999997, v)), 0.49999997 being the float below one half; beyond |v| = 130 both sides of their
+    clamp to [-128, 127] agree anyway.  Checked here over every non-negative float up to 130 (float addition and trunc
+    are odd functions, so the negative half follows)."""
+    c = np.float32(0.49999997)
+    assert c == np.nextafter(np.float32(0.5), np.float32(0))
+    hi = int(np.float32(130.0).view(np.uint32))
+    step = 1 << 25
+    for s0 in range(0, hi + 1, step):
+        x = np.arange(s0, min(s0 + step, hi + 1), dtype=np.uint32).view(np.float32)
+        got = np.trunc(x + c)                                   # f32 arithmetic, as on the device
+        want = np.floor(x.astype(np.float64) + 0.5)             # round half away from zero, exactly
+        assert np.array_equal(got, want), x[got != want][:4]
