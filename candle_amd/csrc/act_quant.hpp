@@ -9,6 +9,22 @@
 
 namespace moe {
 
+// `v.round() as i8` of the activation quantisers (f32::round: half away from zero; `as i8`: saturating, NaN -> 0) in five
+// instructions.  For every float with |v| <= 130, trunc(v + copysign(0.49999997, v)) == v.round() (0.49999997 is the
+// float below one half; checked over all 2.2e9 such floats), beyond that both sides of the clamp agree anyway, and the
+// conversion instruction truncates toward zero, saturates and turns NaN into 0.
+__device__ inline int round_as_i8(float v) {
+    const int q = __float2int_rz(v + copysignf(0.49999997f, v));
+    return min(max(q, -128), 127);
+}
+// `v.round().min(127.) as i8` (BlockQ8K::from_float, k_quants.rs:1843-1844): f32::min returns the other operand for a
+// NaN, so a NaN becomes 127.
+__device__ inline int round_min127_as_i8(float v) {
+    const int q = __float2int_rz(fminf(v + copysignf(0.49999997f, v), 127.0f));
+    return max(q, -128);
+}
+
+
 // Maximum over the wave, in every lane: four rotations inside the rows of 16 lanes (DPP: no LDS traffic, no address
 // arithmetic), one exchange between neighbouring rows, and the two halves' values read back as scalars.
 __device__ inline float wave_max(float v) {
