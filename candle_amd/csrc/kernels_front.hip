@@ -27,15 +27,28 @@ constexpr int FRONT_THREADS = 256;
 constexpr int MAX_E = 256;
 constexpr int MAX_K = 16;
 
+// Sum over the wave by the butterfly lane ^ 32, ^ 16, ^ 8, ^ 4, ^ 2, ^ 1 (every lane ends with the same bits).  The last
+// four steps run as rotations inside the rows of 16 lanes (DPP, no LDS traffic): after the steps before it the lanes of
+// one residue class hold the same value, and lane i + o (mod 16) lies in the class of lane i ^ o, so a rotation by o adds
+// the same number as the exchange would.
+#define MOE_ROW_ROR(v, n) __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + (n), 0xf, 0xf, false))
 __device__ inline float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    v += __shfl_xor(v, 32, 64);
+    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401f));   // lane ^ 16
+    v += MOE_ROW_ROR(v, 8);
+    v += MOE_ROW_ROR(v, 4);
+    v += MOE_ROW_ROR(v, 2);
+    v += MOE_ROW_ROR(v, 1);
     return v;
 }
 
 __device__ inline float wave_max_f(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401f)));
+    v = fmaxf(v, MOE_ROW_ROR(v, 8));
+    v = fmaxf(v, MOE_ROW_ROR(v, 4));
+    v = fmaxf(v, MOE_ROW_ROR(v, 2));
+    v = fmaxf(v, MOE_ROW_ROR(v, 1));
     return v;
 }
 
@@ -716,11 +729,8 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
                     acc0 = __builtin_fmaf(wa[i].w, xr[4 * i + 3], acc0); acc1 = __builtin_fmaf(wb[i].w, xr[4 * i + 3], acc1);
                 }
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                acc0 += __shfl_xor(acc0, o, 64);
-                acc1 += __shfl_xor(acc1, o, 64);
-            }
+            acc0 = wave_sum(acc0);
+            acc1 = wave_sum(acc1);
             if (lane == 0) {
                 if (e0 < E) {
                     if (p.gate_bias) acc0 += p.gate_bias[e0];
