@@ -616,9 +616,13 @@ __device__ inline float ordered_sum_of_squares(const float* xr, int tid, bool se
     return result;
 }
 
-template <int VDT, int NCH, bool LEAN>
+// WIDE (layers with dozens of experts, small batches): all eight waves take gate products, after sharing out the
+// quantisation -- a token's gate rows are a megabyte at 128 experts, and a workgroup that requests two rows per wave at a
+// time from four waves spends its time waiting for them (one token, 128 experts of 2048: 28 us).
+template <int VDT, int NCH, bool LEAN, bool WIDE = false>
 __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
-    __shared__ float logit_lds[64];
+    __shared__ float logit_lds[MAX_E];
+    __shared__ int sel_lds[MAX_K];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t t = blockIdx.x;
@@ -637,7 +641,7 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     const int n_dot = E + (p.shared_gate ? 1 : 0);
     float4 wa[NCH], wb[NCH];
     auto load_gate_pair = [&](int e0) {
-        const int e1 = e0 + 4 < n_dot ? e0 + 4 : e0;
+        const int e1 = e0 + (WIDE ? 8 : 4) < n_dot ? e0 + (WIDE ? 8 : 4) : e0;
         const float* w0 = (e0 < E) ? p.gate + (int64_t)e0 * H : p.shared_gate;
         const float* w1 = (e1 < E) ? p.gate + (int64_t)e1 * H : p.shared_gate;
 #pragma unroll
@@ -649,7 +653,7 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     // (only with an rms-norm ahead: without one the early request measured 0.9 us slower on a gate that is still in the
     // L2; and not for rows beyond 4096, where two gate rows and the token's row exceed the registers)
     const bool early_gate = !LEAN && NCH <= 16 && p.rms_alpha != nullptr;
-    if (early_gate && wave < 4 && wave < n_dot) load_gate_pair(wave);
+    if (early_gate && wave < (WIDE ? 8 : 4) && wave < n_dot) load_gate_pair(wave);
     if (!LEAN && p.rms_alpha) {
         // rms_norm (candle-nn/src/ops.rs:504-515) sums the squares left to right in f32.  A different
         // order changes the divisor in the last ulp, which flips quantised activations now and then
@@ -676,7 +680,8 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     // rows of 4096 and more leave no registers for a second buffer (and few experts per wave to run ahead over)
     // gate products: waves 0..3 while waves 4..7 quantise (all eight waves on the products with the quantisation shared
     // out afterwards measured no better at 61 products per token and worse at 8)
-    constexpr int GW = 4;
+    static_assert(!(LEAN && WIDE), "one or the other");
+    constexpr int GW = WIDE ? 8 : 4;
     constexpr bool LEAN_PIPE = NCH < 16;
     constexpr int LEAN_PIECE = LEAN_PIPE ? 2 : 4, LEAN_NP = LEAN ? NCH / LEAN_PIECE : 2;
     static_assert(!LEAN || (NCH % LEAN_PIECE == 0 && LEAN_NP % 2 == 0), "the pieces alternate between two buffers");
@@ -691,6 +696,14 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
             qb[buf][j] = *reinterpret_cast<const float4*>(w1 + (pc * LEAN_PIECE + j) * 256 + lane * 4);
         }
     };
+    if constexpr (WIDE) {   // every wave quantises its share of the row (chunks wave, wave + 8, ...), then joins the products
+#pragma unroll
+        for (int i = 0; i < NCH; i++)
+            if ((i & 7) == wave) {
+                const float e4[4] = {xr[4 * i], xr[4 * i + 1], xr[4 * i + 2], xr[4 * i + 3]};
+                quantize_chunk<VDT>(p, t, H, i, e4, lane);
+            }
+    }
     if (wave < GW) {
         // gate products
         if (LEAN && LEAN_PIPE && wave < n_dot) load_piece(wave, 0, 0);
@@ -751,27 +764,35 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
             }
         }
     }
-    if (wave >= GW) {
-        // quantise: wave 4+q owns chunks q, q+4, ...; the branches are wave-uniform
-        const int q = wave - GW;
+    if constexpr (!WIDE) {
+        if (wave >= GW) {
+            // quantise: wave 4+q owns chunks q, q+4, ...; the branches are wave-uniform
+            const int q = wave - GW;
 #pragma unroll
-        for (int i = 0; i < NCH; i++)
-            if ((i & 3) == q) {
-                const float e4[4] = {xr[4 * i], xr[4 * i + 1], xr[4 * i + 2], xr[4 * i + 3]};
-                quantize_chunk<VDT>(p, t, H, i, e4, lane);
-            }
+            for (int i = 0; i < NCH; i++)
+                if ((i & 3) == q) {
+                    const float e4[4] = {xr[4 * i], xr[4 * i + 1], xr[4 * i + 2], xr[4 * i + 3]};
+                    quantize_chunk<VDT>(p, t, H, i, e4, lane);
+                }
+        }
     }
     __syncthreads();
     // every wave read the row of x at the start (the output may be the input buffer): clear the token's output row if
     // the down kernels are to accumulate into it
     if (p.y_zero)
         for (int i = tid; i < H / 4; i += FAST_THREADS) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (wave == 0) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk,
-                                        p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+    if (wave == 0) {
+        if (E <= 64) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+        else route_one_token_wave_lds(logit_lds, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds);
+    }
 }
 template <int VDT, int NCH>
 __global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel(FrontParams p) {
     front_fast_body<VDT, NCH, false>(p);
+}
+template <int VDT, int NCH>
+__global__ __launch_bounds__(FAST_THREADS) void front_fast_kernel_wide(FrontParams p) {
+    front_fast_body<VDT, NCH, false, true>(p);
 }
 // The same for large batches: at most 128 registers, so that two workgroups share a CU (a batch of thousands of tokens
 // is bound by how many of these latency chains run at once, a decode batch by the length of one).
@@ -947,7 +968,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs
 // ---------------------------------------------------------------------------------------------
 template <int VDT>
 static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
-    if (p.E > 64 || p.H % 256) return false;
+    if (p.E > MAX_E || p.H % 256) return false;
     dim3 grid((unsigned)p.T), block(FAST_THREADS);
     switch (p.H / 256) {
         case 1: hipLaunchKernelGGL((front_fast_kernel<VDT, 1>), grid, block, 0, s, p); return true;
@@ -955,11 +976,13 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
         case 4: hipLaunchKernelGGL((front_fast_kernel<VDT, 4>), grid, block, 0, s, p); return true;
         case 8:
             if (p.T >= 256 && !p.rms_alpha) hipLaunchKernelGGL((front_fast_kernel_dense<VDT, 8>), grid, block, 0, s, p);
+            else if (p.E > 32) hipLaunchKernelGGL((front_fast_kernel_wide<VDT, 8>), grid, block, 0, s, p);
             else hipLaunchKernelGGL((front_fast_kernel<VDT, 8>), grid, block, 0, s, p);
             return true;
         case 12: hipLaunchKernelGGL((front_fast_kernel<VDT, 12>), grid, block, 0, s, p); return true;
         case 16:
             if (p.T >= 1024 && !p.rms_alpha) hipLaunchKernelGGL((front_fast_kernel_dense<VDT, 16>), grid, block, 0, s, p);
+            else if (p.E > 32) hipLaunchKernelGGL((front_fast_kernel_wide<VDT, 16>), grid, block, 0, s, p);
             else hipLaunchKernelGGL((front_fast_kernel<VDT, 16>), grid, block, 0, s, p);
             return true;
         case 20: hipLaunchKernelGGL((front_fast_kernel<VDT, 20>), grid, block, 0, s, p); return true;

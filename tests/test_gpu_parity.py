@@ -451,6 +451,17 @@ def test_block_more_than_64_experts(E, k):
     gpu.close()
 
 
+@pytest.mark.parametrize("H,E,k,shared,rms", [(2048, 128, 8, 0, False), (2048, 61, 4, 512, False), (4096, 40, 2, 0, False), (2048, 130, 6, 0, True)])
+def test_block_dozens_of_experts_at_small_batches(H, E, k, shared, rms):
+    # more than 32 experts and rows of 2048 or 4096: all eight waves of the front kernel take gate products (the quantisation
+    # of the row is shared out first); with and without the always-on expert's gate row and the pre-norm; 300 tokens take
+    # the large-batch variant of the kernel
+    ref, gpu = make_pair(H, 256, E, k, O.Q4K, seed=60 + E, Fs=shared, rms=rms)
+    for T in (1, 5, 33, 300):
+        check_block(ref, gpu, T, tol=block_tol(O.Q4K, 256))
+    gpu.close()
+
+
 def test_block_rms_residual_chain():
     ref, gpu = make_pair(512, 512, 4, 2, O.Q4K, seed=5, rms=True)
     xs = activations(6, 512, 9)
