@@ -461,14 +461,6 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     // (w2 may be Q4K, Q5K or Q6K whatever w1 / w3 are: mixed files store part of it as Q6K)
     pl.tiled = !sw.no_gemm && q4k_gemm_up_format(L->dt) && L->F % 64 == 0 && L->H % 128 == 0 && T * L->k > 34 * L->E;
     pl.tiled_down = pl.tiled && q4k_gemm_down_format(L->dt_down) && T * L->k > 64 * L->E;
-    // small batches: slots are numbered t*k + r and no dispatch pass runs
-    pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS;
-    pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 72 * L->E ? 128 : 64;
-    // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
-    // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
-    // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches
-    // served without a dispatch pass only: a prefill's tens of millions of atomic adds cost more than its combine pass.
-    pl.accumulate = pl.direct && L->k == 2 && !shared && !L->has_rms && !sw.combine_pass;
     // 16-slot tiles a workgroup carries per pass over the weights, from the expected rows per expert
     // (a list longer than a pass covers is finished by further workgroups that stream the weights again)
     // (measured at the Mixtral shape: two tiles per pass, with a second pass for the longer lists, beat four
@@ -480,6 +472,18 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     const int64_t two_from = (L->vdt == MOE_GGML_Q8K ? 13 : 9) * L->E;
     pl.slot_tiles = (T * L->k > 34 * L->E) ? 4 : (T * L->k > two_from) ? 2 : 1;
     if (sw.slot_tiles) pl.slot_tiles = sw.slot_tiles;
+    // small batches: slots are numbered t*k + r and no dispatch pass runs; every workgroup then finds its expert's slots
+    // by scanning the assignments, and the grid holds a pass for every 16 * slot_tiles tokens there could be in a list.
+    // With many experts most of those passes are empty: beyond four of them the dispatch pass is worth its 5 us (its
+    // lists let an empty pass leave at once; 128 experts, 512 tokens: 386 -> 303 us).
+    const int64_t passes = (T + 16 * pl.slot_tiles - 1) / (16 * pl.slot_tiles);
+    pl.direct = !pl.tiled && T * L->k <= DIRECT_MAX_SLOTS && T <= DIRECT_MAX_SLOTS && (passes <= 4 || L->E <= 16);
+    pl.tile_slots = sw.tile_slots == 64 || sw.tile_slots == 128 ? sw.tile_slots : T * L->k >= 72 * L->E ? 128 : 64;
+    // Top-2 routing with nothing else to add to a token's result (no shared expert, no residual): the streaming down
+    // kernels add their two terms per token straight into the output, which the front kernel clears, and no combine
+    // pass runs (a + b is the same float in either order; with three or more terms the order would matter).  Batches
+    // served without a dispatch pass only: a prefill's tens of millions of atomic adds cost more than its combine pass.
+    pl.accumulate = pl.direct && L->k == 2 && !shared && !L->has_rms && !sw.combine_pass;
     // very small K-quant batches: at most half of the experts can be active, so the weights are cut
     // into four times as many workgroups; those write f32 h and a small pass quantises it
     pl.narrow = pl.direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && pl.slot_tiles == 1 &&

@@ -585,6 +585,12 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
         tp[RTW + j] = gw.w3 + (size_t)(rt0 + j) * FMT::TILE_BYTES;
     }
     const size_t sb_stride = (size_t)(F / 16) * FMT::TILE_BYTES;
+    // The grid's passes cover the longest list there could be; with many experts most of them find nothing.  A later pass
+    // over a list that the dispatch kernel has measured looks at its length before it requests anything.
+    if (blockIdx.z > 0 && !p.rb.direct && !p.is_shared) {
+        const int gi = p.group0 + grp;
+        if ((int)blockIdx.z * (TT * 16) >= p.rb.offsets[gi + 1] - p.rb.offsets[gi]) return;
+    }
     // first weight tiles go out before anything else; an expert without tokens wastes them
     typename FMT::Tile ring[RING];
     q4k_engine_prefetch<FMT, NT, RING>(tp, sb_stride, 0, nsb - 1, lane, ring);
@@ -684,6 +690,10 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
         for (int j = 0; j < NTD; j++) tp[j] += (size_t)a_off * sb_stride;
         sb_stride *= NW;
         sb_lo = 0; sb_hi = mine;
+    }
+    if (blockIdx.z > 0 && !p.rb.direct && !p.is_shared) {   // (a later pass: see the up kernel)
+        const int gi = p.group0 + grp;
+        if ((int)blockIdx.z * (TT * 16) >= p.rb.offsets[gi + 1] - p.rb.offsets[gi]) return;
     }
     typename FMT::Tile ring[RING];
     if (ILV) q4k_engine_prefetch<FMT, NTD, RING>(tp, sb_stride, 0, sb_hi > 0 ? sb_hi - 1 : 0, lane, ring);
