@@ -270,11 +270,13 @@ struct Workspace {
     ActBuf xq, hq, hq_shared;
     float* yw = nullptr;
     float* hbuf = nullptr;
+    float* ab_shared = nullptr;   // [2][T][Fs]: silu(w1 x) and w3 x of the always-on expert at a few tokens
 };
 
 // Which kernels a forward of T tokens takes.
 struct ForwardPlan {
     bool tiled = false, tiled_down = false, tiled32 = false, direct = false, accumulate = false, narrow = false, hbuf = false;
+    bool shared_rows = false;   // the always-on expert as two dense few-row products
     int tile_slots = 128, slot_tiles = 1;
 };
 
@@ -489,6 +491,17 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
     pl.narrow = pl.direct && L->vdt == MOE_GGML_Q8K && L->F % 64 == 0 && L->H % 32 == 0 && pl.slot_tiles == 1 &&
                 (sw.narrow >= 0 ? sw.narrow > 0 : T * L->k <= L->E);
     pl.hbuf = pl.tiled || pl.narrow;
+    // The always-on expert of a few tokens: its regular up launch has Fs / 256 (K-quants) or Fs / 128 workgroups, a
+    // handful for a matrix of megabytes, and it is the step's critical path then.  The dense few-row kernels split K over
+    // the waves of a workgroup per 16 rows instead (hundreds of workgroups): one launch for w1 and w3, one for w2.
+    if (shared && sw.fused_rows != 1) {
+        const bool kq = L->vdt == MOE_GGML_Q8K;
+        const bool can = kq ? qlinear_fused_usable(L->dt, T, L->Fs, L->H) && qlinear_fused_usable(L->dt_down, T, L->H, L->Fs)
+                            : q32_rows_fused_usable(L->dt, T, L->Fs, L->H) && q32_rows_fused_usable(L->dt_down, T, L->H, L->Fs);
+        // (measured, step with / without: Qwen-MoE shape Q8_0, Fs = 5632: 73 / 94 us at one token, 88 / 100 at two, 103 / 107
+        // at three, 115 / 112 at four; 64 Q4_K experts top-6 with Fs = 3072: 63 / 70, 65 / 75, 67 / 76, 70 / 81)
+        pl.shared_rows = can && (sw.fused_rows == 2 || T <= (kq ? 4 : 3));
+    }
     // Q8_0 / Q4_0 / Q5_0 layers whose slots are grouped by expert (more than DIRECT_MAX_SLOTS assignments): the tiled
     // kernels of kernels_q32.hip read an expert's weights once for up to 64 of its slots
     pl.tiled32 = !sw.no_gemm && !pl.direct && q8_0_gemm_usable(L->dt, L->dt_down, L->H, L->F) && T * L->k > 20 * L->E;
@@ -509,6 +522,7 @@ static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& 
     if (shared) w.hq_shared = c.take_act(L->vdt, T, L->Fs);
     w.yw = c.take<float>((size_t)S * L->H * 4);
     if (pl.hbuf) w.hbuf = c.take<float>((size_t)T * L->k * L->F * 4);
+    if (pl.shared_rows) w.ab_shared = c.take<float>((size_t)2 * T * L->Fs * 4);
     if (ws) *ws = w;
     return c.off;
 }
@@ -568,6 +582,20 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
     // (the timed entry keeps one stream: its stage marks would mean nothing otherwise).
     hipStream_t ss = overlap_shared ? L->side : s;
     auto run_shared = [&]() -> int {
+        if (pl.shared_rows) {
+            const GroupWeights& g = L->host_groups[L->E];
+            const bool kq = L->vdt == MOE_GGML_Q8K;
+            FusedRows up;
+            up.xq = fp.xq; up.m = T; up.n = L->Fs; up.k = L->H;
+            up.w = g.w1; up.y = ws.ab_shared; up.silu_y = 1;
+            up.w_b = g.w3; up.y_b = ws.ab_shared + T * L->Fs;
+            MOE_HIP_CHECK(kq ? launch_qlinear_fused(L->dt, up, ss) : launch_q32_rows_fused(L->dt, up, ss));
+            FusedRows down;   // quantises silu(w1 x) * (w3 x) as the up kernels' epilogues do, scales by the expert's gate
+            down.x = up.y; down.x2 = up.y_b; down.m = T; down.n = L->H; down.k = L->Fs;
+            down.w = g.w2; down.y = ws.yw + T * L->k * L->H; down.row_scale = fp.rb.shared_w;
+            MOE_HIP_CHECK(kq ? launch_qlinear_fused(L->dt_down, down, ss) : launch_q32_rows_fused(L->dt_down, down, ss));
+            return MOE_OK;
+        }
         ExpertParams sp = ep;
         // the always-on expert takes the regular kernels (which quantise its intermediate in their epilogue) also when
         // the routed experts of a tiny batch took the narrow ones with their separate quantisation pass
@@ -998,14 +1026,18 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     // 10.7 / 14.5; 32000 x 4096: 21.2 / 19.5).  fused_rows: 1 = never, 2 = whenever the kernel can (test aid).
     const int fr = switches().fused_rows;
     if (fr != 1 && qlinear_fused_usable(Q->dt, m, Q->n, Q->k) && (fr == 2 || (m <= 2 && Q->n <= 16384))) {
-        MOE_HIP_CHECK(launch_qlinear_fused(Q->dt, d_x, m, Q->n, Q->k, Q->weights.as<uint8_t>(), d_y, s));
+        FusedRows f;
+        f.x = d_x; f.m = m; f.n = Q->n; f.k = Q->k; f.w = Q->weights.as<uint8_t>(); f.y = d_y;
+        MOE_HIP_CHECK(launch_qlinear_fused(Q->dt, f, s));
         return MOE_OK;
     }
     // the 32-element formats: the same, with the block values added in the reference's order by one wave (in a graph,
     // Q8_0, fused / two passes: 4096 x 4096: 9.3 / 22.1 us at one row, 13.6 / 22.4 at two, 21.4 / 22.8 at four; 4096 x 14336:
     // 27.6 / 57.0 at one row; 8192 x 4096: 11.4 / 22.7; 32000 x 4096: 33.1 / 30.3)
     if (fr != 1 && q32_rows_fused_usable(Q->dt, m, Q->n, Q->k) && (fr == 2 || (m <= 3 && Q->n <= 16384))) {
-        MOE_HIP_CHECK(launch_q32_rows_fused(Q->dt, d_x, m, Q->n, Q->k, Q->weights.as<uint8_t>(), d_y, s));
+        FusedRows f;
+        f.x = d_x; f.m = m; f.n = Q->n; f.k = Q->k; f.w = Q->weights.as<uint8_t>(); f.y = d_y;
+        MOE_HIP_CHECK(launch_q32_rows_fused(Q->dt, f, s));
         return MOE_OK;
     }
     // under stream capture nothing may be allocated, the graph carries its own copy of the routing table pass, and the

@@ -133,12 +133,25 @@ hipError_t launch_expert_down(const ExpertParams& p, hipStream_t s);
 // caller re-quantises it), down writes yw.
 bool q4k_gemm_up_format(int dt);
 bool q4k_gemm_down_format(int dt);
-// Dense K-quant matrix [n, k] (device layout) times m <= 4 rows of f32 in one launch (the rows are quantised in the kernel).
+// Dense matrix [n, k] (device layout) times m <= 4 rows of f32 in one launch (the rows are quantised in the kernel).
+struct FusedRows {
+    const float* x = nullptr;          // [m, k] rows ...
+    const float* x2 = nullptr;         // ... optionally times the rows x2 (the two halves of a SwiGLU intermediate in f32)
+    ActBuf xq;                         // x == nullptr: the rows, already quantised to the matrix format's activation type
+    int64_t m = 0, n = 0, k = 0;
+    const uint8_t* w = nullptr;        // the matrix
+    float* y = nullptr;                // [m, n]
+    const uint8_t* w_b = nullptr;      // optional second matrix of the same shape against the same rows ...
+    float* y_b = nullptr;              // ... and its output
+    const float* row_scale = nullptr;  // optional: row r of y is multiplied by row_scale[r]
+    int silu_y = 0;                    // y = silu(w x) (y_b stays w_b x)
+};
+// K-quant matrices:
 bool qlinear_fused_usable(int dt, int64_t m, int64_t n, int64_t k);
-// The same for the 32-element formats (super-tile layout): bit-identical to the streaming kernel's results.
+hipError_t launch_qlinear_fused(int dt, const FusedRows& f, hipStream_t s);
+// The 32-element formats (super-tile layout): bit-identical to the streaming kernel's results.
 bool q32_rows_fused_usable(int dt, int64_t m, int64_t n, int64_t k);
-hipError_t launch_q32_rows_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s);
-hipError_t launch_qlinear_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s);
+hipError_t launch_q32_rows_fused(int dt, const FusedRows& f, hipStream_t s);
 hipError_t launch_q4k_gemm_up(const ExpertParams& p, hipStream_t s);
 hipError_t launch_q4k_gemm_down(const ExpertParams& p, hipStream_t s);
 

@@ -964,9 +964,13 @@ constexpr int GV_STEPS = 4;                     // K steps (of four blocks) a wa
 constexpr int GV_BLOCKS = 4 * GV_STEPS;         // blocks per wave and chunk
 constexpr int GV_CHUNK = 4 * GV_BLOCKS;         // blocks per workgroup and chunk
 
-template <int DT>
-__global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int m, int n, int K, const uint8_t* w, float* y) {
+template <int DT, bool QUANTISED>
+__global__ __launch_bounds__(256) void q32_rows_fused_kernel(FusedRows f) {
     typedef Q32Fmt<DT> F;
+    const float* x = f.x;
+    const int m = (int)f.m, n = (int)f.n, K = (int)f.k;
+    const uint8_t* w = blockIdx.y ? f.w_b : f.w;
+    float* y = blockIdx.y ? f.y_b : f.y;
     constexpr size_t STB = Q32SFmt<DT>::STB;
     constexpr int VDT = F::HAS_M ? MOE_GGML_Q8_1 : MOE_GGML_Q8_0;
     __shared__ float terms[2][GV_CHUNK][4][16];                       // [buffer][block of the chunk][row of x][weight row]
@@ -993,15 +997,58 @@ __global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int
         }
     };
     request(0);
+    auto fetch = [&](uint32_t off) {
+        float a = ldg<float>(x, off);
+        if (f.x2) a *= ldg<float>(f.x2, off);
+        return a;
+    };
     float xnext[8];
+    // rows that arrive quantised: per row and chunk a lane copies 8 quants of the wave's 512, lanes 0..15 a block's scale
+    // and word; requested a chunk ahead like the weights
+    uint2 qnext[GV_MAX_ROWS];
+    float dnext[GV_MAX_ROWS];
+    int wnext[GV_MAX_ROWS];
+    auto request_rows = [&](int ks0) {
+        const int e = ks0 * 128 + lane * 8;
+        const int b = ks0 * 4 + (lane & 15);
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const int e = wave * GV_STEPS * 128 + j * 64 + lane;
-        xnext[j] = ldg<float>(x, (uint32_t)(e < K ? e : K - 1) * 4u);
+        for (int row = 0; row < GV_MAX_ROWS; row++) {
+            const size_t rr = (size_t)(row < m ? row : m - 1);
+            qnext[row] = *reinterpret_cast<const uint2*>(f.xq.qs + rr * K + (e < K ? e : K - 8));
+            dnext[row] = f.xq.d[rr * nkb + (b < nkb ? b : nkb - 1)];
+            wnext[row] = static_cast<const int32_t*>(f.xq.bsum)[rr * nkb + (b < nkb ? b : nkb - 1)];
+        }
+    };
+    if constexpr (QUANTISED) {
+        request_rows(wave * GV_STEPS);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int e = wave * GV_STEPS * 128 + j * 64 + lane;
+            xnext[j] = fetch((uint32_t)(e < K ? e : K - 1) * 4u);
+        }
     }
     for (int c = 0; c < n_chunks; c++) {
         const int ks0 = c * 4 * GV_STEPS + wave * GV_STEPS;       // this wave's first K step of the chunk
         const int n_steps = nks - ks0 < GV_STEPS ? (nks - ks0 < 0 ? 0 : nks - ks0) : GV_STEPS;
+        if constexpr (QUANTISED) {
+            uint2 qc[GV_MAX_ROWS];
+            float dc[GV_MAX_ROWS];
+            int wc[GV_MAX_ROWS];
+#pragma unroll
+            for (int row = 0; row < GV_MAX_ROWS; row++) { qc[row] = qnext[row]; dc[row] = dnext[row]; wc[row] = wnext[row]; }
+            request_rows(ks0 + 4 * GV_STEPS);
+#pragma unroll
+            for (int row = 0; row < GV_MAX_ROWS; row++) {
+                if (row < m) {   // uniform
+                    *reinterpret_cast<uint2*>(&xq[wave][lane >> 2][row][(lane & 3) * 8]) = qc[row];
+                    if (lane < GV_BLOCKS) {
+                        xd[wave][lane][row] = dc[row];
+                        xw[wave][lane][row] = wc[row];
+                    }
+                }
+            }
+        } else
         // the rows' blocks of these steps: 512 elements per row, lane l holds elements l, l + 64, ... (pair of blocks j)
         for (int row = 0; row < m; row++) {
             float xv[8];
@@ -1013,7 +1060,7 @@ __global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
                     const int e = nks0 * 128 + j * 64 + lane;
-                    xnext[j] = ldg<float>(x, ((uint32_t)nrow * (uint32_t)K + (uint32_t)(e < K ? e : K - 1)) * 4u);
+                    xnext[j] = fetch(((uint32_t)nrow * (uint32_t)K + (uint32_t)(e < K ? e : K - 1)) * 4u);
                 }
             }
             float amax[8];
@@ -1086,22 +1133,31 @@ __global__ __launch_bounds__(256) void q32_rows_fused_kernel(const float* x, int
             for (int b = 0; b < nb; b++) acc += terms[buf][b][g][r];
         }
     }
-    if (wave == 0 && g < m) y[(size_t)g * n + (size_t)rt * 16 + r] = acc;
+    if (wave == 0 && g < m) {
+        if (f.row_scale) acc *= f.row_scale[g];
+        if (f.silu_y && blockIdx.y == 0) acc = silu_ref32(acc);
+        y[(size_t)g * n + (size_t)rt * 16 + r] = acc;
+    }
 }
 
 bool q32_rows_fused_usable(int dt, int64_t m, int64_t n, int64_t k) {
     const bool fmt = dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_1;
     return fmt && m >= 1 && m <= GV_MAX_ROWS && n % 16 == 0 && q32_super_layout(k) && k >= 128 && m * k < ((int64_t)1 << 29);
 }
-hipError_t launch_q32_rows_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s) {
-    if (!q32_rows_fused_usable(dt, m, n, k)) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)(n / 16)), block(256);
+template <int DT>
+static void launch_q32_rows_fused_t(const FusedRows& f, hipStream_t s) {
+    const dim3 grid((unsigned)(f.n / 16), f.w_b ? 2u : 1u), block(256);
+    if (f.x) hipLaunchKernelGGL((q32_rows_fused_kernel<DT, false>), grid, block, 0, s, f);
+    else hipLaunchKernelGGL((q32_rows_fused_kernel<DT, true>), grid, block, 0, s, f);
+}
+hipError_t launch_q32_rows_fused(int dt, const FusedRows& f, hipStream_t s) {
+    if (!q32_rows_fused_usable(dt, f.m, f.n, f.k) || !(f.x || f.xq.qs) || !f.w || !f.y || (f.w_b && !f.y_b)) return hipErrorInvalidValue;
     switch (dt) {
-        case MOE_GGML_Q8_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q8_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
-        case MOE_GGML_Q4_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q4_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
-        case MOE_GGML_Q5_0: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q5_0>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
-        case MOE_GGML_Q4_1: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q4_1>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
-        case MOE_GGML_Q5_1: hipLaunchKernelGGL((q32_rows_fused_kernel<MOE_GGML_Q5_1>), grid, block, 0, s, x, (int)m, (int)n, (int)k, w, y); break;
+        case MOE_GGML_Q8_0: launch_q32_rows_fused_t<MOE_GGML_Q8_0>(f, s); break;
+        case MOE_GGML_Q4_0: launch_q32_rows_fused_t<MOE_GGML_Q4_0>(f, s); break;
+        case MOE_GGML_Q5_0: launch_q32_rows_fused_t<MOE_GGML_Q5_0>(f, s); break;
+        case MOE_GGML_Q4_1: launch_q32_rows_fused_t<MOE_GGML_Q4_1>(f, s); break;
+        case MOE_GGML_Q5_1: launch_q32_rows_fused_t<MOE_GGML_Q5_1>(f, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -855,10 +855,13 @@ constexpr size_t FUSED_MAX_LDS = 44 * 1024;   // beside the 16 KiB at most of pa
 __host__ __device__ inline int fused_blocks_per_wave(int K) { return (K / 256 + FUSED_NW - 1) / FUSED_NW; }
 static size_t fused_lds_bytes(int64_t m, int64_t K) { return (size_t)FUSED_NW * (size_t)fused_blocks_per_wave((int)K) * (size_t)m * XQ_BYTES; }
 
-template <class FMT, int NTD>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qlinear_fused_kernel(const float* x, int m, int n, int K,
-                                                                                                         const uint8_t* w, float* y) {
+template <class FMT, int NTD, bool QUANTISED>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qlinear_fused_kernel(FusedRows f) {
     constexpr int NW = FUSED_NW;
+    const float* x = f.x;
+    const int m = (int)f.m, n = (int)f.n, K = (int)f.k;
+    const uint8_t* w = blockIdx.y ? f.w_b : f.w;
+    float* y = blockIdx.y ? f.y_b : f.y;
     constexpr int RING = 4, U = RING / NTD;   // tiles in flight per wave; super-blocks per trip of the loop
     static_assert(RING % NTD == 0, "the ring holds whole super-blocks");
     __shared__ float part[NW][NTD * 4][64];
@@ -889,7 +892,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             ring[q] = FMT::load(tp[q % NTD] + (size_t)it * sb_stride, lane);
         }
         uint8_t* xq = xq_all + (size_t)wave * fused_blocks_per_wave(K) * m * XQ_BYTES;
-        {
+        if constexpr (QUANTISED) {
+            // the wave's blocks of all rows, numbered b = it * m + row, copied from the Q8K rows in memory, four per turn
+            constexpr int NQ = 4;
+            const int n_blk = mine * m;
+            const uint32_t* bsum = static_cast<const uint32_t*>(f.xq.bsum);
+            for (int b0 = 0; b0 < n_blk; b0 += NQ) {
+                uint32_t q[NQ], bs[NQ];
+                float d[NQ];
+#pragma unroll
+                for (int i = 0; i < NQ; i++) {
+                    const int bb = b0 + i < n_blk ? b0 + i : n_blk - 1;
+                    const int it = bb / m, row = bb - it * m;
+                    const size_t blk = (size_t)row * nsb + (size_t)(wave + it * NW);
+                    q[i] = *reinterpret_cast<const uint32_t*>(f.xq.qs + blk * 256 + lane * 4);
+                    bs[i] = bsum[blk * 8 + (lane & 7)];
+                    d[i] = f.xq.d[blk];
+                }
+#pragma unroll
+                for (int i = 0; i < NQ; i++) {
+                    if (b0 + i < n_blk) {   // uniform
+                        uint8_t* blk = xq + (size_t)(b0 + i) * XQ_BYTES;
+                        *reinterpret_cast<uint32_t*>(blk + lane * 4) = q[i];
+                        if (lane < 8) *reinterpret_cast<uint32_t*>(blk + XQ_BSUM + lane * 4) = bs[i];
+                        if (lane == 0) *reinterpret_cast<float*>(blk + XQ_D) = d[i];
+                    }
+                }
+            }
+        } else {
             // the wave's blocks of all rows, numbered b = it * m + row, four at a time side by side (their loads, wave
             // reductions and divisions overlap); 32-bit byte offsets: m * K * 4 < 2^31
             constexpr int NQ = 4;
@@ -899,9 +929,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 const int it = bb / m, row = bb - it * m;
                 return ((uint32_t)row * (uint32_t)K + (uint32_t)((wave + it * NW) * 256 + lane * 4)) * 4u;
             };
+            auto fetch = [&](int b) {
+                const uint32_t off = x_offset(b);
+                float4 a = gload<float4>(x, off);
+                if (f.x2) {
+                    const float4 c = gload<float4>(f.x2, off);
+                    a = make_float4(a.x * c.x, a.y * c.y, a.z * c.z, a.w * c.w);
+                }
+                return a;
+            };
             float4 v[NQ];
 #pragma unroll
-            for (int i = 0; i < NQ; i++) v[i] = gload<float4>(x, x_offset(i));
+            for (int i = 0; i < NQ; i++) v[i] = fetch(i);
             for (int b0 = 0; b0 < n_blk; b0 += NQ) {
                 bool valid[NQ];
                 int8_t* qs_out[NQ];
@@ -918,7 +957,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     cur[i] = v[i];
                 }
 #pragma unroll
-                for (int i = 0; i < NQ; i++) v[i] = gload<float4>(x, x_offset(b0 + NQ + i));
+                for (int i = 0; i < NQ; i++) v[i] = fetch(b0 + NQ + i);
                 quantize_q8k_blocks<NQ>(cur, valid, lane, qs_out, d_out, bs_out);
             }
         }
@@ -972,6 +1011,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int ww = 0; ww < NW; ww++) sum += part[ww][v2][lane];
         const int j = v2 / 4, i = v2 % 4;
         const int row = 4 * g + i;
+        if (f.row_scale && row < m) sum *= f.row_scale[row];
+        if (f.silu_y && blockIdx.y == 0) sum = silu_fast(sum);
         if (row < m && rt0 + j < n_rt) y[(size_t)row * n + (size_t)(rt0 + j) * 16 + r] = sum;
     }
 }
@@ -981,24 +1022,30 @@ bool qlinear_fused_usable(int dt, int64_t m, int64_t n, int64_t k) {
            m * k < ((int64_t)1 << 29) && fused_lds_bytes(m, k) <= FUSED_MAX_LDS;
 }
 
+template <class FMT, bool QUANTISED>
+static void launch_fused_src(const FusedRows& f, hipStream_t s) {
+    // enough workgroups for two per CU where the matrices have the rows for it
+    const int n_rt = (int)(f.n / 16);
+    const unsigned ny = f.w_b ? 2u : 1u;
+    const size_t lds = fused_lds_bytes(f.m, f.k);
+    if (n_rt * (int)ny >= 2048) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 4, QUANTISED>), dim3((unsigned)((n_rt + 3) / 4), ny), dim3(256), lds, s, f);
+    else if (n_rt * (int)ny >= 1024) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 2, QUANTISED>), dim3((unsigned)((n_rt + 1) / 2), ny), dim3(256), lds, s, f);
+    else hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 1, QUANTISED>), dim3((unsigned)n_rt, ny), dim3(256), lds, s, f);
+}
 template <class FMT>
-static void launch_fused_fmt(const float* x, int m, int n, int k, const uint8_t* w, float* y, hipStream_t s) {
-    // enough workgroups for two per CU where the matrix has the rows for it
-    const int n_rt = n / 16;
-    const size_t lds = fused_lds_bytes(m, k);
-    if (n_rt >= 2048) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 4>), dim3((unsigned)((n_rt + 3) / 4)), dim3(256), lds, s, x, m, n, k, w, y);
-    else if (n_rt >= 1024) hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 2>), dim3((unsigned)((n_rt + 1) / 2)), dim3(256), lds, s, x, m, n, k, w, y);
-    else hipLaunchKernelGGL((qlinear_fused_kernel<FMT, 1>), dim3((unsigned)n_rt), dim3(256), lds, s, x, m, n, k, w, y);
+static void launch_fused_fmt(const FusedRows& f, hipStream_t s) {
+    if (f.x) launch_fused_src<FMT, false>(f, s);
+    else launch_fused_src<FMT, true>(f, s);
 }
 
-hipError_t launch_qlinear_fused(int dt, const float* x, int64_t m, int64_t n, int64_t k, const uint8_t* w, float* y, hipStream_t s) {
-    if (!qlinear_fused_usable(dt, m, n, k)) return hipErrorInvalidValue;
+hipError_t launch_qlinear_fused(int dt, const FusedRows& f, hipStream_t s) {
+    if (!qlinear_fused_usable(dt, f.m, f.n, f.k) || !(f.x || f.xq.qs) || !f.w || !f.y || (f.w_b && !f.y_b)) return hipErrorInvalidValue;
     switch (dt) {
-        case MOE_GGML_Q2K: launch_fused_fmt<FmtQ2K>(x, (int)m, (int)n, (int)k, w, y, s); break;
-        case MOE_GGML_Q3K: launch_fused_fmt<FmtQ3K>(x, (int)m, (int)n, (int)k, w, y, s); break;
-        case MOE_GGML_Q4K: launch_fused_fmt<FmtQ4K>(x, (int)m, (int)n, (int)k, w, y, s); break;
-        case MOE_GGML_Q5K: launch_fused_fmt<FmtQ5K>(x, (int)m, (int)n, (int)k, w, y, s); break;
-        case MOE_GGML_Q6K: launch_fused_fmt<FmtQ6K>(x, (int)m, (int)n, (int)k, w, y, s); break;
+        case MOE_GGML_Q2K: launch_fused_fmt<FmtQ2K>(f, s); break;
+        case MOE_GGML_Q3K: launch_fused_fmt<FmtQ3K>(f, s); break;
+        case MOE_GGML_Q4K: launch_fused_fmt<FmtQ4K>(f, s); break;
+        case MOE_GGML_Q5K: launch_fused_fmt<FmtQ5K>(f, s); break;
+        case MOE_GGML_Q6K: launch_fused_fmt<FmtQ6K>(f, s); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

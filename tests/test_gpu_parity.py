@@ -362,6 +362,29 @@ def test_block_kquant_shared_expert_tiny_batches(dt):
     gpu.close()
 
 
+@pytest.mark.parametrize("dt,dt_down,rms_norm", [(O.Q8_0, None, False), (O.Q4_0, O.Q5_0, True), (O.Q5_1, O.Q4_1, False),
+                                                 (O.Q4K, O.Q6K, True), (O.Q5K, None, False), (O.Q3K, O.Q2K, False)])
+def test_block_shared_expert_of_a_few_tokens_as_dense_rows(dt, dt_down, rms_norm):
+    # one to four tokens: the always-on expert runs as two dense few-row launches (w1 and w3 side by side from the quantised
+    # rows, then w2 from silu(w1 x) * (w3 x) quantised in the kernel) instead of the grouped kernels.  Against the oracle in
+    # both settings; the 32-element formats add block values in the reference's order either way: same bits.
+    legacy = dt in (O.Q8_0, O.Q4_0, O.Q5_1)
+    H, F, Fs = (256, 128, 640) if legacy else (512, 256, 1280)
+    ref, gpu = make_pair(H, F, 8, 2, dt, seed=70 + dt, Fs=Fs, dt_down=dt_down, rms=rms_norm)
+    try:
+        for T in (1, 2, 3, 4):
+            out = []
+            for sw in (2, 1):   # whenever the kernels can / never
+                candle_amd.set_switch("fused_rows", sw)
+                ys, _ = check_block(ref, gpu, T, seed=T, tol=None if legacy else block_tol(O.Q4K, F))
+                out.append(ys)
+            if legacy:
+                assert np.array_equal(bits(out[0]), bits(out[1]))
+    finally:
+        candle_amd.set_switch("fused_rows", 0)
+    gpu.close()
+
+
 def test_block_q6k_shared_expert():
     ref, gpu = make_pair(512, 512, 8, 2, O.Q4K, seed=13, Fs=1024, dt_down=O.Q6K)
     for T in (5, 40, 70):
