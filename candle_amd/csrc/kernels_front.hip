@@ -260,13 +260,14 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
 
 // ---------------------------------------------------------------------------------------------
 __device__ inline void route_one_token_wave(float logit, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out);
-__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel);
+__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel, long long* order);
 
 template <int VDT>
 __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     extern __shared__ float xrow[];  // [H]
     __shared__ float probs[MAX_E];
     __shared__ int sel_lds[MAX_K];
+    __shared__ __align__(16) long long order_lds[MAX_E];
     __shared__ float red[FRONT_THREADS / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t t = blockIdx.x;
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void front_kernel(FrontParams p) {
     // ---- wave 0 routes, then joins the others in quantising the row
     if (wave == 0) {
         if (E <= 64) route_one_token_wave(lane < E ? probs[lane] : 0.f, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
-        else route_one_token_wave_lds(probs, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds);
+        else route_one_token_wave_lds(probs, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds, order_lds);
     }
 
     if (VDT == MOE_GGML_Q8K) {
@@ -409,8 +410,21 @@ __device__ inline void route_one_token_wave(float logit, int lane, int E, int k,
 // same float), the exp values summed as vec_sum_ref_order sums them (lane j < 32 carries accumulator j over the blocks
 // of 32, then the tree, then the tail left to right), the rank of an expert = the number of experts that precede it in
 // the (total_cmp key descending, index ascending) order.  `sel` (LDS, k ints) receives the experts in rank order.
-// Call with all 64 lanes of one wave active; p and sel belong to that wave.
-__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel) {
+// Call with all 64 lanes of one wave active; p, sel and order (LDS, MAX_E entries, 16-byte aligned) belong to that wave.
+// Ranks of a lane's NQ experts among all E: order[i] = (total_cmp key of p[i], ~i) as one signed 64-bit integer, so that
+// "i precedes e" is one comparison; four entries per LDS read pair.
+template <int NQ>
+__device__ __forceinline__ void count_ranks(const long long* order, int E, const long long (&mine)[4], int (&rank)[4]) {
+    for (int i = 0; i < E; i += 4) {
+        const longlong2 a = *reinterpret_cast<const longlong2*>(order + i), b = *reinterpret_cast<const longlong2*>(order + i + 2);
+        const long long c[4] = {a.x, a.y, b.x, b.y};
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int q = 0; q < NQ; q++) rank[q] += c[j] > mine[q] ? 1 : 0;
+    }
+}
+__device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k, int norm_topk, int32_t* idx_out, float* w_out, int* sel, long long* order_lds) {
     float mx = -__builtin_inff();
     bool any = false;   // fmaxf skips NaNs; with nothing but NaNs the serial loop is left with one
     for (int e = lane; e < E; e += 64) {
@@ -432,25 +446,29 @@ __device__ inline void route_one_token_wave_lds(float* p, int lane, int E, int k
     const float t3 = lane_bcast(x0, 3) + lane_bcast(x0, 7);
     float s = (t0 + t1) + (t2 + t3);
     for (int i = np; i < E; i++) s += p[i];
+    static_assert(MAX_E == 256, "four experts per lane");
     float pr[4];
-    int key[4], rank[4];
+    long long mine[4];
+    int rank[4];
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int e = lane + 64 * q;
         pr[q] = e < E ? p[e] / s : 0.f;
-        key[q] = total_key(pr[q]);
+        // experts past E sort behind everything (the loop reads the table in fours)
+        mine[q] = e < E ? (long long)(((unsigned long long)(uint32_t)total_key(pr[q]) << 32) | (uint32_t)~(uint32_t)e)
+                        : (long long)0x8000000000000000ull;
         rank[q] = 0;
     }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int q = 0; q < 4; q++)
+    for (int q = 0; q < 4; q++) {
         if (lane + 64 * q < E) p[lane + 64 * q] = pr[q];
-    __builtin_amdgcn_wave_barrier();
-    for (int i = 0; i < E; i++) {
-        const int ki = total_key(p[i]);
-#pragma unroll
-        for (int q = 0; q < 4; q++) rank[q] += (ki > key[q] || (ki == key[q] && i < lane + 64 * q)) ? 1 : 0;
+        order_lds[lane + 64 * q] = mine[q];
     }
+    __builtin_amdgcn_wave_barrier();
+    if (E <= 128) count_ranks<2>(order_lds, E, mine, rank);
+    else if (E <= 192) count_ranks<3>(order_lds, E, mine, rank);
+    else count_ranks<4>(order_lds, E, mine, rank);
 #pragma unroll
     for (int q = 0; q < 4; q++)
         if (lane + 64 * q < E && rank[q] < k) sel[rank[q]] = lane + 64 * q;
@@ -623,6 +641,7 @@ template <int VDT, int NCH, bool LEAN, bool WIDE = false>
 __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     __shared__ float logit_lds[MAX_E];
     __shared__ int sel_lds[MAX_K];
+    __shared__ __align__(16) long long order_lds[MAX_E];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t t = blockIdx.x;
@@ -783,7 +802,7 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
         for (int i = tid; i < H / 4; i += FAST_THREADS) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (wave == 0) {
         if (E <= 64) route_one_token_wave(lane < E ? logit_lds[lane] : 0.f, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
-        else route_one_token_wave_lds(logit_lds, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds);
+        else route_one_token_wave_lds(logit_lds, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds, order_lds);
     }
 }
 template <int VDT, int NCH>
@@ -869,6 +888,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
                                                                          int norm_topk, RouteBufs rb) {
     __shared__ float probs[FRONT_THREADS / 64][MAX_E];
     __shared__ int sel_lds[FRONT_THREADS / 64][MAX_K];
+    __shared__ __align__(16) long long order_lds[FRONT_THREADS / 64][MAX_E];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // one wave per token (4 tokens per workgroup)
     int64_t t = (int64_t)blockIdx.x * (FRONT_THREADS / 64) + wave;
@@ -883,7 +903,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
     if (E <= 64) {
         if (t < T) route_one_token_wave(lane < E ? probs[wave][lane] : 0.f, lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k);
     } else if (t < T) {
-        route_one_token_wave_lds(probs[wave], lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k, sel_lds[wave]);
+        route_one_token_wave_lds(probs[wave], lane, E, k, norm_topk, rb.topk_idx + t * k, rb.topk_w + t * k, sel_lds[wave], order_lds[wave]);
     }
 }
 
@@ -910,20 +930,25 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs
                                                       float* y, int64_t T, int H) {
     const int64_t t = blockIdx.x;
     const int k = rb.k;
-    int slots[MAX_K + 1];
-    int n = k + (shared ? 1 : 0);
-    if (rb.direct) {
-        int es[MAX_K];
-        for (int r = 0; r < k; r++) { es[r] = rb.topk_idx[t * k + r]; slots[r] = (int)(t * k + r); }
-        for (int i = 1; i < k; i++) {
-            int ev = es[i], sv = slots[i], j = i - 1;
-            while (j >= 0 && es[j] > ev) { es[j + 1] = es[j]; slots[j + 1] = slots[j]; j--; }
-            es[j + 1] = ev; slots[j + 1] = sv;
+    const int n = k + (shared ? 1 : 0);
+    // the token's slots in the order of the sum: one wave ranks the selected experts (they are distinct) ...
+    __shared__ int slots[MAX_K + 1];
+    if (threadIdx.x < 64) {
+        const int lane = threadIdx.x;
+        if (rb.direct) {
+            const int e = lane < k ? rb.topk_idx[t * k + lane] : 0x7fffffff;
+            int rank = 0;
+            for (int j = 0; j < k; j++) {
+                const int ej = __shfl(e, j, 64);
+                rank += (ej < e || (ej == e && j < lane)) ? 1 : 0;
+            }
+            if (lane < k) slots[rank] = (int)(t * k + lane);
+            if (shared && lane == 0) slots[k] = (int)(T * k + t);
+        } else if (lane < n) {   // ... or the dispatch pass has
+            slots[lane] = rb.tok_slots[t * n + lane];
         }
-        if (shared) slots[k] = (int)(T * k + t);
-    } else {
-        for (int j = 0; j < n; j++) slots[j] = rb.tok_slots[t * n + j];
     }
+    __syncthreads();
     // a workgroup walks the token's row in steps of 1024 floats, two steps' loads in flight
     const int h0 = (blockIdx.y * 256 + threadIdx.x) * 4, hstep = gridDim.y * 1024;
     for (int h = h0; h < H; h += 2 * hstep) {
@@ -931,24 +956,34 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs
         const bool two = h2 < H;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f), acc2 = acc;
         if (n == 2) {   // the common case: both terms of both steps requested before the first add
-            const float4 a0 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[0] * H + h);
-            const float4 a1 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[1] * H + h);
+            const int s0 = slots[0], s1 = slots[1];
+            const float4 a0 = *reinterpret_cast<const float4*>(yw + (int64_t)s0 * H + h);
+            const float4 a1 = *reinterpret_cast<const float4*>(yw + (int64_t)s1 * H + h);
             float4 b0 = acc, b1 = acc;
             if (two) {
-                b0 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[0] * H + h2);
-                b1 = *reinterpret_cast<const float4*>(yw + (int64_t)slots[1] * H + h2);
+                b0 = *reinterpret_cast<const float4*>(yw + (int64_t)s0 * H + h2);
+                b1 = *reinterpret_cast<const float4*>(yw + (int64_t)s1 * H + h2);
             }
             acc.x += a0.x; acc.y += a0.y; acc.z += a0.z; acc.w += a0.w;
             acc.x += a1.x; acc.y += a1.y; acc.z += a1.z; acc.w += a1.w;
             acc2.x += b0.x; acc2.y += b0.y; acc2.z += b0.z; acc2.w += b0.w;
             acc2.x += b1.x; acc2.y += b1.y; acc2.z += b1.z; acc2.w += b1.w;
         } else {
-            for (int j = 0; j < n; j++) {
-                const float4 v = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h);
-                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
-                if (two) {
-                    const float4 u = *reinterpret_cast<const float4*>(yw + (int64_t)slots[j] * H + h2);
-                    acc2.x += u.x; acc2.y += u.y; acc2.z += u.z; acc2.w += u.w;
+            // four terms requested at a time, added in order
+            for (int j0 = 0; j0 < n; j0 += 4) {
+                float4 v[4], u[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int sl = slots[j0 + i < n ? j0 + i : n - 1];
+                    v[i] = *reinterpret_cast<const float4*>(yw + (int64_t)sl * H + h);
+                    if (two) u[i] = *reinterpret_cast<const float4*>(yw + (int64_t)sl * H + h2);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    if (j0 + i < n) {   // uniform
+                        acc.x += v[i].x; acc.y += v[i].y; acc.z += v[i].z; acc.w += v[i].w;
+                        if (two) { acc2.x += u[i].x; acc2.y += u[i].y; acc2.z += u[i].z; acc2.w += u[i].w; }
+                    }
                 }
             }
         }
