@@ -252,6 +252,7 @@ Switches& switches() {
         g_sw.max_tokens_per_pass = num("MOE_MAX_TOKENS_PER_PASS", 0);
         g_sw.no_gemm = getenv("MOE_NO_GEMM") != nullptr;
         g_sw.front_generic = getenv("MOE_FRONT_GENERIC") != nullptr;
+        g_sw.front_split = (int)num("MOE_FRONT_SPLIT", -1);
         g_sw.tile_slots = (int)num("MOE_TILE_SLOTS", 0);
         g_sw.slot_tiles = (int)num("MOE_SLOT_TILES", 0);
         g_sw.narrow = (int)num("MOE_NARROW", -1);
@@ -1246,6 +1247,7 @@ extern "C" int moe_debug_set_switch(const char* name, int64_t value) {
     else if (n == "slot_tiles") sw.slot_tiles = (int)value;
     else if (n == "narrow") sw.narrow = (int)value;
     else if (n == "fused_rows") sw.fused_rows = (int)value;
+    else if (n == "front_split") sw.front_split = (int)value;
     else return fail(MOE_E_INVALID, "moe_debug_set_switch: unknown switch '" + n + "'");
     return MOE_OK;
 }

@@ -12,6 +12,7 @@ struct Switches {
     int64_t max_tokens_per_pass = 0;  // MOE_MAX_TOKENS_PER_PASS: lower the per-pass token bound (0 = the real bound)
     int no_gemm = 0;                  // MOE_NO_GEMM: never take the tiled kernels
     int front_generic = 0;            // MOE_FRONT_GENERIC: generic front kernel
+    int front_split = -1;             // MOE_FRONT_SPLIT: gate product as a kernel of its own ahead of routing: 0 | 1 (-1 = by shape)
     int tile_slots = 0;               // MOE_TILE_SLOTS: 64 | 128 (0 = by batch size)
     int slot_tiles = 0;               // MOE_SLOT_TILES: 16-slot tiles per streaming pass (0 = by batch size)
     int narrow = -1;                  // MOE_NARROW: 0 | 1 (-1 = by batch size)

@@ -116,9 +116,6 @@ struct DispatchShared {
     int tot[MAX_E];
 };
 
-// tok_slots is written and re-read inside one workgroup: bypass the vector cache on the re-read
-__device__ inline int ld_i32(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-
 // Mask of the valid lanes whose expert index equals this lane's: one ballot per bit of the index, whatever the number
 // of distinct experts among the 64 lanes (a loop over the distinct values takes ~40 rounds with 60 experts and top-4).
 __device__ inline unsigned long long same_expert_lanes(int e, bool valid, int ebits) {
@@ -206,8 +203,11 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         }
         rb.tile_tab[0] = n;
     }
-    // phase 3: stable placement
+    // phase 3: stable placement; the token's row of tok_slots lists its slots by ascending expert index (the order
+    // of the combine pass): an assignment's place there is the number of the token's experts below its own.  With k a
+    // power of two a token's assignments lie in one wave's 64 lanes, otherwise its experts are read back.
     const int kk = k + (shared ? 1 : 0);
+    const bool in_wave = (k & (k - 1)) == 0;   // k <= 16
     {
         int e_next = (lo + lane < hi) ? rb.topk_idx[lo + lane] : -1;
         float w_next = (lo + lane < hi) ? rb.topk_w[lo + lane] : 0.f;
@@ -219,6 +219,21 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
             e_next = (a + 64 < hi) ? rb.topk_idx[a + 64] : -1;
             w_next = (a + 64 < hi) ? rb.topk_w[a + 64] : 0.f;
             const unsigned long long m = same_expert_lanes(e, valid, ebits);
+            const int t = (int)((uint32_t)a / (uint32_t)k), r0 = (int)a - t * k;
+            int place = 0;
+            if (in_wave) {
+                const int first = lane - r0;
+                for (int j = 0; j < k; j++) {
+                    const int ej = __shfl(e, first + j, 64);
+                    place += (ej < e || (ej == e && j < r0)) ? 1 : 0;
+                }
+            } else if (valid) {
+#pragma unroll 4
+                for (int j = 0; j < k; j++) {
+                    const int ej = rb.topk_idx[(int64_t)t * k + j];
+                    place += (ej < e || (ej == e && j < r0)) ? 1 : 0;
+                }
+            }
             int slot = -1;
             if (valid) {
                 const int cur = sh.cnt[wave][e];
@@ -227,35 +242,20 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
                 if ((m & lt) == 0) sh.cnt[wave][e] = cur + __popcll(m);
             }
             if (valid) {
-                int t = (int)(a / k);
                 rb.perm_token[slot] = t;
                 rb.perm_w[slot] = w;
-                // stash (slot) per assignment in tok_slots, unsorted for now
-                rb.tok_slots[(int64_t)t * kk + (int)(a % k)] = slot;
+                rb.tok_slots[(int64_t)t * kk + place] = slot;
             }
         }
     }
-    __syncthreads();
-    // phase 4: per token, order its slots by ascending expert index (combine order); append shared
-    for (int64_t t = tid; t < T; t += DISPATCH_THREADS) {
-        int es[MAX_K], ss[MAX_K];
-        for (int r = 0; r < k; r++) {
-            es[r] = rb.topk_idx[t * k + r];
-            ss[r] = ld_i32(rb.tok_slots + t * kk + r);
-        }
-        for (int i = 1; i < k; i++) {
-            int ev = es[i], sv = ss[i], j = i - 1;
-            while (j >= 0 && es[j] > ev) { es[j + 1] = es[j]; ss[j + 1] = ss[j]; j--; }
-            es[j + 1] = ev; ss[j + 1] = sv;
-        }
-        for (int r = 0; r < k; r++) rb.tok_slots[t * kk + r] = ss[r];
-        if (shared) {
-            int slot = (int)(A + t);
+    // phase 4: the always-on expert's slots follow the routed ones
+    if (shared)
+        for (int64_t t = tid; t < T; t += DISPATCH_THREADS) {
+            const int slot = (int)(A + t);
             rb.tok_slots[t * kk + k] = slot;
             rb.perm_token[slot] = (int)t;
             rb.perm_w[slot] = rb.shared_w[t];
         }
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1001,6 +1001,143 @@ __global__ __launch_bounds__(256) void combine_kernel(const float* yw, RouteBufs
 }
 
 // ---------------------------------------------------------------------------------------------
+// The front end in two launches, for layers with dozens of experts and for large batches (no pre-norm): the gate product
+// of all tokens as an f32 matrix product on the matrix cores, then routing and quantisation per token.  One workgroup per
+// token computing its own E products reads the whole gate (a megabyte at 128 experts of 2048) through one CU.
+//
+// logits[t, e] = x[t, :] . gate[e, :] (+ bias[e]); row E of the product is the always-on expert's gate, whose sigmoid goes
+// to shared_w[t].  A workgroup owns 16 tokens x NB * 16 gate rows; its four waves split K and add their parts in wave
+// order (v_mfma_f32_16x16x4_f32: lane l holds A[l % 16][l / 16], B[l / 16][l % 16] and D[4 (l / 16) + r][l % 16]).
+typedef float v4f_front __attribute__((ext_vector_type(4)));
+template <int NB>
+__global__ __launch_bounds__(256) void gate_logits_kernel(FrontParams p) {
+    __shared__ float part[4][NB][4][64];
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int H = p.H, E = p.E;
+    const int NE = E + (p.shared_gate ? 1 : 0);
+    const int64_t t0 = (int64_t)blockIdx.x * 16;
+    const int e0 = blockIdx.y * (NB * 16);
+    const int64_t trow = t0 + m < p.T ? t0 + m : p.T - 1;
+    const int kw = (H / 64) * 16;   // K of a wave: a multiple of 64
+    // a batch is 16 * DEPTH consecutive k: lane group kq takes 4 * DEPTH consecutive ones of them (whole cache lines per
+    // row and batch; which k a lane group multiplies only permutes the sum), DEPTH loads of four
+    constexpr int DEPTH = NB == 1 ? 4 : 2;
+    const float* xp = p.x + trow * H + wave * kw + 4 * DEPTH * kq;
+    const float* gp[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) {
+        int e = e0 + nb * 16 + m;
+        e = e < NE ? e : NE - 1;   // rows past the last are computed and dropped
+        gp[nb] = (e < E ? p.gate + (int64_t)e * H : p.shared_gate) + wave * kw + 4 * DEPTH * kq;
+    }
+    v4f_front acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) acc[nb] = v4f_front{0.f, 0.f, 0.f, 0.f};
+    // a batch is requested ahead of the one being multiplied
+    float4 xa[DEPTH], ga[DEPTH][NB];
+    auto request = [&](int kc, float4 (&xo)[DEPTH], float4 (&go)[DEPTH][NB]) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            xo[d] = *reinterpret_cast<const float4*>(xp + kc + 4 * d);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) go[d][nb] = *reinterpret_cast<const float4*>(gp[nb] + kc + 4 * d);
+        }
+    };
+    request(0, xa, ga);
+    for (int kc = 0; kc < kw; kc += 16 * DEPTH) {
+        float4 xn[DEPTH], gn[DEPTH][NB];
+        request(kc + 16 * DEPTH < kw ? kc + 16 * DEPTH : kc, xn, gn);
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            const float xs[4] = {xa[d].x, xa[d].y, xa[d].z, xa[d].w};
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) {
+                const float gs[4] = {ga[d][nb].x, ga[d][nb].y, ga[d][nb].z, ga[d][nb].w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(xs[j], gs[j], acc[nb], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            xa[d] = xn[d];
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) ga[d][nb] = gn[d][nb];
+        }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) part[wave][nb][r][lane] = acc[nb][r];
+    __syncthreads();
+    for (int v = wave; v < NB * 4; v += 4) {
+        const int nb = v >> 2, r = v & 3;
+        float sum = part[0][nb][r][lane];
+        sum += part[1][nb][r][lane];
+        sum += part[2][nb][r][lane];
+        sum += part[3][nb][r][lane];
+        const int64_t t = t0 + 4 * kq + r;
+        const int e = e0 + nb * 16 + m;
+        if (t < p.T && e < NE) {
+            if (e < E) p.rb.logits[t * E + e] = p.gate_bias ? sum + p.gate_bias[e] : sum;
+            else p.rb.shared_w[t] = 1.0f / (expf_glibc(-sum) + 1.0f);
+        }
+    }
+}
+
+// Routing and quantisation of one token whose logits are in memory: wave 0 routes, waves 1 to 3 quantise the row.
+template <int VDT>
+__global__ __launch_bounds__(256) void front_route_kernel(FrontParams p) {
+    __shared__ float logit_lds[MAX_E];
+    __shared__ int sel_lds[MAX_K];
+    __shared__ __align__(16) long long order_lds[MAX_E];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t t = blockIdx.x;
+    const int H = p.H, E = p.E, nch = H / 256;
+    if (wave == 0) {
+        if (E <= 64) {
+            const float v = lane < E ? p.rb.logits[t * E + lane] : 0.f;
+            route_one_token_wave(v, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k);
+        } else {
+            for (int e = lane; e < E; e += 64) logit_lds[e] = p.rb.logits[t * E + e];
+            __builtin_amdgcn_wave_barrier();
+            route_one_token_wave_lds(logit_lds, lane, E, p.k, p.norm_topk, p.rb.topk_idx + t * p.k, p.rb.topk_w + t * p.k, sel_lds, order_lds);
+        }
+    } else {
+        // chunks wave - 1, wave + 2, ...: two of them side by side
+        for (int i = wave - 1; i < nch; i += 6) {
+            const int i2 = i + 3;
+            const float4 a = *reinterpret_cast<const float4*>(p.x + t * H + i * 256 + lane * 4);
+            float4 b = a;
+            if (i2 < nch) b = *reinterpret_cast<const float4*>(p.x + t * H + i2 * 256 + lane * 4);
+            const float ea[4] = {a.x, a.y, a.z, a.w}, eb[4] = {b.x, b.y, b.z, b.w};
+            quantize_chunk<VDT>(p, t, H, i, ea, lane);
+            if (i2 < nch) quantize_chunk<VDT>(p, t, H, i2, eb, lane);
+        }
+    }
+    if (p.y_zero)
+        for (int i = tid; i < H / 4; i += 256) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
+static bool launch_front_split(const FrontParams& p, hipStream_t s) {
+    const int sw = switches().front_split;
+    const int NE = p.E + (p.shared_gate ? 1 : 0);
+    if (sw == 0 || p.rms_alpha || p.H % 256 || p.E > MAX_E || p.T * (int64_t)p.H >= ((int64_t)1 << 31)) return false;
+    // (measured, front stage fused / split: 128 experts of 2048: 25 / 17 us at 512 tokens, 179 / 57 at 4096; 64 experts and
+    // the always-on gate: 18 / 18 at 512, 118 / 51 at 4096; 60 experts and that gate: 19 / 21 at 512, 112 / 42 at 4096; 8 experts
+    // of 4096: 54 / 46 at 4096, 5 / 18 at 32: a wave of the product waits ~1.7 us for every batch of loads, whatever its shape)
+    if (sw < 0 && !(NE >= 32 && p.T * (int64_t)NE >= 49152)) return false;
+    const unsigned tiles = (unsigned)((p.T + 15) / 16);
+    // four blocks of gate rows per workgroup when that still leaves a workgroup per CU
+    if (NE > 16 && (int64_t)tiles * ((NE + 63) / 64) >= 256) hipLaunchKernelGGL(gate_logits_kernel<4>, dim3(tiles, (unsigned)((NE + 63) / 64)), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(gate_logits_kernel<1>, dim3(tiles, (unsigned)((NE + 15) / 16)), dim3(256), 0, s, p);
+    if (p.vdt == MOE_GGML_Q8K) hipLaunchKernelGGL(front_route_kernel<MOE_GGML_Q8K>, dim3((unsigned)p.T), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(front_route_kernel<MOE_GGML_Q8_0>, dim3((unsigned)p.T), dim3(256), 0, s, p);
+    return true;
+}
+
+// ---------------------------------------------------------------------------------------------
 template <int VDT>
 static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
     if (p.E > MAX_E || p.H % 256) return false;
@@ -1056,6 +1193,7 @@ hipError_t launch_front(const FrontParams& p_in, hipStream_t s) {
     const FrontParams& p = p_in;
     const bool no_fast = switches().front_generic != 0;
     const bool q8k = p.vdt == MOE_GGML_Q8K;
+    if (!no_fast && launch_front_split(p, s)) return hipGetLastError();
     if (!no_fast && (q8k ? launch_front_fast<MOE_GGML_Q8K>(p, s) : launch_front_fast<MOE_GGML_Q8_0>(p, s))) return hipGetLastError();
     size_t lds = (size_t)p.H * sizeof(float);
     if (q8k)

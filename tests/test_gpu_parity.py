@@ -485,6 +485,31 @@ def test_block_dozens_of_experts_at_small_batches(H, E, k, shared, rms):
     gpu.close()
 
 
+@pytest.mark.parametrize("H,E,k,dt,shared,bias", [(512, 8, 2, O.Q4K, 0, False), (2048, 128, 8, O.Q4K, 256, False), (256, 60, 4, O.Q8_0, 64, True),
+                                                  (768, 33, 3, O.Q5_1, 0, True)])
+def test_block_gate_product_as_a_launch_of_its_own(H, E, k, dt, shared, bias):
+    # the front end in two launches (large batches of layers with dozens of experts take it by default: 400 tokens of the
+    # 128-expert case): the gate product on the matrix cores -- logits within 1e-4 of the oracle's and of the one-launch
+    # kernel's --, then routing (bit-exact given those logits) and quantisation per token
+    F = 256 if dt == O.Q4K else 64
+    gb = np.random.default_rng(E).normal(0, 0.3, E).astype(np.float32) if bias else None
+    ref, gpu = make_pair(H, F, E, k, dt, seed=90 + E, Fs=shared, gate_bias=gb)
+    try:
+        for T in (1, 17, 400):
+            xs = activations(T, H, 2)
+            candle_amd.set_switch("front_split", 0)
+            gpu.forward(xs)
+            one = gpu.last_logits(T)
+            candle_amd.set_switch("front_split", 1)
+            check_block(ref, gpu, T, tol=block_tol(dt, F))
+            assert np.abs(gpu.last_logits(T) - one).max() < 1e-4
+            candle_amd.set_switch("front_split", -1)
+            check_block(ref, gpu, T, tol=block_tol(dt, F))
+    finally:
+        candle_amd.set_switch("front_split", -1)
+    gpu.close()
+
+
 def test_block_rms_residual_chain():
     ref, gpu = make_pair(512, 512, 4, 2, O.Q4K, seed=5, rms=True)
     xs = activations(6, 512, 9)
