@@ -100,7 +100,7 @@ struct ActStore {
 };
 
 struct RouteStore {
-    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots, tile_tab;
+    DevBuf logits, topk_idx, topk_w, shared_w, offsets, perm_token, perm_w, tok_slots, tile_tab, wg_counts;
     int reserve(int64_t T, int E, int k, bool shared) {
         int rc;
         const int64_t S = T * k + (shared ? T : 0);
@@ -113,6 +113,7 @@ struct RouteStore {
         if ((rc = perm_w.reserve((size_t)S * 4))) return rc;
         if ((rc = tok_slots.reserve((size_t)T * (k + 1) * 4))) return rc;
         if ((rc = tile_tab.reserve((size_t)(1 + 2 * max_gemm_tiles(S, E + 1)) * 4))) return rc;
+        if ((rc = wg_counts.reserve((size_t)DISPATCH_MAX_WGS * DISPATCH_COUNT_STRIDE * 4))) return rc;
         return MOE_OK;
     }
     RouteBufs view() const {
@@ -126,6 +127,7 @@ struct RouteStore {
         r.perm_w = perm_w.as<float>();
         r.tok_slots = tok_slots.as<int32_t>();
         r.tile_tab = tile_tab.as<int32_t>();
+        r.wg_counts = wg_counts.as<int32_t>();
         return r;
     }
 };
@@ -160,6 +162,7 @@ struct Carver {
         r.perm_w = take<float>((size_t)S * 4);
         r.tok_slots = take<int32_t>((size_t)T * (k + 1) * 4);
         r.tile_tab = tile_tab ? take<int32_t>((size_t)(1 + 2 * max_gemm_tiles(S, E + 1)) * 4) : nullptr;
+        if (T * k > 16384) r.wg_counts = take<int32_t>((size_t)DISPATCH_MAX_WGS * DISPATCH_COUNT_STRIDE * 4);
         return r;
     }
 };
@@ -253,6 +256,7 @@ Switches& switches() {
         g_sw.no_gemm = getenv("MOE_NO_GEMM") != nullptr;
         g_sw.front_generic = getenv("MOE_FRONT_GENERIC") != nullptr;
         g_sw.front_split = (int)num("MOE_FRONT_SPLIT", -1);
+        g_sw.dispatch_one = (int)num("MOE_DISPATCH_ONE", 0);
         g_sw.tile_slots = (int)num("MOE_TILE_SLOTS", 0);
         g_sw.slot_tiles = (int)num("MOE_SLOT_TILES", 0);
         g_sw.narrow = (int)num("MOE_NARROW", -1);
@@ -1248,6 +1252,7 @@ extern "C" int moe_debug_set_switch(const char* name, int64_t value) {
     else if (n == "narrow") sw.narrow = (int)value;
     else if (n == "fused_rows") sw.fused_rows = (int)value;
     else if (n == "front_split") sw.front_split = (int)value;
+    else if (n == "dispatch_one") sw.dispatch_one = (int)value;
     else return fail(MOE_E_INVALID, "moe_debug_set_switch: unknown switch '" + n + "'");
     return MOE_OK;
 }

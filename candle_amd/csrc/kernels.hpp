@@ -12,6 +12,7 @@ struct Switches {
     int64_t max_tokens_per_pass = 0;  // MOE_MAX_TOKENS_PER_PASS: lower the per-pass token bound (0 = the real bound)
     int no_gemm = 0;                  // MOE_NO_GEMM: never take the tiled kernels
     int front_generic = 0;            // MOE_FRONT_GENERIC: generic front kernel
+    int dispatch_one = 0;             // MOE_DISPATCH_ONE: the dispatch pass always as one workgroup
     int front_split = -1;             // MOE_FRONT_SPLIT: gate product as a kernel of its own ahead of routing: 0 | 1 (-1 = by shape)
     int tile_slots = 0;               // MOE_TILE_SLOTS: 64 | 128 (0 = by batch size)
     int slot_tiles = 0;               // MOE_SLOT_TILES: 16-slot tiles per streaming pass (0 = by batch size)
@@ -35,6 +36,7 @@ struct RouteBufs {
     // of tiles of `tile_slots` slots, then (group, first position inside the group) per tile.  Built
     // from the real list lengths, so a skewed routing yields tiles in proportion to each expert's load.
     int32_t* tile_tab = nullptr;
+    int32_t* wg_counts = nullptr;   // [DISPATCH_MAX_WGS][DISPATCH_COUNT_STRIDE] assignments per expert of each workgroup of a dispatch pass in two launches
     int tile_slots = 128;           // 128, or 64 when the lists are short
     // Slot numbering.  direct == 0: slots are grouped by expert (offsets / perm_* built by the
     // dispatch kernel).  direct == 1 (small batches): slot of assignment (token t, rank r) is
@@ -43,6 +45,8 @@ struct RouteBufs {
     int direct = 0;
     int T = 0, k = 0;
 };
+constexpr int DISPATCH_MAX_WGS = 32;      // workgroups of a dispatch pass in two launches
+constexpr int DISPATCH_COUNT_STRIDE = 256;  // ints per workgroup in wg_counts: the largest expert count
 constexpr int DIRECT_MAX_SLOTS = 1024;  // largest T*k (and T) served without a dispatch pass
 constexpr int GEMM_MIN_TILE_SLOTS = 64;  // smallest tile of the tiled expert kernels
 inline int64_t max_gemm_tiles(int64_t slots, int64_t groups, int tile_slots = GEMM_MIN_TILE_SLOTS) { return slots / tile_slots + groups + 1; }

@@ -25,6 +25,7 @@ namespace moe {
 
 constexpr int FRONT_THREADS = 256;
 constexpr int MAX_E = 256;
+static_assert(MAX_E == DISPATCH_COUNT_STRIDE, "a workgroup's row of wg_counts holds every expert");
 constexpr int MAX_K = 16;
 
 // Sum over the wave by the butterfly lane ^ 32, ^ 16, ^ 8, ^ 4, ^ 2, ^ 1 (every lane ends with the same bits).  The last
@@ -114,6 +115,7 @@ struct DispatchShared {
     int cnt[DISPATCH_THREADS / 64][MAX_E];
     int off[MAX_E + 2];
     int tot[MAX_E];
+    int before[MAX_E];
 };
 
 // Mask of the valid lanes whose expert index equals this lane's: one ballot per bit of the index, whatever the number
@@ -127,12 +129,19 @@ __device__ inline unsigned long long same_expert_lanes(int e, bool valid, int eb
     return m;
 }
 
-__device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, bool shared, DispatchShared& sh) {
+// One workgroup of G (`pass` 0 with G = 1: everything in one launch).  With G > 1 the assignments are cut into G stretches
+// and the work into two launches: pass 1 counts a stretch's assignments per expert into rb.wg_counts[g][:], pass 2 repeats
+// its own count, reads the others' and places its stretch behind the earlier ones'.
+__device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, bool shared, DispatchShared& sh, int g, int G, int pass) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int NW = DISPATCH_THREADS / 64;
     const int64_t A = T * k;
-    const int64_t chunk = ((A + NW - 1) / NW + 63) / 64 * 64;
-    const int64_t lo = wave * chunk, hi = (lo + chunk < A) ? lo + chunk : A;
+    // a workgroup's stretch is a multiple of 64 * NW assignments, a wave's chunk of 64 (and so of every k <= 16 that is a
+    // power of two: such a token's assignments stay in one wave's 64 lanes)
+    const int64_t stretch = ((A + G - 1) / G + 64 * NW - 1) / (64 * NW) * (64 * NW);
+    const int64_t a_lo = g * stretch, a_hi = a_lo + stretch < A ? a_lo + stretch : A;
+    const int64_t chunk = stretch / NW;
+    const int64_t lo = a_lo + wave * chunk, hi = lo + chunk < a_hi ? lo + chunk : a_hi;
     const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));   // the lanes below this one
     const int ebits = 32 - __clz(E > 1 ? E - 1 : 1);                              // bits of an expert index
     for (int i = tid; i < NW * MAX_E; i += DISPATCH_THREADS) (&sh.cnt[0][0])[i] = 0;
@@ -151,13 +160,26 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         }
     }
     __syncthreads();
-    // phase 2: totals per expert, exclusive scan over experts (one wave, four experts per lane), per-wave bases
+    // phase 2: totals per expert (over all workgroups), exclusive scan over experts (one wave, four experts per lane),
+    // per-wave bases behind the earlier workgroups' assignments
     for (int e = tid; e < MAX_E; e += DISPATCH_THREADS) {
-        int t = 0;
-        if (e < E)
-            for (int w = 0; w < NW; w++) t += sh.cnt[w][e];
-        sh.tot[e] = t;
+        int mine = 0, all = 0, before = 0;
+        if (e < E) {
+            for (int w = 0; w < NW; w++) mine += sh.cnt[w][e];
+            all = mine;
+            if (pass == 2)
+                for (int gg = 0; gg < G; gg++) {
+                    if (gg == g) continue;
+                    const int c = rb.wg_counts[gg * MAX_E + e];
+                    all += c;
+                    if (gg < g) before += c;
+                }
+        }
+        if (pass == 1) rb.wg_counts[g * MAX_E + e] = mine;
+        sh.tot[e] = all;
+        sh.before[e] = before;
     }
+    if (pass == 1) return;
     __syncthreads();
     if (wave == 0) {
         static_assert(MAX_E == 256, "four experts per lane");
@@ -181,7 +203,7 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         sh.off[E + 1] = (int)A + (shared ? (int)T : 0);
     }
     for (int e = tid; e < E; e += DISPATCH_THREADS) {
-        int run = sh.off[e];
+        int run = sh.off[e] + sh.before[e];
         for (int w = 0; w < NW; w++) {
             int c = sh.cnt[w][e];
             sh.cnt[w][e] = run;  // becomes the wave's running cursor
@@ -189,19 +211,21 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         }
     }
     __syncthreads();
-    for (int e = tid; e <= E + (shared ? 1 : 0); e += DISPATCH_THREADS) rb.offsets[e] = sh.off[e];
-    if (tid == 0 && rb.tile_tab) {  // work list of the tiled expert kernels
-        int n = 0;
-        const int G = E + (shared ? 1 : 0);
-        for (int gi = 0; gi < G; gi++) {
-            const int len = sh.off[gi + 1] - sh.off[gi];
-            for (int pos = 0; pos < len; pos += rb.tile_slots) {
-                rb.tile_tab[1 + 2 * n] = gi;
-                rb.tile_tab[2 + 2 * n] = pos;
-                n++;
+    if (g == 0) {
+        for (int e = tid; e <= E + (shared ? 1 : 0); e += DISPATCH_THREADS) rb.offsets[e] = sh.off[e];
+        if (tid == 0 && rb.tile_tab) {  // work list of the tiled expert kernels
+            int n = 0;
+            const int NG = E + (shared ? 1 : 0);
+            for (int gi = 0; gi < NG; gi++) {
+                const int len = sh.off[gi + 1] - sh.off[gi];
+                for (int pos = 0; pos < len; pos += rb.tile_slots) {
+                    rb.tile_tab[1 + 2 * n] = gi;
+                    rb.tile_tab[2 + 2 * n] = pos;
+                    n++;
+                }
             }
+            rb.tile_tab[0] = n;
         }
-        rb.tile_tab[0] = n;
     }
     // phase 3: stable placement; the token's row of tok_slots lists its slots by ascending expert index (the order
     // of the combine pass): an assignment's place there is the number of the token's experts below its own.  With k a
@@ -250,7 +274,7 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
     }
     // phase 4: the always-on expert's slots follow the routed ones
     if (shared)
-        for (int64_t t = tid; t < T; t += DISPATCH_THREADS) {
+        for (int64_t t = (int64_t)g * DISPATCH_THREADS + tid; t < T; t += (int64_t)G * DISPATCH_THREADS) {
             const int slot = (int)(A + t);
             rb.tok_slots[t * kk + k] = slot;
             rb.perm_token[slot] = (int)t;
@@ -907,9 +931,9 @@ __global__ __launch_bounds__(FRONT_THREADS) void route_from_logits_kernel(const 
     }
 }
 
-__global__ __launch_bounds__(DISPATCH_THREADS) void dispatch_kernel(RouteBufs rb, int64_t T, int E, int k, int shared) {
+__global__ __launch_bounds__(DISPATCH_THREADS) void dispatch_kernel(RouteBufs rb, int64_t T, int E, int k, int shared, int pass) {
     __shared__ DispatchShared dsh;
-    dispatch_block(rb, T, E, k, shared != 0, dsh);
+    dispatch_block(rb, T, E, k, shared != 0, dsh, (int)blockIdx.x, (int)gridDim.x, pass);
 }
 
 __global__ void identity_routing_kernel(RouteBufs rb, int64_t rows) {
@@ -1220,7 +1244,15 @@ hipError_t launch_identity_routing(const RouteBufs& rb, int64_t rows, hipStream_
 
 hipError_t launch_dispatch(const RouteBufs& rb, int64_t T, int E, int k, bool shared, hipStream_t s) {
     if (T == 0) return hipSuccess;
-    hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(DISPATCH_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0);
+    // one workgroup up to 16k assignments (8192: 13 us); beyond, a counting and a placing launch of a workgroup per 4096
+    const int64_t A = T * k;
+    const unsigned G = (unsigned)std::min<int64_t>(DISPATCH_MAX_WGS, (A + 4095) / 4096);
+    if (A <= 16384 || !rb.wg_counts || switches().dispatch_one) {
+        hipLaunchKernelGGL(dispatch_kernel, dim3(1), dim3(DISPATCH_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0, 0);
+    } else {
+        hipLaunchKernelGGL(dispatch_kernel, dim3(G), dim3(DISPATCH_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0, 1);
+        hipLaunchKernelGGL(dispatch_kernel, dim3(G), dim3(DISPATCH_THREADS), 0, s, rb, T, E, k, shared ? 1 : 0, 2);
+    }
     return hipGetLastError();
 }
 

@@ -258,7 +258,7 @@ const char* moe_device_arch(void);
 
 /* Test aid (no counterpart in the reference): sets one of the process-wide tuning switches that are otherwise
  * read once from the MOE_* environment variables: "combine_pass", "rms_serial", "max_tokens_per_pass", "no_gemm",
- * "front_generic", "tile_slots", "slot_tiles", "narrow", "fused_rows", "front_split".  Not for use while forwards are in flight. */
+ * "front_generic", "tile_slots", "slot_tiles", "narrow", "fused_rows", "front_split", "dispatch_one".  Not for use while forwards are in flight. */
 int moe_debug_set_switch(const char* name, int64_t value);
 
 /* Host restatement of the exp used by the device router (same source, compiled for the CPU), so

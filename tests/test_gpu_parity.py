@@ -109,7 +109,9 @@ def test_activation_quantiser_bit_exact(vdt):
 
 @pytest.mark.parametrize("T,E,k,norm", [(16, 8, 2, True), (1, 8, 2, True), (333, 60, 4, True), (4096, 8, 2, True),
                                          (65, 64, 6, False), (7, 3, 3, True), (50, 160, 8, True), (9, 1, 1, True),
-                                         (33, 256, 16, True), (12, 65, 3, False), (20, 100, 5, True), (40, 224, 1, True)])
+                                         (33, 256, 16, True), (12, 65, 3, False), (20, 100, 5, True), (40, 224, 1, True),
+                                         # more than 16384 assignments: the dispatch pass as two launches of several workgroups
+                                         (3000, 128, 8, True), (5000, 60, 6, False), (2100, 256, 16, True), (40000, 8, 2, True)])
 def test_route_bit_exact_given_logits(T, E, k, norm):
     logits = O.fill_normal(T * 31 + E, T * E, 0.0, 1.5).reshape(T, E)
     if T > 4:
@@ -507,6 +509,21 @@ def test_block_gate_product_as_a_launch_of_its_own(H, E, k, dt, shared, bias):
             check_block(ref, gpu, T, tol=block_tol(dt, F))
     finally:
         candle_amd.set_switch("front_split", -1)
+    gpu.close()
+
+
+@pytest.mark.parametrize("E,k,shared", [(60, 4, 64), (16, 3, 0)])
+def test_block_dispatch_pass_of_several_workgroups(E, k, shared):
+    # more than 16384 assignments: every workgroup of the dispatch pass places its stretch of the assignments behind the
+    # earlier ones' and writes its tokens' slots in the order of the combine pass; same result with one workgroup
+    T = 16384 // k + 600
+    ref, gpu = make_pair(256, 64, E, k, O.Q8_0, seed=95 + E, Fs=shared)
+    try:
+        ys, _ = check_block(ref, gpu, T)
+        candle_amd.set_switch("dispatch_one", 1)
+        assert np.array_equal(bits(gpu.forward(activations(T, 256, 2))), bits(ys))
+    finally:
+        candle_amd.set_switch("dispatch_one", 0)
     gpu.close()
 
 
