@@ -1147,7 +1147,7 @@ __global__ __launch_bounds__(256) void front_route_kernel(FrontParams p) {
 static bool launch_front_split(const FrontParams& p, hipStream_t s) {
     const int sw = switches().front_split;
     const int NE = p.E + (p.shared_gate ? 1 : 0);
-    if (sw == 0 || p.rms_alpha || p.H % 256 || p.E > MAX_E || p.T * (int64_t)p.H >= ((int64_t)1 << 31)) return false;
+    if (sw == 0 || p.rms_alpha || p.H % 256 || p.E > MAX_E) return false;
     // (measured, front stage fused / split: 128 experts of 2048: 25 / 17 us at 512 tokens, 179 / 57 at 4096; 64 experts and
     // the always-on gate: 18 / 18 at 512, 118 / 51 at 4096; 60 experts and that gate: 19 / 21 at 512, 112 / 42 at 4096; 8 experts
     // of 4096: 54 / 46 at 4096, 5 / 18 at 32: a wave of the product waits ~1.7 us for every batch of loads, whatever its shape)
