@@ -1150,7 +1150,7 @@ static bool launch_front_split(const FrontParams& p, hipStream_t s) {
     if (sw == 0 || p.rms_alpha || p.H % 256 || p.E > MAX_E) return false;
     // (measured, front stage fused / split: 128 experts of 2048: 25 / 17 us at 512 tokens, 179 / 57 at 4096; 64 experts and
     // the always-on gate: 18 / 18 at 512, 118 / 51 at 4096; 60 experts and that gate: 19 / 21 at 512, 112 / 42 at 4096; 8 experts
-    // of 4096: 54 / 46 at 4096, 5 / 18 at 32: a wave of the product waits ~1.7 us for every batch of loads, whatever its shape)
+    // of 4096: 54 / 46 at 4096, 5 / 18 at 32: the product kernel takes 2 us + 3.3 us per 1024 of H whatever its grid)
     if (sw < 0 && !(NE >= 32 && p.T * (int64_t)NE >= 49152)) return false;
     const unsigned tiles = (unsigned)((p.T + 15) / 16);
     // four blocks of gate rows per workgroup when that still leaves a workgroup per CU
