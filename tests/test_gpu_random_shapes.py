@@ -21,7 +21,7 @@ Q81 = [O.Q4_1, O.Q5_1]           # ... with Q8_1 activations
 @pytest.mark.parametrize("seed", [2, 3])
 def test_random_layers(seed):
     rnd = random.Random(seed)
-    for case in range(30):
+    for case in range(18):
         fam = rnd.choice(["k", "k", "80", "81"])
         if fam == "k":
             dt, dtd, mult = rnd.choice(KQ), rnd.choice(KQ + [None, None]), 256
