@@ -652,6 +652,32 @@ def test_long_inputs_go_through_in_several_passes(monkeypatch):
     gpu.close()
 
 
+def test_large_batch_front_end_and_dispatch_recorded_into_a_hip_graph():
+    # 4200 tokens of a 60-expert top-4 layer with an always-on expert: the gate product as a launch of its own, the dispatch
+    # pass as two launches of several workgroups -- kernels only, so a capture holds them; replays equal the eager result
+    torch = pytest.importorskip("torch")
+    ref, gpu = make_pair(256, 64, 60, 4, O.Q8_0, seed=97, Fs=64)
+    T = 4200
+    xs = [torch.from_numpy(activations(T, 256, 50 + i)).cuda() for i in range(2)]
+    eager = [gpu.forward(x).clone() for x in xs]
+    x_in, y_out = xs[0].clone(), torch.empty_like(xs[0])
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        gpu.forward(x_in, out=y_out)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        gpu.forward(x_in, out=y_out)
+    for rep in range(2):
+        for x, want in zip(xs, eager):
+            x_in.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_out, want)
+            assert torch.equal(gpu.forward(x), want)
+    gpu.close()
+
+
 @pytest.mark.parametrize("T", [4, 32, 200])
 def test_forward_recorded_into_a_hip_graph(T):
     # a decode loop records the layer into a graph and replays it: narrow (4), direct (32) and tiled (200)
