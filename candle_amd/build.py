@@ -40,6 +40,11 @@ def build_library(verbose=False, out_dir=None, extra_flags=()):
     out_dir = out_dir or OUT_DIR
     lib_path = os.path.join(out_dir, os.path.basename(LIB_PATH))
     os.makedirs(out_dir, exist_ok=True)
+    # objects of sources that are no longer part of the library do not ship with it
+    wanted = {os.path.splitext(src)[0] + ".o" for src in SOURCES}
+    for name in os.listdir(out_dir):
+        if name.endswith(".o") and name not in wanted:
+            os.remove(os.path.join(out_dir, name))
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         results = list(ex.map(lambda src: _compile(src, out_dir, extra_flags), SOURCES))
     objs = [o for o, _ in results]

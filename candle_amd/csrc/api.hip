@@ -775,9 +775,14 @@ extern "C" int moe_layer_forward_device_noalloc(moe_layer* L, const void* d_x, i
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    // An earlier call on this layer may still run on another stream: it shares the layer's side stream and events (and
+    // a later allocating call must find this one in the order).  An event record and a stream wait: no allocation.
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    if (!capturing)
+        if (int rc = L->order.enter(s)) return rc;
     if (int rc = enqueue_forward(L, pl, ws, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s)) return rc;
     // the hooks that read the last call's logits and routing wait for this stream
-    if (cap == hipStreamCaptureStatusNone) L->order.leave(s);
+    if (!capturing) L->order.leave(s);
     return MOE_OK;
 }
 
@@ -1058,7 +1063,7 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
         if (int rc = Q->ws.reserve(need)) return rc;
         Q->routed_m = -1;   // the table has moved
     }
-    if (capturing) { Q->ws.captured = true; Q->routed_m = -1; }
+    if (capturing) Q->ws.captured = true;
     RouteBufs rb;
     ActBuf xq;
     carve_qlinear(Q, m, static_cast<uint8_t*>(Q->ws.p), &rb, &xq);
@@ -1078,11 +1083,12 @@ static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d
     rb.tile_slots = tiled32 ? 64 : tile_slots;
     if (!tiled) rb.tile_tab = nullptr;
     MOE_HIP_CHECK(launch_quantize_rows(Q->vdt, d_x, m, (int)Q->k, xq, s));
-    // the identity table depends on the row count only: a decode loop that calls with the same m finds it in place
-    if (Q->routed_m != m || Q->routed_tile != tile_slots || Q->routed_tab != tiled || Q->routed_stream != s) {
+    // The identity table depends on the row count only: a decode loop that calls with the same m finds it in place.
+    // Once a graph has been captured on this object the host no longer knows what the table holds -- a replay rewrites
+    // it for the captured row count, in the workspace eager calls share -- so from then on every call writes it again.
+    if (Q->ws.captured || Q->routed_m != m || Q->routed_tile != tile_slots || Q->routed_tab != tiled || Q->routed_stream != s) {
         MOE_HIP_CHECK(launch_identity_routing(rb, m, s));
         Q->routed_m = m; Q->routed_tile = tile_slots; Q->routed_tab = tiled; Q->routed_stream = s;
-        if (capturing) Q->routed_m = -1;   // an eager call after the capture writes the table again
     }
     ExpertParams ep;
     ep.dt = Q->dt; ep.H = (int)Q->n; ep.F = (int)Q->k; ep.n_groups = 1; ep.group0 = 0;

@@ -340,9 +340,13 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     if (!g || !out || layer_index < 0) return fail(MOE_E_INVALID, "moe_layer_create_from_gguf: bad argument");
     *out = nullptr;
     // quantized_llama.rs:507-512: both keys default to 0 when absent
-    uint64_t n_expert = 0, n_used = 0;
-    if (g->metadata.count("llama.expert_count") && moe_gguf_metadata_u64(g, "llama.expert_count", &n_expert)) return MOE_E_INVALID;
-    if (g->metadata.count("llama.expert_used_count") && moe_gguf_metadata_u64(g, "llama.expert_used_count", &n_used)) return MOE_E_INVALID;
+    // (`md_get(..).and_then(|v| v.to_u32()).unwrap_or(0)`: `Value::to_u32`, gguf_file.rs:249-254, takes the U32 variant
+    // only, so a key of any other type counts as 0 too instead of failing the load)
+    auto u32_or_zero = [&](const char* key) -> uint64_t {
+        const Value* v = find_value(g, key);
+        return v && v->type == 4 ? v->u : 0;
+    };
+    const uint64_t n_expert = u32_or_zero("llama.expert_count"), n_used = u32_or_zero("llama.expert_used_count");
     if (n_expert <= 1) return fail(MOE_E_INVALID, "llama.expert_count is " + std::to_string(n_expert) + ": the file has dense feed-forward layers, no MoE block");
     // n_used == 0 (key absent or zero): the reference builds the block all the same and its forward selects no expert
     // (`take(0)`, quantized_llama.rs:167): a layer with top_k = 0 whose output is zero

@@ -26,6 +26,8 @@ __device__ inline GroupSlots group_slots(const ExpertParams& p, int grp, int* li
     if (!p.rb.direct) {
         gs.s_begin = p.rb.offsets[p.group0 + grp];
         gs.n = p.rb.offsets[p.group0 + grp + 1] - gs.s_begin;
+        // the grid and the output hold max_rows rows per group: a table that says more is never followed past them
+        if (gs.n > (int)p.max_rows) gs.n = (int)p.max_rows;
         gs.list = nullptr;
         return gs;
     }

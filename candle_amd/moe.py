@@ -312,6 +312,14 @@ class GgufFile:
         _check(L.moe_gguf_metadata_array_len(self._h, k, C.byref(n), C.byref(et)))
         return ("array", n.value, et.value)
 
+    def metadata_u32_or_zero(self, key):
+        """`md_get(key).and_then(|v| v.to_u32()).unwrap_or(0)`: the value of a U32 key, 0 for a missing key and for
+        one of any other type (`Value::to_u32`, gguf_file.rs:249-254, takes the U32 variant only)."""
+        vt = C.c_int()
+        if load_library().moe_gguf_metadata_type(self._h, key.encode(), C.byref(vt)) or vt.value != 4:
+            return 0
+        return int(self.metadata(key))
+
     def tensor(self, name):
         """(ggml dtype id, shape, bytes as a numpy uint8 view of the mapping)."""
         L = load_library()
@@ -389,11 +397,9 @@ class SparseMoeBlock:
             self._h = h
             self.hidden, self.ffn, self.dtype = hdim, f, dt
             self.dtype_down = g.tensor(prefix + ".ffn_down.0.weight")[0]
-            self.n_experts = g.metadata("llama.expert_count")
-            try:
-                self.top_k = g.metadata("llama.expert_used_count")
-            except MoeError:
-                self.top_k = 0   # the reference's default for a missing key (quantized_llama.rs:510-512)
+            # the reference's default for a missing key or one that is not a U32 is 0 (quantized_llama.rs:507-512)
+            self.n_experts = g.metadata_u32_or_zero("llama.expert_count")
+            self.top_k = g.metadata_u32_or_zero("llama.expert_used_count")
             self.shared_ffn = 0
             return self
         finally:

@@ -73,6 +73,20 @@ def test_both_magics_are_accepted(tmp_path):
             assert g.tensor_names() == []
 
 
+def test_expert_count_keys_of_another_type_read_as_zero(tmp_path):
+    # `md_get(key).and_then(|v| v.to_u32()).unwrap_or(0)` (quantized_llama.rs:507-512): `Value::to_u32`
+    # (gguf_file.rs:249-254) takes the U32 variant only, so a string, a u64 or a missing key all give 0
+    p = tmp_path / "keys.gguf"
+    W.write_gguf(p, [("llama.expert_count", W.U32, 8), ("llama.expert_used_count", W.STRING, "2"),
+                     ("llama.block_count", W.U64, 32)], [("t", 0, (4,), np.zeros(4, np.float32).tobytes())])
+    with candle_amd.GgufFile(str(p)) as g:
+        assert g.metadata_u32_or_zero("llama.expert_count") == 8
+        assert g.metadata_u32_or_zero("llama.expert_used_count") == 0
+        assert g.metadata_u32_or_zero("llama.block_count") == 0
+        assert g.metadata_u32_or_zero("llama.absent") == 0
+        assert g.metadata("llama.expert_used_count") == "2"
+
+
 def test_malformed_files_are_rejected(tmp_path):
     good = tmp_path / "good.gguf"
     W.write_gguf(good, [("k", W.U32, 1)], [("t", 12, (256,), rnd(144))])

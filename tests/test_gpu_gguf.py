@@ -81,6 +81,27 @@ def test_missing_expert_used_count_gives_the_reference_zeros(tmp_path):
     layer.close()
 
 
+def test_expert_used_count_of_another_type_counts_as_zero(tmp_path):
+    # a string-typed (or u64) `llama.expert_used_count` is not an error in the reference: `to_u32` fails and
+    # `unwrap_or(0)` makes it 0 (quantized_llama.rs:507-512), the same layer as with the key absent
+    H, F, E, k = 512, 1024, 8, 2
+    gate, w1, w3, w2 = build(O.Q4K)
+    for i, (vt, v) in enumerate(((W.STRING, "2"), (W.U64, 2))):
+        p = tmp_path / ("typed%d.gguf" % i)
+        W.moe_layer_file(p, 0, gate, w1, w3, w2, O.Q4K, k, expert_keys=False,
+                         extra_metadata=[("llama.expert_count", W.U32, E), ("llama.expert_used_count", vt, v)])
+        layer = candle_amd.SparseMoeBlock.from_gguf(str(p), 0)
+        assert layer.top_k == 0 and layer.n_experts == E
+        assert not layer.forward(activations(5, H, 6)).any()
+        layer.close()
+    # the expert count itself as a u64: 0 experts to the reference, i.e. the dense arm
+    p = tmp_path / "typed_count.gguf"
+    W.moe_layer_file(p, 0, gate, w1, w3, w2, O.Q4K, k, expert_keys=False,
+                     extra_metadata=[("llama.expert_count", W.U64, E), ("llama.expert_used_count", W.U32, k)])
+    with pytest.raises(candle_amd.MoeError, match="expert_count is 0"):
+        candle_amd.SparseMoeBlock.from_gguf(str(p), 0)
+
+
 def test_loader_errors(tmp_path):
     H, F, E, k = 512, 1024, 8, 2
     gate, w1, w3, w2 = build(O.Q4K)

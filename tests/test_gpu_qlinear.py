@@ -125,15 +125,24 @@ def test_projection_recorded_into_a_hip_graph(m):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
         lin.forward(x_in, out=y_out)
+    # Eager calls with another row count between the replays: a replay rewrites the routing table in the workspace the
+    # eager calls share, so an eager call after it must write the table again (a stale table of 8 rows would have the
+    # product of 3 rows write rows 3..7 past its output: the rows behind the output are a canary).
+    x3 = torch.from_numpy(activations(3, k, seed=1)).cuda()
+    want3 = lin.forward(x3).clone()
+    check(dt, want3.cpu().numpy(), O.matmul(dt, x3.cpu().numpy(), w, n))
+    out3 = torch.empty(3 + 8, n, device="cuda")
     for rep in range(2):
         for x, want in zip(xs, eager):
             x_in.copy_(x)
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(y_out, want)
-            # eager calls with other row counts in between rewrite the routing table; the graph carries its own pass
-            lin.forward(torch.from_numpy(activations(3, k, seed=1)).cuda())
+            out3.fill_(-7.0)
+            lin.forward(x3, out=out3[:3])
             torch.cuda.synchronize()
+            assert torch.equal(out3[:3], want3)
+            assert bool((out3[3:] == -7.0).all()), "the eager product wrote past its output"
     # a larger eager call moves the workspace to new memory; the graph's nodes keep using the old, which stays alive
     big = torch.from_numpy(activations(m + 300, k, seed=2)).cuda()
     want_big = O.matmul(dt, big.cpu().numpy(), w, n)

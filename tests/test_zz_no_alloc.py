@@ -76,3 +76,23 @@ def test_noalloc_entry_under_stream_capture():
             assert torch.equal(y_out, want)
             assert torch.equal(gpu.forward(x), want)
     gpu.close()
+
+
+def test_noalloc_entry_between_allocating_calls_on_three_streams():
+    # allocating call on stream A, the entry that allocates nothing on B, allocating call on C: each has to wait for
+    # the one before it (they share the layer's side stream and events, and the two allocating calls its workspace)
+    torch = pytest.importorskip("torch")
+    ref, gpu = make_pair(256, 512, 12, 4, O.Q8_0, seed=35, Fs=1024)
+    xs = [torch.from_numpy(activations(T, 256, 40 + i)).cuda() for i, T in enumerate((48, 20, 33))]
+    want = [gpu.forward(x).clone() for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        outs = []
+        for i, (x, st) in enumerate(zip(xs, streams)):
+            with torch.cuda.stream(st):
+                outs.append(gpu.forward(x, noalloc=(i == 1)))
+        torch.cuda.synchronize()
+        for y, w in zip(outs, want):
+            assert torch.equal(y, w), rep
+    gpu.close()
