@@ -254,6 +254,35 @@ def measure_decode(args, np, torch, timer, layer, B, fmt="q4_k"):
             "roofline": roofline, "xs": xs, "ys": ys}
 
 
+def measure_decode_batches(args, np, torch, timer, layer, batches=(1, 8, 64)):
+    """The other batch sizes BASELINE config 2 names, briefly (200 timed steps each): step time and the share of the HBM
+    peak the step's algorithmic bytes reach.  Batch 1 also as a HIP graph of four forwards (the four rotating inputs,
+    whose routings differ) replayed back to back: what the step takes without the host's launch gaps."""
+    out = []
+    for B in batches:
+        xs, ys = activations(torch, B, H)
+        ms, _, _ = timer.run(lambda i: layer.forward(xs[i % 4], out=ys[i % 4]), MIN_TIMED_STEPS, 10, min_warm_seconds=0.3)
+        active = []
+        for i in range(4):   # the four inputs select different experts: bytes are those of their mean
+            layer.forward(xs[i], out=ys[i])
+            active.append(int((np.diff(layer.last_routing(B)[2])[:E] > 0).sum()))
+        n_active = sum(active) / 4.0
+        step_bytes = n_active * EXPERT_BYTES + E * H * 4 + 2 * B * H * 4
+        rec = {"batch": B, "active_experts": n_active, "us_per_step": ms * 1e3, "tokens_per_s": B / (ms * 1e-3),
+               "step_algorithmic_bytes": step_bytes, "step_hbm_frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        if B == 1:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=timer.stream):
+                for i in range(4):
+                    layer.forward(xs[i], out=ys[i])
+            g_ms, _, _ = timer.run(lambda i: graph.replay(), 50, 5, min_warm_seconds=0.2)
+            rec["graph_us_per_step"] = g_ms * 1e3 / 4
+            rec["graph_step_hbm_frac"] = step_bytes / (g_ms * 1e-3 / 4) / 1e9 / HBM_PEAK_GBS
+            del graph
+        out.append(rec)
+    return out
+
+
 def measure_prefill(args, np, torch, timer, layer, B):
     xs, ys = activations(torch, B, H, n=2)
     n_steps = max(20, min(args.steps, 50))
@@ -474,6 +503,9 @@ def main():
             layer.forward(m["xs"][0], out=m["ys"][0])
             torch.cuda.synchronize()
             cpu = cpu_baseline(w, m["xs"][0].cpu().numpy(), layer.last_logits(B), args.cpu_seconds)
+        if wl == "all" or (wl == "decode" and q4k and args.batch is None):
+            # the other batch sizes of BASELINE config 2, on the same layer
+            cfg["decode_batches"] = measure_decode_batches(args, np, torch, timer, layer)
         if wl == "all":
             out["metric"] = "MoE layer tokens/s; decode HBM GB/s %peak; prefill MFMA util, Mixtral-8x7B Q4_K"
             # prefill on the same weights, with the router bias that skews the load

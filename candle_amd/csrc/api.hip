@@ -269,6 +269,9 @@ Switches& switches() {
 
 using namespace moe;
 
+struct moe_qlinear;
+static int enqueue_qlinear(moe_qlinear* Q, const float* d_x, int64_t m, float* d_y, hipStream_t s);
+
 // The pieces of one forward's workspace (device pointers).
 struct Workspace {
     RouteBufs rb;
@@ -276,6 +279,8 @@ struct Workspace {
     float* yw = nullptr;
     float* hbuf = nullptr;
     float* ab_shared = nullptr;   // [2][T][Fs]: silu(w1 x) and w3 x of the always-on expert at a few tokens
+    float* xn = nullptr;          // quantised router, layers with the pre-norm: the normed rows [T][H]
+    float* logits_pad = nullptr;  // quantised router: the dense product's rows [T][E rounded up to 16]
 };
 
 // Which kernels a forward of T tokens takes.
@@ -292,6 +297,10 @@ struct moe_layer {
     float rms_eps = 0.f;
     DevBuf weights;                 // all re-laid expert matrices
     DevBuf gate, gate_bias, shared_gate, rms_alpha, groups;
+    // a router tensor kept quantised (moe_desc.gate_dtype): the [E, H] blocks as a dense projection of E16 = E rounded up
+    // to the layout's 16-row tiles (the extra rows are zero blocks), applied to the rows the experts see
+    moe_qlinear* gate_q = nullptr;
+    int64_t E16 = 0;
     std::vector<GroupWeights> host_groups;  // E routed (+1 shared)
     std::mutex mu;
     GrowBuf ws;                     // per-call workspace, grown on demand, cut anew for every call
@@ -331,7 +340,13 @@ static int check_desc(const moe_desc* d) {
     if (d->top_k < 0 || d->top_k > d->n_experts || d->top_k > 16)
         return fail(MOE_E_INVALID, "top_k must be in 0..min(n_experts,16)");
     if (d->top_k == 0 && d->shared_ffn > 0) return fail(MOE_E_INVALID, "top_k = 0 with a shared expert is not supported");
-    if (!d->gate || !d->w1 || !d->w2 || !d->w3) return fail(MOE_E_INVALID, "gate, w1, w2, w3 must be set");
+    if ((!d->gate && !d->gate_dtype) || !d->w1 || !d->w2 || !d->w3) return fail(MOE_E_INVALID, "gate, w1, w2, w3 must be set");
+    if (d->gate_dtype) {
+        if (!weight_dtype_supported(d->gate_dtype)) return fail(MOE_E_INVALID, "unsupported gate_dtype " + std::to_string(d->gate_dtype));
+        if (!d->gate_blocks) return fail(MOE_E_INVALID, "gate_dtype is set but gate_blocks is NULL");
+        if (d->hidden % 256) return fail(MOE_E_INVALID, "a quantised router needs hidden to be a multiple of 256");
+        if (d->shared_ffn > 0) return fail(MOE_E_INVALID, "a quantised router together with a shared expert is not supported");
+    }
     for (int64_t e = 0; e < d->n_experts; e++)
         if (!d->w1[e] || !d->w2[e] || !d->w3[e]) return fail(MOE_E_INVALID, "expert " + std::to_string(e) + " has a NULL matrix");
     if (d->shared_ffn < 0) return fail(MOE_E_INVALID, "shared_ffn < 0");
@@ -365,7 +380,15 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
     L->dt = d->ggml_dtype; L->dt_down = d->ggml_dtype_down ? d->ggml_dtype_down : L->dt;
     L->vdt = vecdot_dtype(L->dt); L->norm_topk = d->norm_topk ? 1 : 0;
     L->rms_eps = d->rms_eps;
-    if ((rc = upload_f32(L->gate, d->gate, (size_t)L->E * L->H))) return bail(rc);
+    if (d->gate_dtype) {
+        // QMatMul::QTensor arm (quantized/mod.rs:428-447, 533-537): the blocks stay as they are, padded with zero blocks
+        // (every format reads all-zero bytes as zeros) to the 16-row tiles of the dense projections
+        L->E16 = (L->E + 15) / 16 * 16;
+        const size_t row_bytes = (size_t)(L->H / block_elems(d->gate_dtype) * block_bytes(d->gate_dtype));
+        std::vector<uint8_t> padded((size_t)L->E16 * row_bytes, 0);
+        memcpy(padded.data(), d->gate_blocks, (size_t)L->E * row_bytes);
+        if ((rc = moe_qlinear_create(d->gate_dtype, padded.data(), L->E16, L->H, &L->gate_q))) return bail(rc);
+    } else if ((rc = upload_f32(L->gate, d->gate, (size_t)L->E * L->H))) return bail(rc);
     if (d->gate_bias) {
         L->has_bias = true;
         if ((rc = upload_f32(L->gate_bias, d->gate_bias, (size_t)L->E))) return bail(rc);
@@ -433,6 +456,7 @@ extern "C" int moe_layer_create(const moe_desc* d, moe_layer** out) {
 extern "C" void moe_layer_destroy(moe_layer* L) {
     if (!L) return;
     (void)hipDeviceSynchronize();
+    if (L->gate_q) moe_qlinear_destroy(L->gate_q);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->side) (void)hipStreamDestroy(L->side);
     if (L->fork) (void)hipEventDestroy(L->fork);
@@ -528,6 +552,10 @@ static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& 
     w.yw = c.take<float>((size_t)S * L->H * 4);
     if (pl.hbuf) w.hbuf = c.take<float>((size_t)T * L->k * L->F * 4);
     if (pl.shared_rows) w.ab_shared = c.take<float>((size_t)2 * T * L->Fs * 4);
+    if (L->gate_q) {
+        if (L->has_rms) w.xn = c.take<float>((size_t)T * L->H * 4);
+        w.logits_pad = c.take<float>((size_t)T * L->E16 * 4);
+    }
     if (ws) *ws = w;
     return c.off;
 }
@@ -560,6 +588,18 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
     fp.rb.tile_slots = pl.tile_slots;
     if (pl.accumulate) fp.y_zero = d_y;
     MOE_MARK(ST_BEGIN);
+    if (L->gate_q) {
+        // The quantised router: logits = the gate matrix's quantised product over the rows the experts see, quantised to
+        // the gate dtype's own activation format; then routing and the experts' activation quantisation from those logits.
+        if (L->has_rms) {
+            MOE_HIP_CHECK(launch_add_rms_norm(d_x, nullptr, fp.rms_alpha, fp.rms_eps, T, (int)L->H, nullptr, ws.xn, s));
+            fp.x = ws.xn;
+            fp.rms_alpha = nullptr;
+        }
+        if (int rc = enqueue_qlinear(L->gate_q, fp.x, T, ws.logits_pad, s)) return rc;
+        MOE_HIP_CHECK(launch_logits_unpad(ws.logits_pad, (int)L->E16, fp.gate_bias, fp.rb.logits, T, (int)L->E, s));
+        MOE_HIP_CHECK(launch_front_route(fp, s));
+    } else
     MOE_HIP_CHECK(launch_front(fp, s));
     MOE_MARK(ST_FRONT);
     if (!pl.direct) MOE_HIP_CHECK(launch_dispatch(fp.rb, T, (int)L->E, (int)L->k, shared, s));
@@ -762,6 +802,7 @@ extern "C" int moe_layer_forward_device_noalloc(moe_layer* L, const void* d_x, i
     if (T == 0) { L->last_T = 0; return MOE_OK; }
     if (T > max_tokens_per_pass(L))
         return fail(MOE_E_INVALID, "moe_layer_forward_device_noalloc: " + std::to_string(T) + " tokens are more than one pass carries");
+    if (L->gate_q) return fail(MOE_E_INVALID, "moe_layer_forward_device_noalloc: a layer with a quantised router allocates the workspace of its gate product; use moe_layer_forward_device");
     const ForwardPlan pl = plan_forward(L, T);
     const size_t need = L->k > 0 ? carve_workspace(L, T, pl, nullptr, nullptr) : 0;
     if (need > STATIC_SCRATCH_BYTES)

@@ -360,6 +360,8 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     if (rc) return rc;
     if (nd != 2 || (uint64_t)dims[0] != n_expert) return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: expected shape [expert_count, hidden]");
     const int64_t E = dims[0], H = dims[1];
+    int gate_dtype = 0;
+    const void* gate_blocks = nullptr;
     std::vector<float> gate((size_t)(E * H));
     if (dt == 0) memcpy(gate.data(), data, gate.size() * 4);
     else if (dt == 1) {
@@ -371,11 +373,12 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
             const uint32_t bits = (uint32_t)h[i] << 16;
             memcpy(&gate[i], &bits, 4);
         }
-    } else
-        // QMatMul::from_arc (candle-core/src/quantized/mod.rs:429-443) dequantises F32, F16 and BF16 only; a quantised
-        // router would run as a quantised product over Q8-quantised activations, with other logits than an f32 gate
-        // gives.  llama.cpp never quantises this tensor; such a file is refused rather than routed differently.
-        return fail(MOE_E_INVALID, prefix + ".ffn_gate_inp.weight: dtype " + std::to_string(dt) + " is not supported for the router (supported: F32, F16, BF16)");
+    } else {
+        // QMatMul::from_arc (candle-core/src/quantized/mod.rs:429-443) dequantises F32, F16 and BF16 only; any other
+        // router tensor stays a QTensor and its logits are a quantised product over Q8-quantised rows (moe_desc.gate_dtype)
+        gate_dtype = dt;
+        gate_blocks = data;
+    }
 
     std::vector<const void*> w1((size_t)E), w2((size_t)E), w3((size_t)E);
     int up_dt = -1, down_dt = -1;   // gate / up matrices share one dtype, down matrices one
@@ -404,6 +407,7 @@ extern "C" int moe_layer_create_from_gguf(const moe_gguf* g, int layer_index, in
     d.hidden = H; d.ffn = F; d.n_experts = E; d.top_k = (int64_t)n_used;
     d.ggml_dtype = up_dt; d.ggml_dtype_down = down_dt == up_dt ? 0 : down_dt; d.norm_topk = norm_topk;
     d.gate = gate.data();
+    d.gate_dtype = gate_dtype; d.gate_blocks = gate_blocks;
     d.w1 = w1.data(); d.w3 = w3.data(); d.w2 = w2.data();
     return moe_layer_create(&d, out);
 }

@@ -90,6 +90,10 @@ struct FrontParams {
 };
 // rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token.
 hipError_t launch_front(const FrontParams& p, hipStream_t s);
+// The front end of a layer whose router stays quantised: logits from the dense product's padded rows, then routing and
+// activation quantisation from rb.logits.
+hipError_t launch_logits_unpad(const float* padded, int n_pad, const float* bias, float* logits, int64_t T, int E, hipStream_t s);
+hipError_t launch_front_route(const FrontParams& p, hipStream_t s);
 // softmax + top-k from given logits (parity hook).
 hipError_t launch_route_from_logits(const float* logits, int64_t T, int E, int k, int norm_topk,
                                     const RouteBufs& rb, hipStream_t s);

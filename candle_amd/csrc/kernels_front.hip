@@ -1144,6 +1144,30 @@ __global__ __launch_bounds__(256) void front_route_kernel(FrontParams p) {
         for (int i = tid; i < H / 4; i += 256) reinterpret_cast<float4*>(p.y_zero + t * H)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
+// Logits of a quantised router: the dense product's [T, n_pad] rows cut to E columns, the optional bias added.
+__global__ void logits_unpad_kernel(const float* padded, int n_pad, const float* bias, float* logits, int64_t T, int E) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T * E) return;
+    const int64_t t = i / E;
+    const int e = (int)(i - t * E);
+    const float v = padded[t * n_pad + e];
+    logits[i] = bias ? v + bias[e] : v;
+}
+hipError_t launch_logits_unpad(const float* padded, int n_pad, const float* bias, float* logits, int64_t T, int E, hipStream_t s) {
+    if (T == 0) return hipSuccess;
+    hipLaunchKernelGGL(logits_unpad_kernel, dim3((unsigned)((T * E + 255) / 256)), dim3(256), 0, s, padded, n_pad, bias, logits, T, E);
+    return hipGetLastError();
+}
+// Routing and activation quantisation from logits that are already in p.rb.logits (no gate product, no pre-norm: p.x is
+// the row the experts see).
+hipError_t launch_front_route(const FrontParams& p, hipStream_t s) {
+    if (p.T == 0) return hipSuccess;
+    if (p.H % 256 || p.E > MAX_E) return hipErrorInvalidValue;
+    if (p.vdt == MOE_GGML_Q8K) hipLaunchKernelGGL(front_route_kernel<MOE_GGML_Q8K>, dim3((unsigned)p.T), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(front_route_kernel<MOE_GGML_Q8_0>, dim3((unsigned)p.T), dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
 static bool launch_front_split(const FrontParams& p, hipStream_t s) {
     const int sw = switches().front_split;
     const int NE = p.E + (p.shared_gate ? 1 : 0);

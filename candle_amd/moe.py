@@ -36,6 +36,7 @@ class _Desc(C.Structure):
         ("shared_ffn", C.c_int64), ("shared_w1", C.c_void_p), ("shared_w3", C.c_void_p), ("shared_w2", C.c_void_p),
         ("shared_gate", C.c_void_p), ("rms_alpha", C.c_void_p), ("rms_eps", C.c_float),
         ("ggml_dtype_down", C.c_int32),
+        ("gate_dtype", C.c_int32), ("gate_blocks", C.c_void_p),
     ]
 
 
@@ -338,7 +339,10 @@ class SparseMoeBlock:
 
     def __init__(self, hidden, ffn, n_experts, top_k, ggml_dtype, gate, w1, w3, w2, norm_topk=True,
                  gate_bias=None, shared_ffn=0, shared_w1=None, shared_w3=None, shared_w2=None,
-                 shared_gate=None, rms_alpha=None, rms_eps=1e-5, ggml_dtype_down=None):
+                 shared_gate=None, rms_alpha=None, rms_eps=1e-5, ggml_dtype_down=None, gate_dtype=None, gate_blocks=None):
+        """gate_dtype / gate_blocks: a router tensor kept quantised, as the reference keeps every `ffn_gate_inp` that is
+        not F32 / F16 / BF16 (`QMatMul::from_arc`, quantized/mod.rs:428-447): the raw blocks of the [E, H] tensor; `gate`
+        is then ignored and may be None."""
         L = load_library()
         dtype_down = ggml_dtype if ggml_dtype_down is None else ggml_dtype_down
         for dt in (ggml_dtype, dtype_down):
@@ -349,8 +353,16 @@ class SparseMoeBlock:
             raise MoeError("need one w1/w2/w3 per expert")
         self.hidden, self.ffn, self.n_experts, self.top_k, self.dtype = hidden, ffn, n_experts, top_k, ggml_dtype
         self.shared_ffn = shared_ffn
-        gate = _f32(gate).reshape(n_experts, hidden)
-        keep = [gate]
+        if gate_dtype:
+            if gate_dtype not in _BLOCK or gate_dtype in (GGML_Q8K, GGML_Q8_1):
+                raise MoeError("unsupported gate_dtype %r" % (gate_dtype,))
+            gate_q = _blocks(gate_blocks, gate_dtype, n_experts * hidden, "gate_blocks")
+            gate = np.zeros((n_experts, hidden), dtype=np.float32)   # not read by the library
+            keep = [gate, gate_q]
+        else:
+            gate_q = None
+            gate = _f32(gate).reshape(n_experts, hidden)
+            keep = [gate]
         mats = {}
         for name, ws in (("w1", w1), ("w3", w3), ("w2", w2)):
             arrs = [_blocks(w, dtype_down if name == "w2" else ggml_dtype, hidden * ffn, name) for w in ws]
@@ -375,7 +387,7 @@ class SparseMoeBlock:
                      C.cast(mats["w1"], C.POINTER(C.c_void_p)), C.cast(mats["w3"], C.POINTER(C.c_void_p)),
                      C.cast(mats["w2"], C.POINTER(C.c_void_p)), shared_ffn, ptr(sh["shared_w1"]), ptr(sh["shared_w3"]),
                      ptr(sh["shared_w2"]), ptr(opt["shared_gate"]), ptr(opt["rms_alpha"]), float(rms_eps),
-                     0 if dtype_down == ggml_dtype else dtype_down)
+                     0 if dtype_down == ggml_dtype else dtype_down, int(gate_dtype or 0), ptr(gate_q))
         handle = C.c_void_p()
         self._h = None
         _check(L.moe_layer_create(C.byref(desc), C.byref(handle)))

@@ -90,6 +90,14 @@ typedef struct {
      * dtypes must quantise activations the same way (Q2K ... Q6K use Q8K; Q4_0, Q5_0 and Q8_0 use Q8_0;
      * Q4_1 and Q5_1 use Q8_1). */
     int32_t ggml_dtype_down;
+    /* A router tensor that is not F32 / F16 / BF16 stays quantised in the reference: `QMatMul::from_arc`
+     * (candle-core/src/quantized/mod.rs:428-447) dequantises those three only, any other `ffn_gate_inp` runs as
+     * `QMatMul::QTensor`, i.e. the logits are a quantised product over the rows quantised to the gate dtype's
+     * activation format (mod.rs:533-537 -> k_quants::matmul, k_quants.rs:1873-1920).  gate_dtype != 0 selects that arm:
+     * gate_blocks holds the raw GGML blocks of the [E, H] tensor in that dtype (any dtype ggml_dtype accepts) and `gate`
+     * is not read.  hidden has to be a multiple of 256; not accepted together with a shared expert. */
+    int32_t gate_dtype;
+    const void* gate_blocks;
 } moe_desc;
 
 /* Uploads and re-lays the weights.  Replaces the construction at quantized_llama.rs:553-578. */

@@ -200,8 +200,16 @@ class Layer:
     """Block-level oracle: candle's MlpOrMoe::MoE forward on raw GGUF blocks."""
 
     def __init__(self, H, F, E, k, dtype, gate, w1, w3, w2, norm_topk=True, gate_bias=None,
-                 Fs=0, sw1=None, sw3=None, sw2=None, shared_gate=None, rms_alpha=None, rms_eps=1e-5, dtype_down=None):
+                 Fs=0, sw1=None, sw3=None, sw2=None, shared_gate=None, rms_alpha=None, rms_eps=1e-5, dtype_down=None,
+                 gate_dtype=None, gate_blocks=None):
+        """gate_dtype / gate_blocks: the router tensor kept quantised, the `QMatMul::QTensor` arm that
+        `QMatMul::from_arc` (candle-core/src/quantized/mod.rs:428-447) takes for every dtype but F32 / F16 / BF16: the
+        logits are then `k_quants::matmul` (k_quants.rs:1873-1920) of the rows the block sees against those blocks."""
         self.H, self.F, self.E, self.k, self.dtype = H, F, E, k, dtype
+        self.gate_dtype, self.gate_blocks, self.rms_eps = gate_dtype, gate_blocks, rms_eps
+        if gate_dtype:
+            assert np.asarray(gate_blocks).size == nbytes(gate_dtype, E * H)
+            gate = np.zeros((E, H), dtype=np.float32) if gate is None else gate
         self.dtype_down = dtype if dtype_down is None else dtype_down
         self._keep = []
 
@@ -233,9 +241,18 @@ class Layer:
                         ptr(self.sw[2]), ptr(self.shared_gate), ptr(self.rms_alpha), rms_eps,
                         0 if self.dtype_down == dtype else self.dtype_down)
 
+    def router_logits(self, xs, simd=False):
+        """Logits of the quantised router (`self.gate_blocks`) on the rows the block sees: after the pre-norm when the
+        layer carries one (quantized_llama.rs:886-890), plus the bias."""
+        seen = _f32(xs) if self.rms_alpha is None else rms_norm(xs, self.rms_alpha, self.rms_eps)
+        lo = matmul(self.gate_dtype, seen, self.gate_blocks, self.E, simd=simd)
+        return lo if self.gate_bias is None else (lo + self.gate_bias[None, :]).astype(np.float32)
+
     def forward(self, xs, logits=None, simd=False, threads=1, return_logits=False):
         xs = _f32(xs)
         T = xs.shape[0]
+        if logits is None and self.gate_dtype:
+            logits = self.router_logits(xs, simd=simd)
         ys = np.empty((T, self.H), dtype=np.float32)
         lo = np.empty((T, self.E), dtype=np.float32)
         li = None if logits is None else _f32(logits)

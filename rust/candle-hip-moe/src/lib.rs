@@ -56,6 +56,8 @@ pub mod ffi {
         pub rms_alpha: *const f32,
         pub rms_eps: f32,
         pub ggml_dtype_down: i32,
+        pub gate_dtype: i32,
+        pub gate_blocks: *const c_void,
     }
 
     extern "C" {
@@ -154,6 +156,8 @@ pub struct SharedExpert<'a> {
 /// library covers.  `experts[e] = (w1, w2, w3)` in the order of `Mlp` (feed_forward_w1 / w2 / w3, :117-122).
 pub struct HipSparseMoeConfig<'a> {
     pub gate: &'a Tensor,                         // ffn_gate_inp, dequantised: [n_experts, hidden]
+    pub gate_quantized: Option<&'a QTensor>,      // the same tensor kept quantised (any dtype but F32 / F16 / BF16): its logits
+                                                  // are then the quantised product the reference's QMatMul::QTensor arm computes
     pub experts: &'a [(QTensor, QTensor, QTensor)],
     pub n_expert_used: usize,                     // 0 is accepted: the reference then returns zeros (:167, :507-512)
     pub norm_topk: bool,                          // Mixtral: true (:175-178); qwen2-moe's norm_topk_prob
@@ -177,6 +181,7 @@ impl HipSparseMoe {
     pub fn new(gate: &Tensor, experts: &[(QTensor, QTensor, QTensor)], n_expert_used: usize) -> Result<Self> {
         Self::with_config(HipSparseMoeConfig {
             gate,
+            gate_quantized: None,
             experts,
             n_expert_used,
             norm_topk: true,
@@ -206,6 +211,16 @@ impl HipSparseMoe {
             }
         }
         let gate = f32_vec(cfg.gate)?;
+        // `gate_quantized`: the router as the reference runs it when `ffn_gate_inp` is not F32 / F16 / BF16
+        let gate_q = match cfg.gate_quantized {
+            Some(q) => {
+                if q.shape().dims2()? != (n_experts, hidden) {
+                    bail!("HipSparseMoe: the quantised gate is {:?}, expected [{n_experts}, {hidden}]", q.shape())
+                }
+                Some((q.dtype(), q.data()?))
+            }
+            None => None,
+        };
         let gate_bias = cfg.gate_bias.map(f32_vec).transpose()?;
         if let Some(b) = &gate_bias {
             if b.len() != n_experts {
@@ -279,6 +294,9 @@ impl HipSparseMoe {
             rms_eps: eps,
             // Q4_K_M files store ffn_down of some layers as Q6K beside Q4K gate / up matrices (0 = same dtype)
             ggml_dtype_down: if id_down == id { 0 } else { id_down },
+            // a router tensor the reference keeps quantised (QMatMul::from_arc, quantized/mod.rs:428-447)
+            gate_dtype: gate_q.as_ref().map_or(Ok(0), |(d, _)| ggml_id(*d))?,
+            gate_blocks: gate_q.as_ref().map_or(null, |(_, b)| b.as_ptr() as *const c_void),
         };
         let mut handle = std::ptr::null_mut();
         // SAFETY: every pointer in desc refers to a live buffer of the size the header states; the library only

@@ -58,13 +58,22 @@ def test_router_stored_as_f16_bf16_or_quantised(tmp_path):
     b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, (gb.astype(np.uint32) << 16).view(np.float32).reshape(E, H), w1, w3, w2)
     assert np.array_equal(bits(a.forward(xs)), bits(b.forward(xs)))
     a.close(); b.close()
-    # Q8_0 router: the reference would run it as a quantised product over Q8_0-quantised activations (QMatMul::QTensor
-    # arm), which gives other logits than the f32 gate; llama.cpp never quantises this tensor.  Refused, not approximated.
+    # Q8_0 router: the reference runs it as a quantised product over Q8_0-quantised rows (the QMatMul::QTensor arm of
+    # QMatMul::from_arc, quantized/mod.rs:428-447), which gives other logits than the dequantised gate would
     gq = O.quantize(O.Q8_0, gate.reshape(-1))
     pq = tmp_path / "q8.gguf"
     W.moe_layer_file(pq, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=O.Q8_0, gate_blocks=gq)
-    with pytest.raises(candle_amd.MoeError, match="not supported for the router"):
-        candle_amd.SparseMoeBlock.from_gguf(str(pq), 0)
+    a = candle_amd.SparseMoeBlock.from_gguf(str(pq), 0)
+    b = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, None, w1, w3, w2, gate_dtype=O.Q8_0, gate_blocks=gq)
+    ya = a.forward(xs)
+    assert np.array_equal(bits(ya), bits(b.forward(xs)))
+    assert np.array_equal(bits(a.last_logits(xs.shape[0])), bits(O.matmul(O.Q8_0, xs, gq, E)))
+    a.close(); b.close()
+    # a dtype no quantised product exists for (Q8_1 = 9 is an activation format)
+    pq1 = tmp_path / "q81.gguf"
+    W.moe_layer_file(pq1, 0, gate, w1, w3, w2, O.Q4K, k, gate_dtype=9, gate_blocks=np.zeros(E * H // 32 * 36, np.uint8))
+    with pytest.raises(candle_amd.MoeError, match="unsupported gate_dtype 9"):
+        candle_amd.SparseMoeBlock.from_gguf(str(pq1), 0)
 
 
 def test_missing_expert_used_count_gives_the_reference_zeros(tmp_path):

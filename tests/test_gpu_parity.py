@@ -8,7 +8,7 @@ import pytest
 
 import candle_amd
 import pyoracle as O
-from helpers import CONFIGS, activations, make_pair, rms
+from helpers import CONFIGS, activations, make_pair, make_weights, rms
 
 pytestmark = pytest.mark.gpu
 
@@ -890,3 +890,47 @@ def test_concurrent_forward_from_several_threads():
         t.join()
     assert not errors, errors
     gpu_a.close(); gpu_b.close()
+
+
+@pytest.mark.parametrize("gate_dt,rms_norm,bias", [(O.Q8_0, False, False), (O.Q4_0, True, True), (O.Q5_1, False, False),
+                                                   (O.Q4K, True, False), (O.Q6K, False, True)])
+def test_quantised_router(gate_dt, rms_norm, bias):
+    # A router tensor that is not F32 / F16 / BF16 stays quantised in the reference (QMatMul::from_arc,
+    # quantized/mod.rs:428-447): the logits are k_quants::matmul of the rows the block sees (quantised to the gate dtype's
+    # activation format) against the gate's blocks.  Logits against the oracle's matmul (the 32-element formats add their
+    # block values in the reference's order: bit for bit), routing bit-exact given the logits, outputs at the usual bar.
+    H, F, E, k = 512, 1024, 8, 2
+    w1, w3, w2, _ = make_weights(H, F, E, O.Q4K, 61)
+    gate = O.fill_normal(6161, E * H, 0.0, 0.02)
+    gq = O.quantize(gate_dt, gate)
+    gb = O.fill_normal(6162, E, 0.0, 0.5) if bias else None
+    alpha = (1.0 + 0.1 * O.fill_normal(6163, H)).astype(np.float32) if rms_norm else None
+    ref = O.Layer(H, F, E, k, O.Q4K, None, w1, w3, w2, gate_bias=gb, rms_alpha=alpha, gate_dtype=gate_dt, gate_blocks=gq)
+    gpu = candle_amd.SparseMoeBlock(H, F, E, k, O.Q4K, None, w1, w3, w2, gate_bias=gb, rms_alpha=alpha, gate_dtype=gate_dt, gate_blocks=gq)
+    for T in (1, 7, 40, 300):
+        xs = activations(T, H, 33 + T)
+        ys = gpu.forward(xs)
+        logits = gpu.last_logits(T)
+        want_logits = ref.router_logits(xs)
+        if O.BLOCK_ELEMS[gate_dt] == 32:
+            assert np.array_equal(bits(logits), bits(want_logits)), (gate_dt, T)
+        else:
+            assert np.abs(logits - want_logits).max() <= 1e-4 * rms(want_logits), (gate_dt, T)
+        gi, gw, goff, gperm, gpw = gpu.last_routing(T)
+        ri, rw, roff, rperm, rpw = O.route(O.softmax_last_dim(logits), k)
+        assert np.array_equal(gi, ri) and np.array_equal(bits(gw), bits(rw))
+        assert np.array_equal(goff, roff) and np.array_equal(gperm, rperm) and np.array_equal(bits(gpw), bits(rpw))
+        want = ref.forward(xs, logits=logits)
+        moe = want - xs if rms_norm else want
+        assert np.abs(ys - want).max() <= block_tol(O.Q4K, F) * rms(moe), (gate_dt, T)
+        # the device entry takes the same path
+        import torch
+        yd = gpu.forward(torch.from_numpy(xs).cuda()).cpu().numpy()
+        assert np.array_equal(bits(yd), bits(ys))
+    with pytest.raises(candle_amd.MoeError, match="quantised router"):
+        import torch
+        gpu.forward(torch.from_numpy(activations(4, H, 1)).cuda(), noalloc=True)
+    gpu.close()
+    with pytest.raises(candle_amd.MoeError, match="multiple of 256"):
+        candle_amd.SparseMoeBlock(128, 256, 4, 2, O.Q8_0, None, [np.zeros(128 * 256 // 32 * 34, np.uint8)] * 4, [np.zeros(128 * 256 // 32 * 34, np.uint8)] * 4,
+                                  [np.zeros(128 * 256 // 32 * 34, np.uint8)] * 4, gate_dtype=O.Q8_0, gate_blocks=np.zeros(4 * 128 // 32 * 34, np.uint8))

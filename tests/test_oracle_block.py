@@ -121,3 +121,27 @@ def test_scalar_and_avx2_paths_of_the_reference_flip_requantised_values(O):
     # without a flip the two paths agree to 1e-5; every flip shows up as an O(1e-3) outlier
     assert (flips == 0 and diff < 1e-4) or (flips > 0 and 2e-4 < diff < 2e-2)
     assert np.sqrt(((y0 - y1).astype(np.float64) ** 2).mean()) / r < 5e-4
+
+
+def test_quantised_router_logits_follow_the_quantised_product(O):
+    # QMatMul::from_arc (candle-core/src/quantized/mod.rs:428-447) keeps a router tensor of any dtype but F32 / F16 / BF16
+    # as a QTensor: logits = k_quants::matmul on the rows the block sees.  Close to the dequantised gate's logits (the
+    # gate and the rows are each quantised once), and what forward() routes by when no logits are handed in.
+    H, F, E, k = 256, 512, 8, 2
+    rng = np.random.default_rng(5)
+    gate = (rng.standard_normal((E, H)) * 0.02).astype(np.float32)
+    xs = rng.standard_normal((6, H)).astype(np.float32)
+    w = [O.fill_normal_quantized(70 + e, O.Q8_0, F, H, 0.02) for e in range(E)]
+    w2 = [O.fill_normal_quantized(80 + e, O.Q8_0, H, F, 0.02) for e in range(E)]
+    alpha = (1.0 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    for dt in (O.Q8_0, O.Q4K):
+        gq = O.quantize(dt, gate.reshape(-1))
+        layer = O.Layer(H, F, E, k, O.Q8_0, None, w, w, w2, rms_alpha=alpha, gate_dtype=dt, gate_blocks=gq)
+        seen = O.rms_norm(xs, alpha, 1e-5)
+        lo = layer.router_logits(xs)
+        assert np.array_equal(lo, O.matmul(dt, seen, gq, E))
+        dense = seen.astype(np.float64) @ O.dequantize(dt, gq, E * H).reshape(E, H).astype(np.float64).T
+        assert np.abs(lo - dense).max() < (0.02 if dt == O.Q8_0 else 0.05) * np.abs(dense).max()
+        ys, lo2 = layer.forward(xs, return_logits=True)
+        assert np.array_equal(lo2, lo)
+        assert np.array_equal(ys, layer.forward(xs, logits=lo))

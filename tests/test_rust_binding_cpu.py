@@ -101,7 +101,7 @@ def rust_items():
 def test_moe_desc_layout_matches_the_header():
     c_fields = c_desc_fields()
     r_fields, _ = rust_items()
-    assert len(c_fields) == 19
+    assert len(c_fields) == 21
     assert r_fields == c_fields
 
 
