@@ -359,13 +359,22 @@ def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32
     x_next = torch.empty_like(x0)
 
     def step(_):
+        # one call for the 32 layers (moe_stack_forward_device): a layer's combine pass + residual and the next layer's
+        # rms-norm / router / quantiser are one launch
+        h = candle_amd.stack_forward(layers, state["h"], out=bufs[0])
+        noise.normal_(0.0, 0.1, generator=g)
+        state["h"] = torch.add(h, noise, out=x_next)   # the next step's input
+
+    def step_layer_by_layer(_):
         h = state["h"]
         for i, layer in enumerate(layers):
             layer.forward(h, out=bufs[i & 1])
             h = bufs[i & 1]
         noise.normal_(0.0, 0.1, generator=g)
-        state["h"] = torch.add(h, noise, out=x_next)   # the next step's input
+        state["h"] = torch.add(h, noise, out=x_next)
 
+    lbl_ms, _, _ = timer.run(step_layer_by_layer, 32, 2, min_warm_seconds=0.2)
+    state["h"] = x0
     ms, wall_ms, warmed = timer.run(step, n_steps, min(args.warmup, 3), min_warm_seconds=0.3)
     finite = bool(torch.isfinite(state["h"]).all())
     # stage times of a mid-stack layer, measured right after its predecessors ran (its weights and gate are cold)
@@ -389,6 +398,7 @@ def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32
         layer.close()
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "layers": n_layers, "batch": B, "resident_gb": n_layers * E * EXPERT_BYTES / 1e9, "us_per_layer": ms * 1e3 / n_layers,
+            "entry": "moe_stack_forward_device (one call per step)", "layer_by_layer_ms_per_step": lbl_ms,
             "mid_stack_stage_us": stage_us, "output_finite": finite, "step_algorithmic_bytes": step_bytes,
             "step_hbm_frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "roofline": {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation), layer %d of the stack" % mid,

@@ -279,6 +279,7 @@ struct Workspace {
     float* yw = nullptr;
     float* hbuf = nullptr;
     float* ab_shared = nullptr;   // [2][T][Fs]: silu(w1 x) and w3 x of the always-on expert at a few tokens
+    float* xin = nullptr;         // stacks: the layer's input row [T][H] when the layer before leaves its combine pass to this one
     float* xn = nullptr;          // quantised router, layers with the pre-norm: the normed rows [T][H]
     float* logits_pad = nullptr;  // quantised router: the dense product's rows [T][E rounded up to 16]
 };
@@ -539,7 +540,7 @@ static ForwardPlan plan_forward(const moe_layer* L, int64_t T) {
 }
 
 // Cuts the workspace of a forward of T tokens out of `base`; returns the bytes it takes (base == nullptr: only that).
-static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& pl, uint8_t* base, Workspace* ws) {
+static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& pl, uint8_t* base, Workspace* ws, bool stack_input = false) {
     Carver c;
     c.base = base;
     const bool shared = L->Fs > 0;
@@ -552,6 +553,7 @@ static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& 
     w.yw = c.take<float>((size_t)S * L->H * 4);
     if (pl.hbuf) w.hbuf = c.take<float>((size_t)T * L->k * L->F * 4);
     if (pl.shared_rows) w.ab_shared = c.take<float>((size_t)2 * T * L->Fs * 4);
+    if (stack_input) w.xin = c.take<float>((size_t)T * L->H * 4);
     if (L->gate_q) {
         if (L->has_rms) w.xn = c.take<float>((size_t)T * L->H * 4);
         w.logits_pad = c.take<float>((size_t)T * L->E16 * 4);
@@ -561,8 +563,10 @@ static size_t carve_workspace(const moe_layer* L, int64_t T, const ForwardPlan& 
 }
 
 // Enqueues one forward of T tokens on `s` with the workspace `ws`.  Caller holds L->mu.
+// In a stack (moe_stack_forward_device): `prev` = the layer before left its combine pass to this layer's front kernel,
+// which writes this layer's input to ws.xin (d_x is not read); `leave_combine` = this layer leaves its own to the next.
 static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace& ws, const float* d_x, int64_t T, float* d_y,
-                           hipStream_t s, hipEvent_t* marks = nullptr) {
+                           hipStream_t s, hipEvent_t* marks = nullptr, const PrevCombine* prev = nullptr, bool leave_combine = false) {
 #define MOE_MARK(i) do { if (marks) MOE_HIP_CHECK(hipEventRecord(marks[i], s)); } while (0)
     if (L->k == 0) {
         // nothing is selected: the block's output is zero (quantized_llama.rs:167 `take(0)`), plus the residual of a
@@ -587,6 +591,11 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
     fp.rb.direct = pl.direct ? 1 : 0;
     fp.rb.tile_slots = pl.tile_slots;
     if (pl.accumulate) fp.y_zero = d_y;
+    if (prev) {
+        fp.prev = *prev;
+        fp.prev.x_out = ws.xin;
+        d_x = ws.xin;   // this layer's residual
+    }
     MOE_MARK(ST_BEGIN);
     if (L->gate_q) {
         // The quantised router: logits = the gate matrix's quantised product over the rows the experts see, quantised to
@@ -714,7 +723,7 @@ static int enqueue_forward(moe_layer* L, const ForwardPlan& pl, const Workspace&
     else if (shared)
         if (int rc = run_shared()) return rc;
     MOE_MARK(ST_SHARED);
-    if (!pl.accumulate) MOE_HIP_CHECK(launch_combine(ws.yw, fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
+    if (!pl.accumulate && !leave_combine) MOE_HIP_CHECK(launch_combine(ws.yw, fp.rb, shared, L->has_rms ? d_x : nullptr, d_y, T, (int)L->H, s));
     MOE_MARK(ST_COMBINE);
 #undef MOE_MARK
     L->last_direct = pl.direct;
@@ -766,6 +775,91 @@ extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T
         if (rc) return rc;
     }
     if (T > step && L->k > 0) L->last_T = -1;   // the routing hooks describe one pass only
+    return MOE_OK;
+}
+
+// ------------------------------------------------------------------ a stack of layers
+// y = layer[n-1](... layer[1](layer[0](x))), quantized_llama.rs:886-892 for the MoE blocks of consecutive transformer layers.
+// Between two layers of a decode batch the first one's combine pass (+ residual) and the second one's front kernel
+// (rms-norm, gate, routing, quantisation) are one launch: the front kernel forms its input row from the first layer's
+// weighted expert outputs with the combine pass's own additions, in its order.  Where a boundary does not qualify (a
+// dispatch pass, a shared expert, top-2 layers that accumulate in place, a front end in two launches, a quantised router)
+// the two launches stay apart; the results are the same bits either way.
+static bool stack_boundary_fuses(const moe_layer* A, const ForwardPlan& pa, const moe_layer* B, int64_t T) {
+    if (A->k == 0 || B->k == 0 || A->Fs > 0 || !pa.direct || pa.accumulate || B->gate_q) return false;
+    FrontParams fp;
+    fp.T = T; fp.H = (int)B->H; fp.E = (int)B->E;
+    fp.shared_gate = B->Fs > 0 ? B->shared_gate.as<float>() : nullptr;
+    fp.rms_alpha = B->has_rms ? B->rms_alpha.as<float>() : nullptr;
+    return front_takes_prev_combine(fp);
+}
+
+extern "C" int moe_stack_forward_device(moe_layer* const* layers, int64_t n_layers, const void* d_x, int64_t T, void* d_y, void* hip_stream) {
+    if (!layers || n_layers <= 0 || T < 0 || (T > 0 && (!d_x || !d_y))) return fail(MOE_E_INVALID, "bad argument to moe_stack_forward_device");
+    if (d_x == d_y && T > 0) return fail(MOE_E_INVALID, "d_x and d_y must not alias");
+    for (int64_t l = 0; l < n_layers; l++) {
+        if (!layers[l]) return fail(MOE_E_INVALID, "moe_stack_forward_device: layer " + std::to_string(l) + " is NULL");
+        if (layers[l]->H != layers[0]->H) return fail(MOE_E_INVALID, "moe_stack_forward_device: the layers differ in hidden size");
+        for (int64_t m = 0; m < l; m++)
+            if (layers[m] == layers[l]) return fail(MOE_E_INVALID, "moe_stack_forward_device: a layer appears twice (every layer owns one workspace)");
+    }
+    if (T == 0) return MOE_OK;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    // every layer of the stack is locked for the call (in address order: two stacks that share layers cannot deadlock)
+    std::vector<moe_layer*> order(layers, layers + n_layers);
+    std::sort(order.begin(), order.end());
+    std::vector<std::unique_lock<std::mutex>> locks;
+    for (moe_layer* L : order) locks.emplace_back(L->mu);
+    for (int64_t l = 0; l < n_layers; l++)
+        if (T > max_tokens_per_pass(layers[l])) return fail(MOE_E_INVALID, "moe_stack_forward_device: more tokens than one pass carries; call the layers one by one");
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (s) MOE_HIP_CHECK(hipStreamIsCapturing(s, &cap));
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    // plans, workspaces and which boundaries fuse
+    std::vector<ForwardPlan> plans((size_t)n_layers);
+    std::vector<char> fused_in((size_t)n_layers, 0);   // layer l takes layer l-1's combine pass
+    for (int64_t l = 0; l < n_layers; l++) plans[(size_t)l] = plan_forward(layers[l], T);
+    for (int64_t l = 1; l < n_layers; l++) fused_in[(size_t)l] = stack_boundary_fuses(layers[l - 1], plans[(size_t)l - 1], layers[l], T) ? 1 : 0;
+    std::vector<Workspace> wss((size_t)n_layers);
+    for (int64_t l = 0; l < n_layers; l++) {
+        moe_layer* L = layers[l];
+        // the layer's input row lives in its own workspace when the layer before writes it (fused) and, otherwise, in
+        // the workspace too: every layer but the last writes its output into the next layer's xin
+        const size_t need = L->k > 0 ? carve_workspace(L, T, plans[(size_t)l], nullptr, nullptr, l > 0) : (l > 0 ? (size_t)T * L->H * 4 + 256 : 0);
+        if (capturing && need > L->ws.cap)
+            return fail(MOE_E_INVALID, "moe_stack_forward_device under stream capture needs its workspaces: run the stack once with the same number of tokens before capturing");
+        if (need > L->ws.cap) {
+            if (int rc = L->order.wait()) return rc;
+            if (int rc = L->ws.reserve(need)) return rc;
+        }
+        if (L->k > 0) carve_workspace(L, T, plans[(size_t)l], static_cast<uint8_t*>(L->ws.p), &wss[(size_t)l], l > 0);
+        else if (l > 0) wss[(size_t)l].xin = reinterpret_cast<float*>(L->ws.p);
+        if (capturing) L->ws.captured = true;
+        if (!capturing)
+            if (int rc = L->order.enter(s)) return rc;
+    }
+    // Layer l reads its input from d_x (l = 0) or from its own xin, which either the layer before wrote (its combine pass)
+    // or this layer's front kernel writes (the combine pass folded in); its output goes to the next layer's xin, or to d_y.
+    const float* in_prev = nullptr;
+    for (int64_t l = 0; l < n_layers; l++) {
+        moe_layer* L = layers[l];
+        const bool last = l + 1 == n_layers;
+        const bool leave = !last && fused_in[(size_t)l + 1];
+        const float* in = l == 0 ? static_cast<const float*>(d_x) : wss[(size_t)l].xin;
+        float* out = last ? static_cast<float*>(d_y) : wss[(size_t)l + 1].xin;
+        PrevCombine prev;
+        if (fused_in[(size_t)l]) {
+            const moe_layer* P = layers[l - 1];
+            prev.yw = wss[(size_t)l - 1].yw;
+            prev.topk_idx = wss[(size_t)l - 1].rb.topk_idx;
+            prev.k = (int)P->k;
+            prev.residual = P->has_rms ? in_prev : nullptr;
+        }
+        if (int rc = enqueue_forward(L, plans[(size_t)l], wss[(size_t)l], in, T, out, s, nullptr, fused_in[(size_t)l] ? &prev : nullptr, leave)) return rc;
+        in_prev = in;
+    }
+    if (!capturing)
+        for (int64_t l = 0; l < n_layers; l++) layers[l]->order.leave(s);
     return MOE_OK;
 }
 

@@ -73,6 +73,18 @@ inline unsigned patch_grid(int64_t n_rb, int64_t tiles, int edge) {
     return (unsigned)((RG * TG + 7) / 8 * 8 * edge * edge);
 }
 
+// The combine pass of the layer BEFORE this one, folded into this layer's front kernel (stacks of layers, small batches):
+// the token's input row is  sum of that layer's weighted expert outputs in ascending expert order (+ that layer's
+// input, its residual) -- the additions of combine_kernel in combine_kernel's order -- and is stored to x_out, where this
+// layer's own residual is read from later.  Slots are numbered t * k + r (no dispatch pass ran in that layer).
+struct PrevCombine {
+    const float* yw = nullptr;          // [T * k, H] weighted expert outputs of the previous layer
+    const int32_t* topk_idx = nullptr;  // [T, k] its routing
+    int k = 0;
+    const float* residual = nullptr;    // [T, H] its input, or null for a layer without the pre-norm
+    float* x_out = nullptr;             // [T, H]
+};
+
 struct FrontParams {
     const float* x = nullptr;       // [T, H]
     int64_t T = 0;
@@ -87,7 +99,10 @@ struct FrontParams {
     ActBuf xq;                          // token-indexed quantised activations (output)
     float* y_zero = nullptr;            // [T, H] or null: rows the kernel clears for the down kernels to accumulate into
     RouteBufs rb;
+    PrevCombine prev;                   // fast kernel only (front_takes_prev_combine): x is not read then
 };
+// whether launch_front will take the kernel that can fold the previous layer's combine pass in
+bool front_takes_prev_combine(const FrontParams& p);
 // rms-norm (optional) + gate product + softmax + top-k + activation quantisation per token.
 hipError_t launch_front(const FrontParams& p, hipStream_t s);
 // The front end of a layer whose router stays quantised: logits from the dense product's padded rows, then routing and

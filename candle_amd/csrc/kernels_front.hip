@@ -671,12 +671,64 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
     const int64_t t = blockIdx.x;
     constexpr int H = NCH * 256;
     const int E = p.E;
-    const float* x = p.x + t * H;
     float xr[NCH * 4];
+    // the rms-norm's workspace; also the row exchange of a folded-in combine pass
+    __shared__ float row_lds[LEAN ? 1 : 64 * (NCH * 4 + 1)];
+    if (!LEAN && p.prev.yw) {
+        // the previous layer's combine pass: its terms in ascending expert order onto zero, then its residual
+        // (combine_kernel's additions in combine_kernel's order).  Wave i % 8 sums chunk i -- all of a wave's loads are in
+        // flight together -- stores it as the previous layer's output and shares it through the LDS.
+        constexpr int PK = 8;   // terms requested together
+        const int pk = p.prev.k;
+        const int e = lane < pk ? p.prev.topk_idx[t * pk + lane] : 0x7fffffff;
+        int rank = 0;
+        for (int j = 0; j < pk; j++) {
+            const int ej = __shfl(e, j, 64);
+            rank += (ej < e || (ej == e && j < lane)) ? 1 : 0;
+        }
+        // lane j learns which of the token's slots comes j-th
+        int nth = 0;
+        for (int j = 0; j < pk; j++) {
+            const int rj = __shfl(rank, j, 64);
+            if (rj == lane) nth = j;
+        }
+        const int64_t slot0 = t * pk;
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-        const float4 v = *reinterpret_cast<const float4*>(x + i * 256 + lane * 4);
-        xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        for (int i = 0; i < NCH; i++)
+            if ((i & 7) == wave) {
+                float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+                float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (p.prev.residual) r = *reinterpret_cast<const float4*>(p.prev.residual + t * H + i * 256 + lane * 4);
+                for (int j0 = 0; j0 < pk; j0 += PK) {
+                    float4 a[PK];
+#pragma unroll
+                    for (int j = 0; j < PK; j++)
+                        if (j0 + j < pk) {
+                            const int64_t slot = slot0 + __builtin_amdgcn_readlane(nth, (j0 + j) & 63);
+                            a[j] = *reinterpret_cast<const float4*>(p.prev.yw + slot * H + i * 256 + lane * 4);
+                        }
+#pragma unroll
+                    for (int j = 0; j < PK; j++)
+                        if (j0 + j < pk) { acc.x += a[j].x; acc.y += a[j].y; acc.z += a[j].z; acc.w += a[j].w; }
+                }
+                if (p.prev.residual) { acc.x += r.x; acc.y += r.y; acc.z += r.z; acc.w += r.w; }
+                *reinterpret_cast<float4*>(p.prev.x_out + t * H + i * 256 + lane * 4) = acc;
+                *reinterpret_cast<float4*>(row_lds + i * 256 + lane * 4) = acc;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const float4 v = *reinterpret_cast<const float4*>(row_lds + i * 256 + lane * 4);
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        }
+        __syncthreads();   // the norm below writes row_lds again
+    } else {
+        const float* x = p.x + t * H;
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const float4 v = *reinterpret_cast<const float4*>(x + i * 256 + lane * 4);
+            xr[4 * i] = v.x; xr[4 * i + 1] = v.y; xr[4 * i + 2] = v.z; xr[4 * i + 3] = v.w;
+        }
     }
     // Gate rows of experts e0 and e0 + 4 (the shared-expert gate counts as expert E).  Waves 0..3 request their first
     // pair here, ahead of the rms-norm: nothing has touched the gate since the layer last ran, and the fetch from HBM
@@ -701,7 +753,6 @@ __device__ __forceinline__ void front_fast_body(const FrontParams& p) {
         // rms_norm (candle-nn/src/ops.rs:504-515) sums the squares left to right in f32.  A different
         // order changes the divisor in the last ulp, which flips quantised activations now and then
         // and moves a whole output row by 1e-3 of its rms, so the sum keeps the reference's order.
-        __shared__ float row_lds[64 * (NCH * 4 + 1)];
         const float sum2 = ordered_sum_of_squares<NCH>(xr, tid, p.rms_serial != 0, row_lds);
         const float m = sqrtf(sum2 / (float)H + p.rms_eps);
         // every wave holds the whole row: each normalises an eighth of it (a correctly rounded division per element)
@@ -1211,6 +1262,19 @@ static bool launch_front_fast(const FrontParams& p, hipStream_t s) {
         case 32: hipLaunchKernelGGL((front_fast_kernel<VDT, 32>), grid, block, 0, s, p); return true;
     }
     return false;
+}
+
+// The fast kernel in its plain or wide form (not the two-launch front end, not the lean form of large batches without a
+// pre-norm, not the generic kernel): the one that can fold the previous layer's combine pass in.
+bool front_takes_prev_combine(const FrontParams& p) {
+    if (switches().front_generic || p.E > MAX_E || p.H % 256 || p.T == 0) return false;
+    const int nch = p.H / 256;
+    if (!(nch == 1 || nch == 2 || (nch % 4 == 0 && nch <= 32))) return false;
+    const int sw = switches().front_split;
+    const int NE = p.E + (p.shared_gate ? 1 : 0);
+    if (!p.rms_alpha && sw != 0 && (sw > 0 || (NE >= 32 && p.T * (int64_t)NE >= 49152))) return false;   // two launches
+    if (!p.rms_alpha && ((nch == 8 && p.T >= 256) || (nch == 16 && p.T >= 1024))) return false;              // lean form
+    return true;
 }
 
 hipError_t launch_fill_or_copy(const float* src, float* y, int64_t n, hipStream_t s) {

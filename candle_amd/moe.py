@@ -68,6 +68,7 @@ def load_library():
     L.moe_layer_forward_device.argtypes = [vp, vp, i64, vp, vp]
     L.moe_layer_forward_device_noalloc.argtypes = [vp, vp, i64, vp, vp]
     L.moe_static_scratch_bytes.restype = i64
+    L.moe_stack_forward_device.argtypes = [C.POINTER(vp), i64, vp, i64, vp, vp]
     L.moe_layer_forward_timed.argtypes = [vp, vp, i64, vp, vp, vp]
     L.moe_rms_norm.argtypes = [vp, vp, C.c_float, i64, i64, vp]
     L.moe_add_rms_norm_device.argtypes = [vp, vp, vp, C.c_float, i64, i64, vp, vp, vp]
@@ -493,6 +494,28 @@ class SparseMoeBlock:
 
 
 MlpOrMoe = SparseMoeBlock  # the reference's name for the enum that holds the MoE arm
+
+
+def stack_forward(layers, xs, out=None):
+    """`layers[-1](... layers[1](layers[0](xs)))` for a list of SparseMoeBlocks on a contiguous f32 torch CUDA tensor
+    (torch's current stream): the same bits as calling the layers one by one, with each layer's combine pass folded
+    into the next layer's front kernel where the batch is small (moe_stack_forward_device)."""
+    import torch
+    if not layers:
+        raise MoeError("stack_forward needs at least one layer")
+    if not (isinstance(xs, torch.Tensor) and xs.is_cuda and xs.dtype == torch.float32 and xs.is_contiguous()):
+        raise MoeError("stack_forward takes a contiguous f32 torch CUDA tensor")
+    hidden = layers[0].hidden
+    if xs.dim() not in (2, 3) or xs.shape[-1] != hidden:
+        raise MoeError("expected [b, seq, %d] or [tokens, %d], got %s" % (hidden, hidden, tuple(xs.shape)))
+    for layer in layers:
+        if layer._h is None:
+            raise MoeError("layer is closed")
+    y = torch.empty_like(xs) if out is None else out
+    handles = (C.c_void_p * len(layers))(*[layer._h for layer in layers])
+    stream = torch.cuda.current_stream(xs.device).cuda_stream
+    _check(load_library().moe_stack_forward_device(handles, len(layers), xs.data_ptr(), xs.numel() // hidden, y.data_ptr(), stream))
+    return y
 
 
 class QMatMul:

@@ -127,6 +127,15 @@ int moe_layer_forward(moe_layer* layer, const float* x, int64_t n_tokens, float*
  * caller that already keeps activations on the GPU uses (no PCIe in the path). */
 int moe_layer_forward_device(moe_layer* layer, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
 
+/* The MoE blocks of consecutive transformer layers as one call: y = layer[n-1](... layer[1](layer[0](x))), each layer's own
+ * forward (with rms_alpha: x + moe(rms_norm(x)), `ModelWeights::forward`, quantized_llama.rs:886-892, without the attention
+ * half of the layer).  Same results, bit for bit, as n calls of moe_layer_forward_device; what the call adds is that
+ * between two layers of a small (decode) batch the first layer's combine pass and residual add and the second layer's
+ * rms-norm, router and activation quantiser are ONE launch.  The layers must be distinct objects of one hidden size;
+ * n_tokens at most what one pass carries.  Like moe_layer_forward_device it can be recorded into a HIP graph after one
+ * eager call of the same size.  d_x and d_y must not overlap. */
+int moe_stack_forward_device(moe_layer* const* layers, int64_t n_layers, const void* d_x, int64_t n_tokens, void* d_y, void* hip_stream);
+
 /* No counterpart in the reference.  For callers that cannot allocate device memory while they run: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  The same forward as
  * moe_layer_forward_device (same kernels, same results), but its workspace (routing lists, quantised activations,

@@ -68,6 +68,7 @@ pub mod ffi {
         pub fn moe_layer_forward_device(layer: *mut MoeLayer, d_x: *const c_void, n_tokens: i64, d_y: *mut c_void, hip_stream: *mut c_void) -> i32;
         pub fn moe_layer_forward_device_noalloc(layer: *mut MoeLayer, d_x: *const c_void, n_tokens: i64, d_y: *mut c_void, hip_stream: *mut c_void) -> i32;
         pub fn moe_static_scratch_bytes() -> i64;
+        pub fn moe_stack_forward_device(layers: *const *mut MoeLayer, n_layers: i64, d_x: *const c_void, n_tokens: i64, d_y: *mut c_void, hip_stream: *mut c_void) -> i32;
         pub fn moe_qmatmul(ggml_dtype: i32, w_blocks: *const c_void, n: i64, k: i64, x: *const f32, m: i64, y: *mut f32) -> i32;
         pub fn moe_qlinear_create(ggml_dtype: i32, w_blocks: *const c_void, n: i64, k: i64, out: *mut *mut MoeQLinear) -> i32;
         pub fn moe_qlinear_destroy(q: *mut MoeQLinear);
@@ -331,6 +332,14 @@ impl HipSparseMoe {
         };
         check(rc)
     }
+}
+
+/// The MoE blocks of consecutive layers on device pointers (HIP memory the caller owns), enqueued on `hip_stream`
+/// without synchronising: `y = layers[n-1](... layers[0](x))`, the same bits as the layers' own forwards one after
+/// the other, with each layer's combine pass folded into the next layer's front kernel at decode batch sizes.
+pub unsafe fn stack_forward_device(layers: &[&HipSparseMoe], d_x: *const c_void, n_tokens: usize, d_y: *mut c_void, hip_stream: *mut c_void) -> Result<()> {
+    let handles: Vec<*mut ffi::MoeLayer> = layers.iter().map(|l| l.handle).collect();
+    check(ffi::moe_stack_forward_device(handles.as_ptr(), handles.len() as i64, d_x, n_tokens as i64, d_y, hip_stream))
 }
 
 impl CustomOp1 for HipSparseMoe {

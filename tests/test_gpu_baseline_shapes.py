@@ -378,10 +378,15 @@ def test_cfg5_stack_128_chained_steps(mixtral_stack, request):
     g.manual_seed(77)
     x = torch.randn((32, 4096), generator=g, device="cuda", dtype=torch.float32)
     bufs = [torch.empty_like(x) for _ in range(2)]
+    gpus = [gpu for _, gpu in mixtral_stack]
     for step in range(N_STEPS - 1):
-        h = x
-        for i, (_, gpu) in enumerate(mixtral_stack):
-            h = gpu.forward(h, out=bufs[i & 1])
+        h = candle_amd.stack_forward(gpus, x, out=bufs[0])   # the 32 layers as one call
+        if step == 0:   # the same bits as the layers one by one
+            hh = x
+            for i, gpu in enumerate(gpus):
+                hh = gpu.forward(hh, out=bufs[1] if i & 1 else torch.empty_like(x))
+            assert torch.equal(h, hh)
+            h = candle_amd.stack_forward(gpus, x, out=bufs[0])
         x = h + 0.1 * torch.randn((32, 4096), generator=g, device="cuda", dtype=torch.float32)
         if step % 32 == 31:
             assert bool(torch.isfinite(x).all()), step
