@@ -189,32 +189,36 @@ def cpu_baseline(w, xs_host, logits_host, min_seconds, gate_bias=None, cfg4=Fals
                       "(AVX2 vec_dot, %d threads over output columns)" % (reps, xs_host.shape[0], dt, cores)}
 
 
-def profiled_value(name, label, key):
-    """A `label[key]: value` line of a committed profile summary (a float), or None."""
+def profile_build_id(name):
+    """The `library_build_id: <id>` line of a committed profile summary: the sources the profiled library was built from."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", name)):
+            m = re.match(r"library_build_id:\s*([0-9a-f]+)", line.strip())
+            if m:
+                return m.group(1)
+    except OSError:
+        pass
+    return None
+
+
+def counter_figure(name, label, key):
+    """(value, note) for a `label[key]: value` line of a committed rocprofv3 counter summary.  Such a figure belongs to
+    the build it was measured on: it is given only when the summary's recorded build id equals the loaded library's
+    (moe_build_id); otherwise the value is None and the note says which ids differ.  Never a reading of this run."""
+    import candle_amd
+    lib_id, prof_id = candle_amd.build_id(), profile_build_id(name)
+    if prof_id != lib_id:
+        return None, "profiles/%s was measured on build %s, the loaded library is build %s: figure withheld" % (name, prof_id, lib_id)
     try:
         for line in open(os.path.join(ROOT, "profiles", name)):
             m = re.match(r"%s\[([^\]]+)\]:\s*([0-9.eE+-]+)" % re.escape(label), line.strip())
             if m and m.group(1) == key:
-                return float(m.group(2))
+                v = float(m.group(2))
+                return (int(v) if v == int(v) and "." not in m.group(2) else v), \
+                    "profiles/%s (committed rocprofv3 --pmc summary of build %s, the build loaded now; not a reading of this run)" % (name, prof_id)
     except OSError:
         pass
-    return None
-
-
-def profiled_traffic(batch, name="q4k_up_decode_hbm_traffic.md", key=None):
-    """HBM bytes per launch of the dominant kernel as the committed rocprofv3 counter summary gives them (FETCH_SIZE +
-    WRITE_SIZE, scaled by the copy kernel): a figure from that profile, not a reading of this run; None when the summary
-    does not cover this batch size."""
-    path = os.path.join(ROOT, "profiles", name)
-    key = key or "batch=%d" % batch
-    try:
-        for line in open(path):
-            m = re.match(r"traffic_bytes_per_launch\[([^\]]+)\]:\s*(\d+)", line.strip())
-            if m and m.group(1) == key:
-                return int(m.group(2))
-    except OSError:
-        pass
-    return None
+    return None, "profiles/%s holds no %s[%s]" % (name, label, key)
 
 
 def activations(torch, B, hid, seed=2, n=4):
@@ -243,10 +247,10 @@ def measure_decode(args, np, torch, timer, layer, B, fmt="q4_k"):
     up_bytes = n_active * (2 * H * F * fmt_bb // fmt_be) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
     achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
     q4k = fmt == "q4_k"
-    traffic = profiled_traffic(B) if q4k else None
+    traffic, traffic_note = counter_figure("q4k_up_decode_hbm_traffic.md", "traffic_bytes_per_launch", "batch=%d" % B) if q4k else (None, None)
     roofline = {"bound": "hbm", "kernel": "q4k_up (w1, w3, SiLU, Q8K re-quantisation)" if q4k else "up projection (w1, w3, SiLU, re-quantisation), %s" % fmt,
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                "traffic_source": "profiles/q4k_up_decode_hbm_traffic.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
+                "traffic_source": traffic_note,
                 "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "batch": B, "active_experts": n_active, "stage_us": stage_us, "empty_stage_us": min(stage_us.values()),
@@ -297,6 +301,7 @@ def measure_prefill(args, np, torch, timer, layer, B):
     step_ops = 2.0 * B * TOPK * 3 * H * F
     one_plane = args.weights == "q2_k"   # a 4-bit scale times a 2-bit code fits a byte: one plane, every multiply-add issued once
     q4k = args.weights == "q4_k"
+    busy, busy_note = counter_figure("q4k_gemm_prefill_4096_kernel_trace.md", "mfma_busy_frac", "prefill_up") if B == 4096 and q4k else (None, None)
     roofline = {"bound": "mfma", "kernel": "q4k_gemm up (w1, w3, SiLU; int8 MFMA 16x16x64, %s)" % ("one plane of scaled codes" if one_plane else "two scale planes"),
                 "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": achieved / INT8_PEAK_TOPS,
                 "traffic": None, "algorithmic_ops_per_launch": up_ops, "launch_us": stage_us["up"],
@@ -306,8 +311,7 @@ def measure_prefill(args, np, torch, timer, layer, B):
                 "mfma_issued_frac": (1.0 if one_plane else 2.0) * achieved / INT8_PEAK_TOPS,
                 # share of the cycles the matrix pipe is busy (SQ_VALU_MFMA_BUSY_CYCLES over the kernel's SIMD cycles)
                 # as the committed rocprofv3 counter summary gives it: a figure of that profile, not a reading of this run
-                "mfma_pipe_busy_frac": profiled_value("q4k_gemm_prefill_4096_kernel_trace.md", "mfma_busy_frac", "prefill_up") if B == 4096 and q4k else None,
-                "mfma_pipe_busy_source": "profiles/q4k_gemm_prefill_4096_kernel_trace.md (rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES, SQ_CYCLES)"}
+                "mfma_pipe_busy_frac": busy, "mfma_pipe_busy_source": busy_note}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "tokens": B, "expert_loads": [int(v) for v in loads], "stage_us": stage_us, "step_int8_ops": step_ops,
             "step_mfma_frac": step_ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, "roofline": roofline, "xs": xs, "ys": ys}
@@ -329,10 +333,10 @@ def measure_cfg4(args, np, torch, timer, layer, B):
     step_bytes = n_active * expert_bytes + shared_bytes + c["E"] * c["H"] * 4 + 2 * B * c["H"] * 4
     up_bytes = n_active * (2 * c["H"] * c["F"] * 34 // 32)
     achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
-    traffic = profiled_traffic(B, "q8_0_gemm_config4_kernel_trace.md", "config4") if B == 512 else None
+    traffic, traffic_note = counter_figure("q8_0_gemm_config4_kernel_trace.md", "traffic_bytes_per_launch", "config4") if B == 512 else (None, None)
     roofline = {"bound": "hbm", "kernel": "q8_0_gemm<0>: routed up projection (w1, w3, SiLU, Q8_0 re-quantisation), 64-slot tiles",
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                "traffic_source": "profiles/q8_0_gemm_config4_kernel_trace.md (committed rocprofv3 --pmc summary, not a reading of this run)" if traffic else None,
+                "traffic_source": traffic_note,
                 "algorithmic_bytes_per_launch": up_bytes, "launch_us": stage_us["up"]}
     return {"tokens_per_s": B / (ms * 1e-3), "ms_per_step": ms, "wall_ms_per_step": wall_ms, "timed_steps": n_steps, "warmup_steps_run": warmed,
             "tokens": B, "active_experts": n_active, "max_expert_load": int(loads.max()), "stage_us": stage_us, "dispatch_us": stage_us["dispatch"],
@@ -456,7 +460,7 @@ def main():
         sys.exit("bench.py: --weights-down applies to the prefill workload only")
     timer = Timer(torch)
     out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-           "dtype": "i8", "data": "synthetic", "unit": "tokens/s"}
+           "dtype": "i8", "data": "synthetic", "unit": "tokens/s", "library_build_id": candle_amd.build_id()}
     bias = np.array(ZIPF_BIAS, dtype=np.float32)
     cpu = None
 

@@ -1,5 +1,6 @@
 """Builds libcandle_amd_moe.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
 import concurrent.futures
+import hashlib
 import os
 import shutil
 import subprocess
@@ -26,9 +27,25 @@ def hipcc():
     return exe
 
 
+def source_id():
+    """Sixteen hex digits of the SHA-256 over the library's source files (names and contents, in name order): what
+    moe_build_id() of a library built from them returns."""
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".hpp", ".cpp", ".h")):
+            h.update(name.encode() + b"\0")
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(f.read())
+            h.update(b"\0")
+    return h.hexdigest()[:16]
+
+
 def _compile(src, out_dir=None, extra_flags=()):
     obj = os.path.join(out_dir or OUT_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [hipcc()] + HIPCC_FLAGS + list(extra_flags) + ["-c", os.path.join(CSRC, src), "-o", obj]
+    flags = list(extra_flags)
+    if src == "api.hip":
+        flags.append('-DMOE_BUILD_ID="%s"' % source_id())
+    cmd = [hipcc()] + HIPCC_FLAGS + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))

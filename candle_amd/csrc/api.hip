@@ -1400,6 +1400,11 @@ extern "C" int moe_debug_set_switch(const char* name, int64_t value) {
 
 extern "C" const char* moe_last_error(void) { return g_err.c_str(); }
 
+#ifndef MOE_BUILD_ID
+#define MOE_BUILD_ID "unknown"
+#endif
+extern "C" const char* moe_build_id(void) { return MOE_BUILD_ID; }
+
 extern "C" const char* moe_device_arch(void) {
     if (ensure_device()) return nullptr;
     return g_arch.c_str();

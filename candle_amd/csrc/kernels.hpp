@@ -57,20 +57,31 @@ inline int64_t max_gemm_tiles(int64_t slots, int64_t groups, int tile_slots = GE
 // edge is 8 when that still gives every XCD at least two patches, else 4 or 2: a grid of a few hundred workgroups cut
 // into 8 x 8 patches would leave XCDs without work.
 struct PatchPos { int rblk, tile; };
-__host__ __device__ inline PatchPos patch_position(int block, int n_rb, int edge) {
-    const int per = edge * edge, RG = (n_rb + edge - 1) / edge;
+// `patch` = rows edge + 256 * tiles edge (a tiles edge of 0: a square patch)
+__host__ __device__ inline PatchPos patch_position(int block, int n_rb, int patch) {
+    const int er = patch & 255, et = (patch >> 8) ? (patch >> 8) : er;
+    const int per = er * et, RG = (n_rb + er - 1) / er;
     const int xcd = block & 7, q = block >> 3;
     const int st = (q / per) * 8 + xcd, within = q % per;
-    return PatchPos{(st % RG) * edge + within % edge, (st / RG) * edge + within / edge};
+    return PatchPos{(st % RG) * er + within % er, (st / RG) * et + within / er};
 }
 inline int patch_edge(int64_t n_rb, int64_t tiles) {
     for (int e = 8; e > 2; e >>= 1)
         if (((n_rb + e - 1) / e) * ((tiles + e - 1) / e) >= 16) return e;
     return 2;
 }
-inline unsigned patch_grid(int64_t n_rb, int64_t tiles, int edge) {
-    const int64_t RG = (n_rb + edge - 1) / edge, TG = (tiles + edge - 1) / edge;
-    return (unsigned)((RG * TG + 7) / 8 * 8 * edge * edge);
+// One group of a few tiles (the always-on expert, a dense product): a patch holds every tile of its row blocks, so that
+// each weight row is fetched into one XCD's L2 only (square patches of 4 x 4 fetched the rows of eight tiles twice).
+inline int patch_all_tiles(int64_t n_rb, int64_t tiles) {
+    if (tiles < 1 || tiles > 16) return patch_edge(n_rb, tiles);
+    int er = 4;
+    while (er > 1 && (n_rb + er - 1) / er < 16) er >>= 1;
+    return er + 256 * (int)tiles;
+}
+inline unsigned patch_grid(int64_t n_rb, int64_t tiles, int patch) {
+    const int er = patch & 255, et = (patch >> 8) ? (patch >> 8) : er;
+    const int64_t RG = (n_rb + er - 1) / er, TG = (tiles + et - 1) / et;
+    return (unsigned)((RG * TG + 7) / 8 * 8 * er * et);
 }
 
 // The combine pass of the layer BEFORE this one, folded into this layer's front kernel (stacks of layers, small batches):

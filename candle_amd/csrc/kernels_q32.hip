@@ -723,9 +723,15 @@ __device__ __forceinline__ void qg_dma16(const void* gbase, uint32_t voff, uint3
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(gbase), "s"(lds));
 }
 
-template <int DT, int MODE>
+// WOPS (MODE 1): 16-slot operands per wave.  With 4 the eight waves hold eight weight operands (128 rows) and every one of
+// them takes the tile's four slot operands; with 2 (1) they hold four (two) weight operands, 64 (32) rows, and split
+// the slot operands between them: a grid of few tiles -- the always-on expert's down projection, 16 row blocks of 128 x 8
+// tiles at 512 tokens of 2048 -- becomes twice (four times) as many workgroups, each of half (a quarter of) the length.
+template <int DT, int MODE, int WOPS = QG_NOP>
 __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q8_0_gemm_kernel(ExpertParams p) {
     static_assert(DT == MOE_GGML_Q8_0 || DT == MOE_GGML_Q4_0 || DT == MOE_GGML_Q5_0, "formats with Q8_0 activations and no minimum");
+    static_assert(MODE == 1 || WOPS == QG_NOP, "the up projection pairs w1 and w3 waves");
+    constexpr int RTW = 8 * WOPS / QG_NOP;   // MODE 1: weight operands (16 rows) per workgroup
     constexpr int OFFSET = Q32Fmt<DT>::OFFSET;
     constexpr size_t STB = Q32SFmt<DT>::STB;
     __shared__ QGemmLds L;
@@ -733,7 +739,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // workgroup -> (row block, slot tile), in patches per XCD (patch_position)
-    const int n_rb = MODE == 0 ? p.F / 64 : p.H / 128;
+    const int n_rb = MODE == 0 ? p.F / 64 : p.H / (16 * RTW);
     const PatchPos pp = patch_position((int)blockIdx.x, n_rb, p.patch);
     const int rblk = pp.rblk, tile = pp.tile;
     if (rblk >= n_rb) return;
@@ -761,9 +767,13 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
         const int slot = s_begin + (pos < n_g ? pos : n_g - 1);
         return MODE == 0 ? p.rb.perm_token[slot] : slot - p.slot_origin;
     };
+    // Row r of a 16-slot operand holds the tile's position 4 (r % 4) + r / 4, so that a lane's result register i (rows
+    // 4 g + i of the matrix instruction's output) covers positions 4 i .. 4 i + 3: the result arithmetic of a short last
+    // operand then follows the list length in steps of four slots, not sixteen.
+    auto pos_of_row = [](int r) { return (r & ~15) + ((r & 3) << 2) + ((r >> 2) & 3); };
     // transfers of a step: wave w stages half w % 2 (pieces 4 (w % 2) .. +3) of operand w / 2; wave 0 also the scales
-    const uint32_t q_src = (uint32_t)act_row(16 * (wave >> 1) + (lane & 15)) * (uint32_t)K + (uint32_t)((4 * (wave & 1) + (lane >> 4)) * 16);
-    const uint32_t d_src = (uint32_t)act_row(lane) * (uint32_t)nkb * 4u;
+    const uint32_t q_src = (uint32_t)act_row(pos_of_row(16 * (wave >> 1) + (lane & 15))) * (uint32_t)K + (uint32_t)((4 * (wave & 1) + (lane >> 4)) * 16);
+    const uint32_t d_src = (uint32_t)act_row(pos_of_row(lane)) * (uint32_t)nkb * 4u;
     auto stage = [&](int ks, int buf) {
         qg_dma16(ab.qs, q_src + (uint32_t)(ks * 128), qg_lds_address(&L.q[buf][wave >> 1][4 * (wave & 1)][0]));
         if (wave == 0) qg_dma16(ab.d, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.yd[buf][0][0]));
@@ -777,13 +787,14 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
         row0 = rblk * 64 + (wave & 3) * 16;
         wp = (wave < 4 ? gw.w1 : gw.w3) + (size_t)(row0 / 16) * STB;
     } else {
-        row0 = rblk * 128 + wave * 16;
+        row0 = rblk * (16 * RTW) + (wave % RTW) * 16;
         wp = gw.w2 + (size_t)(row0 / 16) * STB;
     }
+    const int ob = MODE == 0 ? 0 : (wave / RTW) * WOPS;   // the wave's first slot operand
     const int m = lane & 15, g = lane >> 4;
-    float acc[QG_NOP][4];
+    float acc[WOPS][4];
 #pragma unroll
-    for (int o = 0; o < QG_NOP; o++)
+    for (int o = 0; o < WOPS; o++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[o][i] = 0.f;
 
@@ -793,6 +804,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     __syncthreads();
     const v4i magic = {Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS, Q32S_MAGIC_BITS};
+    const int last_regs = __builtin_amdgcn_readfirstlane((n_here - 16 * (n_op - 1) + 3) >> 2);   // live result registers of the last operand
     for (int ks = 0; ks < nks; ks++) {
         const int buf = ks & 1;
         const int ks1 = ks + 1 < nks ? ks + 1 : ks, ks2 = ks + 2 < nks ? ks + 2 : nks - 1;
@@ -807,7 +819,8 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
         for (int b = 0; b < 4; b++) cneg[b] = -(Q32S_MAGIC * dwv[b]);
 #pragma unroll
-        for (int o = 0; o < QG_NOP; o++) {
+        for (int ow = 0; ow < WOPS; ow++) {
+            const int o = ob + ow;
             if (o < n_op) {   // wave-uniform
                 f32x4g ydv[4];
 #pragma unroll
@@ -828,14 +841,18 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                     D[b] = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, addend, 0, 0, 0);
                 }
                 __builtin_amdgcn_s_setprio(0);
-                // ascending block order per (row, slot), every product rounded where the reference rounds it
+                // ascending block order per (row, slot), every product rounded where the reference rounds it; result
+                // registers beyond the end of the list are left alone
+                const int regs = o + 1 < n_op ? 4 : last_regs;
 #pragma unroll
-                for (int b = 0; b < 4; b++)
+                for (int i = 0; i < 4; i++)
+                    if (i < regs) {   // wave-uniform
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        float t = __builtin_fmaf(__int_as_float(D[b][i]), dwv[b], cneg[b]);
-                        t = t * ydv[i][b];
-                        acc[o][i] += t;
+                        for (int b = 0; b < 4; b++) {
+                            float t = __builtin_fmaf(__int_as_float(D[b][i]), dwv[b], cneg[b]);
+                            t = t * ydv[i][b];
+                            acc[ow][i] += t;
+                        }
                     }
             }
         }
@@ -843,7 +860,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
         __syncthreads();
     }
 
-    // epilogue: lane holds weight row n = lane % 16 and slots 16 o + 4 (lane / 16) + i
+    // epilogue: lane holds weight row n = lane % 16 and the tile's positions 16 o + 4 i + lane / 16
     const int n = lane & 15;
     if (MODE == 0) {
         // w3 waves (4-7) park their sums in LDS (the staging buffers are free now), w1 waves combine
@@ -862,7 +879,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const float up = xch[((wave * QG_NOP + o) * 4 + i) * 64 + lane];
-                    hx[o * 16 + 4 * g + i][wave * 16 + n] = silu_ref32(acc[o][i]) * up;
+                    hx[o * 16 + 4 * i + g][wave * 16 + n] = silu_ref32(acc[o][i]) * up;
                 }
         }
         __syncthreads();
@@ -895,13 +912,13 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
         }
     } else {
 #pragma unroll
-        for (int o = 0; o < QG_NOP; o++)
+        for (int ow = 0; ow < WOPS; ow++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int pos = o * 16 + g * 4 + i;
+                const int pos = (ob + ow) * 16 + i * 4 + g;
                 if (pos >= n_here) continue;
                 const int slot = s_begin + pos0 + pos;
-                p.yw[(int64_t)slot * p.H + row0 + n] = acc[o][i] * p.rb.perm_w[slot];
+                p.yw[(int64_t)slot * p.H + row0 + n] = acc[ow][i] * p.rb.perm_w[slot];
             }
     }
 }
@@ -913,12 +930,12 @@ bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F) {
 static int64_t qg_tiles(const ExpertParams& p) {
     return p.is_shared ? (p.max_rows + QG_NOP * 16 - 1) / (QG_NOP * 16) : max_gemm_tiles(p.n_slots, p.n_groups + 1, QG_NOP * 16);
 }
-template <int MODE>
+template <int MODE, int WOPS = QG_NOP>
 static hipError_t qg_launch(int dt, const ExpertParams& p, dim3 grid, hipStream_t s) {
     switch (dt) {
-        case MOE_GGML_Q8_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q8_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
-        case MOE_GGML_Q4_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q4_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
-        case MOE_GGML_Q5_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q5_0, MODE>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q8_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q8_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q4_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q4_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q5_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q5_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -926,14 +943,19 @@ static hipError_t qg_launch(int dt, const ExpertParams& p, dim3 grid, hipStream_
 hipError_t launch_q8_0_gemm_up(const ExpertParams& p_in, hipStream_t s) {
     if (p_in.max_rows == 0 || p_in.n_groups == 0) return hipSuccess;
     ExpertParams p = p_in;
-    p.patch = patch_edge(p.F / 64, qg_tiles(p));
+    p.patch = p.is_shared ? patch_all_tiles(p.F / 64, qg_tiles(p)) : patch_edge(p.F / 64, qg_tiles(p));
     return qg_launch<0>(p.dt, p, dim3(patch_grid(p.F / 64, qg_tiles(p), p.patch)), s);
 }
 hipError_t launch_q8_0_gemm_down(const ExpertParams& p_in, hipStream_t s) {
     if (p_in.max_rows == 0 || p_in.n_groups == 0) return hipSuccess;
     ExpertParams p = p_in;
-    p.patch = patch_edge(p.H / 128, qg_tiles(p));
-    return qg_launch<1>(p.dt_down ? p.dt_down : p.dt, p, dim3(patch_grid(p.H / 128, qg_tiles(p), p.patch)), s);
+    const int dt = p.dt_down ? p.dt_down : p.dt;
+    const int64_t tiles = qg_tiles(p);
+    // fewer than a workgroup per CU: narrower workgroups (64 or 32 rows), whose waves split the slot operands
+    const int rows = (p.H / 128) * tiles >= 256 ? 128 : (p.H / 64) * tiles >= 256 ? 64 : 32;
+    p.patch = p.is_shared ? patch_all_tiles(p.H / rows, tiles) : patch_edge(p.H / rows, tiles);
+    const dim3 grid(patch_grid(p.H / rows, tiles, p.patch));
+    return rows == 128 ? qg_launch<1, 4>(dt, p, grid, s) : rows == 64 ? qg_launch<1, 2>(dt, p, grid, s) : qg_launch<1, 1>(dt, p, grid, s);
 }
 
 // ---------------------------------------------------------------------------------------------

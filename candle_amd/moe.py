@@ -110,6 +110,7 @@ def load_library():
     L.moe_layer_create_from_gguf.argtypes = [vp, C.c_int, C.c_int, C.POINTER(vp)]
     L.moe_last_error.restype = C.c_char_p
     L.moe_device_arch.restype = C.c_char_p
+    L.moe_build_id.restype = C.c_char_p
     L.moe_debug_expf.restype = C.c_float
     L.moe_debug_expf.argtypes = [C.c_float]
     _lib = L
@@ -145,6 +146,11 @@ def device_arch():
     if r is None:
         raise MoeError(load_library().moe_last_error().decode())
     return r.decode()
+
+
+def build_id():
+    """The id of the sources the loaded library was compiled from (moe_build_id)."""
+    return load_library().moe_build_id().decode()
 
 
 def debug_expf(x):

@@ -273,6 +273,11 @@ const char* moe_last_error(void);
 /* Name of the device the library runs on, e.g. "gfx950"; NULL (and an error message) if none. */
 const char* moe_device_arch(void);
 
+/* Identifies the sources this library was compiled from (no counterpart in the reference): sixteen hex digits of the
+ * SHA-256 over the library's source files, as the build step computed it; "unknown" for a build that did not pass it.
+ * Counter summaries of a kernel are tied to a build with it: a figure measured on other sources is not this library's. */
+const char* moe_build_id(void);
+
 /* Test aid (no counterpart in the reference): sets one of the process-wide tuning switches that are otherwise
  * read once from the MOE_* environment variables: "combine_pass", "rms_serial", "max_tokens_per_pass", "no_gemm",
  * "front_generic", "tile_slots", "slot_tiles", "narrow", "fused_rows", "front_split", "dispatch_one".  Not for use while forwards are in flight. */

@@ -27,6 +27,13 @@ def test_library_exports_every_declared_symbol():
         assert getattr(lib, n) is not None, n
 
 
+def test_build_id_names_the_sources_on_disk():
+    # the library in the tree was compiled from the sources in the tree (a stale library would carry another id)
+    from candle_amd import build
+    assert re.fullmatch(r"[0-9a-f]{16}", candle_amd.build_id())
+    assert candle_amd.build_id() == build.source_id()
+
+
 def test_header_is_plain_c(tmp_path):
     # the boundary is a C ABI: the header has to compile as C99 (no C++ in the signatures), and a C caller has to link
     import shutil
