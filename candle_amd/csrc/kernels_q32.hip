@@ -152,6 +152,11 @@ __device__ inline void q32_mac(const Q32Tile<DT>& w, const Q8_0Operand& A, float
 }
 
 __device__ inline float silu_ref32(float v) { return v / (1.0f + expf_glibc(-v)); }
+// the same with the exp table in LDS (32 entries, filled by the caller): a table fetched from memory per element makes
+// a run of these a chain of memory latencies
+__device__ inline float silu_ref32(float v, const uint64_t* lds_tab) {
+    return v / (1.0f + expf_glibc_with(-v, [lds_tab](int i) { return lds_tab[i]; }));
+}
 
 constexpr int Q32_THREADS = 256;
 
@@ -736,7 +741,9 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     constexpr size_t STB = Q32SFmt<DT>::STB;
     __shared__ QGemmLds L;
     __shared__ float hx[MODE == 0 ? QG_NOP * 16 : 1][MODE == 0 ? 65 : 1];   // MODE 0: h of the tile's slots x the workgroup's 64 rows
+    __shared__ uint64_t exp_tab[MODE == 0 ? 32 : 1];
     const int tid = threadIdx.x, lane = tid & 63;
+    if (MODE == 0 && tid < 32) exp_tab[tid] = exp2f_tab(tid);   // published by the barrier ahead of the K loop
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // workgroup -> (row block, slot tile), in patches per XCD (patch_position)
     const int n_rb = MODE == 0 ? p.F / 64 : p.H / (16 * RTW);
@@ -863,25 +870,28 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     // epilogue: lane holds weight row n = lane % 16 and the tile's positions 16 o + 4 i + lane / 16
     const int n = lane & 15;
     if (MODE == 0) {
-        // w3 waves (4-7) park their sums in LDS (the staging buffers are free now), w1 waves combine
-        float* xch = reinterpret_cast<float*>(&L.q[0][0][0][0]);   // [4 waves][QG_NOP][4 i][64 lanes] floats
-        static_assert(4 * QG_NOP * 4 * 64 * 4 <= sizeof(L.q), "exchange area");
-        if (wave >= 4) {
+        // Wave w < 4 holds w1 x of 16 rows, wave w + 4 holds w3 x of the same rows.  Each of the two parks half of its sums
+        // in LDS (the staging buffers are free now) and combines the other half: the w1 wave slot operands 0 and 1, the
+        // w3 wave operands 2 and 3 -- a wave's silu evaluations are a chain of dependent double-precision operations, and
+        // eight waves carry eight of them each instead of four waves sixteen.
+        float* xch = reinterpret_cast<float*>(&L.q[0][0][0][0]);   // [8 waves][2 operands][4 i][64 lanes] floats
+        static_assert(8 * 2 * 4 * 64 * 4 <= sizeof(L.q) && QG_NOP == 4, "exchange area");
 #pragma unroll
-            for (int o = 0; o < QG_NOP; o++)
+        for (int oo = 0; oo < 2; oo++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) xch[(((wave - 4) * QG_NOP + o) * 4 + i) * 64 + lane] = acc[o][i];
-        }
+            for (int i = 0; i < 4; i++) xch[((wave * 2 + oo) * 4 + i) * 64 + lane] = wave < 4 ? acc[2 + oo][i] : acc[oo][i];
         __syncthreads();
-        if (wave < 4) {
+        const int partner = wave ^ 4;
 #pragma unroll
-            for (int o = 0; o < QG_NOP; o++)
+        for (int oo = 0; oo < 2; oo++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float up = xch[((wave * QG_NOP + o) * 4 + i) * 64 + lane];
-                    hx[o * 16 + 4 * i + g][wave * 16 + n] = silu_ref32(acc[o][i]) * up;
-                }
-        }
+            for (int i = 0; i < 4; i++) {
+                const float other = xch[((partner * 2 + oo) * 4 + i) * 64 + lane];
+                const int o = (wave < 4 ? 0 : 2) + oo;
+                // silu(w1 x) * (w3 x): the operand this wave kept, times / under the partner's
+                const float gate_v = wave < 4 ? acc[oo][i] : other, up_v = wave < 4 ? other : acc[2 + oo][i];
+                hx[o * 16 + 4 * i + g][(wave & 3) * 16 + n] = silu_ref32(gate_v, exp_tab) * up_v;
+            }
         __syncthreads();
         // Q8_0 blocks of h (BlockQ8_0::from_float, k_quants.rs:605-634): the workgroup's 64 rows are two blocks per slot;
         // half a wave quantises one (slot, block)

@@ -185,7 +185,9 @@ __host__ __device__ inline uint64_t exp2f_tab(int i) {
     return T[i];
 }
 
-__host__ __device__ inline float expf_glibc(float x) {
+// `tab(i)`: entry i of the table above, from wherever the caller keeps it
+template <class Tab>
+__host__ __device__ inline float expf_glibc_with(float x, Tab tab) {
     if (x != x) return x;
     if (x > 0x1.62e42ep6f) return __builtin_inff();      // overflow
     if (x < -0x1.9fe368p6f) return 0.0f;                 // underflow (also -inf)
@@ -201,7 +203,7 @@ __host__ __device__ inline float expf_glibc(float x) {
     __builtin_memcpy(&ki, &kd, 8);
     kd -= Shift;
     double r = z - kd;
-    uint64_t t = exp2f_tab((int)(ki % 32));
+    uint64_t t = tab((int)(ki % 32));
     t += ki << (52 - 5);
     double s;
     __builtin_memcpy(&s, &t, 8);
@@ -212,6 +214,9 @@ __host__ __device__ inline float expf_glibc(float x) {
     y = __builtin_fma(z, r2, y);
     y = y * s;
     return (float)y;
+}
+__host__ __device__ inline float expf_glibc(float x) {
+    return expf_glibc_with(x, [](int i) { return exp2f_tab(i); });
 }
 
 // Total order of Rust's f32::total_cmp as a sortable signed integer.
