@@ -27,10 +27,12 @@ def hipcc():
     return exe
 
 
-def source_id():
-    """Sixteen hex digits of the SHA-256 over the library's source files (names and contents, in name order): what
-    moe_build_id() of a library built from them returns."""
+def source_id(extra_flags=()):
+    """Sixteen hex digits of the SHA-256 over the library's source files (names and contents, in name order) and any
+    extra compiler flags: what moe_build_id() of a library built from them returns."""
     h = hashlib.sha256()
+    for flag in extra_flags:
+        h.update(flag.encode() + b"\0")
     for name in sorted(os.listdir(CSRC)):
         if name.endswith((".hip", ".hpp", ".cpp", ".h")):
             h.update(name.encode() + b"\0")
@@ -44,7 +46,7 @@ def _compile(src, out_dir=None, extra_flags=()):
     obj = os.path.join(out_dir or OUT_DIR, os.path.splitext(src)[0] + ".o")
     flags = list(extra_flags)
     if src == "api.hip":
-        flags.append('-DMOE_BUILD_ID="%s"' % source_id())
+        flags.append('-DMOE_BUILD_ID="%s"' % source_id(extra_flags))
     cmd = [hipcc()] + HIPCC_FLAGS + flags + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -78,4 +80,10 @@ def build_library(verbose=False, out_dir=None, extra_flags=()):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    import argparse
+    ap = argparse.ArgumentParser(description="Builds libcandle_amd_moe.so; --out-dir / --flag: a second library beside the "
+                                             "product's (measurement variants such as -DMOE_WHATIF=N of kernels_q4k_gemm.hip)")
+    ap.add_argument("--out-dir", default=None)
+    ap.add_argument("--flag", action="append", default=[])
+    a = ap.parse_args()
+    print(build_library(verbose=True, out_dir=a.out_dir, extra_flags=tuple(a.flag)))

@@ -90,6 +90,17 @@ __device__ __forceinline__ void dma4(const void* gbase, uint32_t voff, uint32_t 
 }
 __device__ __forceinline__ void wait_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
 
+// Measurement aid, Q4K only, never set in the product (`python -m candle_amd.build --out-dir DIR --flag=-DMOE_WHATIF=N`
+// builds a second library; its results are WRONG by construction, only its kernel times mean something).  Each bit
+// takes one cost out of the tiled kernel's K loop, to show what the loop's other parts alone would take:
+//   1  the result step: one vector instruction per result keeps the matrix instructions alive, no mins product
+//   2  the unpacking of the weights into two scaled digit planes (the raw bytes go to the matrix cores)
+//   4  the transfers of the next super-block's activations into LDS
+//   8  the LDS reads of the activation operands (one register set for every operand)
+#ifndef MOE_WHATIF
+#define MOE_WHATIF 0
+#endif
+
 // What a lane fetches for the tile.  Quants: the NOP*4 (operand, pair) stretches of 1 KiB are dealt to
 // the eight waves, NOP/2 each: lane (m = l%16, g = l/16) fetches piece (P, g) of row 16 o + m.  Block
 // sums: one transfer covers two operands: lane fetches half (l/16)%2 of row 32 x + 16 (l/32) + l%16.
@@ -163,6 +174,18 @@ struct BPlanes {
 __device__ __forceinline__ BPlanes b_prepare(const BRegs& b, int lane) {
     const int g = lane >> 4;
     const uint32_t M4 = 0x0f0f0f0fu;
+    if (MOE_WHATIF & 2) {   // measurement aid: no unpacking
+        BPlanes o;
+        o.d = __uint_as_float(b.hdr.x); o.dmin = __uint_as_float(b.hdr.y);
+#pragma unroll
+        for (int P = 0; P < 4; P++) {
+            const u32x4 c = b.c[P >> 1];
+            o.lo[P] = v4i{(int)c.x, (int)c.y, (int)c.z, (int)c.w};
+            o.hi[P] = v4i{(int)c.y, (int)c.z, (int)c.w, (int)c.x};
+        }
+        o.mB = v4h{0, 0, 0, 0};
+        return o;
+    }
     const uint32_t u0 = b.hdr.y, u1 = b.hdr.z, u2 = b.hdr.w;
     BPlanes o;
     o.d = __half2float(__ushort_as_half((unsigned short)(b.hdr.x & 0xffffu)));
@@ -342,7 +365,9 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
     __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int P = 0; P < 4; P++) {
-        const v4i a = *reinterpret_cast<const v4i*>(arow + P * 1024);
+        v4i a;
+        if (MOE_WHATIF & 8) a = v4i{lane, lane + 1, lane + 2, lane + 3};   // measurement aid: no LDS read (one register set for all)
+        else a = *reinterpret_cast<const v4i*>(arow + P * 1024);
         acc_lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.lo[P], P == 0 ? zero4 : acc_lo, 0, 0, 0);
         if constexpr (FMT != MOE_GGML_Q2K) acc_hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, B.hi[P], P == 0 ? zero4 : acc_hi, 0, 0, 0);
     }
@@ -356,6 +381,10 @@ __device__ __forceinline__ void gemm_operand(const BPlanes& B, const GemmLds<NOP
             const int isum = (acc_hi[i] << 8) + acc_lo[i];
             facc[i] = __builtin_fmaf(B.d * yd[i], (float)isum, facc[i]);
         }
+    } else if ((MOE_WHATIF & 1) && FMT == MOE_GGML_Q4K) {   // measurement aid: no result step
+        while_busy();
+#pragma unroll
+        for (int i = 0; i < 4; i++) facc[i] = __int_as_float(acc_lo[i] + acc_hi[i] + __float_as_int(facc[i]));
     } else {
         const v4h mA = *reinterpret_cast<const v4h*>(&L.bs[buf][o][g >> 1][m][(g & 1) * 4]);
         const v4f zf = {0.f, 0.f, 0.f, 0.f};
@@ -442,6 +471,7 @@ __global__ __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4)
 
     // transfer t of the wave's share (quant stretches, sums, scales), then the weight tile
     auto stage = [&](auto I, int sb, int buf) {
+        if ((MOE_WHATIF & 4) && sb > 0) return;   // measurement aid: the first super-block's transfers only
         if constexpr (!kSums && decltype(I)::value == NB) return;
         stage_piece<decltype(I)::value, NOP>(ab, rows, nsb, sb, L, buf, wave, lane);
     };
