@@ -23,6 +23,7 @@
 //                    quantised to Q8K in the epilogue (Mlp::forward, quantized_llama.rs:124-131;
 //                    the re-quantisation is what k_quants::matmul does to the lhs of w2).
 //   q4k_down_kernel  yw[slot, :] = (W2 h[slot]) * routing weight (quantized_llama.rs:199-201).
+#include <type_traits>
 #include <cstdlib>
 
 #include "act_quant.hpp"
@@ -599,64 +600,71 @@ __device__ inline void q4k_up_body(const ExpertParams& p, float (*hbuf)[HBUF_STR
     const int tg0 = blockIdx.z * (TT * 16);
     if (tg0 >= gs.n) return;
 
-    int rowA[TT];
+    // A two-tile pass over a list that ends inside its first tile runs the one-tile arithmetic (wave-uniform): the second
+    // tile's matrix instructions and result steps are a fifth of the vector work of such a workgroup.
+    auto run = [&](auto ttl_tag) {
+        constexpr int TTL = decltype(ttl_tag)::value;   // live slot tiles of this pass
+        int rowA[TTL];
 #pragma unroll
-    for (int tt = 0; tt < TT; tt++) {
-        int i = tg0 + tt * 16 + r;
-        rowA[tt] = slot_token(p, gs.slot(i < gs.n ? i : gs.n - 1));
-    }
-    float acc[NT][TT][4];
+        for (int tt = 0; tt < TTL; tt++) {
+            int i = tg0 + tt * 16 + r;
+            rowA[tt] = slot_token(p, gs.slot(i < gs.n ? i : gs.n - 1));
+        }
+        float acc[NT][TTL][4];
 #pragma unroll
-    for (int j = 0; j < NT; j++)
+        for (int j = 0; j < NT; j++)
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++)
+            for (int tt = 0; tt < TTL; tt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
+                for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
 
-    q4k_engine<FMT, TT, NT, RING>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
+        q4k_engine<FMT, TTL, NT, RING>(tp, sb_stride, ring, p.xq, H, nsb, 0, nsb, rowA, lane, g, acc);
 
-    if (UP_ROWS != 256) {   // h = silu(w1 x) * (w3 x) straight to memory
+        if (UP_ROWS != 256) {   // h = silu(w1 x) * (w3 x) straight to memory
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++)
+            for (int tt = 0; tt < TTL; tt++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int pos = tg0 + tt * 16 + 4 * g + i;
-                if (pos >= gs.n) continue;
-                const int64_t hrow = gs.slot(pos) - p.slot_origin;
+                for (int i = 0; i < 4; i++) {
+                    const int pos = tg0 + tt * 16 + 4 * g + i;
+                    if (pos >= gs.n) continue;
+                    const int64_t hrow = gs.slot(pos) - p.slot_origin;
 #pragma unroll
-                for (int j = 0; j < RTW; j++)
-                    p.hbuf[hrow * F + rb * UP_ROWS + (wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
-            }
-        return;
-    }
-    // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
+                    for (int j = 0; j < RTW; j++)
+                        p.hbuf[hrow * F + rb * UP_ROWS + (wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
+                }
+            return;
+        }
+        // epilogue: h = silu(w1 x) * (w3 x), then Q8K-quantise the 256-row block of every slot
 #pragma unroll
-    for (int tt = 0; tt < TT; tt++)
+        for (int tt = 0; tt < TTL; tt++)
 #pragma unroll
-        for (int j = 0; j < RTW; j++)
+            for (int j = 0; j < RTW; j++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
-    __syncthreads();
-    const int nfb = F / 256;
-    // every wave quantises its TT*16/NW tokens side by side
-    constexpr int NQ = TT * 16 / NW;
-    float4 v[NQ];
-    bool valid[NQ];
-    int8_t* qs_out[NQ];
-    float* d_out[NQ];
-    __half* bs_out[NQ];
+                for (int i = 0; i < 4; i++)
+                    hbuf[tt * 16 + 4 * g + i][(wave * RTW + j) * 16 + r] = silu_fast(acc[j][tt][i]) * acc[RTW + j][tt][i];
+        __syncthreads();
+        const int nfb = F / 256;
+        // every wave quantises its TTL*16/NW tokens side by side
+        constexpr int NQ = TTL * 16 / NW;
+        float4 v[NQ];
+        bool valid[NQ];
+        int8_t* qs_out[NQ];
+        float* d_out[NQ];
+        __half* bs_out[NQ];
 #pragma unroll
-    for (int n = 0; n < NQ; n++) {
-        const int tok = wave + n * NW;
-        valid[n] = tg0 + tok < gs.n;
-        v[n] = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
-        const int64_t hrow = gs.slot(valid[n] ? tg0 + tok : gs.n - 1) - p.slot_origin;
-        qs_out[n] = p.hq.qs + hrow * F + rb * 256;
-        d_out[n] = p.hq.d + hrow * nfb + rb;
-        bs_out[n] = reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16;
-    }
-    quantize_q8k_blocks<NQ>(v, valid, lane, qs_out, d_out, bs_out);
+        for (int n = 0; n < NQ; n++) {
+            const int tok = wave + n * NW;
+            valid[n] = tg0 + tok < gs.n;
+            v[n] = *reinterpret_cast<const float4*>(&hbuf[tok][lane * 4]);
+            const int64_t hrow = gs.slot(valid[n] ? tg0 + tok : gs.n - 1) - p.slot_origin;
+            qs_out[n] = p.hq.qs + hrow * F + rb * 256;
+            d_out[n] = p.hq.d + hrow * nfb + rb;
+            bs_out[n] = reinterpret_cast<__half*>(p.hq.bsum) + (hrow * nfb + rb) * 16;
+        }
+        quantize_q8k_blocks<NQ>(v, valid, lane, qs_out, d_out, bs_out);
+    };
+    if (TT == 2 && gs.n - tg0 <= 16) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, TT>{});
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -703,46 +711,52 @@ __device__ inline void q4k_down_body(const ExpertParams& p, float (*part)[NTD * 
     const int tg0 = blockIdx.z * (TT * 16);
     if (tg0 >= gs.n) return;
 
-    int rowA[TT];
+    // (a two-tile pass over a list that ends inside its first tile: the one-tile arithmetic, as in the up kernel)
+    auto run = [&](auto ttl_tag) {
+        constexpr int TTL = decltype(ttl_tag)::value;
+        int rowA[TTL];
 #pragma unroll
-    for (int tt = 0; tt < TT; tt++) {
-        int i = tg0 + tt * 16 + r;
-        rowA[tt] = gs.slot(i < gs.n ? i : gs.n - 1) - p.slot_origin;
-    }
-    float acc[NTD][TT][4];
-#pragma unroll
-    for (int j = 0; j < NTD; j++)
-#pragma unroll
-        for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
-
-    q4k_engine<FMT, TT, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc, a_step, a_off);
-
-#pragma unroll
-    for (int j = 0; j < NTD; j++)
-#pragma unroll
-        for (int tt = 0; tt < TT; tt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) part[wave][(j * TT + tt) * 4 + i][lane] = acc[j][tt][i];
-    __syncthreads();
-    // NTD*TT*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ... (a fixed trip count, so that the routing
-    // weights of all its planes are fetched together rather than one per trip)
-    constexpr int NPL = NTD * TT * 4;
-#pragma unroll
-    for (int n = 0; n < (NPL + NW - 1) / NW; n++) {
-        const int v = wave + n * NW;
-        if (NPL % NW != 0 && v >= NPL) break;
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; w++) sum += part[w][v][lane];
-        const int j = v / (TT * 4), tt = (v / 4) % TT, i = v % 4;
-        const int pos = tg0 + tt * 16 + 4 * g + i;
-        if (pos < gs.n && rt0 + j < n_rt) {
-            const int slot = gs.slot(pos);
-            emit_expert_output(p, slot, (rt0 + j) * 16 + r, sum * slot_weight(p, slot));
+        for (int tt = 0; tt < TTL; tt++) {
+            int i = tg0 + tt * 16 + r;
+            rowA[tt] = gs.slot(i < gs.n ? i : gs.n - 1) - p.slot_origin;
         }
-    }
+        float acc[NTD][TTL][4];
+#pragma unroll
+        for (int j = 0; j < NTD; j++)
+#pragma unroll
+            for (int tt = 0; tt < TTL; tt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[j][tt][i] = 0.f;
+
+        q4k_engine<FMT, TTL, NTD, RING>(tp, sb_stride, ring, p.hq, F, nsb, sb_lo, sb_hi, rowA, lane, g, acc, a_step, a_off);
+
+#pragma unroll
+        for (int j = 0; j < NTD; j++)
+#pragma unroll
+            for (int tt = 0; tt < TTL; tt++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) part[wave][(j * TTL + tt) * 4 + i][lane] = acc[j][tt][i];
+        __syncthreads();
+        // NTD*TTL*4 value planes of 64 lanes; wave w reduces planes w, w+NW, ... (a fixed trip count, so that the routing
+        // weights of all its planes are fetched together rather than one per trip)
+        constexpr int NPL = NTD * TTL * 4;
+#pragma unroll
+        for (int n = 0; n < (NPL + NW - 1) / NW; n++) {
+            const int v = wave + n * NW;
+            if (NPL % NW != 0 && v >= NPL) break;
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) sum += part[w][v][lane];
+            const int j = v / (TTL * 4), tt = (v / 4) % TTL, i = v % 4;
+            const int pos = tg0 + tt * 16 + 4 * g + i;
+            if (pos < gs.n && rt0 + j < n_rt) {
+                const int slot = gs.slot(pos);
+                emit_expert_output(p, slot, (rt0 + j) * 16 + r, sum * slot_weight(p, slot));
+            }
+        }
+    };
+    if (TT == 2 && gs.n - tg0 <= 16) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, TT>{});
 }
 
 #define DEF_UP_NARROW(NAME, FMT, NW, RING, WPE)                                                               \
