@@ -377,7 +377,11 @@ def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32
         noise.normal_(0.0, 0.1, generator=g)
         state["h"] = torch.add(h, noise, out=x_next)
 
-    lbl_ms, _, _ = timer.run(step_layer_by_layer, 32, 2, min_warm_seconds=0.2)
+    # the same stack as 32 calls of moe_layer_forward_device, for comparison (--stack-entry-only leaves it out, so that a
+    # kernel trace of the run holds the one-call path's launches only)
+    lbl_ms = None
+    if not args.stack_entry_only:
+        lbl_ms, _, _ = timer.run(step_layer_by_layer, 32, 2, min_warm_seconds=0.2)
     state["h"] = x0
     ms, wall_ms, warmed = timer.run(step, n_steps, min(args.warmup, 3), min_warm_seconds=0.3)
     finite = bool(torch.isfinite(state["h"]).all())
@@ -385,7 +389,7 @@ def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32
     mid = len(layers) // 2
     stage = {k: 0.0 for k in layers[mid].STAGES}
     with torch.cuda.stream(timer.stream):
-        for _ in range(5):
+        for _ in range(0 if args.stack_entry_only else 5):
             hh = x0
             for i, layer in enumerate(layers[:mid]):
                 layer.forward(hh, out=bufs[i & 1])
@@ -396,7 +400,7 @@ def measure_stack(args, np, torch, candle_amd, timer, w, n_layers, n_steps, B=32
     n_active = E   # a 32-token batch reaches every expert (64 assignments over 8 experts)
     act = 36 / 256
     up_bytes = n_active * (2 * H * F * 144 // 256) + int(B * H * (1 + act)) + int(B * TOPK * F * (1 + act))
-    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9
+    achieved = up_bytes / (stage["up"] * 1e-3) / 1e9 if stage["up"] else 0.0
     step_bytes = len(layers) * (n_active * EXPERT_BYTES + E * H * 4 + 3 * B * H * 4)
     for layer in layers:
         layer.close()
@@ -430,6 +434,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--stage-iters", type=int, default=50)
+    ap.add_argument("--stack-entry-only", action="store_true",
+                    help="stack workload: skip the layer-by-layer comparison run and the per-stage timing of layer 16")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 1 GiB device copy (the known-size kernel that scales rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings) and exit")
