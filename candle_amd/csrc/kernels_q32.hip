@@ -697,7 +697,7 @@ static hipError_t launch_q32_down_t(const ExpertParams& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Tiled grouped products for Q8_0 weights, and for Q4_0 / Q5_0 (batches whose slots are grouped by expert): one pass over an expert's
+// Tiled grouped products for Q8_0 weights, and for Q4_0 / Q5_0 / Q4_1 / Q5_1 (batches whose slots are grouped by expert): one pass over an expert's
 // weights for up to 64 of its slots, where the streaming kernels above take a pass per 32.
 //
 // Same arithmetic and the same order of additions as q32s_mac (bit-identical results): one
@@ -734,10 +734,12 @@ __device__ __forceinline__ void qg_dma16(const void* gbase, uint32_t voff, uint3
 // tiles at 512 tokens of 2048 -- becomes twice (four times) as many workgroups, each of half (a quarter of) the length.
 template <int DT, int MODE, int WOPS = QG_NOP>
 __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void q8_0_gemm_kernel(ExpertParams p) {
-    static_assert(DT == MOE_GGML_Q8_0 || DT == MOE_GGML_Q4_0 || DT == MOE_GGML_Q5_0, "formats with Q8_0 activations and no minimum");
+    static_assert(DT == MOE_GGML_Q8_0 || DT == MOE_GGML_Q4_0 || DT == MOE_GGML_Q5_0 || DT == MOE_GGML_Q4_1 || DT == MOE_GGML_Q5_1, "the 32-element formats");
     static_assert(MODE == 1 || WOPS == QG_NOP, "the up projection pairs w1 and w3 waves");
     constexpr int RTW = 8 * WOPS / QG_NOP;   // MODE 1: weight operands (16 rows) per workgroup
     constexpr int OFFSET = Q32Fmt<DT>::OFFSET;
+    constexpr bool HAS_M = Q32Fmt<DT>::HAS_M;    // Q4_1 / Q5_1: the block minimum times the activation block's s (Q8_1 rows)
+    constexpr bool WORDS = OFFSET != 0 || HAS_M;   // the activation blocks' words (sum of quants, or s) are staged too
     constexpr size_t STB = Q32SFmt<DT>::STB;
     __shared__ QGemmLds L;
     __shared__ float hx[MODE == 0 ? QG_NOP * 16 : 1][MODE == 0 ? 65 : 1];   // MODE 0: h of the tile's slots x the workgroup's 64 rows
@@ -784,7 +786,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     auto stage = [&](int ks, int buf) {
         qg_dma16(ab.qs, q_src + (uint32_t)(ks * 128), qg_lds_address(&L.q[buf][wave >> 1][4 * (wave & 1)][0]));
         if (wave == 0) qg_dma16(ab.d, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.yd[buf][0][0]));
-        if (OFFSET && wave == 1) qg_dma16(ab.bsum, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.bs[buf][0][0]));
+        if (WORDS && wave == 1) qg_dma16(ab.bsum, d_src + (uint32_t)(ks * 16), qg_lds_address(&L.bs[buf][0][0]));
     };
 
     const GroupWeights gw = p.groups[grp];
@@ -821,6 +823,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
         nxt = load_q32s<DT, false>(wp + (size_t)ks2 * step_stride, lane);
         const Q32Tile<DT> w0 = q32s_block<DT, 0>(w, g), w1 = q32s_block<DT, 1>(w, g), w2 = q32s_block<DT, 2>(w, g), w3 = q32s_block<DT, 3>(w, g);
         const float dwv[4] = {w0.d, w1.d, w2.d, w3.d};
+        const float wm[4] = {w0.m, w1.m, w2.m, w3.m};
         const uint2 wq[4] = {w0.q, w1.q, w2.q, w3.q};
         float cneg[4];
 #pragma unroll
@@ -832,6 +835,11 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                 f32x4g ydv[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) ydv[i] = *reinterpret_cast<const f32x4g*>(&L.yd[buf][o * 16 + 4 * g + i][0]);
+                f32x4g ysv[4];   // the activation blocks' s
+                if (HAS_M) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) ysv[i] = *reinterpret_cast<const f32x4g*>(&L.bs[buf][o * 16 + 4 * g + i][0]);
+                }
                 v4i D[4];
                 __builtin_amdgcn_s_setprio(2);   // issue priority while the matrix instructions go out (as in q4k_gemm_kernel)
 #pragma unroll
@@ -858,6 +866,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                         for (int b = 0; b < 4; b++) {
                             float t = __builtin_fmaf(__int_as_float(D[b][i]), dwv[b], cneg[b]);
                             t = t * ydv[i][b];
+                            if (HAS_M) t = t + wm[b] * ysv[i][b];   // (isum d_w) d_x + m_w s_x, then the sum (k_quants.rs:294-295)
                             acc[ow][i] += t;
                         }
                     }
@@ -916,7 +925,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
                 if (e == 0) {
                     const float dh = __half2float(__float2half_rn(d));
                     p.hq.d[hrow * nfb + rblk * 2 + blk] = dh;
-                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + rblk * 2 + blk] = q8_block_word(MOE_GGML_Q8_0, sum, dh);
+                    reinterpret_cast<int32_t*>(p.hq.bsum)[hrow * nfb + rblk * 2 + blk] = q8_block_word(vecdot_dtype(DT), sum, dh);
                 }
             }
         }
@@ -933,7 +942,7 @@ __global__ __launch_bounds__(QG_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
     }
 }
 
-static bool qg_format(int dt) { return dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q5_0; }
+static bool qg_format(int dt) { return dt == MOE_GGML_Q8_0 || dt == MOE_GGML_Q4_0 || dt == MOE_GGML_Q5_0 || dt == MOE_GGML_Q4_1 || dt == MOE_GGML_Q5_1; }
 bool q8_0_gemm_usable(int dt, int dt_down, int64_t H, int64_t F) {
     return qg_format(dt) && (dt_down == 0 || qg_format(dt_down)) && H % 128 == 0 && F % 128 == 0;
 }
@@ -946,6 +955,8 @@ static hipError_t qg_launch(int dt, const ExpertParams& p, dim3 grid, hipStream_
         case MOE_GGML_Q8_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q8_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
         case MOE_GGML_Q4_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q4_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
         case MOE_GGML_Q5_0: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q5_0, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q4_1: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q4_1, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
+        case MOE_GGML_Q5_1: hipLaunchKernelGGL((q8_0_gemm_kernel<MOE_GGML_Q5_1, MODE, WOPS>), grid, dim3(QG_THREADS), 0, s, p); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

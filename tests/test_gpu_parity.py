@@ -432,9 +432,10 @@ def test_block_32_element_formats_ragged_row_tiles(dt):
         assert np.array_equal(bits(candle_amd.qmatmul(dt, w, n, k, x)), bits(O.matmul(dt, x, w, n)))
 
 
-@pytest.mark.parametrize("dt,dt_down", [(O.Q4_0, None), (O.Q5_0, None), (O.Q8_0, None), (O.Q4_0, O.Q8_0), (O.Q5_0, O.Q4_0)])
+@pytest.mark.parametrize("dt,dt_down", [(O.Q4_0, None), (O.Q5_0, None), (O.Q8_0, None), (O.Q4_0, O.Q8_0), (O.Q5_0, O.Q4_0),
+                                        (O.Q4_1, None), (O.Q5_1, None), (O.Q5_1, O.Q4_1)])
 def test_block_32_element_formats_tiled_kernels(dt, dt_down):
-    # beyond 1024 assignments the slots are grouped by expert and the Q8_0-activation formats take the tiled kernels
+    # beyond 1024 assignments the slots are grouped by expert and the 32-element formats take the tiled kernels
     # (64-slot tiles): lists of ~300 and ~650 rows, a last tile of every length, and a shared expert beside them
     ref, gpu = make_pair(256, 384, 4, 2, dt, seed=50, dt_down=dt_down)
     for T in (600, 1301):

@@ -44,6 +44,19 @@ def test_resident_projection_over_batch_sizes(dt, n, k):
         lin.forward(activations(1, k, seed=1))
 
 
+@pytest.mark.parametrize("dt", [O.Q8_0, O.Q4_0, O.Q5_0, O.Q4_1, O.Q5_1])
+def test_dense_product_on_the_tiled_kernel_of_the_32_element_formats(dt):
+    # 1024 x 256: eight row blocks of 128; from 2048 rows on the grid holds a workgroup per CU and the product takes the
+    # tiled kernel (64-row tiles, the last one ragged), bit for bit what the reference's loop adds up
+    n, k = 1024, 256
+    w = O.fill_normal_quantized(7 + dt, dt, n, k, 0.02)
+    lin = candle_amd.QMatMul(dt, w, n, k)
+    for m in (2100, 2049, 130):
+        x = activations(m, k, seed=m + dt)
+        assert np.array_equal(bits(lin.forward(x)), bits(O.matmul(dt, x, w, n))), m
+    lin.close()
+
+
 def test_device_entry_equals_host_entry_and_keeps_leading_dims():
     torch = pytest.importorskip("torch")
     dt, n, k = O.Q4K, 384, 768
