@@ -757,9 +757,9 @@ static int forward_pass(moe_layer* L, const float* d_x, int64_t T, float* d_y, h
     // a previous call may still be running on another stream and shares the workspace
     if (!capturing)
         if (int rc = L->order.enter(s)) return rc;
-    if (int rc = enqueue_forward(L, pl, ws, d_x, T, d_y, s, marks)) return rc;
-    if (!capturing) L->order.leave(s);
-    return MOE_OK;
+    const int rc = enqueue_forward(L, pl, ws, d_x, T, d_y, s, marks);
+    if (!capturing) L->order.leave(s);   // also after a failure: what was enqueued before it is pending work on s
+    return rc;
 }
 
 extern "C" int moe_layer_forward_device(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream) {
@@ -821,6 +821,16 @@ extern "C" int moe_stack_forward_device(moe_layer* const* layers, int64_t n_laye
     for (int64_t l = 0; l < n_layers; l++) plans[(size_t)l] = plan_forward(layers[l], T);
     for (int64_t l = 1; l < n_layers; l++) fused_in[(size_t)l] = stack_boundary_fuses(layers[l - 1], plans[(size_t)l - 1], layers[l], T) ? 1 : 0;
     std::vector<Workspace> wss((size_t)n_layers);
+    // Whatever was enqueued for a layer counts as its pending work on this stream, also when a later step of the call
+    // fails: a following call from another stream then still waits for it.
+    struct Entered {
+        moe_layer* const* layers;
+        hipStream_t s;
+        int64_t n = 0;
+        ~Entered() {
+            for (int64_t l = 0; l < n; l++) layers[l]->order.leave(s);
+        }
+    } entered{layers, s};
     for (int64_t l = 0; l < n_layers; l++) {
         moe_layer* L = layers[l];
         // the layer's input row lives in its own workspace when the layer before writes it (fused) and, otherwise, in
@@ -835,8 +845,10 @@ extern "C" int moe_stack_forward_device(moe_layer* const* layers, int64_t n_laye
         if (L->k > 0) carve_workspace(L, T, plans[(size_t)l], static_cast<uint8_t*>(L->ws.p), &wss[(size_t)l], l > 0);
         else if (l > 0) wss[(size_t)l].xin = reinterpret_cast<float*>(L->ws.p);
         if (capturing) L->ws.captured = true;
-        if (!capturing)
+        if (!capturing) {
             if (int rc = L->order.enter(s)) return rc;
+            entered.n = l + 1;
+        }
     }
     // Layer l reads its input from d_x (l = 0) or from its own xin, which either the layer before wrote (its combine pass)
     // or this layer's front kernel writes (the combine pass folded in); its output goes to the next layer's xin, or to d_y.
@@ -858,9 +870,7 @@ extern "C" int moe_stack_forward_device(moe_layer* const* layers, int64_t n_laye
         if (int rc = enqueue_forward(L, plans[(size_t)l], wss[(size_t)l], in, T, out, s, nullptr, fused_in[(size_t)l] ? &prev : nullptr, leave)) return rc;
         in_prev = in;
     }
-    if (!capturing)
-        for (int64_t l = 0; l < n_layers; l++) layers[l]->order.leave(s);
-    return MOE_OK;
+    return MOE_OK;   // `entered` marks the layers' work as pending on s
 }
 
 // ------------------------------------------------------------------ the entry point that allocates nothing
@@ -915,10 +925,11 @@ extern "C" int moe_layer_forward_device_noalloc(moe_layer* L, const void* d_x, i
     const bool capturing = cap != hipStreamCaptureStatusNone;
     if (!capturing)
         if (int rc = L->order.enter(s)) return rc;
-    if (int rc = enqueue_forward(L, pl, ws, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s)) return rc;
-    // the hooks that read the last call's logits and routing wait for this stream
+    const int rc = enqueue_forward(L, pl, ws, static_cast<const float*>(d_x), T, static_cast<float*>(d_y), s);
+    // the hooks that read the last call's logits and routing wait for this stream (after a failure too: what was
+    // enqueued before it is pending work on s)
     if (!capturing) L->order.leave(s);
-    return MOE_OK;
+    return rc;
 }
 
 extern "C" int moe_layer_forward_timed(moe_layer* L, const void* d_x, int64_t T, void* d_y, void* hip_stream, float* stage_ms) {

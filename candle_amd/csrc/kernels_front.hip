@@ -114,8 +114,9 @@ constexpr int DISPATCH_THREADS = 1024;
 struct DispatchShared {
     int cnt[DISPATCH_THREADS / 64][MAX_E];
     int off[MAX_E + 2];
-    int tot[MAX_E];
+    int tot[MAX_E];      // per expert: its assignments over all workgroups; after the scan: the tiles of the experts before it
     int before[MAX_E];
+    int n_tiles;         // tiles of the E routed experts
 };
 
 // Mask of the valid lanes whose expert index equals this lane's: one ballot per bit of the index, whatever the number
@@ -196,6 +197,21 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
         sh.off[4 * lane + 2] = base + t0 + t1;
         sh.off[4 * lane + 3] = base + t0 + t1 + t2;
         if (lane == 63) sh.off[MAX_E] = incl;   // = A
+        // the same scan over the experts' tile counts (work list of the tiled kernels; the tile size is a power of two)
+        const int tsh = 31 - __clz(rb.tile_slots > 0 ? rb.tile_slots : 1), tm = (1 << tsh) - 1;
+        const int l0 = (t0 + tm) >> tsh, l1 = (t1 + tm) >> tsh, l2 = (t2 + tm) >> tsh, l3 = (t3 + tm) >> tsh;
+        int tincl = l0 + l1 + l2 + l3;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(tincl, o, 64);
+            if (lane >= o) tincl += v;
+        }
+        const int tbase = tincl - (l0 + l1 + l2 + l3);
+        sh.tot[4 * lane] = tbase;
+        sh.tot[4 * lane + 1] = tbase + l0;
+        sh.tot[4 * lane + 2] = tbase + l0 + l1;
+        sh.tot[4 * lane + 3] = tbase + l0 + l1 + l2;
+        if (lane == 63) sh.n_tiles = tincl;
     }
     __syncthreads();
     if (tid == 0) {   // experts past E have no assignments: off[E] == A already; the shared expert follows
@@ -213,18 +229,17 @@ __device__ void dispatch_block(const RouteBufs& rb, int64_t T, int E, int k, boo
     __syncthreads();
     if (g == 0) {
         for (int e = tid; e <= E + (shared ? 1 : 0); e += DISPATCH_THREADS) rb.offsets[e] = sh.off[e];
-        if (tid == 0 && rb.tile_tab) {  // work list of the tiled expert kernels
-            int n = 0;
-            const int NG = E + (shared ? 1 : 0);
-            for (int gi = 0; gi < NG; gi++) {
+        if (rb.tile_tab) {  // work list of the tiled expert kernels: a group's tiles follow those of the groups before it
+            const int NG = E + (shared ? 1 : 0), ts = rb.tile_slots;
+            for (int gi = tid; gi < NG; gi += DISPATCH_THREADS) {
+                int n = gi < E ? sh.tot[gi] : sh.n_tiles;
                 const int len = sh.off[gi + 1] - sh.off[gi];
-                for (int pos = 0; pos < len; pos += rb.tile_slots) {
+                for (int pos = 0; pos < len; pos += ts, n++) {
                     rb.tile_tab[1 + 2 * n] = gi;
                     rb.tile_tab[2 + 2 * n] = pos;
-                    n++;
                 }
+                if (gi == NG - 1) rb.tile_tab[0] = n;
             }
-            rb.tile_tab[0] = n;
         }
     }
     // phase 3: stable placement; the token's row of tok_slots lists its slots by ascending expert index (the order
